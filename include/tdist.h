@@ -1,0 +1,248 @@
+/*
+ * tdist.h — C ABI of libtdist_hip.so: hand-written gfx950 (MI355X) kernels for the per-GPU compute
+ * half of Triton-distributed's overlapped ops.
+ *
+ * Conventions
+ *   - every entry point is extern "C", returns 0 (TDIST_OK) or a negative tdist_status, never aborts;
+ *     tdist_last_error_string() gives the text of the calling thread's last failure;
+ *   - pointers are DEVICE pointers unless the parameter name ends in _host;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the legacy default stream);
+ *   - no entry point allocates or frees memory; scratch comes from the caller (see *_workspace_bytes);
+ *   - leading dimensions (lda, ldb, ...) are in ELEMENTS, sizes in elements unless named *_bytes;
+ *   - launches are asynchronous on `stream`; a non-zero return means nothing was launched.
+ *
+ * Each declaration cites the reference interface (file:line under python/triton_dist of
+ * Triton-distributed) whose device work it replaces.
+ */
+#ifndef TDIST_H_
+#define TDIST_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum tdist_status {
+  TDIST_OK = 0,
+  TDIST_ERR_INVALID = -1,     /* bad argument (null pointer, misaligned, non-positive size) */
+  TDIST_ERR_UNSUPPORTED = -2, /* shape / dtype outside what the kernels implement */
+  TDIST_ERR_LAUNCH = -3,      /* HIP reported an error at launch */
+  TDIST_ERR_TIMEOUT = -4,     /* a bounded flag wait expired (reported through a status word) */
+  TDIST_ERR_WORKSPACE = -5,   /* caller's scratch buffer is too small */
+  TDIST_ERR_DEVICE = -6       /* not a gfx950 device / no device */
+} tdist_status;
+
+typedef enum tdist_dtype {
+  TDIST_BF16 = 0,
+  TDIST_F16 = 1,
+  TDIST_F8E4M3 = 2, /* OCP e4m3fn, the gfx950 hardware format */
+  TDIST_F32 = 3
+} tdist_dtype;
+
+/* ---------------------------------------------------------------------------------------------
+ * Library
+ * ------------------------------------------------------------------------------------------- */
+int tdist_version(void);
+const char* tdist_last_error_string(void);
+/* Caches properties of the current device (CU count, XCD count). Optional: every entry point calls
+ * it lazily. Returns TDIST_ERR_DEVICE when the current device is not gfx950. */
+int tdist_init(void);
+int tdist_num_cus(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * (a) chunk-gated tile GEMM — the AG-GEMM consumer.
+ *   replaces kernel_consumer_gemm_persistent      kernels/amd/all_gather_gemm.py:140-254
+ *            wait_eq_sys                          kernels/amd/common_ops.py:39-46
+ *
+ * C[M,N] = A[M,K] * B[N,K]^T, fp32 accumulate, output bf16 (or f16 for f16 inputs).
+ *   A     gathered workspace, row-major, lda elements between rows (K contiguous)
+ *   A_local / local_row_begin / local_rows
+ *         rows [local_row_begin, local_row_begin+local_rows) are the caller's own shard: they are read
+ *         from A_local (row 0 of A_local = row local_row_begin) and are never gated
+ *         (all_gather_gemm.py:201-218). Pass A_local = NULL, local_rows = 0 to gate every row.
+ *   B     [N,K] row-major (K contiguous), the reference's non-transposed weight layout (:308-309)
+ *   flags int32[ceil(M/m_per_chunk)]: rows of chunk c may be read only once flags[c] == wait_value
+ *         (acquire, system scope). flags = NULL disables gating (plain GEMM).
+ *   chunk_order  device int32[n_chunks] permutation giving the order in which chunks are consumed,
+ *         or NULL for the reference's order (own rank's chunks first, then rank+1, ... :193-199,
+ *         which needs rank / world_size).
+ *   spin_limit   > 0: polls per wait before giving up; <= 0: library default (seconds of polling).
+ *         On expiry the tile is skipped (its C rows are left untouched) and status[0] is set to
+ *         TDIST_ERR_TIMEOUT, status[1] to the chunk index. status may be NULL.
+ * Requirements: K % 64 == 0 (bf16/f16) or K % 128 == 0 (fp8), lda/ldb multiples of 8 (16 for fp8)
+ * elements, 16-byte aligned bases, m_per_chunk % 256 == 0 when flags != NULL.
+ * ------------------------------------------------------------------------------------------- */
+int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
+                                int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
+                                int64_t ldc, int M, int N, int K, const int32_t* flags, int m_per_chunk,
+                                int wait_value, const int32_t* chunk_order, int rank, int world_size,
+                                int spin_limit, int32_t* status, void* stream);
+
+int tdist_gemm_chunk_gated_f16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
+                               int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
+                               int64_t ldc, int M, int N, int K, const int32_t* flags, int m_per_chunk,
+                               int wait_value, const int32_t* chunk_order, int rank, int world_size,
+                               int spin_limit, int32_t* status, void* stream);
+
+/* fp8-e4m3 inputs, bf16 output, C = (sum_k A8*B8) * row_scale[m] * col_scale[n].
+ * The scale epilogue has no counterpart in the reference (fp8 is a dtype passthrough there,
+ * kernels/nvidia/allgather_gemm.py:313); row_scale / col_scale may be NULL (= 1.0). */
+int tdist_gemm_chunk_gated_fp8e4m3(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
+                                   int local_row_begin, int local_rows, const void* B, int64_t ldb,
+                                   void* C, int64_t ldc, int M, int N, int K, const float* row_scale,
+                                   const float* col_scale, const int32_t* flags, int m_per_chunk,
+                                   int wait_value, const int32_t* chunk_order, int rank, int world_size,
+                                   int spin_limit, int32_t* status, void* stream);
+
+/* Producer side of the gate on the same GPU: copy one chunk, then release its flag, both ordered on
+ * `stream`.   replaces cp_engine_producer_all_gather_full_mesh_push_multi_stream
+ *             kernels/amd/all_gather_gemm.py:41-100 (data copy + 4-byte flag copy per chunk).
+ * `one` is a device int32 holding the value to publish (the reference copies from a tensor of ones
+ * because a stream write-value disturbs the GEMM, :88-100). use_sdma != 0 requests the copy-engine
+ * path (hipMemcpyDeviceToDeviceNoCU) so the copy takes no compute unit. */
+int tdist_producer_push_chunk(void* dst, const void* src, int64_t nbytes, int32_t* flag, const int32_t* one,
+                              int use_sdma, void* stream);
+
+/* Stream-ordered store of `value` into *flag by a one-thread kernel (release, system scope).
+ *   replaces set_signal  kernels/amd/common_ops.py:97-112 */
+int tdist_flag_set(int32_t* flag, int value, void* stream);
+/* Stream-ordered fill of n int32 flags (the reference resets with barrier_ptr.fill_(0),
+ * kernels/amd/all_gather_gemm.py:460-461). Safe to record into a HIP graph. */
+int tdist_flag_fill(int32_t* flags, int n, int value, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (b) GEMM-RS: GEMM whose epilogue scatters each row block to its owner's buffer, then the
+ *     reduction of the per-rank slices.
+ *   replaces kernel_gemm_rs_producer_fuse_scatter  kernels/amd/gemm_reduce_scatter.py:125-229
+ *            kernel_consumer_reduce                kernels/amd/gemm_reduce_scatter.py:232-258
+ * ------------------------------------------------------------------------------------------- */
+/* P = A[M,K] * B[N,K]^T (fp32 accumulate) rounded to the input dtype; the rows of P that belong to
+ * rank o (rows [o*M/world, (o+1)*M/world)) are stored into scatter_bufs[o] at rows
+ * [rank*M/world, (rank+1)*M/world) (gemm_reduce_scatter.py:222-229), every buffer [M, ldc].
+ * scatter_bufs is a DEVICE array of world_size device pointers (the reference's scatter_bufs_ptr).
+ * Tiles are visited starting with the rows of rank+1 (:171-180).
+ * Requirements: M % (256*world_size) == 0, K % 64 == 0. */
+int tdist_gemm_rs_scatter_bf16(const void* A, int64_t lda, const void* B, int64_t ldb,
+                               void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank,
+                               int world_size, void* stream);
+int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t ldb,
+                              void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank,
+                              int world_size, void* stream);
+
+/* out[e] = round( sum_{i=0..n_slices-1} float(c[((i + first_slice) % n_slices) * slice_stride + e]) )
+ * for e in [0, n_elems): fp32 accumulation in exactly that order (the reference's order is
+ * first_slice = rank+1, gemm_reduce_scatter.py:252-256; it accumulates in the output dtype, this
+ * kernel in fp32). dtype: TDIST_BF16 or TDIST_F16 for both c and out. */
+int tdist_reduce_slices(const void* c, int64_t slice_stride, int n_slices, int first_slice, int64_t n_elems,
+                        void* out, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (c) MoE low-latency dispatch / combine permute.
+ *   replaces the test-side preprocessing  test/nvidia/test_all_to_all.py:42-96,314-329
+ *            all_to_all_kernel            kernels/nvidia/low_latency_all_to_all.py:35-118
+ *            all_to_all_post_process      kernels/nvidia/low_latency_all_to_all.py:251-270
+ *            combine + index_add_         test/nvidia/test_all_to_all.py:360-370
+ *            weighted top-k reduce        test/nvidia/test_moe_reduce_rs.py:103-129
+ * ------------------------------------------------------------------------------------------- */
+/* Scratch bytes needed by tdist_moe_scatter_index / tdist_moe_splits_cumsum for n_ids ids. */
+int64_t tdist_moe_workspace_bytes(int64_t n_ids, int num_experts);
+
+/* splits[g] = #{i : ids[i] == g} (torch.bincount(..., minlength=G), test_all_to_all.py:314);
+ * cumsum[0] = 0, cumsum[g+1] = splits[0] + ... + splits[g] (splits_to_cumsum, :42-46).
+ * ids int32[n_ids] with values in [0, G); splits int32[G]; cumsum int32[G+1]. */
+int tdist_moe_splits_cumsum(const int32_t* ids, int64_t n_ids, int num_experts, int32_t* splits,
+                            int32_t* cumsum, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Everything tdist_moe_splits_cumsum writes, plus
+ *   scatter_idx[i] = position of flat entry i in the stable sort of ids by expert
+ *                    (argsort(stable).argsort(), calc_scatter_index_stable, test_all_to_all.py:95-96)
+ *   gather_idx[p]  = token (i / topk) of the entry sorted to position p (calc_gather_index, :49-92)
+ *   topk_idx[p]    = i % topk of that entry (may be NULL)
+ * all int32; splits may be NULL. */
+int tdist_moe_scatter_index(const int32_t* ids, int64_t n_ids, int topk, int num_experts, int32_t* splits,
+                            int32_t* cumsum, int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx,
+                            void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Dispatch: sorted row p (0 <= p < cumsum[G]) of expert e goes to destination d = e / experts_per_rank,
+ * slot row d*max_m + (p - cumsum[d*experts_per_rank]) of slot_rows / slot_scales
+ * (low_latency_all_to_all.py:59-103 with every destination's receive slot for this sender kept on the
+ * one GPU). Row p is read from rows[gather_idx[p]] (gather_idx = NULL: rows[p], i.e. already sorted
+ * input as fast_all_to_all takes it, :189-215). Rows are row_bytes bytes (any dtype); scales fp32 per
+ * row or NULL. splits_out int32[G] receives cumsum[g+1]-cumsum[g] (:70-74), or may be NULL.
+ * n_rows is the caller's count of sorted rows (T*topk); rows p >= cumsum[G] and rows that would land
+ * beyond max_m in their destination slot are not written (the reference asserts the latter away). */
+int tdist_moe_dispatch(const void* rows, int64_t row_bytes, const float* scales, const int32_t* gather_idx,
+                       const int32_t* cumsum, int64_t n_rows, int world_size, int experts_per_rank,
+                       int max_m, void* slot_rows, float* slot_scales, int32_t* splits_out, void* stream);
+
+/* Compaction of the slots into one [sum, row_bytes] tensor in destination order
+ * (all_to_all_post_process, low_latency_all_to_all.py:251-270): output row p comes from slot row
+ * d*max_m + (p - start_d) where start_d = sum of splits of destinations < d.
+ * splits int32[world_size*experts_per_rank]; n_rows = number of output rows (the caller knows the
+ * total, as the reference does when it slices). out_scales / slot_scales may be NULL. */
+int tdist_moe_post_process(const void* slot_rows, int64_t row_bytes, const float* slot_scales,
+                           const int32_t* splits, int64_t n_rows, int world_size, int experts_per_rank,
+                           int max_m, void* out_rows, float* out_scales, void* stream);
+
+/* Weighted combine back to token order:
+ *   y[t, :] = sum_{k=0..topk-1} w[t,k] * scale[p] * float(row[p]),  p = scatter_idx[t*topk + k],
+ * fp32 accumulation in k order, output bf16 [T, hidden]. Rows are read from the slot layout written by
+ * tdist_moe_dispatch (max_m > 0) or from a compact sorted [n, hidden] tensor (max_m == 0, cumsum
+ * ignored). row_dtype: TDIST_F8E4M3 (scales required unless NULL = 1.0) or TDIST_BF16.
+ * topk_w fp32 [T, topk] or NULL (= 1.0, the index_add_ form of test_all_to_all.py:366-367). */
+int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_scales, const int32_t* scatter_idx,
+                      const float* topk_w, const int32_t* cumsum, int64_t n_tokens, int topk, int hidden,
+                      int world_size, int experts_per_rank, int max_m, void* out_bf16, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (d) split-KV GQA flash decode + LSE combine.
+ *   replaces kernel_gqa_fwd_batch_decode_split_kv               kernels/nvidia/flash_decode.py:129-239
+ *            kernel_intra_rank_gqa_fwd_batch_decode_combine_kv  kernels/nvidia/flash_decode.py:392-449
+ *            kernel_inter_rank_gqa_fwd_batch_decode_combine_kv  kernels/nvidia/flash_decode.py:481-532
+ * ------------------------------------------------------------------------------------------- */
+/* One query token per sequence. For split s of sequence b (keys [s*per, min((s+1)*per, len)),
+ * per = ceil(len/num_splits), flash_decode.py:193-195) and every query head h:
+ *   out_split[b,h,s,:] = softmax(q.k*sm_scale [soft-capped]) . v   over the split's keys (fp32)
+ *   lse_split[b,h,s]   = log(sum exp(scores))  (natural log, fp32; -inf for an empty split)
+ * q [B,Hq,D] (strides q_stride_b, q_stride_h, last dim contiguous); k_cache / v_cache
+ * [num_pages, page_size, Hkv, D] with element strides kv_stride_page (between pages),
+ * kv_stride_token, kv_stride_head; block_table int32 [B, table_stride]; kv_lens int32 [B].
+ * out_split fp32 [B,Hq,S,Dv] contiguous; lse_split fp32 [B,Hq,S] contiguous.
+ * The reference keeps LSE in-band in the q dtype (column Dv of its [.., Dv+1] buffer, :235-239);
+ * here it is a separate fp32 tensor. Supported: D == Dv in {64,128,256}, dtype bf16 / f16. */
+int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cache, float* out_split,
+                          float* lse_split, float sm_scale, float soft_cap, const int32_t* block_table,
+                          const int32_t* kv_lens, int batch, int q_heads, int kv_heads, int head_dim,
+                          int page_size, int num_splits, int64_t q_stride_b, int64_t q_stride_h,
+                          int64_t k_stride_page, int64_t k_stride_token, int64_t k_stride_head,
+                          int64_t v_stride_page, int64_t v_stride_token, int64_t v_stride_head,
+                          int64_t table_stride, int dtype, void* stream);
+
+/* LSE-weighted merge of P partial results per (b,h) — used for the splits of one shard and for the
+ * shards of several ranks:
+ *   m = max_j lse[j];  w_j = exp(lse[j]-m);  out = sum_j w_j*part[j] / sum_j w_j;  lse_out = m + log(sum_j w_j)
+ * over the partials j that are not skipped. part_dtype TDIST_F32 / TDIST_BF16 / TDIST_F16.
+ * Partial j of (b,h) lives at part + j*part_stride_p + b*part_stride_b + h*part_stride_h (+ d), its
+ * LSE at lse + j*lse_stride_p + b*lse_stride_b + h*lse_stride_h (fp32).
+ * Skipping (mode): 0 = none; 1 = split ranges: partial j is skipped when split j of a sequence of
+ * lens[b] keys is empty (flash_decode.py:423-428); 2 = shard lengths: lens is int32 [P, B] and partial j
+ * is skipped when lens[j*B+b] == 0 (:512-515). A (b,h) whose partials are all skipped gets out = 0,
+ * lse_out = -inf. out has out_dtype (TDIST_BF16 / TDIST_F16 / TDIST_F32), [B,Hq,Dv] with strides
+ * out_stride_b, out_stride_h; lse_out fp32 [B,Hq] or NULL. */
+int tdist_decode_combine(const void* part, int part_dtype, const float* lse, int num_partials, int mode,
+                         const int32_t* lens, int batch, int q_heads, int head_dim_v, int64_t part_stride_p,
+                         int64_t part_stride_b, int64_t part_stride_h, int64_t lse_stride_p,
+                         int64_t lse_stride_b, int64_t lse_stride_h, void* out, int out_dtype,
+                         int64_t out_stride_b, int64_t out_stride_h, float* lse_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Measurement helper: plain 16-byte-vector device copy of nbytes (multiple of 16). Used to calibrate
+ * rocprof FETCH_SIZE / WRITE_SIZE readings and as the HBM streaming yardstick; not on the hot path.
+ * ------------------------------------------------------------------------------------------- */
+int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TDIST_H_ */

@@ -1,0 +1,28 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.join(ROOT, "triton-distributed_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def cuda():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from triton_dist import _lib
+    _lib.check(_lib.load().tdist_init())  # fails loudly if the HIP library is missing or the GPU is not gfx950
+    return torch.device("cuda", 0)
+
+
+def announce(msg):
+    """Print and flush the case about to touch the GPU, so that a fault names its test."""
+    print("[gpu-case] " + msg, flush=True)

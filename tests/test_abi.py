@@ -1,0 +1,82 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/tdist.h declares; argument
+validation that needs no device returns error codes instead of aborting. No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from triton_dist import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tdist.h")
+
+
+def header_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tdist_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_functions():
+    names = header_functions()
+    assert "tdist_gemm_chunk_gated_bf16" in names and "tdist_decode_split_kv" in names
+    assert len(names) >= 20
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    for name in header_functions():
+        assert hasattr(lib, name), "libtdist_hip.so does not export %s" % name
+
+
+def test_python_prototypes_cover_header():
+    assert sorted(_lib.PROTOTYPES) == header_functions()
+
+
+def test_prototype_arity_matches_header():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    for name, (_, argtypes) in _lib.PROTOTYPES.items():
+        m = re.search(r"\b%s\s*\((.*?)\)\s*;" % name, text, flags=re.S)
+        assert m, name
+        params = m.group(1).strip()
+        n = 0 if params in ("", "void") else params.count(",") + 1
+        assert n == len(argtypes), "%s: header has %d parameters, binding %d" % (name, n, len(argtypes))
+
+
+def test_version_and_error_string():
+    lib = _lib.load()
+    assert lib.tdist_version() >= 100
+    assert isinstance(_lib.last_error(), str)
+
+
+def test_null_pointers_are_rejected_without_touching_the_gpu():
+    lib = _lib.load()
+    assert lib.tdist_reduce_slices(None, 0, 8, 0, 16, None, _lib.TDIST_BF16, None) == _lib.TDIST_ERR_INVALID
+    assert "null" in _lib.last_error()
+    assert lib.tdist_flag_set(None, 1, None) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_moe_dispatch(None, 16, None, None, None, 0, 1, 1, 1, None, None, None, None) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_copy_bytes(None, None, 16, None) == _lib.TDIST_ERR_INVALID
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    # bad sizes are caught before any launch
+    assert lib.tdist_reduce_slices(p, 0, 0, 0, 16, p, _lib.TDIST_BF16, None) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_reduce_slices(p, 0, 4, 7, 16, p, _lib.TDIST_BF16, None) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_reduce_slices(p, 0, 4, 0, 16, p, _lib.TDIST_F8E4M3, None) == _lib.TDIST_ERR_UNSUPPORTED
+    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 6, 4, 128, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                     _lib.TDIST_BF16, None) == _lib.TDIST_ERR_INVALID  # 6 % 4 != 0
+    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 96, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                     _lib.TDIST_BF16, None) == _lib.TDIST_ERR_UNSUPPORTED  # head_dim 96
+    assert lib.tdist_moe_workspace_bytes(32768, 256) == (32 + 1) * 256 * 4
+
+
+def test_ops_fail_loudly_without_gpu():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    from triton_dist.kernels.amd import create_gemm_rs_intra_node_context, moe_dispatch_preprocess
+    with pytest.raises(RuntimeError):
+        create_gemm_rs_intra_node_context(1024, 256, torch.bfloat16, 0, 8, None)
+    with pytest.raises(RuntimeError):
+        moe_dispatch_preprocess(torch.zeros((4, 2), dtype=torch.int32), 8)

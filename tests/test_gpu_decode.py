@@ -1,0 +1,170 @@
+"""(d) split-KV flash decode and the LSE merges on the GPU against the oracle.
+Bars: <= 2e-3 absolute on the fp32 partial / merged outputs and on the LSE (against the exact fp64 closed
+form); the 16-bit final output against the reference's own golden at the reference test's tolerance
+(atol = rtol = 1e-2, test/nvidia/test_decode_attn.py:164)."""
+import math
+
+import pytest
+import torch
+
+from oracle import golden
+from tests.conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+ATOL = 2e-3
+
+
+def build_case(kv_lens, heads, head_size, block_size, dtype, seed, num_pages=None):
+    g = torch.Generator().manual_seed(seed)
+    Hq, Hkv = heads
+    B = len(kv_lens)
+    q = torch.randn((B, Hq, head_size), generator=g).to(dtype)
+    k_cache, v_cache, table = golden.make_paged_kv(B, max(max(kv_lens), 1), Hkv, head_size, block_size, dtype, g)
+    return q, k_cache, v_cache, table
+
+
+# the reference's own grid (test/nvidia/test_decode_attn.py:126-131) in both 16-bit dtypes
+@pytest.mark.parametrize("kv_lens", [[1320, 18, 463], [1, 54, 293, 70]])
+@pytest.mark.parametrize("num_heads", [(16, 16), (32, 8), (64, 8), (6, 1)])
+@pytest.mark.parametrize("head_size", [128, 256])
+@pytest.mark.parametrize("block_size", [1, 16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("soft_cap", [0, 30, 50])
+def test_decode_with_paged_kv(cuda, kv_lens, num_heads, head_size, dtype, block_size, soft_cap):
+    from triton_dist.kernels.nvidia import gqa_fwd_batch_decode
+    announce("decode kv_lens=%s heads=%s D=%d page=%d %s cap=%s" % (kv_lens, num_heads, head_size, block_size, dtype, soft_cap))
+    q, k_cache, v_cache, table = build_case(kv_lens, num_heads, head_size, block_size, dtype, seed=sum(kv_lens) + head_size)
+    scale = head_size**-0.5
+    B = len(kv_lens)
+    workspace = torch.zeros([B * num_heads[0] * 32], dtype=torch.int32, device=cuda)
+    lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
+    out = gqa_fwd_batch_decode(q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), workspace, [1] * B, lens_dev, table.to(cuda),
+                               scale, soft_cap)
+    torch.cuda.synchronize()
+    ref = golden.ref_paged_attn(q, k_cache, v_cache, [1] * B, kv_lens, table, scale, soft_cap)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), atol=1e-2, rtol=1e-2)
+    exact, _ = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, scale, soft_cap)
+    # the final output is rounded to 16 bits: allow that rounding on top of the 2e-3 bar
+    eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    assert ((out.cpu().double() - exact).abs() <= ATOL + eps * exact.abs()).all()
+
+
+@pytest.mark.parametrize("kv_lens,S", [([1320, 18, 463, 5], 32), ([1, 54, 293, 70], 16), ([2048, 2047, 33, 16], 8), ([100], 1)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_split_partials_and_lse(cuda, kv_lens, S, dtype):
+    from triton_dist.kernels.amd.flash_decode import _split_kv
+    announce("decode partials kv_lens=%s S=%d %s" % (kv_lens, S, dtype))
+    heads, D, page = (64, 8), 128, 16
+    q, k_cache, v_cache, table = build_case(kv_lens, heads, D, page, dtype, seed=S)
+    scale = D**-0.5
+    lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
+    out_split, lse_split, _ = _split_kv(q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), lens_dev, table.to(cuda), scale, 0.0, S)
+    torch.cuda.synchronize()
+    w_out, w_lse = golden.decode_split_exact(q, k_cache, v_cache, kv_lens, table, scale, S)
+    got_lse = lse_split.cpu().double()
+    empty = torch.isinf(w_lse)
+    assert torch.equal(torch.isinf(got_lse), empty), "empty splits must carry LSE = -inf"
+    assert (got_lse[~empty] - w_lse[~empty]).abs().max() <= ATOL
+    assert (out_split.cpu().double() - w_out).abs().max() <= ATOL
+    assert (out_split.cpu()[empty] == 0).all()
+
+
+def test_page_indices_beyond_2_31_bytes(cuda):
+    """Pages far apart: byte offsets above 2^31 (the reference sizes NUM_BLOCKS = 32000 for this,
+    test_decode_attn.py:123)."""
+    from triton_dist.kernels.nvidia import gqa_fwd_batch_decode
+    announce("decode large page indices")
+    Hq, Hkv, D, page = 16, 8, 128, 16
+    num_pages = 100000                     # 100000 * 16*8*128*2 B = 3.3 GB per cache
+    kv_lens = [70, 300]
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn((2, Hq, D), generator=g).to(torch.bfloat16)
+    k_dev = torch.zeros((num_pages, page, Hkv, D), dtype=torch.bfloat16, device=cuda)
+    v_dev = torch.zeros_like(k_dev)
+    pages_per_seq = (max(kv_lens) + page - 1) // page
+    table = torch.stack([torch.arange(num_pages - 1 - b, num_pages - 1 - b - 2 * pages_per_seq, -2)[:pages_per_seq] for b in range(2)]).int()
+    used = table.flatten().long()
+    k_small = torch.randn((used.numel(), page, Hkv, D), generator=g).to(torch.bfloat16)
+    v_small = torch.randn((used.numel(), page, Hkv, D), generator=g).to(torch.bfloat16)
+    k_dev[used.to(cuda)] = k_small.to(cuda)
+    v_dev[used.to(cuda)] = v_small.to(cuda)
+    lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
+    out = gqa_fwd_batch_decode(q.to(cuda), k_dev, v_dev, None, [1, 1], lens_dev, table.to(cuda), D**-0.5, kv_split=4)
+    torch.cuda.synchronize()
+    small_table = torch.arange(used.numel(), dtype=torch.int32).view(2, pages_per_seq)
+    exact, _ = golden.decode_exact(q, k_small, v_small, kv_lens, small_table, D**-0.5)
+    assert ((out.cpu().double() - exact).abs() <= ATOL + 2.0**-8 * exact.abs()).all()
+
+
+def test_inter_rank_combine_and_layer(cuda):
+    """One rank's shard plus synthetic peers, merged by LSE (layers/nvidia/sp_flash_decode_layer.py:142-182,
+    kernels/nvidia/flash_decode.py:512-532); a peer with kv_len 0 is skipped."""
+    from triton_dist.layers.nvidia import SpGQAFlashDecodeAttention
+    announce("SP decode layer, 4 ranks")
+    R, rank, B, Hq, Hkv, D, page = 4, 1, 3, 32, 4, 128, 16
+    kv_lens = [500, 64, 1]
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn((B, Hq, D), generator=g).to(torch.bfloat16)
+    k_cache, v_cache, table = golden.make_paged_kv(B, max(kv_lens), Hkv, D, page, torch.bfloat16, g)
+    global_lens = torch.tensor([[300, 0, 7], kv_lens, [0, 0, 0], [10, 20, 30]], dtype=torch.int32)
+    peer_out = torch.randn((R, B, Hq, D), generator=g)
+    peer_lse = torch.randn((R, B, Hq), generator=g) * 2 + math.log(100.0)
+    layer = SpGQAFlashDecodeAttention(rank, 0, R, 1, Hq, Hkv, D, D, page_size=page, scale=D**-0.5, max_allowed_batch=B)
+    out = layer(q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), global_lens.to(cuda), table.to(cuda),
+                peer_partials=(peer_out.to(cuda), peer_lse.to(cuda)))
+    torch.cuda.synchronize()
+    own, own_lse = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, D**-0.5)
+    all_out = peer_out.double().clone()
+    all_lse = peer_lse.double().clone()
+    all_out[rank], all_lse[rank] = own, own_lse
+    skip = (global_lens == 0)[:, :, None].expand(R, B, Hq)
+    want, _ = golden.lse_merge(all_out, all_lse, skip)
+    assert out.dtype == torch.bfloat16 and out.shape == (B, Hq, D)
+    assert ((out.cpu().double() - want).abs() <= ATOL + 2.0**-8 * want.abs()).all()
+
+
+def test_combine_all_partials_skipped_gives_zero(cuda):
+    from triton_dist.kernels.amd import gqa_fwd_batch_decode_inter_rank_combine
+    announce("inter-rank combine, everything skipped")
+    out = gqa_fwd_batch_decode_inter_rank_combine(torch.ones((2, 1, 4, 64), device=cuda), torch.zeros((2, 1, 4), device=cuda),
+                                                  torch.zeros((2, 1), dtype=torch.int32, device=cuda))
+    torch.cuda.synchronize()
+    assert (out == 0).all()
+
+
+def test_full_size_shard_sampled(cuda):
+    """BASELINE config 5 at full size (B 32, Hq 64, Hkv 8, D 128, 32768 keys, 16 splits, page 16), checked on
+    two sequences against the exact closed form, and through the merge identity on all of them."""
+    from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine
+    announce("decode full size C5")
+    B, Hq, Hkv, D, L, S, page = 32, 64, 8, 128, 32768, 16, 16
+    g = torch.Generator(device="cuda").manual_seed(5)
+    pages_per_seq = L // page
+    num_pages = B * pages_per_seq
+    k_dev = torch.randn((num_pages, page, Hkv, D), generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    v_dev = torch.randn((num_pages, page, Hkv, D), generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    q_dev = torch.randn((B, Hq, D), generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    table = torch.randperm(num_pages, generator=torch.Generator().manual_seed(6)).view(B, pages_per_seq).int()
+    lens_dev = torch.full((B, ), L, dtype=torch.int32, device=cuda)
+    scale = D**-0.5
+    out_split, lse_split, _ = _split_kv(q_dev, k_dev, v_dev, lens_dev, table.to(cuda), scale, 0.0, S)
+    merged = torch.empty((B, Hq, D), dtype=torch.float32, device=cuda)
+    merged_lse = torch.empty((B, Hq), dtype=torch.float32, device=cuda)
+    decode_combine(out_split, lse_split, S, 1, lens_dev, B, Hq, D,
+                   (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
+                   (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), merged, merged_lse)
+    torch.cuda.synchronize()
+    # merge identity on every sequence: the closed-form merge of the GPU's partials equals the GPU's merge
+    w_merged, w_lse = golden.lse_merge(out_split.cpu().permute(2, 0, 1, 3), lse_split.cpu().permute(2, 0, 1))
+    assert (merged.cpu().double() - w_merged).abs().max() <= 1e-5
+    assert (merged_lse.cpu().double() - w_lse).abs().max() <= 1e-4
+    # exact closed form on two sequences (their pages only)
+    for b in (0, 31):
+        pages = table[b].long()
+        k_b = k_dev[pages.to(cuda)].cpu()
+        v_b = v_dev[pages.to(cuda)].cpu()
+        t_b = torch.arange(pages_per_seq, dtype=torch.int32).view(1, -1)
+        exact, exact_lse = golden.decode_exact(q_dev[b:b + 1].cpu(), k_b, v_b, [L], t_b, scale)
+        assert (merged[b].cpu().double() - exact[0]).abs().max() <= ATOL
+        assert (merged_lse[b].cpu().double() - exact_lse[0]).abs().max() <= ATOL

@@ -1,0 +1,253 @@
+"""(a)/(b1) chunk-gated GEMM and the GEMM-RS scatter GEMM on the GPU against the oracle.
+Bar: max relative error <= 1e-2 against the fp32 reference; exact on integer-valued inputs; gating checked
+through host-forced conditions (held flags with a tiny spin limit, shuffled arrival, poisoned workspace)."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cref, golden
+from tests.conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+
+def plain_gemm(a, b, out_dtype, cuda, row_scale=None, col_scale=None):
+    from triton_dist.kernels.amd import gated_gemm
+    c = torch.full((a.shape[0], b.shape[0]), float("nan"), dtype=out_dtype, device=cuda)
+    gated_gemm(a.to(cuda), None, 0, b.to(cuda), c, None, 0, 0, 1,
+               row_scale=None if row_scale is None else row_scale.to(cuda),
+               col_scale=None if col_scale is None else col_scale.to(cuda))
+    torch.cuda.synchronize()
+    return c.cpu()
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 128, 128), (200, 72, 96), (1, 1, 32), (130, 257, 64), (512, 384, 256)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_small_gemm_exact_on_integer_inputs(cuda, M, N, K, dtype):
+    announce("gemm exact M=%d N=%d K=%d %s" % (M, N, K, dtype))
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randint(-3, 4, (M, K), generator=g).to(dtype)
+    b = torch.randint(-3, 4, (N, K), generator=g).to(dtype)
+    want = torch.from_numpy(cref.gemm_nt_f64(a.float().numpy(), b.float().numpy()))   # |entries| <= 9*K < 2^8 * 16: check range
+    got = plain_gemm(a, b, dtype, cuda)
+    assert not torch.isnan(got.float()).any(), "part of C was not written"
+    assert torch.equal(got.double(), want.to(dtype).double())
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (200, 72, 128), (256, 256, 256), (64, 48, 192)])
+def test_small_fp8_gemm_exact_and_scaled(cuda, M, N, K):
+    announce("fp8 gemm M=%d N=%d K=%d" % (M, N, K))
+    g = torch.Generator().manual_seed(M * 7 + K)
+    a = torch.randint(-2, 3, (M, K), generator=g).float().to(torch.float8_e4m3fn)
+    b = torch.randint(-2, 3, (N, K), generator=g).float().to(torch.float8_e4m3fn)
+    want = cref.gemm_e4m3_nt_f64(a.view(torch.uint8).numpy(), b.view(torch.uint8).numpy(), None, None)
+    got = plain_gemm(a, b, torch.bfloat16, cuda)
+    assert torch.equal(got.double(), torch.from_numpy(want).to(torch.bfloat16).double())
+    # random e4m3 data with scales: closed form, <= 1e-2 relative
+    a = torch.randn((M, K), generator=g).to(torch.float8_e4m3fn)
+    b = torch.randn((N, K), generator=g).to(torch.float8_e4m3fn)
+    sa = torch.rand(M, generator=g) * 0.09 + 0.01
+    sb = torch.rand(N, generator=g) * 0.009 + 0.001
+    ref = golden.fp8_scaled_gemm_fp32(a, sa, b, sb)
+    got = plain_gemm(a, b, torch.bfloat16, cuda, sa, sb)
+    assert golden.max_rel_err(got.float(), ref) <= 1e-2
+    assert torch.allclose(got.float(), ref, rtol=2.0**-7, atol=1e-6)   # nothing but the bf16 rounding of C
+
+
+def make_ag_case(world, m_per_rank, K, N, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    if dtype == torch.float8_e4m3fn:
+        shards = [torch.randn((m_per_rank, K), generator=g).to(dtype) for _ in range(world)]
+        b = torch.randn((N, K), generator=g).to(dtype)
+    else:
+        shards = [torch.randn((m_per_rank, K), generator=g).to(dtype) for _ in range(world)]
+        b = (torch.randn((N, K), generator=g) * 0.02).to(dtype)
+    return shards, b
+
+
+def run_ag_gemm(cuda, shards, b, rank, m_per_chunk, **ctx_kw):
+    from triton_dist.kernels.amd import ag_gemm_intra_node, create_ag_gemm_intra_node_context
+    world = len(shards)
+    m_per_rank, K = shards[0].shape
+    ctx = create_ag_gemm_intra_node_context(world * m_per_rank, b.shape[0], K, shards[0].dtype, torch.bfloat16, rank, world,
+                                            None, M_PER_CHUNK=m_per_chunk)
+    for k, v in ctx_kw.items():
+        setattr(ctx, k, v)
+    ctx.set_peer_shards({r: s.to(cuda) for r, s in enumerate(shards) if r != rank})
+    # garbage in the workspace must never leak into C (test/nvidia/test_ag_gemm_intra_node.py:122-127)
+    ctx.workspace_tensors[rank].view(torch.uint8).fill_(0x7B)
+    return ctx
+
+
+def test_ag_gemm_config1(cuda):
+    """BASELINE config 1: 4 chunks of [1024, 4096] bf16, B [1536, 4096], flags released by the copy streams."""
+    from triton_dist.kernels.amd import ag_gemm_intra_node
+    announce("ag_gemm C1")
+    shards, b = make_ag_case(4, 1024, 4096, 1536, torch.bfloat16, seed=3 + 0)
+    ref = golden.ag_gemm_fp32(shards, b)
+    gold = golden.torch_ag_gemm(shards, b)
+    for rank, order in [(0, None), (2, [(3, 0), (1, 0), (0, 0)])]:
+        ctx = run_ag_gemm(cuda, shards, b, rank, 1024, arrival_order=order)
+        for it in range(2):   # flags are reset between calls
+            c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx)
+            ctx.check_status()
+            assert c.shape == (4096, 1536) and c.dtype == torch.bfloat16
+            assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
+            torch.testing.assert_close(c.cpu().float(), gold.float(), atol=1e-2, rtol=1e-2)   # test_ag_gemm_intra_node.py:257
+            assert int(ctx.barrier_tensors[rank].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
+def test_ag_gemm_any_arrival_order(cuda, dtype):
+    """Result independent of the order in which chunks arrive: all 3! orders of the peers of rank 1, two chunks each."""
+    from triton_dist.kernels.amd import ag_gemm_intra_node
+    announce("ag_gemm arrival orders %s" % dtype)
+    world, rank, m_per_rank, mpc, K, N = 4, 1, 256, 128, 256, 384
+    shards, b = make_ag_case(world, m_per_rank, K, N, dtype, seed=11)
+    if dtype == torch.float8_e4m3fn:
+        ref = golden.fp8_scaled_gemm_fp32(torch.cat(shards), None, b, None)
+    else:
+        ref = golden.ag_gemm_fp32(shards, b)
+    first = None
+    for perm in itertools.permutations([0, 2, 3]):
+        order = [(r, c) for c in (1, 0) for r in perm]
+        ctx = run_ag_gemm(cuda, shards, b, rank, mpc, arrival_order=order)
+        c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx)
+        ctx.check_status()
+        assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
+        if first is None:
+            first = c.clone()
+        assert torch.equal(first, c), "output depends on the arrival order"
+
+
+def test_gate_holds_and_times_out(cuda):
+    """A chunk whose flag is never released: with a small spin limit the call reports TDIST_ERR_TIMEOUT, the rows
+    of that chunk stay untouched and every other row is correct (the 1-GPU pattern of test_distributed_wait.py:206-243)."""
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import gated_gemm
+    announce("gate timeout")
+    M, N, K, mpc = 1024, 256, 128, 256
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    b = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    flags = torch.tensor([1, 1, 0, 1], dtype=torch.int32, device=cuda)
+    status = torch.zeros(2, dtype=torch.int32, device=cuda)
+    c = torch.full((M, N), -7.0, dtype=torch.bfloat16, device=cuda)
+    gated_gemm(a.to(cuda), None, 0, b.to(cuda), c, flags, mpc, 0, 1, spin_limit=50, status=status)
+    torch.cuda.synchronize()
+    assert status.tolist() == [_lib.TDIST_ERR_TIMEOUT, 2]
+    ref = golden.ag_gemm_fp32([a], b)
+    got = c.float().cpu()
+    assert (got[512:768] == -7.0).all(), "rows of the held chunk were written"
+    keep = torch.ones(M, dtype=torch.bool)
+    keep[512:768] = False
+    assert golden.max_rel_err(got[keep], ref[keep]) <= 1e-2
+    # released later (wait_value 1 present from the start this time): complete result
+    status.zero_()
+    flags.fill_(1)
+    gated_gemm(a.to(cuda), None, 0, b.to(cuda), c, flags, mpc, 0, 1, spin_limit=50, status=status)
+    torch.cuda.synchronize()
+    assert status.tolist() == [0, 0]
+    assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
+
+
+def test_gate_released_by_a_stream_while_the_gemm_waits(cuda):
+    """Flags are set by a second stream after the GEMM has been launched (explicit chunk order, last chunk first)."""
+    from triton_dist.kernels.amd import gated_gemm
+    from triton_dist.kernels.amd.common_ops import set_signal
+    announce("gate released late")
+    M, N, K, mpc = 1024, 256, 256, 256
+    g = torch.Generator().manual_seed(6)
+    a = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    b = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    flags = torch.zeros(4, dtype=torch.int32, device=cuda)
+    status = torch.zeros(2, dtype=torch.int32, device=cuda)
+    order = torch.tensor([3, 1, 0, 2], dtype=torch.int32, device=cuda)
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=cuda)
+    a_dev, b_dev = a.to(cuda), b.to(cuda)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    gated_gemm(a_dev, None, 0, b_dev, c, flags, mpc, 0, 1, chunk_order=order, status=status)
+    for chunk in (3, 1, 0, 2):
+        set_signal(flags.data_ptr() + 4 * chunk, 1, side)
+    torch.cuda.synchronize()
+    assert status.tolist() == [0, 0]
+    assert golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32([a], b)) <= 1e-2
+
+
+def test_gemm_rs_small_and_owner_mapping(cuda):
+    from triton_dist.kernels.amd import create_gemm_rs_intra_node_context, gemm_rs_intra_node
+    announce("gemm_rs small")
+    W, rank, M, N, K = 4, 2, 1024, 512, 256
+    g = torch.Generator().manual_seed(8)
+    a = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    b = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    m_per = M // W
+    peers = [None if r == rank else torch.randn((m_per, N), generator=g).to(torch.bfloat16) for r in range(W)]
+    ctx = create_gemm_rs_intra_node_context(M, N, torch.bfloat16, rank, W, None)
+    ctx.set_peer_partials(peers)
+    out = gemm_rs_intra_node(a.to(cuda), b.to(cuda), ctx)
+    torch.cuda.synchronize()
+    assert out.shape == (m_per, N)
+    ref = golden.gemm_rs_fp32(a, b, peers, rank, W)
+    assert golden.max_rel_err(out.float().cpu(), ref) <= 1e-2
+    gold = golden.torch_gemm_rs(a, b, peers, rank, W)
+    torch.testing.assert_close(out.float().cpu(), gold.float(), atol=1e-2, rtol=1e-2)   # test_gemm_rs_intra_node.py:261
+    # epilogue placement (gemm_reduce_scatter.py:222-229): owner o's rows sit in scatter_bufs[o] at row block `rank`
+    full = golden.ag_gemm_fp32([a], b)
+    for o in range(W):
+        blk = ctx.scatter_bufs[o][rank * m_per:(rank + 1) * m_per].float().cpu()
+        assert golden.max_rel_err(blk, full[o * m_per:(o + 1) * m_per]) <= 1e-2, "owner %d" % o
+    # the reduction is bit-exact given what the GEMM stored
+    stored = ctx.scatter_bufs[rank][:M].cpu().view(W, m_per, N)
+    assert torch.equal(out.cpu().view(torch.int16), golden.reduce_slices_ordered(stored, (rank + 1) % W).view(torch.int16))
+
+
+def test_gemm_rs_config2_full_size(cuda):
+    """BASELINE config 2: A [8192, 3584] x B [3584, 8192] (stored [8192, 3584]), rank 0 of 8, 7 synthetic peers."""
+    from triton_dist.kernels.amd import create_gemm_rs_intra_node_context, gemm_rs_intra_node
+    announce("gemm_rs C2 full size")
+    W, rank, M, N, K = 8, 0, 8192, 8192, 3584
+    g = torch.Generator().manual_seed(3 + 1)
+    a = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    b = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    peers = [None if r == rank else torch.randn((M // W, N), generator=g).to(torch.bfloat16) for r in range(W)]
+    ctx = create_gemm_rs_intra_node_context(M, N, torch.bfloat16, rank, W, None)
+    ctx.set_peer_partials(peers)
+    out = gemm_rs_intra_node(a.to(cuda), b.to(cuda), ctx)
+    torch.cuda.synchronize()
+    ref = golden.gemm_rs_fp32(a, b, peers, rank, W)
+    assert golden.max_rel_err(out.float().cpu(), ref) <= 1e-2
+    # the partial of a far row block (owner 5) against the fp32 product of those rows
+    blk = ctx.scatter_bufs[5][rank * 1024:(rank + 1) * 1024].float().cpu()
+    assert golden.max_rel_err(blk, a[5 * 1024:6 * 1024].float() @ b.float().T) <= 1e-2
+
+
+def test_fp8_ag_gemm_config3_full_size(cuda):
+    """BASELINE config 3: 8 chunks of [2048, 8192] e4m3, B [7168, 8192] e4m3, per-row and per-column fp32 scales."""
+    from triton_dist.kernels.amd import ag_gemm_intra_node
+    announce("fp8 ag_gemm C3 full size")
+    world, rank, m_per_rank, K, N = 8, 0, 2048, 8192, 7168
+    g = torch.Generator().manual_seed(3 + 2)
+    shards = [torch.randn((m_per_rank, K), generator=g).to(torch.float8_e4m3fn) for _ in range(world)]
+    b = torch.randn((N, K), generator=g).to(torch.float8_e4m3fn)
+    sa = torch.rand(world * m_per_rank, generator=g) * 0.09 + 0.01
+    sb = torch.rand(N, generator=g) * 0.009 + 0.001
+    ctx = run_ag_gemm(cuda, shards, b, rank, 2048)
+    c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx, row_scale=sa.to(cuda), col_scale=sb.to(cuda))
+    ctx.check_status()
+    assert c.shape == (16384, 7168) and c.dtype == torch.bfloat16
+    got = c.float().cpu()
+    # closed form on a band of rows from every chunk (the full fp32 product is 1.9 TFLOP on the CPU)
+    for r in range(world):
+        rows = slice(r * m_per_rank + 37, r * m_per_rank + 37 + 64)
+        ref = golden.fp8_scaled_gemm_fp32(shards[r][37:37 + 64], sa[rows], b, sb)
+        assert golden.max_rel_err(got[rows], ref) <= 1e-2, "chunk %d" % r
+    # linearity in the scales: doubling a row scale doubles that row (size-independent property)
+    sa2 = sa.clone()
+    sa2[::2] *= 2
+    c2 = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx, row_scale=sa2.to(cuda), col_scale=sb.to(cuda))
+    ctx.check_status()
+    assert torch.equal(c2[::2].float(), c[::2].float() * 2) and torch.equal(c2[1::2], c[1::2])

@@ -1,0 +1,185 @@
+"""(c) MoE dispatch / combine on the GPU against the oracle: indices, splits and moved bytes bit-exact;
+the weighted combine within 1e-2 relative (fp32 accumulation, fixed k order)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import golden
+from tests.conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+
+def make_case(T, topk, G, H, seed, distinct=True):
+    g = torch.Generator().manual_seed(seed)
+    if distinct and topk <= G:
+        ids = golden.random_distinct_experts(T, G, topk, g)
+    else:
+        ids = torch.randint(0, G, (T, topk), generator=g).to(torch.int32)
+    x = torch.randn((T, H), generator=g)
+    q, s = golden.quantize_per_token_e4m3(x)
+    w = torch.softmax(torch.randn((T, topk), generator=g), dim=-1).float().contiguous()
+    return ids, x, q, s, w
+
+
+@pytest.mark.parametrize("T,topk,G", [(4096, 8, 256), (64, 8, 16), (1, 1, 1), (1, 8, 256), (1000, 6, 48), (257, 4, 7),
+                                      (5000, 2, 1024), (3, 2, 3)])
+def test_preprocess_bit_exact(cuda, T, topk, G):
+    from triton_dist.kernels.amd import moe_dispatch_preprocess
+    announce("moe preprocess T=%d topk=%d G=%d" % (T, topk, G))
+    ids, *_ = make_case(T, topk, G, 16, seed=T + topk + G)
+    splits, cumsum, scatter, gather, topk_idx = moe_dispatch_preprocess(ids.to(cuda), G, want_topk_index=True)
+    torch.cuda.synchronize()
+    w_splits, w_cumsum, w_scatter, w_gather, w_topk = golden.moe_preprocess(ids, G)
+    assert torch.equal(splits.cpu(), w_splits)
+    assert torch.equal(cumsum.cpu(), w_cumsum)
+    assert torch.equal(scatter.cpu(), w_scatter)
+    assert torch.equal(gather.cpu(), w_gather)
+    assert torch.equal(topk_idx.cpu(), w_topk)
+
+
+def test_preprocess_repeated_ids_and_skewed_load(cuda):
+    from triton_dist.kernels.amd import moe_dispatch_preprocess
+    announce("moe preprocess skewed")
+    g = torch.Generator().manual_seed(77)
+    ids = torch.randint(0, 4, (3000, 8), generator=g).to(torch.int32)   # every wave sees long runs of equal ids
+    ids[:, 0] = 0
+    out = moe_dispatch_preprocess(ids.to(cuda), 64)
+    torch.cuda.synchronize()
+    want = golden.moe_preprocess(ids, 64)
+    for a, b in zip(out, want[:4]):
+        assert torch.equal(a.cpu(), b)
+
+
+def test_splits_cumsum_entry_point(cuda):
+    from triton_dist import _lib
+    announce("moe splits_cumsum")
+    ids, *_ = make_case(777, 8, 100, 16, seed=5)
+    dev_ids = ids.to(cuda)
+    splits = torch.empty(100, dtype=torch.int32, device=cuda)
+    cumsum = torch.empty(101, dtype=torch.int32, device=cuda)
+    ws = torch.empty(_lib.load().tdist_moe_workspace_bytes(ids.numel(), 100), dtype=torch.uint8, device=cuda)
+    _lib.call("tdist_moe_splits_cumsum", dev_ids.data_ptr(), ids.numel(), 100, splits.data_ptr(), cumsum.data_ptr(),
+              ws.data_ptr(), ws.numel(), _lib.stream_ptr())
+    torch.cuda.synchronize()
+    want = torch.bincount(ids.view(-1).long(), minlength=100).int()
+    assert torch.equal(splits.cpu(), want) and torch.equal(cumsum.cpu(), golden.splits_to_cumsum(want))
+    # too small a workspace is refused
+    assert _lib.load().tdist_moe_splits_cumsum(dev_ids.data_ptr(), ids.numel(), 100, splits.data_ptr(), cumsum.data_ptr(),
+                                               ws.data_ptr(), 16, None) == _lib.TDIST_ERR_WORKSPACE
+
+
+@pytest.mark.parametrize("T,topk,G,W,H,max_m,fused", [(4096, 8, 256, 32, 7168, 4096, True), (4096, 8, 256, 32, 7168, 4096, False),
+                                                     (96, 4, 16, 4, 48, 160, True), (50, 3, 6, 2, 24, 40, False),
+                                                     (10, 2, 8, 8, 1024, 8, True)])
+def test_dispatch_bytes_bit_exact_and_round_trip(cuda, T, topk, G, W, H, max_m, fused):
+    from triton_dist.kernels.amd import (all_to_all_post_process, create_all_to_all_context, fast_all_to_all,
+                                         moe_dispatch_preprocess)
+    announce("moe dispatch T=%d topk=%d G=%d W=%d H=%d max_m=%d fused=%s" % (T, topk, G, W, H, max_m, fused))
+    Er = G // W
+    ids, x, q, s, w = make_case(T, topk, G, H, seed=T * 3 + H)
+    ctx = create_all_to_all_context(max_m, H, 0, G, W, Er, dtype=torch.float8_e4m3fn)
+    ctx.recv_buf.view(torch.uint8).fill_(0xAB)
+    splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids.to(cuda), G)
+    dq, ds = q.to(cuda), s.to(cuda)
+    if fused:
+        out_splits, recv, recv_scale = fast_all_to_all(ctx, dq, cumsum, ds, gather_index=gather)
+    else:
+        rows = torch.index_select(dq.view(torch.uint8), 0, gather.long()).view(torch.float8_e4m3fn)
+        scales = torch.index_select(ds, 0, gather.long())
+        out_splits, recv, recv_scale = fast_all_to_all(ctx, rows, cumsum, scales)
+    torch.cuda.synchronize()
+    w_splits, w_cumsum, w_scatter, w_gather, _ = golden.moe_preprocess(ids, G)
+    sorted_rows = q.view(torch.uint8)[w_gather.long()]
+    sorted_scales = s[w_gather.long()]
+    assert torch.equal(out_splits.cpu(), w_splits)
+    recv_u8 = recv.view(torch.uint8).cpu()
+    recv_scale = recv_scale.cpu()
+    for d in range(W):
+        st, ed = int(w_cumsum[d * Er]), int(w_cumsum[(d + 1) * Er])
+        n = min(ed - st, max_m)
+        assert torch.equal(recv_u8[d * max_m:d * max_m + n], sorted_rows[st:st + n]), "slot %d rows" % d
+        assert torch.equal(recv_scale[d * max_m:d * max_m + n], sorted_scales[st:st + n]), "slot %d scales" % d
+        assert (recv_u8[d * max_m + n:(d + 1) * max_m] == 0xAB).all(), "slot %d: rows past the split were written" % d
+    if max(int(w_cumsum[(d + 1) * Er] - w_cumsum[d * Er]) for d in range(W)) <= max_m:
+        out, out_scale = all_to_all_post_process(ctx, out_splits, recv, recv_scale.to(cuda))
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.uint8).cpu(), sorted_rows)
+        assert torch.equal(out_scale.cpu(), sorted_scales)
+
+
+def test_dispatch_bf16_rows_without_scales_and_odd_row_bytes(cuda):
+    from triton_dist.kernels.amd import create_all_to_all_context, fast_all_to_all, moe_dispatch_preprocess
+    announce("moe dispatch bf16 H=36 (72-byte rows: scalar copy path)")
+    T, topk, G, W, H, max_m = 40, 2, 4, 2, 36, 64
+    g = torch.Generator().manual_seed(12)
+    ids = golden.random_distinct_experts(T, G, topk, g)
+    x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+    ctx = create_all_to_all_context(max_m, H, 0, G, W, G // W, dtype=torch.bfloat16)
+    splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids.to(cuda), G)
+    rows = x.to(cuda)[gather.long()]
+    out_splits, recv, none = fast_all_to_all(ctx, rows, cumsum, None)
+    torch.cuda.synchronize()
+    assert none is None
+    w_splits, w_cumsum, _, w_gather, _ = golden.moe_preprocess(ids, G)
+    _, want, _ = golden.dispatch_slots(x[w_gather.long()], None, w_cumsum, W, G // W, max_m)
+    got = recv.view(torch.uint8).cpu()
+    for d in range(W):
+        n = int(w_cumsum[(d + 1) * (G // W)] - w_cumsum[d * (G // W)])
+        assert torch.equal(got[d * max_m:d * max_m + n], want[d * max_m:d * max_m + n])
+    assert torch.equal(out_splits.cpu(), w_splits)
+
+
+def test_context_double_buffering(cuda):
+    from triton_dist.kernels.amd import create_all_to_all_context, fast_all_to_all
+    announce("moe ctx act_pos alternates")
+    ctx = create_all_to_all_context(8, 16, 0, 2, 2, 1, dtype=torch.bfloat16)
+    cumsum = torch.tensor([0, 2, 4], dtype=torch.int32, device=cuda)
+    a = torch.ones((4, 16), dtype=torch.bfloat16, device=cuda)
+    r1 = fast_all_to_all(ctx, a, cumsum, None)[1]
+    r2 = fast_all_to_all(ctx, a * 2, cumsum, None)[1]
+    r3 = fast_all_to_all(ctx, a * 3, cumsum, None)[1]
+    torch.cuda.synchronize()
+    assert r1.data_ptr() != r2.data_ptr() and r1.data_ptr() == r3.data_ptr()   # reference :195, :239
+    assert float(r2[0, 0]) == 2.0 and float(r3[0, 0]) == 3.0 and float(r3[8, 0]) == 3.0
+
+
+@pytest.mark.parametrize("T,topk,G,W,H,max_m", [(4096, 8, 256, 32, 7168, 4096), (96, 4, 16, 4, 64, 160), (7, 3, 8, 2, 16, 32)])
+def test_weighted_combine(cuda, T, topk, G, W, H, max_m):
+    from triton_dist.kernels.amd import (create_all_to_all_context, fast_all_to_all, moe_dispatch_preprocess,
+                                         moe_weighted_combine)
+    announce("moe combine T=%d topk=%d G=%d H=%d" % (T, topk, G, H))
+    ids, x, q, s, w = make_case(T, topk, G, H, seed=T + 99)
+    ctx = create_all_to_all_context(max_m, H, 0, G, W, G // W, dtype=torch.float8_e4m3fn)
+    splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids.to(cuda), G)
+    out_splits, recv, recv_scale = fast_all_to_all(ctx, q.to(cuda), cumsum, s.to(cuda), gather_index=gather)
+    y = moe_weighted_combine(ctx, recv, recv_scale, scatter, w.to(cuda), cumsum)
+    torch.cuda.synchronize()
+    _, _, w_scatter, w_gather, _ = golden.moe_preprocess(ids, G)
+    ref = golden.weighted_combine(q[w_gather.long()].float(), s[w_gather.long()], w_scatter, w)
+    assert golden.max_rel_err(y.float().cpu(), ref) <= 1e-2
+    # the weights of a token sum to 1 and its topk copies are one row: y is the dequantised token
+    deq = q.float() * s[:, None]
+    assert golden.max_rel_err(y.float().cpu(), deq) <= 1e-2
+
+
+def test_combine_reference_round_trip_bf16(cuda):
+    """dispatch -> combine with unit weights gives topk * input (test_all_to_all.py:366-370)."""
+    from triton_dist.kernels.amd import (all_to_all_post_process, create_all_to_all_context, fast_all_to_all,
+                                         moe_dispatch_preprocess, moe_weighted_combine, splits_to_cumsum)
+    announce("moe round trip bf16")
+    T, topk, G, W, H, max_m = 128, 4, 32, 8, 256, 128
+    g = torch.Generator().manual_seed(21)
+    ids = golden.random_distinct_experts(T, G, topk, g)
+    x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+    ctx = create_all_to_all_context(max_m, H, 0, G, W, G // W, dtype=torch.bfloat16)
+    splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids.to(cuda), G)
+    d_splits, d_tok, _ = fast_all_to_all(ctx, x.to(cuda), cumsum, None, gather_index=gather)
+    tok, _ = all_to_all_post_process(ctx, d_splits, d_tok)
+    c_splits, c_tok, _ = fast_all_to_all(ctx, tok, splits_to_cumsum(d_splits), None)
+    y_slots = moe_weighted_combine(ctx, c_tok, None, scatter, None, cumsum)
+    tok2, _ = all_to_all_post_process(ctx, c_splits, c_tok)
+    y_compact = moe_weighted_combine(None, tok2, None, scatter, None, from_slots=False)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(y_slots.float().cpu(), x.float() * topk, rtol=1e-2, atol=1e-2)
+    assert torch.equal(y_slots, y_compact)

@@ -1,0 +1,547 @@
+// (d) split-KV GQA flash decode and the LSE-weighted combine.
+//
+// Restates kernel_gqa_fwd_batch_decode_split_kv (kernels/nvidia/flash_decode.py:129-239) and the
+// combine kernels (:392-449, :481-532) for CDNA4:
+//
+//  * one workgroup per (split, kv head [x block of 16 query heads], sequence); its NW waves each stream
+//    an interleaved subset of the split's 16-key blocks and keep a private online-softmax state, merged
+//    through LDS at the end, so the main loop has no workgroup barrier;
+//  * K and V rows go HBM → LDS with asynchronous 16-byte-per-lane LDS-DMA loads into a per-wave ring of
+//    NST stages (P = NST-1 stages in flight), so the only synchronisation is the wave's own vmcnt;
+//    the page-table entries a stage needs travel the same way, two rounds ahead of the rows;
+//  * scores:  S^T[key, head] = K[16 keys, D] . Q^T[D, 16 heads]   v_mfma_f32_16x16x32 (D/32 steps);
+//    the result layout (lane = head, 4 keys per lane) is exactly the B operand of
+//    O^T[dv, head] += V^T[16 dv, 16 keys] . P^T[16 keys, 16 heads]  v_mfma_f32_16x16x16 (D/16 tiles),
+//    so probabilities never leave registers; V^T fragments are 16-bit LDS reads from the swizzled rows;
+//  * probabilities enter the PV product as a hi+lo pair of 16-bit values, which keeps the product at
+//    fp32-level accuracy for the cost of a second (idle anyway) MFMA.
+//
+// HBM traffic per launch: every K and V row of the split once (2 * len * Hkv * D * 2 B per sequence).
+#include "common.h"
+
+namespace tdist {
+
+struct DecodeParams {
+  const unsigned char* q;
+  const unsigned char* k;
+  const unsigned char* v;
+  float* out;  // [B,Hq,S,D]
+  float* lse;  // [B,Hq,S]
+  const int32_t* table;
+  const int32_t* lens;
+  float sm_scale;
+  float soft_cap;
+  int B, Hq, Hkv, S;
+  int page_size;
+  // n / page_size for 0 <= n < 2^31 as (n * page_magic) >> page_shift with
+  // page_shift = 31 + ceil(log2 page_size), page_magic = ceil(2^page_shift / page_size)  (exact, Granlund-Montgomery)
+  int page_shift;
+  uint64_t page_magic;
+  // byte strides
+  int64_t q_sb, q_sh;
+  int64_t k_sp, k_st, k_sh;
+  int64_t v_sp, v_st, v_sh;
+  int64_t t_s;  // table stride in entries
+};
+
+struct MmaBF16 {
+  typedef bf16x8v frag8;
+  typedef short4v frag4;
+  __device__ static __forceinline__ float4v qk(frag8 a, frag8 b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ float4v pv(frag4 a, frag4 b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+  }
+  // p → (hi, lo) 16-bit patterns with hi + lo ≈ p to ~16 mantissa bits
+  __device__ static __forceinline__ void split(float p, uint32_t& hi, uint32_t& lo) {
+    hi = f32_to_bf16_bits(p);
+    lo = f32_to_bf16_bits(p - bf16_bits_to_f32(hi));
+  }
+};
+struct MmaF16 {
+  typedef f16x8v frag8;
+  typedef f16x4v frag4;
+  __device__ static __forceinline__ float4v qk(frag8 a, frag8 b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ float4v pv(frag4 a, frag4 b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ void split(float p, uint32_t& hi, uint32_t& lo) {
+    _Float16 h = (_Float16)p;
+    _Float16 l = (_Float16)(p - (float)h);
+    hi = __builtin_bit_cast(unsigned short, h);
+    lo = __builtin_bit_cast(unsigned short, l);
+  }
+};
+
+constexpr int kBlockKeys = 16;
+constexpr int kTableSlots = 8;          // ring of page-table rows per wave (>= 2P+2)
+constexpr int kTableSlotBytes = 16 * 4; // 16 entries
+
+template <int D, int NST>
+struct DecodeCfg {
+  static constexpr int kRowBytes = D * 2;
+  static constexpr int kLanesPerRow = kRowBytes / 16;       // 16-byte chunks per row
+  static constexpr int kRowsPerInstr = 64 / kLanesPerRow;   // rows one wave-wide DMA covers
+  static constexpr int kInstrPerTensor = kBlockKeys / kRowsPerInstr;
+  static constexpr int kTensorBytes = kBlockKeys * kRowBytes;
+  static constexpr int kStageBytes = 2 * kTensorBytes;
+  static constexpr int kLoadsPerGroup = 1 + 2 * kInstrPerTensor;  // table row + K + V
+  static constexpr int kP = NST - 1;
+  static constexpr int kSwz = (kLanesPerRow < 16 ? kLanesPerRow : 16) - 1;
+  static constexpr int kWaveBytes = NST * kStageBytes + kTableSlots * kTableSlotBytes;
+  static_assert(kP >= 1 && kP <= 3, "1..3 stages in flight");
+  static_assert(kP * kLoadsPerGroup < 64, "vmcnt is 6 bits");
+  static_assert(2 * kP + 2 <= kTableSlots, "table ring too small");
+  static_assert(D % 32 == 0 && D >= 64 && D <= 256, "head dim");
+};
+
+template <int N>
+__device__ __forceinline__ void wait_groups(int rem) {
+  // rem in [0, P]: number of younger load groups allowed to stay in flight
+  if (rem >= 3) wait_vmcnt<(3 * N < 64 ? 3 * N : 63)>();
+  else if (rem == 2) wait_vmcnt<(2 * N < 64 ? 2 * N : 63)>();
+  else if (rem == 1) wait_vmcnt<N>();
+  else wait_vmcnt<0>();
+}
+
+template <typename MMA, int D, int NW, int NST, bool kSoftCap>
+__global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodeParams prm) {
+  typedef DecodeCfg<D, NST> C;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  const int split = blockIdx.x;
+  const int group = prm.Hq / prm.Hkv;
+  const int head_blocks = (group + 15) >> 4;
+  const int kvh = blockIdx.y / head_blocks;
+  const int hb = blockIdx.y - kvh * head_blocks;
+  const int b = blockIdx.z;
+  const int h0 = kvh * group + hb * 16;
+  const int nvalid = min(16, group - hb * 16);
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform for the compiler too
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;   // lane group 0..3
+  const int x = lane & 15;   // head (QK result column) / dv within tile (V^T row)
+
+  const int len = prm.lens[b];
+  const int per = (len + prm.S - 1) / prm.S;
+  const int start = per * split;
+  const int end = min(start + per, len);
+
+  float* out_base = prm.out + (((int64_t)b * prm.Hq + h0) * prm.S + split) * D;
+  float* lse_base = prm.lse + ((int64_t)b * prm.Hq + h0) * prm.S + split;
+  if (end <= start) {
+    // empty split: zeros and LSE = -inf so that any merge gives it weight 0
+    for (int i = threadIdx.x; i < nvalid * D; i += NW * 64) {
+      const int h = i / D, d = i - h * D;
+      out_base[(int64_t)h * prm.S * D + d] = 0.f;
+    }
+    if (threadIdx.x < nvalid) lse_base[(int64_t)threadIdx.x * prm.S] = -INFINITY;
+    return;
+  }
+
+  typedef TDIST_AS3 unsigned char* lds_u8;  // explicit LDS pointers: a generic pointer would turn reads into
+                                            // flat loads, which count on vmcnt and break the DMA accounting
+  lds_u8 const smem3 = (lds_u8)smem;
+  lds_u8 const wbase = smem3 + wave * C::kWaveBytes;
+  lds_u8 const tbl_base = wbase + NST * C::kStageBytes;
+
+  const int nb_total = (end - start + kBlockKeys - 1) / kBlockKeys;
+  const int n_w = nb_total > wave ? (nb_total - wave + NW - 1) / NW : 0;  // this wave's blocks
+
+  // ---- Q fragments (B operand of the score MFMA): head x, dims 32s + 8g .. +8 -------------------
+  typename MMA::frag8 qf[D / 32];
+  {
+    const unsigned char* qrow = prm.q + (int64_t)b * prm.q_sb + (int64_t)(h0 + x) * prm.q_sh;
+#pragma unroll
+    for (int s = 0; s < D / 32; ++s) {
+      int4v raw = {0, 0, 0, 0};
+      if (x < nvalid) raw = *(const int4v*)(qrow + (32 * s + 8 * g) * 2);
+      qf[s] = __builtin_bit_cast(typename MMA::frag8, raw);
+    }
+  }
+
+  constexpr float kLog2e = 1.4426950408889634f;
+  const float scale_log2 = prm.sm_scale * kLog2e;
+
+  float m_run = -INFINITY;  // running max (log2 domain) of head x, identical in the 4 lane groups
+  float l_run = 0.f;        // this lane group's share of the running sum
+  float4v acc[D / 16];
+#pragma unroll
+  for (int d = 0; d < D / 16; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // first key of the wave's j-th block
+  auto block_key0 = [&](int j) { return start + (wave + j * NW) * kBlockKeys; };
+
+  // page-table row of block j → table ring slot j % kTableSlots (lanes 0..15, one entry per key)
+  auto issue_table = [&](int j) {
+    if (lane < 16) {
+      int n = block_key0(j) + lane;
+      n = min(n, end - 1);
+      n = max(n, start);
+      const int e = (int)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift);
+      const int32_t* src = prm.table + (int64_t)b * prm.t_s + e;
+      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)src,
+                                       (TDIST_AS3 void*)(tbl_base + (j % kTableSlots) * kTableSlotBytes), 4, 0, 0);
+    }
+  };
+
+  // K and V rows of block j → stage j % NST. LDS position i of a row holds 16-byte chunk i ^ (key & swz).
+  auto issue_rows = [&](int j) {
+    const int key0 = block_key0(j);
+    const volatile TDIST_AS3 int32_t* tbl =
+        (const volatile TDIST_AS3 int32_t*)(tbl_base + (j % kTableSlots) * kTableSlotBytes);
+    lds_u8 const kst = wbase + (j % NST) * C::kStageBytes;
+    lds_u8 const vst = kst + C::kTensorBytes;
+    const int chunk = lane % C::kLanesPerRow;
+#pragma unroll
+    for (int i = 0; i < C::kInstrPerTensor; ++i) {
+      const int key = i * C::kRowsPerInstr + lane / C::kLanesPerRow;
+      int n = min(key0 + key, end - 1);
+      n = max(n, start);
+      const int page = tbl[key];
+      const int in_page = n - (int)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift) * prm.page_size;
+      const int src_chunk = chunk ^ (key & C::kSwz);
+      const unsigned char* ksrc = prm.k + (int64_t)page * prm.k_sp + (int64_t)in_page * prm.k_st +
+                                  (int64_t)kvh * prm.k_sh + src_chunk * 16;
+      const unsigned char* vsrc = prm.v + (int64_t)page * prm.v_sp + (int64_t)in_page * prm.v_st +
+                                  (int64_t)kvh * prm.v_sh + src_chunk * 16;
+      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)ksrc, (TDIST_AS3 void*)(kst + i * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)vsrc, (TDIST_AS3 void*)(vst + i * 1024), 16, 0, 0);
+    }
+  };
+
+  auto compute = [&](int j) {
+    const int key0 = block_key0(j);
+    lds_u8 const kst = wbase + (j % NST) * C::kStageBytes;
+    lds_u8 const vst = kst + C::kTensorBytes;
+    // scores: A = K rows (key x, dims 32s+8g..), B = Q
+    float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < D / 32; ++s) {
+      const int c = 4 * s + g;
+      const int4v raw = *(const TDIST_AS3 int4v*)(kst + x * C::kRowBytes + ((c ^ (x & C::kSwz)) << 4));
+      sc = MMA::qk(__builtin_bit_cast(typename MMA::frag8, raw), qf[s], sc);
+    }
+    // sc[i]: key 4g+i, head x
+    float t[4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v;
+      if (kSoftCap) {
+        v = prm.soft_cap * tanhf(sc[i] * prm.sm_scale / prm.soft_cap) * kLog2e;
+      } else {
+        v = sc[i] * scale_log2;
+      }
+      const bool valid = key0 + 4 * g + i < end;
+      t[i] = valid ? v : -INFINITY;
+      mx = fmaxf(mx, t[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    if (__any(m_new > m_run)) {
+      const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+      l_run *= alpha;
+#pragma unroll
+      for (int d = 0; d < D / 16; ++d) acc[d] *= alpha;
+      m_run = m_new;
+    }
+    const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = __builtin_amdgcn_exp2f(t[i] - m_safe);
+      l_run += p;
+      MMA::split(p, hi[i], lo[i]);
+    }
+    int2v ph = {(int)(hi[0] | (hi[1] << 16)), (int)(hi[2] | (hi[3] << 16))};
+    int2v pl = {(int)(lo[0] | (lo[1] << 16)), (int)(lo[2] | (lo[3] << 16))};
+    const typename MMA::frag4 p_hi = __builtin_bit_cast(typename MMA::frag4, ph);
+    const typename MMA::frag4 p_lo = __builtin_bit_cast(typename MMA::frag4, pl);
+    // O^T tiles: A = V^T (dv 16d+x, keys 4g..4g+3), B = P^T
+#pragma unroll
+    for (int d = 0; d < D / 16; ++d) {
+      const int dv = 16 * d + x;
+      uint32_t e[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = 4 * g + i;
+        e[i] = *(const TDIST_AS3 unsigned short*)(vst + key * C::kRowBytes + (((dv >> 3) ^ (key & C::kSwz)) << 4) + (dv & 7) * 2);
+      }
+      int2v vv = {(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16))};
+      const typename MMA::frag4 vt = __builtin_bit_cast(typename MMA::frag4, vv);
+      acc[d] = MMA::pv(vt, p_hi, acc[d]);
+      acc[d] = MMA::pv(vt, p_lo, acc[d]);
+    }
+  };
+
+  if (n_w > 0) {
+    // page-table rows of the first P+1 blocks, then the first P row groups
+    for (int j = 0; j <= C::kP; ++j) issue_table(j);
+    wait_vmcnt<0>();
+    for (int gi = -C::kP; gi < 0; ++gi) {
+      if (gi + C::kP < n_w) {
+        issue_table(gi + 2 * C::kP + 1);
+        issue_rows(gi + C::kP);
+      }
+    }
+    for (int i = 0; i < n_w; ++i) {
+      if (i + C::kP < n_w) {
+        issue_table(i + 2 * C::kP + 1);
+        issue_rows(i + C::kP);
+      }
+      wait_groups<C::kLoadsPerGroup>(min(C::kP, n_w - 1 - i));
+      compute(i);
+    }
+  }
+
+  // ---- merge the waves' partial states ---------------------------------------------------------
+  l_run += __shfl_xor(l_run, 16);
+  l_run += __shfl_xor(l_run, 32);
+  wait_vmcnt<0>();
+  __syncthreads();  // every wave is done with its ring; reuse it
+  TDIST_AS3 float* s_m = (TDIST_AS3 float*)(wbase);  // [16]
+  TDIST_AS3 float* s_l = s_m + 16;                   // [16]
+  TDIST_AS3 float* s_acc = s_l + 16;                 // [D][16]
+  if (lane < 16) {
+    s_m[lane] = m_run;
+    s_l[lane] = l_run;
+  }
+#pragma unroll
+  for (int d = 0; d < D / 16; ++d)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_acc[(16 * d + 4 * g + i) * 16 + x] = acc[d][i];
+  __syncthreads();
+  constexpr float kLn2 = 0.6931471805599453f;
+  for (int idx = threadIdx.x; idx < nvalid * D; idx += NW * 64) {
+    const int h = idx / D, dv = idx - h * D;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, ((const TDIST_AS3 float*)(smem3 + w * C::kWaveBytes))[h]);
+    float L = 0.f, O = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const TDIST_AS3 float* wm = (const TDIST_AS3 float*)(smem3 + w * C::kWaveBytes);
+      const float mw = wm[h];
+      const float sc = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - M);
+      L += wm[16 + h] * sc;
+      O += wm[32 + dv * 16 + h] * sc;
+    }
+    out_base[(int64_t)h * prm.S * D + dv] = O / L;
+    if (dv == 0) lse_base[(int64_t)h * prm.S] = (M + log2f(L)) * kLn2;
+  }
+}
+
+// ---- combine --------------------------------------------------------------------------------------
+struct CombineParams {
+  const unsigned char* part;
+  const float* lse;
+  const int32_t* lens;
+  unsigned char* out;
+  float* lse_out;
+  int P, mode, B, Hq, Dv;
+  int part_dtype, out_dtype;
+  int64_t p_sp, p_sb, p_sh;  // element strides
+  int64_t l_sp, l_sb, l_sh;
+  int64_t o_sb, o_sh;
+};
+
+__device__ __forceinline__ float load_elem(const unsigned char* base, int64_t idx, int dtype) {
+  if (dtype == TDIST_F32) return ((const float*)base)[idx];
+  const uint32_t bits = ((const unsigned short*)base)[idx];
+  return dtype == TDIST_BF16 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
+}
+__device__ __forceinline__ void store_elem(unsigned char* base, int64_t idx, int dtype, float v) {
+  if (dtype == TDIST_F32) ((float*)base)[idx] = v;
+  else if (dtype == TDIST_BF16) ((unsigned short*)base)[idx] = (unsigned short)f32_to_bf16_bits(v);
+  else ((unsigned short*)base)[idx] = (unsigned short)(pack_f16x2(v, 0.f) & 0xffffu);
+}
+
+// One wave per (b,h); lanes stride over Dv. Partial j is weighted by exp(lse_j - max).
+__global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams prm) {
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int64_t bh = (int64_t)blockIdx.x * 4 + wave;
+  if (bh >= (int64_t)prm.B * prm.Hq) return;
+  const int b = (int)(bh / prm.Hq);
+  const int h = (int)(bh - (int64_t)b * prm.Hq);
+  auto skipped = [&](int j) -> bool {
+    if (prm.mode == 1) {
+      const int len = prm.lens[b];
+      const int per = (len + prm.P - 1) / prm.P;
+      const int st = per * j;
+      return min(st + per, len) <= st;
+    }
+    if (prm.mode == 2) return prm.lens[(int64_t)j * prm.B + b] == 0;
+    return false;
+  };
+  const float* lse = prm.lse + (int64_t)b * prm.l_sb + (int64_t)h * prm.l_sh;
+  float M = -INFINITY;
+  for (int j = 0; j < prm.P; ++j)
+    if (!skipped(j)) M = fmaxf(M, lse[(int64_t)j * prm.l_sp]);
+  float L = 0.f;
+  constexpr int kMaxPerLane = 4;  // Dv <= 256
+  float acc[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f};
+  if (M != -INFINITY) {
+    for (int j = 0; j < prm.P; ++j) {
+      if (skipped(j)) continue;
+      const float lj = lse[(int64_t)j * prm.l_sp];
+      if (lj == -INFINITY) continue;
+      const float w = __expf(lj - M);
+      L += w;
+      const int64_t base = (int64_t)j * prm.p_sp + (int64_t)b * prm.p_sb + (int64_t)h * prm.p_sh;
+#pragma unroll
+      for (int u = 0; u < kMaxPerLane; ++u) {
+        const int d = lane + u * 64;
+        if (d < prm.Dv) acc[u] += w * load_elem(prm.part, base + d, prm.part_dtype);
+      }
+    }
+  }
+  const int64_t obase = (int64_t)b * prm.o_sb + (int64_t)h * prm.o_sh;
+#pragma unroll
+  for (int u = 0; u < kMaxPerLane; ++u) {
+    const int d = lane + u * 64;
+    if (d < prm.Dv) store_elem(prm.out, obase + d, prm.out_dtype, L > 0.f ? acc[u] / L : 0.f);
+  }
+  if (prm.lse_out && lane == 0) prm.lse_out[bh] = L > 0.f ? M + logf(L) : -INFINITY;
+}
+
+template <typename MMA, int D, int NW, int NST, bool kSoftCap>
+static int launch_decode_sc(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
+  typedef DecodeCfg<D, NST> C;
+  const size_t lds = (size_t)NW * C::kWaveBytes;
+  auto kern = decode_split_kv_kernel<MMA, D, NW, NST, kSoftCap>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail(TDIST_ERR_LAUNCH, "decode: cannot reserve %zu B of LDS: %s", lds, hipGetErrorString(e));
+    attr_set = true;
+  }
+  dim3 grid(prm.S, prm.Hkv * head_blocks, prm.B);
+  hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, prm);
+  return launch_status("tdist_decode_split_kv");
+}
+
+template <typename MMA, int D, int NW, int NST>
+static int launch_decode(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
+  return prm.soft_cap > 0.f ? launch_decode_sc<MMA, D, NW, NST, true>(prm, head_blocks, stream)
+                            : launch_decode_sc<MMA, D, NW, NST, false>(prm, head_blocks, stream);
+}
+
+}  // namespace tdist
+
+using namespace tdist;
+
+extern "C" {
+
+int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cache, float* out_split, float* lse_split,
+                          float sm_scale, float soft_cap, const int32_t* block_table, const int32_t* kv_lens, int batch,
+                          int q_heads, int kv_heads, int head_dim, int page_size, int num_splits, int64_t q_stride_b,
+                          int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_token, int64_t k_stride_head,
+                          int64_t v_stride_page, int64_t v_stride_token, int64_t v_stride_head, int64_t table_stride,
+                          int dtype, void* stream) {
+  if (!q || !k_cache || !v_cache || !out_split || !lse_split || !block_table || !kv_lens)
+    return fail(TDIST_ERR_INVALID, "tdist_decode_split_kv: null pointer");
+  if (batch <= 0 || q_heads <= 0 || kv_heads <= 0 || page_size <= 0 || num_splits <= 0)
+    return fail(TDIST_ERR_INVALID, "tdist_decode_split_kv: sizes must be positive");
+  if (q_heads % kv_heads != 0)
+    return fail(TDIST_ERR_INVALID, "tdist_decode_split_kv: q_heads %d not a multiple of kv_heads %d", q_heads, kv_heads);
+  if (dtype != TDIST_BF16 && dtype != TDIST_F16)
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: dtype %d (bf16 and f16 only)", dtype);
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: head_dim %d (64, 128, 256 only)", head_dim);
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (q_stride_b % 8) || (q_stride_h % 8) ||
+      (k_stride_page % 8) || (k_stride_token % 8) || (k_stride_head % 8) || (v_stride_page % 8) ||
+      (v_stride_token % 8) || (v_stride_head % 8))
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: q/k/v rows must be 16-byte aligned");
+  if (num_splits > 65535 || batch > 65535) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: grid too large");
+  DecodeParams prm;
+  prm.q = (const unsigned char*)q;
+  prm.k = (const unsigned char*)k_cache;
+  prm.v = (const unsigned char*)v_cache;
+  prm.out = out_split;
+  prm.lse = lse_split;
+  prm.table = block_table;
+  prm.lens = kv_lens;
+  prm.sm_scale = sm_scale;
+  prm.soft_cap = soft_cap;
+  prm.B = batch;
+  prm.Hq = q_heads;
+  prm.Hkv = kv_heads;
+  prm.S = num_splits;
+  prm.page_size = page_size;
+  int lg = 0;
+  while ((1ll << lg) < page_size) ++lg;
+  prm.page_shift = 31 + lg;
+  prm.page_magic = ((1ull << prm.page_shift) + (uint64_t)page_size - 1) / (uint64_t)page_size;
+  prm.q_sb = q_stride_b * 2;
+  prm.q_sh = q_stride_h * 2;
+  prm.k_sp = k_stride_page * 2;
+  prm.k_st = k_stride_token * 2;
+  prm.k_sh = k_stride_head * 2;
+  prm.v_sp = v_stride_page * 2;
+  prm.v_st = v_stride_token * 2;
+  prm.v_sh = v_stride_head * 2;
+  prm.t_s = table_stride;
+  const int group = q_heads / kv_heads;
+  const int head_blocks = (group + 15) / 16;
+  if ((int64_t)kv_heads * head_blocks > 65535) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: too many heads");
+  hipStream_t st = (hipStream_t)stream;
+  const bool bf = dtype == TDIST_BF16;
+  switch (head_dim) {
+    case 64:
+      return bf ? launch_decode<MmaBF16, 64, 4, 4>(prm, head_blocks, st) : launch_decode<MmaF16, 64, 4, 4>(prm, head_blocks, st);
+    case 128:
+      return bf ? launch_decode<MmaBF16, 128, 4, 4>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 4, 4>(prm, head_blocks, st);
+    default:
+      return bf ? launch_decode<MmaBF16, 256, 2, 3>(prm, head_blocks, st) : launch_decode<MmaF16, 256, 2, 3>(prm, head_blocks, st);
+  }
+}
+
+int tdist_decode_combine(const void* part, int part_dtype, const float* lse, int num_partials, int mode,
+                         const int32_t* lens, int batch, int q_heads, int head_dim_v, int64_t part_stride_p,
+                         int64_t part_stride_b, int64_t part_stride_h, int64_t lse_stride_p, int64_t lse_stride_b,
+                         int64_t lse_stride_h, void* out, int out_dtype, int64_t out_stride_b, int64_t out_stride_h,
+                         float* lse_out, void* stream) {
+  if (!part || !lse || !out) return fail(TDIST_ERR_INVALID, "tdist_decode_combine: null pointer");
+  if (num_partials <= 0 || batch <= 0 || q_heads <= 0 || head_dim_v <= 0)
+    return fail(TDIST_ERR_INVALID, "tdist_decode_combine: sizes must be positive");
+  if (head_dim_v > 256) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_combine: head_dim_v %d > 256", head_dim_v);
+  if (mode < 0 || mode > 2 || (mode != 0 && !lens))
+    return fail(TDIST_ERR_INVALID, "tdist_decode_combine: mode %d needs lens", mode);
+  if ((part_dtype != TDIST_F32 && part_dtype != TDIST_BF16 && part_dtype != TDIST_F16) ||
+      (out_dtype != TDIST_F32 && out_dtype != TDIST_BF16 && out_dtype != TDIST_F16))
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_combine: dtype");
+  CombineParams prm;
+  prm.part = (const unsigned char*)part;
+  prm.lse = lse;
+  prm.lens = lens;
+  prm.out = (unsigned char*)out;
+  prm.lse_out = lse_out;
+  prm.P = num_partials;
+  prm.mode = mode;
+  prm.B = batch;
+  prm.Hq = q_heads;
+  prm.Dv = head_dim_v;
+  prm.part_dtype = part_dtype;
+  prm.out_dtype = out_dtype;
+  prm.p_sp = part_stride_p;
+  prm.p_sb = part_stride_b;
+  prm.p_sh = part_stride_h;
+  prm.l_sp = lse_stride_p;
+  prm.l_sb = lse_stride_b;
+  prm.l_sh = lse_stride_h;
+  prm.o_sb = out_stride_b;
+  prm.o_sh = out_stride_h;
+  const int64_t blocks = ceil_div((int64_t)batch * q_heads, 4);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_combine: grid too large");
+  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, prm);
+  return launch_status("tdist_decode_combine");
+}
+
+}  // extern "C"

@@ -1,0 +1,618 @@
+// (a)/(b1) Persistent MFMA tile GEMM for gfx950: C[M,N] = A[M,K] * B[N,K]^T with
+//   - per-chunk gating of A rows on HBM flag words (the AG-GEMM consumer), and/or
+//   - an epilogue that scatters row blocks to per-rank buffers (the GEMM-RS producer).
+//
+// Restates kernel_consumer_gemm_persistent (kernels/amd/all_gather_gemm.py:140-254), wait_eq_sys
+// (kernels/amd/common_ops.py:39-46) and kernel_gemm_rs_producer_fuse_scatter
+// (kernels/amd/gemm_reduce_scatter.py:125-229) as one hand-scheduled kernel:
+//
+//  * workgroup = WM x WN waves, macro tile BM x BN, each wave owns (BM/WM) x (BN/WN) of it as 32x32
+//    MFMA tiles: v_mfma_f32_32x32x16_{bf16,f16} (16 B of K per lane) or v_mfma_f32_32x32x64_f8f6f4
+//    (32 B of K per lane) with fp32 accumulators;
+//  * A and B tiles go HBM/L2 → LDS with asynchronous 16-byte-per-lane LDS-DMA loads into a ring of NST
+//    stages, P = NST-1 tiles in flight; rows are stored with an XOR swizzle of the 16-byte chunk index
+//    so that the ds_read_b128 operand reads are bank-conflict free; the swizzle is applied on the global
+//    side (which chunk a lane fetches) because the DMA writes lanes to consecutive LDS addresses;
+//  * one s_barrier per K tile, placed before the MFMAs of the tile's last K step, so the first operand
+//    reads of the next tile and the DMA refill overlap those MFMAs;
+//  * the MFMA is issued as D^T = B_tile * A_tile^T so that a lane ends up with 4 consecutive columns
+//    of one row; the epilogue stages the tile through LDS and writes full 16-byte vectors per lane;
+//  * persistent grid (one workgroup per CU). The tile schedule is chunk-major in arrival order, and
+//    within a round of concurrently running tiles the workgroups of one XCD (workgroup id mod 8) get a
+//    compact block of tiles so they share A rows and B rows in that XCD's L2.
+#include "common.h"
+
+namespace tdist {
+
+struct GemmParams {
+  const unsigned char* A;        // gathered workspace
+  const unsigned char* A_local;  // own shard or NULL
+  const unsigned char* B;
+  unsigned char* C;              // plain output (scatter_bufs == NULL)
+  void* const* scatter_bufs;     // GEMM-RS: per-owner buffers
+  const float* row_scale;
+  const float* col_scale;
+  const int32_t* flags;
+  const int32_t* chunk_order;
+  int32_t* status;
+  int64_t lda_b, lda_local_b, ldb_b;  // byte strides
+  int64_t ldc;                         // elements
+  int M, N, K;
+  int local_row_begin, local_rows;
+  int m_per_chunk;   // rows per schedule chunk (multiple of BM)
+  int n_chunks;      // ceil(M / m_per_chunk)
+  int chunks_per_rank;
+  int wait_value;
+  int rank, world_size;
+  int order_mode;    // 0 identity, 1 reference AG order, 2 reference RS order (owner = oc+rank+1), 3 explicit
+  int spin_limit;
+  int m_per_rank;    // GEMM-RS
+  int num_xcds;
+};
+
+// Operand fragment of one lane: K bytes [0, kLaneBytes) of one row; chunk0 / chunk1 are LDS addresses of its
+// 16-byte pieces.
+struct ElemBF16 {
+  static constexpr int kBytes = 2;
+  static constexpr int kLaneBytes = 16;  // K bytes one lane feeds to one MFMA
+  typedef int4v frag;
+  __device__ static __forceinline__ frag load(const TDIST_AS3 unsigned char* c0, const TDIST_AS3 unsigned char*) {
+    return *(const TDIST_AS3 int4v*)c0;
+  }
+  __device__ static __forceinline__ float16v mma(frag a, frag b, float16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8v, a), __builtin_bit_cast(bf16x8v, b), c, 0,
+                                                   0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pack(float a, float b) { return pack_bf16x2(a, b); }
+};
+struct ElemF16 {
+  static constexpr int kBytes = 2;
+  static constexpr int kLaneBytes = 16;
+  typedef int4v frag;
+  __device__ static __forceinline__ frag load(const TDIST_AS3 unsigned char* c0, const TDIST_AS3 unsigned char*) {
+    return *(const TDIST_AS3 int4v*)c0;
+  }
+  __device__ static __forceinline__ float16v mma(frag a, frag b, float16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8v, a), __builtin_bit_cast(f16x8v, b), c, 0, 0,
+                                                  0);
+  }
+  __device__ static __forceinline__ uint32_t pack(float a, float b) { return pack_f16x2(a, b); }
+};
+struct ElemFP8 {
+  static constexpr int kBytes = 1;
+  static constexpr int kLaneBytes = 32;
+  typedef int8v frag;
+  __device__ static __forceinline__ frag load(const TDIST_AS3 unsigned char* c0, const TDIST_AS3 unsigned char* c1) {
+    const int4v lo = *(const TDIST_AS3 int4v*)c0;
+    const int4v hi = *(const TDIST_AS3 int4v*)c1;
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+  __device__ static __forceinline__ float16v mma(frag a, frag b, float16v c) {
+    // cbsz = 0 / blgp = 0 select e4m3 for both operands; scales are 2^0
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pack(float a, float b) { return pack_bf16x2(a, b); }  // bf16 output
+};
+
+// KB = bytes of K per tile row. Chunk c (16 B) of row r is stored at position c ^ swz(r).
+template <int KB>
+__host__ __device__ constexpr int swz(int r) {
+  return KB >= 128 ? (r & 7) : ((r >> 1) & 3);
+}
+
+template <typename E, int BM, int BN, int KB, int WM, int WN, int NST>
+struct GemmCfg {
+  static constexpr int kWaves = WM * WN;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int kChunksPerRow = KB / 16;
+  static constexpr int kRowsPerInstr = 64 / kChunksPerRow;
+  static constexpr int kAInstr = BM / kRowsPerInstr / kWaves;  // DMA instructions per wave per tile
+  static constexpr int kBInstr = BN / kRowsPerInstr / kWaves;
+  static constexpr int kLoadsPerTile = kAInstr + kBInstr;
+  static constexpr int kABytes = BM * KB;
+  static constexpr int kBBytes = BN * KB;
+  static constexpr int kStageBytes = kABytes + kBBytes;
+  static constexpr int kP = NST - 1;
+  static constexpr int kKSteps = KB / (2 * E::kLaneBytes);
+  static constexpr int kFragVecs = E::kLaneBytes / 16;  // 16-byte pieces per operand fragment (1 or 2)
+  static constexpr int kWaveM = BM / WM, kWaveN = BN / WN;
+  static constexpr int kTM = kWaveM / 32, kTN = kWaveN / 32;
+  static constexpr int kLdsBytes = NST * kStageBytes;
+  // epilogue staging: per wave kWaveM rows of kWaveN 16-bit outputs; 16-byte chunk c of row r sits at
+  // position c ^ (r & kEpiSwz) so that the 32 rows one store instruction touches spread over the banks
+  static constexpr int kEpiPitch = kWaveN * 2;
+  static constexpr int kEpiBytes = kWaveM * kEpiPitch;
+  static constexpr int kEpiSwz = (kEpiPitch / 16 < 16 ? kEpiPitch / 16 : 16) - 1;
+  // MFMAs of a K step issued before the next step's operand reads
+  static constexpr int kLeadMfma = (kTM * kTN >= 8) ? 4 : 1;
+  static_assert(KB == 64 || KB == 128, "tile rows of 64 or 128 bytes");
+  static_assert(BM % (kRowsPerInstr * kWaves) == 0 && BN % (kRowsPerInstr * kWaves) == 0, "tile/wave split");
+  static_assert(kP >= 1 && kP <= 3 && kP * kLoadsPerTile < 64, "vmcnt budget");
+  static_assert(kEpiBytes * kWaves <= kLdsBytes, "epilogue staging must fit in the stage ring");
+  static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "wave tile");
+};
+
+template <int N>
+__device__ __forceinline__ void wait_tiles_and_barrier(int rem) {
+  // rem = tiles younger than the awaited one that may stay in flight (0..2)
+  if (rem >= 2) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(2 * N < 64 ? 2 * N : 63) : "memory");
+  else if (rem == 1) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// schedule position → chunk id
+__device__ __forceinline__ int chunk_of(const GemmParams& p, int oc) {
+  switch (p.order_mode) {
+    case 1: {  // own rank's chunks first, then rank+1, ... one chunk of every rank per sweep
+      const int sweep = oc / p.world_size;
+      const int r = (oc % p.world_size + p.rank) % p.world_size;
+      return r * p.chunks_per_rank + sweep;
+    }
+    case 2:  // row blocks of rank+1 first
+      return (oc + p.rank + 1) % p.world_size;
+    case 3:
+      return p.chunk_order[oc];
+    default:
+      return oc;
+  }
+}
+
+template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales>
+__global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams p) {
+  typedef GemmCfg<E, BM, BN, KB, WM, WN, NST> C;
+  typedef TDIST_AS3 unsigned char* lds_u8;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem_generic[];
+  lds_u8 const smem = (lds_u8)smem_generic;
+  __shared__ int s_gate;  // 1 = tile may proceed, 0 = wait expired
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int wm = wave / WN, wn = wave % WN;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  const int num_pid_m = (p.M + BM - 1) / BM;
+  const int num_pid_n = (p.N + BN - 1) / BN;
+  const int cm = p.m_per_chunk / BM;                 // row tiles per chunk
+  const int tiles_per_chunk = cm * num_pid_n;
+  const int total_sched = p.n_chunks * tiles_per_chunk;
+  const int G = gridDim.x;
+  const int KT = p.K * E::kBytes / KB;
+
+  // DMA lane roles: row within an instruction's row group, and the LDS chunk position it fills
+  const int dma_row = lane / C::kChunksPerRow;
+  const int dma_pos = lane % C::kChunksPerRow;
+
+  for (int sbase = 0; sbase < total_sched; sbase += G) {
+    // XCD-aware position within the round: workgroups of XCD x take a contiguous range
+    int u = blockIdx.x;
+    if (p.num_xcds > 1 && G % p.num_xcds == 0) u = (u % p.num_xcds) * (G / p.num_xcds) + u / p.num_xcds;
+    const int sidx = sbase + u;
+    if (sidx >= total_sched) continue;
+    const int oc = sidx / tiles_per_chunk;
+    const int within = sidx - oc * tiles_per_chunk;
+    const int chunk = chunk_of(p, oc);
+    const int pid_m = chunk * cm + within % cm;
+    const int pid_n = within / cm;
+    if (pid_m >= num_pid_m) continue;
+    const int m0 = pid_m * BM, n0 = pid_n * BN;
+
+    // ---- gate ---------------------------------------------------------------------------------
+    const bool is_local = p.A_local != nullptr && m0 >= p.local_row_begin && m0 < p.local_row_begin + p.local_rows;
+    if (p.flags != nullptr && !is_local) {
+      if (threadIdx.x == 0) {
+        const int32_t* f = p.flags + chunk;
+        int ok = 0;
+        int limit = p.spin_limit;
+        if (p.status != nullptr && __hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) limit = 1;
+        for (int it = 0; it < limit; ++it) {
+          if (__hip_atomic_load(f, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == p.wait_value) {
+            ok = 1;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(4);
+        }
+        if (!ok && p.status != nullptr) {
+          if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = chunk;
+        }
+        s_gate = ok;
+      }
+      __syncthreads();
+      const int ok = s_gate;
+      __syncthreads();
+      if (!ok) continue;
+    }
+
+    const unsigned char* Arows = is_local ? p.A_local : p.A;
+    const int64_t a_ld = is_local ? p.lda_local_b : p.lda_b;
+    const int a_row_off = is_local ? p.local_row_begin : 0;
+    const int a_row_max = is_local ? p.local_rows - 1 : p.M - 1;
+
+    // per-lane byte offsets (relative to row 0 / column 0 of the matrix) of this lane's DMA sources
+    int64_t a_off[C::kAInstr], b_off[C::kBInstr];
+#pragma unroll
+    for (int t = 0; t < C::kAInstr; ++t) {
+      const int r = (wave * C::kAInstr + t) * C::kRowsPerInstr + dma_row;  // row within the tile
+      const int gr = min(m0 + r - a_row_off, a_row_max);
+      a_off[t] = (int64_t)gr * a_ld + ((dma_pos ^ swz<KB>(r)) << 4);
+    }
+#pragma unroll
+    for (int t = 0; t < C::kBInstr; ++t) {
+      const int r = (wave * C::kBInstr + t) * C::kRowsPerInstr + dma_row;
+      const int gr = min(n0 + r, p.N - 1);
+      b_off[t] = (int64_t)gr * p.ldb_b + ((dma_pos ^ swz<KB>(r)) << 4);
+    }
+
+    auto issue_tile = [&](int kt) {
+      lds_u8 const sa = smem + (kt % NST) * C::kStageBytes;
+      lds_u8 const sb = sa + C::kABytes;
+      const int64_t kb = (int64_t)kt * KB;
+#pragma unroll
+      for (int t = 0; t < C::kAInstr; ++t)
+        __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(Arows + a_off[t] + kb),
+                                         (TDIST_AS3 void*)(sa + (wave * C::kAInstr + t) * 1024), 16, 0, 0);
+#pragma unroll
+      for (int t = 0; t < C::kBInstr; ++t)
+        __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(p.B + b_off[t] + kb),
+                                         (TDIST_AS3 void*)(sb + (wave * C::kBInstr + t) * 1024), 16, 0, 0);
+    };
+
+    // operand fragments: row (32*i + l32) of the wave's strip, K bytes [ks*2L + lh*L, +L), L = kLaneBytes
+    // operand fragments of the K step being multiplied (cur) and of the one after it (nxt)
+    typename E::frag a_cur[C::kTM], b_cur[C::kTN], a_nxt[C::kTM], b_nxt[C::kTN];
+    auto load_frags = [&](int kt, int ks, typename E::frag* af, typename E::frag* bf) {
+      lds_u8 const sa = smem + (kt % NST) * C::kStageBytes;
+      lds_u8 const sb = sa + C::kABytes;
+      const int c0 = (ks * 2 + lh) * C::kFragVecs;  // first 16-byte chunk of this lane's K bytes
+      const int c1 = c0 + C::kFragVecs - 1;         // last one (== c0 for 16-byte fragments)
+#pragma unroll
+      for (int i = 0; i < C::kTM; ++i) {
+        const int r = wm * C::kWaveM + i * 32 + l32;
+        lds_u8 const row = sa + r * KB;
+        af[i] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
+      }
+#pragma unroll
+      for (int j = 0; j < C::kTN; ++j) {
+        const int r = wn * C::kWaveN + j * 32 + l32;
+        lds_u8 const row = sb + r * KB;
+        bf[j] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
+      }
+    };
+
+    float16v acc[C::kTN][C::kTM];
+#pragma unroll
+    for (int j = 0; j < C::kTN; ++j)
+#pragma unroll
+      for (int i = 0; i < C::kTM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][i][e] = 0.f;
+
+    // ---- prologue: P tiles in flight, wait for tile 0 ------------------------------------------
+#pragma unroll
+    for (int t = 0; t < C::kP; ++t)
+      if (t < KT) issue_tile(t);
+    wait_tiles_and_barrier<C::kLoadsPerTile>(min(C::kP - 1, KT - 1));
+    if (C::kP < KT) issue_tile(C::kP);
+    load_frags(0, 0, a_cur, b_cur);
+
+    // ---- main loop over K tiles -----------------------------------------------------------------
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+      for (int ks = 0; ks < C::kKSteps; ++ks) {
+        // A few MFMAs of this step go first: the wait the compiler puts in front of them then only covers
+        // operand reads issued a whole step ago, and the reads issued below have the rest of the step's
+        // MFMAs to complete.
+#pragma unroll
+        for (int idx = 0; idx < C::kLeadMfma; ++idx) {
+          const int j = idx / C::kTM, i = idx % C::kTM;
+          acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks + 1 < C::kKSteps) {
+          load_frags(kt, ks + 1, a_nxt, b_nxt);
+        } else if (kt + 1 < KT) {
+          // tile kt+1 must have landed; tiles kt+2 .. kt+P may stay in flight
+          wait_tiles_and_barrier<C::kLoadsPerTile>(min(C::kP - 1, KT - 2 - kt));
+          if (kt + 1 + C::kP < KT) issue_tile(kt + 1 + C::kP);
+          load_frags(kt + 1, 0, a_nxt, b_nxt);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int idx = C::kLeadMfma; idx < C::kTN * C::kTM; ++idx) {
+          const int j = idx / C::kTM, i = idx % C::kTM;
+          acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+        }
+#pragma unroll
+        for (int i = 0; i < C::kTM; ++i) a_cur[i] = a_nxt[i];
+#pragma unroll
+        for (int j = 0; j < C::kTN; ++j) b_cur[j] = b_nxt[j];
+      }
+    }
+
+    // ---- epilogue ---------------------------------------------------------------------------------
+    // acc[j][i][e]: output row m = wm*kWaveM + 32i + l32, column n = wn*kWaveN + 32j + 8*(e/4) + 4*lh + e%4
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ring is free
+    lds_u8 const epi = smem + wave * C::kEpiBytes;
+#pragma unroll
+    for (int i = 0; i < C::kTM; ++i) {
+      const int mrow = 32 * i + l32;
+      float rs = 1.f;
+      if (kScales && p.row_scale) rs = p.row_scale[min(m0 + wm * C::kWaveM + mrow, p.M - 1)];
+#pragma unroll
+      for (int j = 0; j < C::kTN; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int ncol = 32 * j + 8 * q + 4 * lh;
+          float v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2],
+                v3 = acc[j][i][4 * q + 3];
+          if (kScales) {
+            float4v cs = {1.f, 1.f, 1.f, 1.f};
+            if (p.col_scale) {
+              const int gn = n0 + wn * C::kWaveN + ncol;
+              if (gn + 3 < p.N) cs = *(const float4v*)(p.col_scale + gn);
+              else
+                for (int e = 0; e < 4; ++e) cs[e] = p.col_scale[min(gn + e, p.N - 1)];
+            }
+            v0 *= rs * cs[0];
+            v1 *= rs * cs[1];
+            v2 *= rs * cs[2];
+            v3 *= rs * cs[3];
+          }
+          const int2v w = {(int)E::pack(v0, v1), (int)E::pack(v2, v3)};
+          *(TDIST_AS3 int2v*)(epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2) = w;
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the accumulator read-out tile by tile (register pressure)
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // destination of this tile's rows
+    unsigned char* Cbase;
+    int64_t crow0;
+    if (p.scatter_bufs != nullptr) {
+      const int owner = m0 / p.m_per_rank;
+      Cbase = (unsigned char*)p.scatter_bufs[owner];
+      crow0 = (int64_t)p.rank * p.m_per_rank + (m0 - owner * p.m_per_rank);
+    } else {
+      Cbase = p.C;
+      crow0 = m0;
+    }
+    constexpr int kLanesPerRow = C::kWaveN * 2 / 16;  // 16-byte vectors per staged row
+    constexpr int kRowsPerPass = 64 / kLanesPerRow;
+    const int er = lane / kLanesPerRow, ec = lane % kLanesPerRow;
+    const bool n_vec_ok = (p.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(Cbase) & 15) == 0);
+#pragma unroll 4
+    for (int pass = 0; pass < C::kWaveM / kRowsPerPass; ++pass) {
+      const int mrow = pass * kRowsPerPass + er;
+      const int gm = m0 + wm * C::kWaveM + mrow;
+      const int gn = n0 + wn * C::kWaveN + ec * 8;
+      const int4v v = *(const TDIST_AS3 int4v*)(epi + mrow * C::kEpiPitch + ((ec ^ (mrow & C::kEpiSwz)) << 4));
+      if (gm < p.M && gn < p.N) {
+        unsigned short* dst = (unsigned short*)Cbase + (crow0 + wm * C::kWaveM + mrow) * p.ldc + gn;
+        if (gn + 8 <= p.N && n_vec_ok) {
+          *(int4v*)dst = v;
+        } else {
+          for (int e = 0; e < 8; ++e)
+            if (gn + e < p.N) dst[e] = (unsigned short)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+        }
+      }
+    }
+    // the next tile's prologue overwrites the ring: every wave must be done reading its staging area
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------------
+enum GemmElem { kElemBF16, kElemF16, kElemFP8 };
+
+struct GemmCall {
+  const void* A;
+  int64_t lda;
+  const void* A_local;
+  int64_t lda_local;
+  int local_row_begin, local_rows;
+  const void* B;
+  int64_t ldb;
+  void* C;
+  void* const* scatter_bufs;
+  int64_t ldc;
+  int M, N, K;
+  const float* row_scale;
+  const float* col_scale;
+  const int32_t* flags;
+  int m_per_chunk, wait_value;
+  const int32_t* chunk_order;
+  int rank, world_size, spin_limit;
+  int32_t* status;
+  hipStream_t stream;
+  const char* who;
+};
+
+template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales>
+static int launch_gemm_cfg(const GemmParams& prm, int grid, hipStream_t stream, const char* who) {
+  typedef GemmCfg<E, BM, BN, KB, WM, WN, NST> C;
+  auto kern = gemm_kernel<E, BM, BN, KB, WM, WN, NST, kScales>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes);
+    if (e != hipSuccess) return fail(TDIST_ERR_LAUNCH, "%s: cannot reserve %d B of LDS: %s", who, C::kLdsBytes, hipGetErrorString(e));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::kThreads), C::kLdsBytes, stream, prm);
+  return launch_status(who);
+}
+
+static int run_gemm(const GemmCall& c, GemmElem elem) {
+  const char* who = c.who;
+  const int esz = elem == kElemFP8 ? 1 : 2;
+  if (!c.A || !c.B || (!c.C && !c.scatter_bufs)) return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
+  if (c.M <= 0 || c.N <= 0 || c.K <= 0) return fail(TDIST_ERR_INVALID, "%s: M, N, K must be positive", who);
+  if (((int64_t)c.K * esz) % 64 != 0)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: K*elem_size = %lld must be a multiple of 64 bytes", who, (long long)c.K * esz);
+  if (!aligned16(c.A) || !aligned16(c.B) || (c.A_local && !aligned16(c.A_local)) || (c.lda * esz) % 16 ||
+      (c.ldb * esz) % 16 || (c.A_local && (c.lda_local * esz) % 16))
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: A/B bases and row strides must be 16-byte aligned", who);
+  if (c.lda < c.K || c.ldb < c.K || c.ldc < c.N) return fail(TDIST_ERR_INVALID, "%s: leading dimension smaller than row", who);
+  const DeviceInfo& di = device_info();
+  if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "%s: current device is not gfx950", who);
+
+  // tile configuration: 256x256 when that fills the chip at least ~1.5 times and the row-block
+  // constraints of the call allow it, else 128x128
+  const int64_t big_tiles = ceil_div(c.M, 256) * ceil_div(c.N, 256);
+  bool big = big_tiles >= (int64_t)di.num_cus * 3 / 2;
+  if (c.scatter_bufs && c.world_size > 0 && (c.M % c.world_size != 0 || (c.M / c.world_size) % 256 != 0)) big = false;
+  if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) big = false;
+  if (c.A_local && (c.local_row_begin % 256 != 0 || c.local_rows % 256 != 0)) big = false;
+  const int BM = big ? 256 : 128;
+
+  GemmParams p;
+  p.A = (const unsigned char*)c.A;
+  p.A_local = (const unsigned char*)c.A_local;
+  p.B = (const unsigned char*)c.B;
+  p.C = (unsigned char*)c.C;
+  p.scatter_bufs = c.scatter_bufs;
+  p.row_scale = c.row_scale;
+  p.col_scale = c.col_scale;
+  p.flags = c.flags;
+  p.chunk_order = c.chunk_order;
+  p.status = c.status;
+  p.lda_b = c.lda * esz;
+  p.lda_local_b = c.lda_local * esz;
+  p.ldb_b = c.ldb * esz;
+  p.ldc = c.ldc;
+  p.M = c.M;
+  p.N = c.N;
+  p.K = c.K;
+  p.local_row_begin = c.A_local ? c.local_row_begin : 0;
+  p.local_rows = c.A_local ? c.local_rows : 0;
+  p.wait_value = c.wait_value;
+  p.rank = c.rank;
+  p.world_size = c.world_size;
+  p.spin_limit = c.spin_limit > 0 ? c.spin_limit : (1 << 22);  // ~seconds of polling
+  p.num_xcds = di.num_xcds;
+  p.m_per_rank = 0;
+  p.chunks_per_rank = 1;
+
+  if (c.scatter_bufs) {
+    if (c.world_size <= 0 || c.rank < 0 || c.rank >= c.world_size)
+      return fail(TDIST_ERR_INVALID, "%s: rank %d / world_size %d", who, c.rank, c.world_size);
+    if (c.M % c.world_size != 0 || (c.M / c.world_size) % BM != 0)
+      return fail(TDIST_ERR_UNSUPPORTED, "%s: M/world_size = %d must be a multiple of the %d-row tile", who,
+                  c.M / c.world_size, BM);
+    p.m_per_rank = c.M / c.world_size;
+    p.m_per_chunk = p.m_per_rank;
+    p.n_chunks = c.world_size;
+    p.order_mode = 2;
+    p.flags = nullptr;
+  } else if (c.flags) {
+    if (c.m_per_chunk <= 0 || c.m_per_chunk % BM != 0)
+      return fail(TDIST_ERR_UNSUPPORTED, "%s: m_per_chunk %d must be a positive multiple of the %d-row tile", who,
+                  c.m_per_chunk, BM);
+    p.m_per_chunk = c.m_per_chunk;
+    p.n_chunks = (int)ceil_div(c.M, c.m_per_chunk);
+    if (c.A_local && (c.local_row_begin % BM != 0 || c.local_rows % BM != 0))
+      return fail(TDIST_ERR_UNSUPPORTED, "%s: the local shard must start and end on a %d-row tile", who, BM);
+    if (c.chunk_order) {
+      p.order_mode = 3;
+    } else if (c.world_size > 1 && c.M % c.world_size == 0 && (c.M / c.world_size) % c.m_per_chunk == 0 &&
+               c.rank >= 0 && c.rank < c.world_size) {
+      p.order_mode = 1;
+      p.chunks_per_rank = (c.M / c.world_size) / c.m_per_chunk;
+    } else {
+      p.order_mode = 0;
+    }
+  } else {
+    // plain GEMM: schedule in groups of 4 row tiles
+    p.m_per_chunk = BM * 4;
+    p.n_chunks = (int)ceil_div(c.M, p.m_per_chunk);
+    p.order_mode = 0;
+    if (c.A_local && (c.local_row_begin % BM != 0 || c.local_rows % BM != 0))
+      return fail(TDIST_ERR_UNSUPPORTED, "%s: the local shard must start and end on a %d-row tile", who, BM);
+  }
+  const int64_t sched = (int64_t)p.n_chunks * (p.m_per_chunk / BM) * ceil_div(c.N, BM);
+  if (sched > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many tiles", who);
+  const int grid = (int)(sched < di.num_cus ? sched : di.num_cus);
+  const bool scales = elem == kElemFP8 && (c.row_scale || c.col_scale);
+
+  if (big) {
+    switch (elem) {
+      case kElemBF16: return launch_gemm_cfg<ElemBF16, 256, 256, 64, 2, 2, 4, false>(p, grid, c.stream, who);
+      case kElemF16: return launch_gemm_cfg<ElemF16, 256, 256, 64, 2, 2, 4, false>(p, grid, c.stream, who);
+      default:
+        return scales ? launch_gemm_cfg<ElemFP8, 256, 256, 64, 2, 2, 4, true>(p, grid, c.stream, who)
+                      : launch_gemm_cfg<ElemFP8, 256, 256, 64, 2, 2, 4, false>(p, grid, c.stream, who);
+    }
+  }
+  switch (elem) {
+    case kElemBF16: return launch_gemm_cfg<ElemBF16, 128, 128, 64, 2, 2, 4, false>(p, grid, c.stream, who);
+    case kElemF16: return launch_gemm_cfg<ElemF16, 128, 128, 64, 2, 2, 4, false>(p, grid, c.stream, who);
+    default:
+      return scales ? launch_gemm_cfg<ElemFP8, 128, 128, 64, 2, 2, 4, true>(p, grid, c.stream, who)
+                    : launch_gemm_cfg<ElemFP8, 128, 128, 64, 2, 2, 4, false>(p, grid, c.stream, who);
+  }
+}
+
+}  // namespace tdist
+
+using namespace tdist;
+
+#define TDIST_GATED_BODY(ELEM, RS, CS, WHO)                                                                         \
+  GemmCall c;                                                                                                       \
+  c.A = A; c.lda = lda; c.A_local = A_local; c.lda_local = lda_local;                                               \
+  c.local_row_begin = local_row_begin; c.local_rows = local_rows;                                                   \
+  c.B = B; c.ldb = ldb; c.C = C; c.scatter_bufs = nullptr; c.ldc = ldc; c.M = M; c.N = N; c.K = K;                  \
+  c.row_scale = RS; c.col_scale = CS; c.flags = flags; c.m_per_chunk = m_per_chunk; c.wait_value = wait_value;      \
+  c.chunk_order = chunk_order; c.rank = rank; c.world_size = world_size; c.spin_limit = spin_limit;                 \
+  c.status = status; c.stream = (hipStream_t)stream; c.who = WHO;                                                   \
+  return run_gemm(c, ELEM);
+
+extern "C" {
+
+int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
+                                int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C, int64_t ldc,
+                                int M, int N, int K, const int32_t* flags, int m_per_chunk, int wait_value,
+                                const int32_t* chunk_order, int rank, int world_size, int spin_limit, int32_t* status,
+                                void* stream) {
+  TDIST_GATED_BODY(kElemBF16, nullptr, nullptr, "tdist_gemm_chunk_gated_bf16")
+}
+
+int tdist_gemm_chunk_gated_f16(const void* A, int64_t lda, const void* A_local, int64_t lda_local, int local_row_begin,
+                               int local_rows, const void* B, int64_t ldb, void* C, int64_t ldc, int M, int N, int K,
+                               const int32_t* flags, int m_per_chunk, int wait_value, const int32_t* chunk_order,
+                               int rank, int world_size, int spin_limit, int32_t* status, void* stream) {
+  TDIST_GATED_BODY(kElemF16, nullptr, nullptr, "tdist_gemm_chunk_gated_f16")
+}
+
+int tdist_gemm_chunk_gated_fp8e4m3(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
+                                   int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
+                                   int64_t ldc, int M, int N, int K, const float* row_scale, const float* col_scale,
+                                   const int32_t* flags, int m_per_chunk, int wait_value, const int32_t* chunk_order,
+                                   int rank, int world_size, int spin_limit, int32_t* status, void* stream) {
+  TDIST_GATED_BODY(kElemFP8, row_scale, col_scale, "tdist_gemm_chunk_gated_fp8e4m3")
+}
+
+static int gemm_rs_scatter(GemmElem elem, const void* A, int64_t lda, const void* B, int64_t ldb,
+                           void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank, int world_size,
+                           void* stream, const char* who) {
+  if (!scatter_bufs) return fail(TDIST_ERR_INVALID, "%s: null scatter_bufs", who);
+  GemmCall c;
+  c.A = A; c.lda = lda; c.A_local = nullptr; c.lda_local = 0; c.local_row_begin = 0; c.local_rows = 0;
+  c.B = B; c.ldb = ldb; c.C = nullptr; c.scatter_bufs = scatter_bufs; c.ldc = ldc; c.M = M; c.N = N; c.K = K;
+  c.row_scale = nullptr; c.col_scale = nullptr; c.flags = nullptr; c.m_per_chunk = 0; c.wait_value = 0;
+  c.chunk_order = nullptr; c.rank = rank; c.world_size = world_size; c.spin_limit = 0; c.status = nullptr;
+  c.stream = (hipStream_t)stream; c.who = who;
+  return run_gemm(c, elem);
+}
+
+int tdist_gemm_rs_scatter_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, void* const* scatter_bufs,
+                               int64_t ldc, int M, int N, int K, int rank, int world_size, void* stream) {
+  return gemm_rs_scatter(kElemBF16, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, stream,
+                         "tdist_gemm_rs_scatter_bf16");
+}
+
+int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t ldb, void* const* scatter_bufs,
+                              int64_t ldc, int M, int N, int K, int rank, int world_size, void* stream) {
+  return gemm_rs_scatter(kElemF16, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, stream,
+                         "tdist_gemm_rs_scatter_f16");
+}
+
+}  // extern "C"

@@ -1,0 +1,497 @@
+// (c) MoE low-latency dispatch / combine permute on one GPU.
+//
+// Index construction (splits, cumsum, stable scatter index, gather index) is a stable counting sort
+// of the flat [T*topk] expert ids, restating in parallel form what the reference does with
+//   torch.bincount / cumsum / argsort(stable).argsort()      test/nvidia/test_all_to_all.py:42-46,95-96,314
+//   calc_gather_index                                         test/nvidia/test_all_to_all.py:49-92
+// Three launches: per-block histograms, one scan block, per-block ranking. Inside a wave the rank of
+// an entry among equal ids is found with ballots (one per id bit), so no sort is involved and the
+// order of equal ids is their flat order (stability).
+//
+// Row movement restates all_to_all_kernel (kernels/nvidia/low_latency_all_to_all.py:56-103): the rows
+// of destination d are contiguous in the sorted order, and land in that destination's receive slot.
+#include "common.h"
+
+namespace tdist {
+
+constexpr int kMoeThreads = 256;              // 4 waves
+constexpr int kMoeItemsPerBlock = 1024;       // ids ranked by one block (256 per wave)
+constexpr int kMoeMaxExperts = 4096;          // LDS: 4 waves * G * 4 B
+constexpr int kScanThreads = 1024;
+
+__host__ __device__ static inline int id_bits(int g) {
+  int b = 1;
+  while ((1 << b) < g) ++b;
+  return b;
+}
+
+// hist[b][g] = #ids equal to g among block b's items.
+__global__ __launch_bounds__(kMoeThreads) void moe_hist_kernel(const int32_t* __restrict__ ids, int64_t n, int G,
+                                                              int32_t* __restrict__ hist) {
+  extern __shared__ int32_t s_hist[];
+  for (int g = threadIdx.x; g < G; g += kMoeThreads) s_hist[g] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kMoeItemsPerBlock;
+#pragma unroll
+  for (int u = 0; u < kMoeItemsPerBlock / kMoeThreads; ++u) {
+    const int64_t i = base + u * kMoeThreads + threadIdx.x;
+    if (i < n) {
+      const int e = ids[i];
+      if (e >= 0 && e < G) atomicAdd(&s_hist[e], 1);
+    }
+  }
+  __syncthreads();
+  int32_t* out = hist + (int64_t)blockIdx.x * G;
+  for (int g = threadIdx.x; g < G; g += kMoeThreads) out[g] = s_hist[g];
+}
+
+// One block. Turns hist[b][g] into the exclusive prefix over b, writes splits[g] and cumsum[0..G].
+// splits is never NULL here: the host substitutes a row of the workspace when the caller has none.
+__global__ __launch_bounds__(kScanThreads) void moe_scan_kernel(int32_t* __restrict__ hist, int num_blocks, int G,
+                                                               int32_t* __restrict__ splits,
+                                                               int32_t* __restrict__ cumsum) {
+  __shared__ int32_t s_part[kScanThreads];
+  const int per = (G + kScanThreads - 1) / kScanThreads;  // consecutive experts per thread
+  const int g0 = threadIdx.x * per;
+  int32_t local_total = 0;
+  for (int j = 0; j < per; ++j) {
+    const int g = g0 + j;
+    if (g < G) {
+      int32_t run = 0;
+      for (int b = 0; b < num_blocks; ++b) {
+        const int64_t at = (int64_t)b * G + g;
+        const int32_t h = hist[at];
+        hist[at] = run;
+        run += h;
+      }
+      splits[g] = run;
+      local_total += run;
+    }
+  }
+  s_part[threadIdx.x] = local_total;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over the per-thread totals.
+  for (int off = 1; off < kScanThreads; off <<= 1) {
+    int32_t v = (threadIdx.x >= off) ? s_part[threadIdx.x - off] : 0;
+    __syncthreads();
+    s_part[threadIdx.x] += v;
+    __syncthreads();
+  }
+  int32_t run = s_part[threadIdx.x] - local_total;  // exclusive prefix of this thread's first expert
+  if (threadIdx.x == 0) cumsum[0] = 0;
+  for (int j = 0; j < per; ++j) {
+    const int g = g0 + j;
+    if (g < G) {
+      run += splits[g];
+      cumsum[g + 1] = run;
+    }
+  }
+}
+
+// Ranks block b's items. base position of expert g for wave w of block b =
+//   cumsum[g] + hist[b][g] (items of earlier blocks) + items of earlier waves of this block.
+__global__ __launch_bounds__(kMoeThreads) void moe_rank_kernel(const int32_t* __restrict__ ids, int64_t n, int topk,
+                                                              int G, int nbits, const int32_t* __restrict__ hist,
+                                                              const int32_t* __restrict__ cumsum,
+                                                              int32_t* __restrict__ scatter_idx,
+                                                              int32_t* __restrict__ gather_idx,
+                                                              int32_t* __restrict__ topk_idx) {
+  extern __shared__ int32_t s_cnt[];  // [4][G]
+  constexpr int kWaves = kMoeThreads / 64;
+  constexpr int kPerWave = kMoeItemsPerBlock / kWaves;
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  for (int g = threadIdx.x; g < kWaves * G; g += kMoeThreads) s_cnt[g] = 0;
+  __syncthreads();
+  const int64_t wbase = (int64_t)blockIdx.x * kMoeItemsPerBlock + wave * kPerWave;
+  int32_t* my_cnt = s_cnt + wave * G;
+  // Pass 1: per-wave counts.
+#pragma unroll
+  for (int u = 0; u < kPerWave / 64; ++u) {
+    const int64_t i = wbase + u * 64 + lane;
+    if (i < n) {
+      const int e = ids[i];
+      if (e >= 0 && e < G) atomicAdd(&my_cnt[e], 1);
+    }
+  }
+  __syncthreads();
+  // Pass 2: counts → base positions (exclusive over waves, plus the block and expert offsets).
+  const int32_t* bh = hist + (int64_t)blockIdx.x * G;
+  for (int g = threadIdx.x; g < G; g += kMoeThreads) {
+    int32_t run = cumsum[g] + bh[g];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const int32_t c = s_cnt[w * G + g];
+      s_cnt[w * G + g] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  // Pass 3: walk the wave's items in flat order, 64 at a time.
+  volatile int32_t* pos = my_cnt;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int u = 0; u < kPerWave / 64; ++u) {
+    const int64_t i = wbase + u * 64 + lane;
+    int e = -1;
+    if (i < n) {
+      e = ids[i];
+      if (e < 0 || e >= G) e = -1;
+    }
+    const bool valid = e >= 0;
+    uint64_t peers = __ballot(valid);
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = (e >> b) & 1;
+      const uint64_t m = __ballot(valid && bit);
+      peers &= bit ? m : ~m;
+    }
+    if (valid) {
+      const int32_t start = pos[e];
+      const int rank_in = __popcll(peers & lt_mask);
+      const int32_t p = start + rank_in;
+      scatter_idx[i] = p;
+      gather_idx[p] = (int32_t)(i / topk);
+      if (topk_idx) topk_idx[p] = (int32_t)(i % topk);
+    } else if (i < n) {
+      scatter_idx[i] = -1;
+    }
+    // every lane of the wave has read pos[] before the leaders advance it
+    __builtin_amdgcn_wave_barrier();
+    if (valid && (peers & lt_mask) == 0) pos[e] = pos[e] + __popcll(peers);
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// ---- row movement ------------------------------------------------------------------------------
+
+// Finds d with bound[d] <= p < bound[d+1] in a non-decreasing bound[0..W] with bound[W] > p.
+__device__ __forceinline__ int find_dest(const int32_t* bound, int stride, int W, int32_t p) {
+  int lo = 0, hi = W;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (bound[mid * stride] <= p) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+constexpr int kRowsPerWave = 2;
+constexpr int kRowsPerBlock = 4 * kRowsPerWave;  // 4 waves
+
+// Copies up to kRowsPerWave rows of n16 16-byte chunks; all loads of a 512-chunk window are issued
+// before its stores so each lane keeps up to 16 vectors in flight.
+__device__ __forceinline__ void copy_rows_vec(const int4v* const* src, int4v* const* dst, const bool* has, int n16,
+                                              int lane) {
+  for (int base = 0; base < n16; base += 8 * 64) {
+    int4v v[kRowsPerWave][8];
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) {
+      if (has[r]) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int c = base + j * 64 + lane;
+          if (c < n16) v[r][j] = __builtin_nontemporal_load(src[r] + c);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) {
+      if (has[r]) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int c = base + j * 64 + lane;
+          if (c < n16) __builtin_nontemporal_store(v[r][j], dst[r] + c);
+        }
+      }
+    }
+  }
+}
+
+// kFromSlots = false: dispatch (sorted/gathered rows → slots); true: post-process (slots → compact).
+// s_bound[d] = first sorted row of destination d, s_bound[W] = total.
+template <bool kVec16, bool kFromSlots>
+__global__ __launch_bounds__(256) void moe_rows_kernel(const unsigned char* __restrict__ in_rows, int64_t row_bytes,
+                                                       const float* __restrict__ in_scales,
+                                                       const int32_t* __restrict__ gather_idx,
+                                                       const int32_t* __restrict__ counts, int64_t n_rows, int W,
+                                                       int Er, int max_m, unsigned char* __restrict__ out_rows,
+                                                       float* __restrict__ out_scales,
+                                                       int32_t* __restrict__ splits_out) {
+  extern __shared__ int32_t s_bound[];  // [W+1]
+  if (kFromSlots) {
+    // counts = splits[G]: per-destination totals, then a serial prefix (W is small).
+    for (int d = threadIdx.x; d < W; d += 256) {
+      int32_t t = 0;
+      for (int j = 0; j < Er; ++j) t += counts[d * Er + j];
+      s_bound[d + 1] = t;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      s_bound[0] = 0;
+      for (int d = 0; d < W; ++d) s_bound[d + 1] += s_bound[d];
+    }
+  } else {
+    // counts = cumsum[G+1]
+    for (int d = threadIdx.x; d <= W; d += 256) s_bound[d] = counts[d * Er];
+    if (splits_out && blockIdx.x == 0) {
+      const int G = W * Er;
+      for (int g = threadIdx.x; g < G; g += 256) splits_out[g] = counts[g + 1] - counts[g];
+    }
+  }
+  __syncthreads();
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int32_t total = s_bound[W];
+  const unsigned char* src[kRowsPerWave];
+  unsigned char* dst[kRowsPerWave];
+  bool has[kRowsPerWave];
+#pragma unroll
+  for (int r = 0; r < kRowsPerWave; ++r) {
+    const int64_t p = (int64_t)blockIdx.x * kRowsPerBlock + wave * kRowsPerWave + r;
+    has[r] = false;
+    src[r] = in_rows;
+    dst[r] = out_rows;
+    if (p >= n_rows || p >= total) continue;
+    const int d = find_dest(s_bound, 1, W, (int32_t)p);
+    const int64_t in_slot = p - s_bound[d];
+    if (in_slot >= max_m) continue;
+    const int64_t slot_row = (int64_t)d * max_m + in_slot;
+    int64_t src_row, dst_row;
+    if (kFromSlots) {
+      src_row = slot_row;
+      dst_row = p;
+    } else {
+      src_row = gather_idx ? (int64_t)gather_idx[p] : p;
+      dst_row = slot_row;
+    }
+    has[r] = true;
+    src[r] = in_rows + src_row * row_bytes;
+    dst[r] = out_rows + dst_row * row_bytes;
+    if (in_scales && out_scales && lane == 0) out_scales[dst_row] = in_scales[src_row];
+  }
+  if (kVec16) {
+    copy_rows_vec((const int4v* const*)src, (int4v* const*)dst, has, (int)(row_bytes >> 4), lane);
+  } else {
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r)
+      if (has[r])
+        for (int64_t c = lane; c < row_bytes; c += 64) dst[r][c] = src[r][c];
+  }
+}
+
+// Weighted combine: one workgroup per token; thread c owns 16-byte column chunk(s) of the row.
+// kFp8: rows are e4m3 bytes (16 elements per chunk), else bf16 (8 elements per chunk).
+constexpr int kCombineMaxTopk = 32;
+
+template <bool kFp8>
+__global__ __launch_bounds__(1024) void moe_combine_kernel(const unsigned char* __restrict__ slot_rows,
+                                                           const float* __restrict__ slot_scales,
+                                                           const int32_t* __restrict__ scatter_idx,
+                                                           const float* __restrict__ topk_w,
+                                                           const int32_t* __restrict__ cumsum, int topk, int hidden,
+                                                           int W, int Er, int max_m,
+                                                           unsigned short* __restrict__ out) {
+  __shared__ int64_t s_row[kCombineMaxTopk];  // source row index, -1 = skip
+  __shared__ float s_coef[kCombineMaxTopk];   // w[t,k] * scale[row]
+  const int64_t t = blockIdx.x;
+  if (threadIdx.x < topk) {
+    const int k = threadIdx.x;
+    const int32_t p = scatter_idx[t * topk + k];
+    int64_t row = -1;
+    if (p >= 0) {
+      if (max_m > 0) {
+        const int32_t total = cumsum[W * Er];
+        if (p < total) {
+          const int d = find_dest(cumsum, Er, W, p);
+          const int64_t in_slot = p - cumsum[d * Er];
+          if (in_slot < max_m) row = (int64_t)d * max_m + in_slot;
+        }
+      } else {
+        row = p;
+      }
+    }
+    float coef = topk_w ? topk_w[t * topk + k] : 1.0f;
+    if (row >= 0 && slot_scales) coef *= slot_scales[row];
+    s_row[k] = row;
+    s_coef[k] = coef;
+  }
+  __syncthreads();
+  constexpr int kElems = kFp8 ? 16 : 8;
+  const int64_t row_bytes = (int64_t)hidden * (kFp8 ? 1 : 2);
+  const int n16 = hidden / kElems;
+  for (int c = threadIdx.x; c < n16; c += blockDim.x) {
+    float acc[kElems];
+#pragma unroll
+    for (int j = 0; j < kElems; ++j) acc[j] = 0.f;
+    int k = 0;
+    // four rows in flight per step
+    for (; k + 4 <= topk; k += 4) {
+      int4v v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t row = s_row[k + j];
+        v[j] = (row >= 0) ? __builtin_nontemporal_load((const int4v*)(slot_rows + row * row_bytes) + c)
+                          : int4v{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float coef = (s_row[k + j] >= 0) ? s_coef[k + j] : 0.f;
+        if (kFp8) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float f[4];
+            e4m3x4_to_f32((uint32_t)v[j][q], f);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[4 * q + r] += coef * f[r];
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            acc[2 * q] += coef * BF16::lo((uint32_t)v[j][q]);
+            acc[2 * q + 1] += coef * BF16::hi((uint32_t)v[j][q]);
+          }
+        }
+      }
+    }
+    for (; k < topk; ++k) {
+      const int64_t row = s_row[k];
+      if (row < 0) continue;
+      const int4v v = __builtin_nontemporal_load((const int4v*)(slot_rows + row * row_bytes) + c);
+      const float coef = s_coef[k];
+      if (kFp8) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float f[4];
+          e4m3x4_to_f32((uint32_t)v[q], f);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[4 * q + r] += coef * f[r];
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc[2 * q] += coef * BF16::lo((uint32_t)v[q]);
+          acc[2 * q + 1] += coef * BF16::hi((uint32_t)v[q]);
+        }
+      }
+    }
+    unsigned short* o = out + t * hidden + (int64_t)c * kElems;
+#pragma unroll
+    for (int q = 0; q < kElems / 8; ++q) {
+      int4v w;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = (int)pack_bf16x2(acc[8 * q + 2 * j], acc[8 * q + 2 * j + 1]);
+      __builtin_nontemporal_store(w, (int4v*)o + q);
+    }
+  }
+}
+
+static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, int32_t* splits, int32_t* cumsum,
+                            int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx, void* workspace,
+                            int64_t workspace_bytes, hipStream_t stream, bool want_index, const char* who) {
+  if (!ids || !cumsum) return fail(TDIST_ERR_INVALID, "%s: null ids or cumsum", who);
+  if (want_index && (!scatter_idx || !gather_idx)) return fail(TDIST_ERR_INVALID, "%s: null index output", who);
+  if (n_ids < 0 || G <= 0 || (want_index && topk <= 0)) return fail(TDIST_ERR_INVALID, "%s: bad sizes", who);
+  if (G > kMoeMaxExperts) return fail(TDIST_ERR_UNSUPPORTED, "%s: num_experts %d > %d", who, G, kMoeMaxExperts);
+  if (n_ids > 0x7fffffffll) return fail(TDIST_ERR_UNSUPPORTED, "%s: more than 2^31-1 ids", who);
+  const int64_t need = tdist_moe_workspace_bytes(n_ids, G);
+  if (!workspace || workspace_bytes < need)
+    return fail(TDIST_ERR_WORKSPACE, "%s: workspace %lld B < %lld B", who, (long long)workspace_bytes, (long long)need);
+  const int num_blocks = (int)ceil_div(n_ids > 0 ? n_ids : 1, kMoeItemsPerBlock);
+  int32_t* hist = (int32_t*)workspace;
+  int32_t* splits_buf = splits ? splits : hist + (int64_t)num_blocks * G;
+  hipLaunchKernelGGL(moe_hist_kernel, dim3(num_blocks), dim3(kMoeThreads), (size_t)G * 4, stream, ids, n_ids, G, hist);
+  hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, hist, num_blocks, G, splits_buf, cumsum);
+  if (want_index && n_ids > 0) {
+    hipLaunchKernelGGL(moe_rank_kernel, dim3(num_blocks), dim3(kMoeThreads), (size_t)G * 4 * (kMoeThreads / 64), stream,
+                       ids, n_ids, topk, G, id_bits(G), hist, cumsum, scatter_idx, gather_idx, topk_idx);
+  }
+  return launch_status(who);
+}
+
+}  // namespace tdist
+
+using namespace tdist;
+
+extern "C" {
+
+int64_t tdist_moe_workspace_bytes(int64_t n_ids, int num_experts) {
+  if (n_ids < 0 || num_experts <= 0) return 0;
+  const int64_t num_blocks = ceil_div(n_ids > 0 ? n_ids : 1, kMoeItemsPerBlock);
+  return (num_blocks + 1) * (int64_t)num_experts * 4;  // block histograms + one splits row
+}
+
+int tdist_moe_splits_cumsum(const int32_t* ids, int64_t n_ids, int num_experts, int32_t* splits, int32_t* cumsum,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
+  return moe_index_common(ids, n_ids, 1, num_experts, splits, cumsum, nullptr, nullptr, nullptr, workspace,
+                          workspace_bytes, (hipStream_t)stream, false, "tdist_moe_splits_cumsum");
+}
+
+int tdist_moe_scatter_index(const int32_t* ids, int64_t n_ids, int topk, int num_experts, int32_t* splits,
+                            int32_t* cumsum, int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
+  return moe_index_common(ids, n_ids, topk, num_experts, splits, cumsum, scatter_idx, gather_idx, topk_idx, workspace,
+                          workspace_bytes, (hipStream_t)stream, true, "tdist_moe_scatter_index");
+}
+
+int tdist_moe_dispatch(const void* rows, int64_t row_bytes, const float* scales, const int32_t* gather_idx,
+                       const int32_t* cumsum, int64_t n_rows, int world_size, int experts_per_rank, int max_m,
+                       void* slot_rows, float* slot_scales, int32_t* splits_out, void* stream) {
+  if (!rows || !cumsum || !slot_rows) return fail(TDIST_ERR_INVALID, "tdist_moe_dispatch: null pointer");
+  if ((scales != nullptr) != (slot_scales != nullptr))
+    return fail(TDIST_ERR_INVALID, "tdist_moe_dispatch: scales and slot_scales must both be given or both NULL");
+  if (row_bytes <= 0 || n_rows < 0 || world_size <= 0 || experts_per_rank <= 0 || max_m <= 0)
+    return fail(TDIST_ERR_INVALID, "tdist_moe_dispatch: bad sizes");
+  if (world_size > 8192) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_dispatch: world_size > 8192");
+  const int64_t blocks = ceil_div(n_rows > 0 ? n_rows : 1, kRowsPerBlock);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_dispatch: too many rows");
+  const bool vec = (row_bytes % 16 == 0) && aligned16(rows) && aligned16(slot_rows);
+  auto kern = vec ? moe_rows_kernel<true, false> : moe_rows_kernel<false, false>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), (size_t)(world_size + 1) * 4, (hipStream_t)stream,
+                     (const unsigned char*)rows, row_bytes, scales, gather_idx, cumsum, n_rows, world_size,
+                     experts_per_rank, max_m, (unsigned char*)slot_rows, slot_scales, splits_out);
+  return launch_status("tdist_moe_dispatch");
+}
+
+int tdist_moe_post_process(const void* slot_rows, int64_t row_bytes, const float* slot_scales, const int32_t* splits,
+                           int64_t n_rows, int world_size, int experts_per_rank, int max_m, void* out_rows,
+                           float* out_scales, void* stream) {
+  if (!slot_rows || !splits || (!out_rows && n_rows > 0))
+    return fail(TDIST_ERR_INVALID, "tdist_moe_post_process: null pointer");
+  if (row_bytes <= 0 || n_rows < 0 || world_size <= 0 || experts_per_rank <= 0 || max_m <= 0)
+    return fail(TDIST_ERR_INVALID, "tdist_moe_post_process: bad sizes");
+  if (world_size > 8192) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_post_process: world_size > 8192");
+  if (n_rows == 0) return TDIST_OK;
+  const int64_t blocks = ceil_div(n_rows, kRowsPerBlock);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_post_process: too many rows");
+  const bool vec = (row_bytes % 16 == 0) && aligned16(out_rows) && aligned16(slot_rows);
+  auto kern = vec ? moe_rows_kernel<true, true> : moe_rows_kernel<false, true>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), (size_t)(world_size + 1) * 4, (hipStream_t)stream,
+                     (const unsigned char*)slot_rows, row_bytes, slot_scales, (const int32_t*)nullptr, splits, n_rows,
+                     world_size, experts_per_rank, max_m, (unsigned char*)out_rows, out_scales, (int32_t*)nullptr);
+  return launch_status("tdist_moe_post_process");
+}
+
+int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_scales, const int32_t* scatter_idx,
+                      const float* topk_w, const int32_t* cumsum, int64_t n_tokens, int topk, int hidden,
+                      int world_size, int experts_per_rank, int max_m, void* out_bf16, void* stream) {
+  if (!slot_rows || !scatter_idx || !out_bf16) return fail(TDIST_ERR_INVALID, "tdist_moe_combine: null pointer");
+  if (max_m > 0 && (!cumsum || world_size <= 0 || experts_per_rank <= 0))
+    return fail(TDIST_ERR_INVALID, "tdist_moe_combine: slot layout needs cumsum, world_size, experts_per_rank");
+  if (n_tokens < 0 || topk <= 0 || topk > kCombineMaxTopk || hidden <= 0)
+    return fail(TDIST_ERR_INVALID, "tdist_moe_combine: bad sizes (topk <= %d)", kCombineMaxTopk);
+  if (row_dtype != TDIST_F8E4M3 && row_dtype != TDIST_BF16)
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: row dtype %d (e4m3 and bf16 only)", row_dtype);
+  const int elems = row_dtype == TDIST_F8E4M3 ? 16 : 8;
+  if (hidden % elems != 0 || !aligned16(slot_rows) || !aligned16(out_bf16))
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: hidden must be a multiple of %d and buffers 16-byte aligned", elems);
+  if (n_tokens == 0) return TDIST_OK;
+  if (n_tokens > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: too many tokens");
+  int threads = ((hidden / elems + 63) / 64) * 64;
+  if (threads > 1024) threads = 1024;
+  if (threads < 64) threads = 64;
+  auto kern = row_dtype == TDIST_F8E4M3 ? moe_combine_kernel<true> : moe_combine_kernel<false>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)n_tokens), dim3(threads), 0, (hipStream_t)stream,
+                     (const unsigned char*)slot_rows, slot_scales, scatter_idx, topk_w, cumsum, topk, hidden,
+                     world_size, experts_per_rank, max_m, (unsigned short*)out_bf16);
+  return launch_status("tdist_moe_combine");
+}
+
+}  // extern "C"

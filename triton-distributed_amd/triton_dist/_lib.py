@@ -1,0 +1,124 @@
+"""ctypes binding of libtdist_hip.so — one prototype per declaration in include/tdist.h."""
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "_lib", "libtdist_hip.so")
+
+TDIST_OK = 0
+TDIST_ERR_INVALID = -1
+TDIST_ERR_UNSUPPORTED = -2
+TDIST_ERR_LAUNCH = -3
+TDIST_ERR_TIMEOUT = -4
+TDIST_ERR_WORKSPACE = -5
+TDIST_ERR_DEVICE = -6
+
+TDIST_BF16 = 0
+TDIST_F16 = 1
+TDIST_F8E4M3 = 2
+TDIST_F32 = 3
+
+_P = c_void_p
+_I = c_int
+_L = c_int64
+_F = c_float
+
+# name -> (restype, argtypes); mirrors include/tdist.h in order
+PROTOTYPES = {
+    "tdist_version": (_I, []),
+    "tdist_last_error_string": (c_char_p, []),
+    "tdist_init": (_I, []),
+    "tdist_num_cus": (_I, []),
+    "tdist_gemm_chunk_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _P]),
+    "tdist_gemm_chunk_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _P]),
+    "tdist_gemm_chunk_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _P]),
+    "tdist_producer_push_chunk": (_I, [_P, _P, _L, _P, _P, _I, _P]),
+    "tdist_flag_set": (_I, [_P, _I, _P]),
+    "tdist_flag_fill": (_I, [_P, _I, _I, _P]),
+    "tdist_gemm_rs_scatter_bf16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P]),
+    "tdist_gemm_rs_scatter_f16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P]),
+    "tdist_reduce_slices": (_I, [_P, _L, _I, _I, _L, _P, _I, _P]),
+    "tdist_moe_workspace_bytes": (_L, [_L, _I]),
+    "tdist_moe_splits_cumsum": (_I, [_P, _L, _I, _P, _P, _P, _L, _P]),
+    "tdist_moe_scatter_index": (_I, [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _L, _P]),
+    "tdist_moe_dispatch": (_I, [_P, _L, _P, _P, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
+    "tdist_moe_post_process": (_I, [_P, _L, _P, _P, _L, _I, _I, _I, _P, _P, _P]),
+    "tdist_moe_combine": (_I, [_P, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P, _P]),
+    "tdist_decode_split_kv": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I,
+                                   _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
+    "tdist_decode_combine": (_I, [_P, _I, _P, _I, _I, _P, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P, _I, _L, _L, _P, _P]),
+    "tdist_copy_bytes": (_I, [_P, _P, _L, _P]),
+}
+
+
+class TdistError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("libtdist_hip error %d: %s" % (code, message))
+        self.code = code
+
+
+_lib = None
+
+
+def load():
+    """Loads the shared library (once). Raises if it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "libtdist_hip.so is missing at %s — build it with `python triton-distributed_amd/build.py` "
+            "(hipcc, gfx950). The ops have no CPU or PyTorch fallback." % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in PROTOTYPES.items():
+        fn = getattr(lib, name)  # AttributeError here means header and library disagree
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def last_error():
+    msg = load().tdist_last_error_string()
+    return msg.decode("utf-8", "replace") if msg else ""
+
+
+def check(code):
+    if code != TDIST_OK:
+        raise TdistError(code, last_error())
+
+
+def call(name, *args):
+    """Calls an entry point that returns a tdist_status and raises TdistError on failure."""
+    check(getattr(load(), name)(*args))
+
+
+def ptr(t):
+    """Device pointer of a tensor (None → NULL)."""
+    return None if t is None else t.data_ptr()
+
+
+def stream_ptr(stream=None):
+    import torch
+    s = torch.cuda.current_stream() if stream is None else stream
+    return s.cuda_stream
+
+
+def dtype_code(dtype):
+    import torch
+    if dtype == torch.bfloat16:
+        return TDIST_BF16
+    if dtype == torch.float16:
+        return TDIST_F16
+    if dtype == torch.float8_e4m3fn:
+        return TDIST_F8E4M3
+    if dtype == torch.float32:
+        return TDIST_F32
+    raise TypeError("unsupported dtype %s" % dtype)
+
+
+def require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("tdist ops run on the GPU only; got a %s tensor" % t.device)

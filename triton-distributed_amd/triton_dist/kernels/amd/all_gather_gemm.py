@@ -1,0 +1,304 @@
+"""AG-GEMM on one MI355X: the consumer GEMM gated per chunk on HBM flag words, with the all-gather's
+arrivals played by copy streams of the same GPU.
+
+Keeps the interface of the reference's kernels/amd/all_gather_gemm.py
+(``create_ag_gemm_intra_node_context`` :360-429, ``ag_gemm_intra_node`` :432-464, context dataclass
+:327-357). What differs is where the peers' rows come from: with one GPU there is no IPC workspace a peer
+pushes into, so the shards of the other ranks are handed to the context (``ctx.set_peer_shards``) and the
+producer copies them chunk by chunk into the workspace and then releases the chunk's flag, exactly the
+per-chunk protocol of the reference's copy-engine producer (:41-100). The GEMM reads the caller's own
+shard directly and never waits for it (:201-218).
+"""
+import dataclasses
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from triton_dist import _lib
+from triton_dist.kernels.amd.common_ops import fill_flags
+
+
+def cp_engine_producer_all_gather_full_mesh_push_multi_stream(
+    rank,
+    num_ranks,
+    peer_shards: Dict[int, torch.Tensor],
+    workspace: torch.Tensor,
+    one: torch.Tensor,
+    M_PER_CHUNK: int,
+    ag_stream_pool: List[torch.cuda.Stream],
+    barrier: torch.Tensor,
+    arrival_order: Optional[Sequence[Tuple[int, int]]] = None,
+    held_chunks: Sequence[int] = (),
+    use_sdma: bool = True,
+):
+    """Delivers the peers' shards into ``workspace`` chunk by chunk: data copy, then a 4-byte copy of
+    ``one`` into the chunk's flag on the same stream (reference :80-100). ``arrival_order`` is a list of
+    (peer_rank, chunk_in_rank); the default is the reference's (:54-66): peers rank+1, rank+2, ... each
+    on its own stream, chunks in order. Chunks listed in ``held_chunks`` (global chunk ids) are never
+    delivered — a test hook for the bounded wait."""
+    some = next(iter(peer_shards.values()))
+    M_per_rank, K = some.shape
+    chunk_num_per_rank = M_per_rank // M_PER_CHUNK
+    esz = some.element_size()
+    nbytes = M_PER_CHUNK * K * esz
+    if arrival_order is None:
+        arrival_order = []
+        for idx in range(1, num_ranks):
+            r = (rank + idx) % num_ranks
+            arrival_order += [(r, c) for c in range(chunk_num_per_rank)]
+    held = set(int(c) for c in held_chunks)
+    n_streams = len(ag_stream_pool)
+    for r, c in arrival_order:
+        if r == rank:
+            continue
+        chunk_pos = r * chunk_num_per_rank + c
+        if chunk_pos in held:
+            continue
+        stream = ag_stream_pool[r % n_streams]
+        src = peer_shards[r]
+        src_ptr = src.data_ptr() + c * M_PER_CHUNK * K * esz
+        dst_ptr = workspace.data_ptr() + (r * M_per_rank + c * M_PER_CHUNK) * K * esz
+        flag_ptr = barrier.data_ptr() + chunk_pos * 4
+        _lib.call("tdist_producer_push_chunk", dst_ptr, src_ptr, nbytes, flag_ptr, one.data_ptr(),
+                  1 if use_sdma else 0, stream.cuda_stream)
+
+
+@dataclasses.dataclass
+class AllGatherGEMMTensorParallelContext:
+    rank: int
+    num_ranks: int
+    workspace_tensors: List[Optional[torch.Tensor]]
+    barrier_tensors: List[Optional[torch.Tensor]]
+    comm_bufs: List[Optional[torch.Tensor]]
+    one: torch.Tensor
+    comm_buf_ptr: Optional[torch.Tensor]
+    ag_streams: Optional[List[torch.cuda.streams.Stream]] = None
+    gemm_stream: Optional[torch.cuda.streams.Stream] = None
+    serial: bool = False
+    M_PER_CHUNK: int = 1024
+    BLOCK_M: int = 128
+    BLOCK_N: int = 256
+    BLOCK_K: int = 64
+    stages: int = 3
+    autotune: bool = False
+    # ---- one-GPU additions -------------------------------------------------------------------
+    output_dtype: torch.dtype = torch.bfloat16
+    peer_shards: Dict[int, torch.Tensor] = dataclasses.field(default_factory=dict)
+    arrival_order: Optional[List[Tuple[int, int]]] = None
+    held_chunks: Tuple[int, ...] = ()
+    spin_limit: int = 0          # 0 = library default (seconds of polling)
+    status: Optional[torch.Tensor] = None  # int32[2]: error code, chunk that timed out
+    use_sdma: bool = True
+    preset_flags: bool = False   # debug: release every flag before the GEMM starts (no overlap)
+
+    def update(self, rank, num_ranks, BLOCK_M=128, BLOCK_N=256, BLOCK_K=64, stages=3, ag_streams=None, gemm_stream=None,
+               serial=False, autotune=False):
+        self.rank = rank
+        self.num_ranks = num_ranks
+        self.BLOCK_M = BLOCK_M
+        self.BLOCK_N = BLOCK_N
+        self.BLOCK_K = BLOCK_K
+        self.stages = stages
+        self.ag_streams = ag_streams
+        self.gemm_stream = gemm_stream
+        self.serial = serial
+        self.autotune = autotune
+
+    def set_peer_shards(self, shards):
+        """``shards``: dict rank -> [M_per_rank, K] tensor, or a list of num_ranks tensors (the entry of
+        ``rank`` is ignored). They stand for the A shards living on the other ranks."""
+        if not isinstance(shards, dict):
+            shards = {r: t for r, t in enumerate(shards) if t is not None}
+        for r, t in shards.items():
+            if r == self.rank:
+                continue
+            _lib.require_cuda(t)
+            if not t.is_contiguous():
+                raise ValueError("peer shard of rank %d must be contiguous" % r)
+        self.peer_shards = {r: t for r, t in shards.items() if r != self.rank}
+
+    def check_status(self):
+        """Synchronises and raises TdistError if a bounded flag wait expired in an earlier call."""
+        torch.cuda.synchronize()
+        code, chunk = self.status.tolist()
+        if code != 0:
+            self.status.zero_()
+            raise _lib.TdistError(code, "flag wait expired for chunk %d" % chunk)
+
+
+def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, rank, num_ranks, tp_group,
+                                      ag_streams=None, gemm_stream=None, M_PER_CHUNK=1024, BLOCK_M=128, BLOCK_N=256,
+                                      BLOCK_K=64, stages=3, serial=False, autotune=False):
+    """create context for allgather gemm intra-node (reference :360-429).
+
+    ``tp_group`` may be None: one GPU holds the only real rank. BLOCK_*/stages/autotune are accepted for
+    signature compatibility; the HIP kernel picks its own tiling.
+    """
+    assert M_PER_CHUNK % BLOCK_M == 0
+    assert max_M % num_ranks == 0
+    M_per_rank = max_M // num_ranks
+    assert M_per_rank % M_PER_CHUNK == 0
+    if not torch.cuda.is_available():
+        raise RuntimeError("create_ag_gemm_intra_node_context needs a GPU")
+    _lib.check(_lib.load().tdist_init())
+    device = torch.device("cuda", torch.cuda.current_device())
+    workspace = torch.empty([max_M, K], dtype=input_dtype, device=device)
+    m_chunk_num = (max_M + M_PER_CHUNK - 1) // M_PER_CHUNK
+    barrier = torch.zeros([m_chunk_num], dtype=torch.int32, device=device)
+    workspaces: List[Optional[torch.Tensor]] = [None] * num_ranks
+    barriers: List[Optional[torch.Tensor]] = [None] * num_ranks
+    workspaces[rank] = workspace
+    barriers[rank] = barrier
+
+    current_stream = torch.cuda.current_stream()
+    # default priority on purpose (the reference asks for priority -1)
+    _ag_streams = [torch.cuda.Stream() for _ in range(num_ranks)] if ag_streams is None else ag_streams
+    _gemm_stream = current_stream if gemm_stream is None else gemm_stream
+    one = torch.ones((1024, ), dtype=torch.int32, device=device)
+    status = torch.zeros((2, ), dtype=torch.int32, device=device)
+    torch.cuda.synchronize()
+
+    return AllGatherGEMMTensorParallelContext(
+        rank=rank,
+        num_ranks=num_ranks,
+        workspace_tensors=workspaces,
+        barrier_tensors=barriers,
+        comm_bufs=[None] * num_ranks,
+        one=one,
+        comm_buf_ptr=None,
+        ag_streams=_ag_streams,
+        gemm_stream=_gemm_stream,
+        serial=serial,
+        M_PER_CHUNK=M_PER_CHUNK,
+        BLOCK_M=BLOCK_M,
+        BLOCK_N=BLOCK_N,
+        BLOCK_K=BLOCK_K,
+        stages=stages,
+        autotune=autotune,
+        output_dtype=output_dtype,
+        status=status,
+    )
+
+
+_GEMM_ENTRY = {
+    torch.bfloat16: "tdist_gemm_chunk_gated_bf16",
+    torch.float16: "tdist_gemm_chunk_gated_f16",
+    torch.float8_e4m3fn: "tdist_gemm_chunk_gated_fp8e4m3",
+}
+
+
+def gated_gemm(a_ws, a_local, local_row_begin, b, c, flags, m_per_chunk, rank, num_ranks, *, row_scale=None,
+               col_scale=None, chunk_order=None, wait_value=1, spin_limit=0, status=None, stream=None):
+    """Thin wrapper over tdist_gemm_chunk_gated_*: C[M,N] = A[M,K] @ B[N,K]^T with per-chunk gating.
+    ``a_ws`` [M,K] gathered rows, ``a_local`` own shard or None, ``b`` [N,K]."""
+    _lib.require_cuda(a_ws, b, c)
+    M, K = a_ws.shape
+    N = b.shape[0]
+    if a_ws.dtype not in _GEMM_ENTRY:
+        raise TypeError("unsupported GEMM dtype %s" % a_ws.dtype)
+    if a_ws.stride(1) != 1 or b.stride(1) != 1 or c.stride(1) != 1:
+        raise ValueError("A, B and C must be row-major with a contiguous last dimension")
+    args = [
+        a_ws.data_ptr(), a_ws.stride(0),
+        _lib.ptr(a_local), a_local.stride(0) if a_local is not None else 0,
+        int(local_row_begin), a_local.shape[0] if a_local is not None else 0,
+        b.data_ptr(), b.stride(0), c.data_ptr(), c.stride(0), M, N, K,
+    ]
+    if a_ws.dtype == torch.float8_e4m3fn:
+        args += [_lib.ptr(row_scale), _lib.ptr(col_scale)]
+    elif row_scale is not None or col_scale is not None:
+        raise ValueError("scales are only defined for fp8 inputs")
+    args += [
+        _lib.ptr(flags), int(m_per_chunk), int(wait_value), _lib.ptr(chunk_order), int(rank), int(num_ranks),
+        int(spin_limit), _lib.ptr(status), _lib.stream_ptr(stream),
+    ]
+    _lib.call(_GEMM_ENTRY[a_ws.dtype], *args)
+    return c
+
+
+def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barrier_tensors, comm_buf_ptr, ag_streams,
+                          gemm_stream, serial=False, M_PER_CHUNK=1024, BLOCK_M=128, BLOCK_N=256, BLOCK_K=64, stages=3,
+                          autotune=False, use_persistent_gemm=True, *, ctx=None, row_scale=None, col_scale=None):
+    """Reference :257-324: start the producer on the all-gather streams, then the gated GEMM on the GEMM
+    stream; the caller's stream waits for the GEMM."""
+    assert a.shape[1] == b.shape[1], "Incompatible dimensions"
+    assert a.dtype == b.dtype, "Incompatible dtypes"
+    if not use_persistent_gemm:
+        raise NotImplementedError("Non-perisitent gemm is not yet supported")
+    M_per_rank, K = a.shape
+    M = M_per_rank * num_ranks
+    workspace = workspace_tensors[rank]
+    barrier = barrier_tensors[rank]
+    peer_shards = ctx.peer_shards if ctx is not None else {}
+    if num_ranks > 1:
+        missing = [r for r in range(num_ranks) if r != rank and r not in peer_shards]
+        if missing:
+            raise RuntimeError(
+                "one GPU holds a single rank: hand the other ranks' A shards to the context first "
+                "(ctx.set_peer_shards); missing ranks %s" % missing)
+
+    current_stream = torch.cuda.current_stream()
+    gemm_stream.wait_stream(current_stream)
+    for ag_stream in ag_streams:
+        ag_stream.wait_stream(current_stream)
+
+    def call_ag():
+        if num_ranks > 1:
+            cp_engine_producer_all_gather_full_mesh_push_multi_stream(
+                rank, num_ranks, peer_shards, workspace, one, M_PER_CHUNK, ag_streams, barrier,
+                arrival_order=ctx.arrival_order if ctx is not None else None,
+                held_chunks=ctx.held_chunks if ctx is not None else (),
+                use_sdma=ctx.use_sdma if ctx is not None else True)
+
+    call_ag()
+    if serial or (ctx is not None and ctx.preset_flags):
+        for ag_stream in ag_streams:
+            gemm_stream.wait_stream(ag_stream)
+        if serial:
+            torch.cuda.synchronize()
+
+    with torch.cuda.stream(gemm_stream):
+        gated_gemm(workspace[:M], a, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
+                   row_scale=row_scale, col_scale=col_scale, wait_value=1,
+                   spin_limit=ctx.spin_limit if ctx is not None else 0,
+                   status=ctx.status if ctx is not None else None, stream=gemm_stream)
+    current_stream.wait_stream(gemm_stream)
+    for ag_stream in ag_streams:
+        current_stream.wait_stream(ag_stream)
+    return None
+
+
+def ag_gemm_intra_node(a, b, transe_b, ctx, *, row_scale=None, col_scale=None):
+    """allgather gemm for intra-node (reference :432-464)
+
+    Allgather global matrix A and do matmul with local matrix B, produces local matrix C
+
+    Args:
+        a (torch.Tensor): local matmul A matrix. shape: [M_per_rank, K]
+        b (torch.Tensor): local matmul B matrix. shape: [N_per_rank, K]
+        transe_b (bool): indicates whether tensor b is transposed (not supported, as in the reference)
+        ctx (AllGatherGEMMTensorParallelContext)
+        row_scale / col_scale: fp8 inputs only — fp32 per-row scales of the gathered A ([M]) and per-column
+            scales of B ([N_per_rank]); no counterpart in the reference.
+
+    Returns:
+        c (torch.Tensor): local matmul C matrix. shape: [M, N_per_rank]; a.dtype for 16-bit inputs,
+        ctx.output_dtype (bf16) for fp8 inputs.
+    """
+    if ctx is None:
+        raise RuntimeError("requires ctx for ipc handle")
+    if transe_b:
+        raise NotImplementedError("transpose weight is not yet supported")
+    _lib.require_cuda(a, b)
+    M_per_rank, K = a.shape
+    N_per_rank = b.shape[0]
+    out_dtype = a.dtype if a.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+    C = torch.empty([ctx.num_ranks * M_per_rank, N_per_rank], dtype=out_dtype, device=a.device)
+
+    ag_gemm_intra_node_op(a, b, C, ctx.rank, ctx.num_ranks, ctx.workspace_tensors, ctx.one, ctx.barrier_tensors,
+                          ctx.comm_buf_ptr, ag_streams=ctx.ag_streams, gemm_stream=ctx.gemm_stream, serial=ctx.serial,
+                          M_PER_CHUNK=ctx.M_PER_CHUNK, autotune=ctx.autotune, use_persistent_gemm=True, ctx=ctx,
+                          row_scale=row_scale, col_scale=col_scale)
+    # reset (reference :459-462); stream-ordered after the GEMM and after every producer copy
+    fill_flags(ctx.barrier_tensors[ctx.rank], 0)
+    return C

@@ -1,0 +1,231 @@
+"""Low-latency MoE dispatch / combine on one MI355X.
+
+Keeps the interface of the reference's kernels/nvidia/low_latency_all_to_all.py (``AllToAllContext``
+:125-164, ``create_all_to_all_context`` :167-186, ``fast_all_to_all`` :189-248,
+``all_to_all_post_process`` :251-270) and moves the index preprocessing the reference does in its test
+(test/nvidia/test_all_to_all.py:42-96,314-329) onto the GPU as ``moe_dispatch_preprocess``.
+
+One GPU stands for the sender ``rank`` and keeps, for every destination d, the slot this sender would
+fill in d's receive buffer: rows of destination d (experts d*E_r .. d*E_r+E_r-1) are contiguous in the
+expert-sorted order and land in ``recv[d*max_m : d*max_m + n_d]`` — the reference's
+``recv[rank*MAX_M + i]`` on destination d (:63-86), stored side by side. The NVSHMEM puts become 16-byte
+vector copies; there is no signal to wait for.
+"""
+from typing import Optional
+
+import torch
+
+from triton_dist import _lib
+
+
+def dtype_size_in_bytes(dtype: torch.dtype) -> int:
+    return torch.tensor([], dtype=dtype).element_size()
+
+
+class AllToAllContext:
+
+    def __init__(
+        self,
+        max_m: int,
+        hidden: int,
+        rank: int,
+        num_tot_experts: int,
+        WORLD_SIZE: int,
+        experts_per_rank: int,
+        dtype=torch.bfloat16,
+        scale_dtype=torch.float,
+    ):
+        """
+        max_m: capacity, in rows, of one destination slot
+        """
+        if not torch.cuda.is_available():
+            raise RuntimeError("AllToAllContext needs a GPU")
+        if scale_dtype != torch.float:
+            raise NotImplementedError("scales are fp32")
+        if num_tot_experts != WORLD_SIZE * experts_per_rank:
+            raise ValueError("num_tot_experts must equal WORLD_SIZE * experts_per_rank")
+        _lib.check(_lib.load().tdist_init())
+        device = torch.device("cuda", torch.cuda.current_device())
+        # double-buffered like the reference (:141-147): a call fills half call_count % 2
+        self.recv_buf = torch.empty([WORLD_SIZE * max_m * 2, hidden], dtype=dtype, device=device)
+        self.scale_recv_buf = torch.empty([WORLD_SIZE * max_m * 2], dtype=scale_dtype, device=device)
+        self.split_recv_buf = torch.zeros([num_tot_experts * 2], dtype=torch.int32, device=device)
+        self.signal_buf = torch.zeros([WORLD_SIZE * 2], dtype=torch.int64, device=device)
+
+        self.max_m = max_m
+        self.hidden = hidden
+        self.dtype = dtype
+        self.scale_dtype = scale_dtype
+        self.ele_size = dtype_size_in_bytes(self.dtype)
+        self.scale_ele_size = dtype_size_in_bytes(self.scale_dtype)
+
+        self.num_tot_experts = num_tot_experts
+        self.experts_per_rank = experts_per_rank
+
+        self.WORLD_SIZE = WORLD_SIZE
+        self.rank = rank
+
+        # start from 1, as the reference does (:161-163)
+        self.call_count = 1
+        self.MOD_VALUE = 1000000
+
+
+def create_all_to_all_context(
+    max_m: int,
+    hidden: int,
+    rank: int,
+    num_tot_experts: int,
+    WORLD_SIZE: int,
+    experts_per_rank: int,
+    dtype=torch.bfloat16,
+    scale_dtype=torch.float,
+):
+    return AllToAllContext(max_m, hidden, rank, num_tot_experts, WORLD_SIZE, experts_per_rank, dtype, scale_dtype)
+
+
+def splits_to_cumsum(splits: torch.Tensor):
+    """[G] -> [G+1] with out[0] = 0 (reference test helper, test/nvidia/test_all_to_all.py:42-46)."""
+    out = torch.empty(splits.shape[0] + 1, dtype=splits.dtype, device=splits.device)
+    out[0] = 0
+    _ = torch.cumsum(splits, 0, out=out[1:])
+    return out
+
+
+def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_topk_index: bool = False):
+    """GPU version of the reference test's index preparation (test/nvidia/test_all_to_all.py:314-320):
+
+        splits       int32[G]        torch.bincount(exp_indices.view(-1), minlength=G)
+        split_cumsum int32[G+1]      splits_to_cumsum(splits)
+        scatter_idx  int32[T, topk]  exp_indices.flatten().argsort(stable=True).argsort()
+        gather_idx   int32[T*topk]   token of each expert-sorted row (calc_gather_index)
+
+    Returns (splits, split_cumsum, scatter_idx, gather_idx[, topk_idx])."""
+    _lib.require_cuda(exp_indices)
+    if exp_indices.dtype != torch.int32:
+        exp_indices = exp_indices.to(torch.int32)
+    exp_indices = exp_indices.contiguous()
+    T, topk = exp_indices.shape
+    n = T * topk
+    dev = exp_indices.device
+    splits = torch.empty(num_experts, dtype=torch.int32, device=dev)
+    cumsum = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+    scatter_idx = torch.empty((T, topk), dtype=torch.int32, device=dev)
+    gather_idx = torch.empty(n, dtype=torch.int32, device=dev)
+    topk_idx = torch.empty(n, dtype=torch.int32, device=dev) if want_topk_index else None
+    ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
+    workspace = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+    _lib.call("tdist_moe_scatter_index", exp_indices.data_ptr(), n, topk, num_experts, splits.data_ptr(),
+              cumsum.data_ptr(), scatter_idx.data_ptr(), gather_idx.data_ptr(), _lib.ptr(topk_idx),
+              workspace.data_ptr(), workspace.numel(), _lib.stream_ptr())
+    if want_topk_index:
+        return splits, cumsum, scatter_idx, gather_idx, topk_idx
+    return splits, cumsum, scatter_idx, gather_idx
+
+
+def fast_all_to_all(
+    ctx: AllToAllContext,
+    send_tensor: torch.Tensor,
+    send_split_cumsum: torch.Tensor,
+    send_scale: Optional[torch.Tensor],
+    gather_index: Optional[torch.Tensor] = None,
+):
+    """
+    low-latency all-to-all communication (reference :189-248).
+
+    send_tensor [n, hidden] rows already sorted by expert, send_split_cumsum int32[G+1], send_scale fp32[n]
+    or None. With ``gather_index`` (int32[n_sorted], an addition) ``send_tensor`` is the unsorted
+    [T, hidden] token tensor (``send_scale`` per token) and sorted row p is read from token
+    gather_index[p], which fuses the reference's index_select (test_all_to_all.py:328-329) into the copy.
+
+    Returns [splits int32[G], recv [W*max_m, hidden], scales [W*max_m] | None] — views into the context's
+    buffers, valid until the call after next.
+    """
+    _lib.require_cuda(send_tensor, send_split_cumsum, send_scale, gather_index)
+    with_scale = send_scale is not None
+    act_pos = ctx.call_count % 2
+
+    split_buf_st = act_pos * ctx.num_tot_experts
+    split_buf_ed = split_buf_st + ctx.num_tot_experts
+    data_buf_st = act_pos * ctx.WORLD_SIZE * ctx.max_m
+    data_buf_ed = data_buf_st + ctx.WORLD_SIZE * ctx.max_m
+
+    assert send_tensor.dim() == 2 and send_tensor.shape[1] == ctx.hidden
+    assert send_tensor.dtype == ctx.dtype, "send_tensor dtype differs from the context's"
+    assert send_split_cumsum.dtype == torch.int32 and send_split_cumsum.numel() == ctx.num_tot_experts + 1
+    send_tensor = send_tensor.contiguous()
+    if gather_index is not None:
+        assert gather_index.dtype == torch.int32
+        n_rows = gather_index.numel()
+    else:
+        n_rows = send_tensor.shape[0]
+    if with_scale:
+        assert send_scale.dtype == torch.float32
+        send_scale = send_scale.contiguous()
+
+    recv = ctx.recv_buf[data_buf_st:data_buf_ed, :]
+    scale_recv = ctx.scale_recv_buf[data_buf_st:data_buf_ed]
+    splits = ctx.split_recv_buf[split_buf_st:split_buf_ed]
+    _lib.call("tdist_moe_dispatch", send_tensor.data_ptr(), ctx.hidden * ctx.ele_size, _lib.ptr(send_scale),
+              _lib.ptr(gather_index), send_split_cumsum.data_ptr(), n_rows, ctx.WORLD_SIZE, ctx.experts_per_rank,
+              ctx.max_m, recv.data_ptr(), scale_recv.data_ptr() if with_scale else None, splits.data_ptr(),
+              _lib.stream_ptr())
+
+    ctx.call_count = (ctx.call_count + 1) % ctx.MOD_VALUE
+    out_lis = [splits, recv]
+    out_lis.append(scale_recv if with_scale else None)
+    return out_lis
+
+
+def all_to_all_post_process(
+    ctx: AllToAllContext,
+    input_splits: torch.Tensor,
+    recv_buffer: torch.Tensor,
+    scale_buffer: Optional[torch.Tensor] = None,
+):
+    """Compacts the slots into one tensor in destination order (reference :251-270). The row count is read
+    back from the device, as the reference's slicing by tensor values does."""
+    _lib.require_cuda(input_splits, recv_buffer, scale_buffer)
+    with_scale = scale_buffer is not None
+    total = int(input_splits.sum().item())
+    row_bytes = recv_buffer.shape[1] * recv_buffer.element_size()
+    output = torch.empty((total, recv_buffer.shape[1]), dtype=recv_buffer.dtype, device=recv_buffer.device)
+    output_scale = torch.empty((total, ), dtype=scale_buffer.dtype, device=recv_buffer.device) if with_scale else None
+    if total > 0:
+        _lib.call("tdist_moe_post_process", recv_buffer.data_ptr(), row_bytes, _lib.ptr(scale_buffer),
+                  input_splits.data_ptr(), total, ctx.WORLD_SIZE, ctx.experts_per_rank, ctx.max_m, output.data_ptr(),
+                  _lib.ptr(output_scale), _lib.stream_ptr())
+    return output, output_scale
+
+
+def moe_weighted_combine(ctx: Optional[AllToAllContext], rows: torch.Tensor, row_scale: Optional[torch.Tensor],
+                         scatter_idx: torch.Tensor, topk_weight: Optional[torch.Tensor],
+                         split_cumsum: Optional[torch.Tensor] = None, from_slots: bool = True):
+    """y[t] = sum_k w[t,k] * scale[p] * rows[p], p = scatter_idx[t,k]: fp32 accumulation in k order, bf16
+    output [T, hidden]. Restates the reduce step of the reference test
+    (``index_add_(0, gather_idx, combine_token)``, test/nvidia/test_all_to_all.py:366-367) with the top-k
+    weighting of TorchGroupGemmReduceRS (test/nvidia/test_moe_reduce_rs.py:117-122).
+
+    ``rows`` is the slot layout returned by fast_all_to_all (from_slots=True, needs ``ctx`` and
+    ``split_cumsum``) or a compact expert-sorted [n, hidden] tensor (from_slots=False)."""
+    _lib.require_cuda(rows, row_scale, scatter_idx, topk_weight, split_cumsum)
+    T, topk = scatter_idx.shape
+    hidden = rows.shape[1]
+    assert scatter_idx.dtype == torch.int32 and scatter_idx.is_contiguous()
+    if topk_weight is not None:
+        assert topk_weight.dtype == torch.float32 and topk_weight.is_contiguous() and topk_weight.shape == (T, topk)
+    if rows.dtype == torch.float8_e4m3fn:
+        code = _lib.TDIST_F8E4M3
+    elif rows.dtype == torch.bfloat16:
+        code = _lib.TDIST_BF16
+    else:
+        raise TypeError("combine takes e4m3 or bf16 rows, got %s" % rows.dtype)
+    out = torch.empty((T, hidden), dtype=torch.bfloat16, device=rows.device)
+    if from_slots:
+        assert ctx is not None and split_cumsum is not None
+        W, Er, max_m = ctx.WORLD_SIZE, ctx.experts_per_rank, ctx.max_m
+    else:
+        W, Er, max_m = 1, 1, 0
+    _lib.call("tdist_moe_combine", rows.data_ptr(), code, _lib.ptr(row_scale), scatter_idx.data_ptr(),
+              _lib.ptr(topk_weight), _lib.ptr(split_cumsum), T, topk, hidden, W, Er, max_m, out.data_ptr(),
+              _lib.stream_ptr())
+    return out
