@@ -1,0 +1,311 @@
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2]
+
+Headline (one JSON line on stdout): BASELINE config 2, the GEMM-RS one-rank share at the Llama-70B TP=8
+MLP-down shape — a "step" is one gemm_rs_intra_node call: the scatter-epilogue GEMM
+A[8192,3584] x B[8192,3584]^T plus the fp32 reduction of 8 partial slices [1024,8192]. ``value`` is the
+algorithmic GEMM work (2*M*N*K) over the whole step time. The same line carries
+  roofline      the dominant kernel (the GEMM) against the bf16 dense MFMA peak, its launch time measured
+                with HIP events on the launch stream,
+  cpu_baseline  the oracle's torch golden for the same step timed on the host cores,
+  kernels       every other hot-path kernel at its BASELINE config with its own roofline fraction.
+Inputs are synthetic, seeded, and resident in HBM before any timed region.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "triton-distributed_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK = {"bf16": 2.5e15, "fp8": 5.0e15, "hbm": 8.0e12}  # MI355X published dense MFMA peaks (FLOP/s) and HBM3E B/s
+METRIC = "AG-GEMM/GEMM-RS TFLOPS (% MFMA peak); decode & A2A GB/s (% HBM peak)"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_launches(fn, steps, warmup):
+    """Average duration in seconds of ``fn`` (which launches on torch's current stream), HIP events on that
+    stream around ``steps`` back-to-back calls."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / steps
+
+
+def roof(bound, work, seconds, peak_key, traffic=None):
+    achieved = work / seconds
+    unit = "TFLOP/s" if bound == "mfma" else "GB/s"
+    scale = 1e12 if bound == "mfma" else 1e9
+    return {
+        "bound": bound,
+        "achieved": round(achieved / scale, 2),
+        "peak": PEAK[peak_key] / scale,
+        "unit": unit,
+        "frac": round(achieved / PEAK[peak_key], 4),
+        "traffic": traffic,
+        "us_per_launch": round(seconds * 1e6, 2),
+    }
+
+
+# ---- workloads ------------------------------------------------------------------------------------------
+def bench_c2(dev, steps, warmup):
+    """GEMM-RS: returns (step seconds, gemm roofline, reduce roofline, cpu baseline)."""
+    import torch
+    from oracle import golden
+    from triton_dist.kernels.amd import create_gemm_rs_intra_node_context, gemm_rs_intra_node
+    from triton_dist.kernels.amd.gemm_reduce_scatter import matmul_fuse_scatter, ring_reduce_after_scatter
+    W, rank, M, N, K = 8, 0, 8192, 8192, 3584
+    g = torch.Generator().manual_seed(3 + 1)
+    a = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    b = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    peers = [None if r == rank else torch.randn((M // W, N), generator=g).to(torch.bfloat16) for r in range(W)]
+    ctx = create_gemm_rs_intra_node_context(M, N, torch.bfloat16, rank, W, None)
+    ctx.set_peer_partials(peers)
+    a_d, b_d = a.to(dev), b.to(dev)
+    flops = 2.0 * M * N * K
+
+    # whole step: barrier + sync on both sides of exactly `steps` steps
+    for _ in range(warmup):
+        out = gemm_rs_intra_node(a_d, b_d, ctx)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = gemm_rs_intra_node(a_d, b_d, ctx)
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / steps
+
+    err = golden.max_rel_err(out.float().cpu(), golden.gemm_rs_fp32(a, b, peers, rank, W))
+    assert err <= 1e-2, "GEMM-RS result off: max rel err %g" % err
+
+    stream = torch.cuda.current_stream()
+    gemm_s = time_launches(lambda: matmul_fuse_scatter(a_d, b_d, ctx.scatter_bufs_ptr, rank, W, False, stream=stream),
+                           steps, warmup)
+    scatter_out = ctx.scatter_bufs[rank][:M]
+    red_s = time_launches(lambda: ring_reduce_after_scatter(rank, W, scatter_out, stream), steps, warmup)
+    red_bytes = (W + 1) * (M // W) * N * 2
+
+    # CPU baseline: the oracle's golden for the same step (bf16 up-cast to fp32, as the torch golden runs on
+    # a CPU), timed on the host cores. A 1/8 row sample first; the full problem if that is quick.
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, 64)))
+    cores = torch.get_num_threads()
+    rows = M // 8
+    t0 = time.perf_counter()
+    (a[:rows].float() @ b.float().T)
+    probe = time.perf_counter() - t0
+    if probe * 8 <= 30.0:
+        t0 = time.perf_counter()
+        golden.gemm_rs_fp32(a, b, peers, rank, W).to(torch.bfloat16)
+        cpu_s = time.perf_counter() - t0
+        cpu = {"value": round(flops / cpu_s / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": "full step once (fp32 up-cast golden: [8192,3584]x[3584,8192] + 8-slice sum), %.2f s" % cpu_s}
+    else:
+        cpu = {"value": round(flops / 8 / probe / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": "1/8 of the rows (1024 of 8192) of the fp32 up-cast golden GEMM, %.2f s" % probe}
+    return step_s, roof("mfma", flops, gemm_s, "bf16"), roof("hbm", red_bytes, red_s, "hbm"), cpu, err
+
+
+def bench_c1(dev, steps, warmup):
+    import torch
+    from oracle import golden
+    from triton_dist.kernels.amd import ag_gemm_intra_node, create_ag_gemm_intra_node_context, gated_gemm
+    world, rank, mpr, K, N = 4, 0, 1024, 4096, 1536
+    g = torch.Generator().manual_seed(3 + 0)
+    shards = [torch.randn((mpr, K), generator=g).to(torch.bfloat16) for _ in range(world)]
+    b = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    ctx = create_ag_gemm_intra_node_context(world * mpr, N, K, torch.bfloat16, torch.bfloat16, rank, world, None, M_PER_CHUNK=1024)
+    ctx.set_peer_shards({r: s.to(dev) for r, s in enumerate(shards) if r != rank})
+    a_d, b_d = shards[rank].to(dev), b.to(dev)
+    flops = 2.0 * world * mpr * N * K
+    live_s = time_launches(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx), steps, warmup)
+    c = ag_gemm_intra_node(a_d, b_d, False, ctx)
+    ctx.check_status()
+    err = golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32(shards, b))
+    assert err <= 1e-2
+    # kernel alone, every flag already released
+    full = torch.cat(shards).to(dev)
+    flags = torch.ones(world, dtype=torch.int32, device=dev)
+    out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
+    pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 1024, rank, world), steps, warmup)
+    r = roof("mfma", flops, pre_s, "bf16")
+    r["with_live_producer_us"] = round(live_s * 1e6, 2)
+    return r
+
+
+def bench_c3(dev, steps, warmup):
+    import torch
+    from oracle import golden
+    from triton_dist.kernels.amd import ag_gemm_intra_node, create_ag_gemm_intra_node_context, gated_gemm
+    world, rank, mpr, K, N = 8, 0, 2048, 8192, 7168
+    g = torch.Generator().manual_seed(3 + 2)
+    shards = [torch.randn((mpr, K), generator=g).to(torch.float8_e4m3fn) for _ in range(world)]
+    b = torch.randn((N, K), generator=g).to(torch.float8_e4m3fn)
+    sa = (torch.rand(world * mpr, generator=g) * 0.09 + 0.01).to(dev)
+    sb = (torch.rand(N, generator=g) * 0.009 + 0.001).to(dev)
+    ctx = create_ag_gemm_intra_node_context(world * mpr, N, K, torch.float8_e4m3fn, torch.bfloat16, rank, world, None,
+                                            M_PER_CHUNK=2048)
+    ctx.set_peer_shards({r: s.to(dev) for r, s in enumerate(shards) if r != rank})
+    a_d, b_d = shards[rank].to(dev), b.to(dev)
+    flops = 2.0 * world * mpr * N * K
+    live_s = time_launches(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb), steps, warmup)
+    c = ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb)
+    ctx.check_status()
+    rows = slice(5 * mpr + 11, 5 * mpr + 75)
+    ref = golden.fp8_scaled_gemm_fp32(shards[5][11:75], sa.cpu()[rows], b, sb.cpu())
+    err = golden.max_rel_err(c[rows].float().cpu(), ref)
+    assert err <= 1e-2
+    full = torch.cat([s.view(torch.uint8) for s in shards]).to(dev).view(torch.float8_e4m3fn)
+    flags = torch.ones(world, dtype=torch.int32, device=dev)
+    out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
+    pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 2048, rank, world, row_scale=sa, col_scale=sb),
+                          steps, warmup)
+    r = roof("mfma", flops, pre_s, "fp8")
+    r["with_live_producer_us"] = round(live_s * 1e6, 2)
+    return r
+
+
+def bench_c4(dev, steps, warmup):
+    import torch
+    from oracle import golden
+    from triton_dist.kernels.amd import (create_all_to_all_context, fast_all_to_all, moe_dispatch_preprocess,
+                                         moe_weighted_combine)
+    T, topk, G, W, H, max_m = 4096, 8, 256, 32, 7168, 4096
+    g = torch.Generator().manual_seed(3 + 3)
+    ids = golden.random_distinct_experts(T, G, topk, g)
+    q, s = golden.quantize_per_token_e4m3(torch.randn((T, H), generator=g))
+    w = torch.softmax(torch.randn((T, topk), generator=g), dim=-1).float().contiguous().to(dev)
+    ctx = create_all_to_all_context(max_m, H, 0, G, W, G // W, dtype=torch.float8_e4m3fn)
+    ids_d, q_d, s_d = ids.to(dev), q.to(dev), s.to(dev)
+    splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids_d, G)
+    pre_s = time_launches(lambda: moe_dispatch_preprocess(ids_d, G), steps, warmup)
+    disp_s = time_launches(lambda: fast_all_to_all(ctx, q_d, cumsum, s_d, gather_index=gather), steps, warmup)
+    _, recv, recv_scale = fast_all_to_all(ctx, q_d, cumsum, s_d, gather_index=gather)
+    comb_s = time_launches(lambda: moe_weighted_combine(ctx, recv, recv_scale, scatter, w, cumsum), steps, warmup)
+    n = T * topk
+    disp_bytes = T * H + n * H + T * 4 + n * 4 + n * 4          # unique row reads + row writes + scales + gather index
+    comb_bytes = n * H + n * 4 + n * 4 + n * 4 + T * H * 2      # row reads + scales + weights + scatter index + bf16 out
+    d = roof("hbm", disp_bytes, disp_s, "hbm")
+    d["index_build_us"] = round(pre_s * 1e6, 2)
+    return d, roof("hbm", comb_bytes, comb_s, "hbm")
+
+
+def bench_c5(dev, steps, warmup):
+    import torch
+    from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine
+    B, Hq, Hkv, D, L, S, page = 32, 64, 8, 128, 32768, 16, 16
+    g = torch.Generator(device="cuda").manual_seed(3 + 4)
+    pages_per_seq = L // page
+    num_pages = B * pages_per_seq
+    k = torch.randn((num_pages, page, Hkv, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    v = torch.randn((num_pages, page, Hkv, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    q = torch.randn((B, Hq, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    table = torch.randperm(num_pages, generator=torch.Generator().manual_seed(6)).view(B, pages_per_seq).int().to(dev)
+    lens = torch.full((B, ), L, dtype=torch.int32, device=dev)
+    out_split = torch.empty((B, Hq, S, D), dtype=torch.float32, device=dev)
+    lse_split = torch.empty((B, Hq, S), dtype=torch.float32, device=dev)
+    scale = D**-0.5
+    split_s = time_launches(lambda: _split_kv(q, k, v, lens, table, scale, 0.0, S, out_split, lse_split), steps, warmup)
+    merged = torch.empty((B, Hq, D), dtype=torch.bfloat16, device=dev)
+    comb_s = time_launches(
+        lambda: decode_combine(out_split, lse_split, S, 1, lens, B, Hq, D,
+                               (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
+                               (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), merged), steps, warmup)
+    kv_bytes = 2 * B * L * Hkv * D * 2
+    split_bytes = kv_bytes + q.numel() * 2 + table.numel() * 4 + out_split.numel() * 4 + lse_split.numel() * 4
+    r = roof("hbm", split_bytes, split_s, "hbm")
+    r["combine_us"] = round(comb_s * 1e6, 2)
+    return r
+
+
+def bench_copy(dev, steps, warmup):
+    import torch
+    from triton_dist import _lib
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev)
+    dst = torch.empty(n, dtype=torch.uint8, device=dev)
+    s = time_launches(lambda: _lib.call("tdist_copy_bytes", dst.data_ptr(), src.data_ptr(), n, _lib.stream_ptr()), steps, warmup)
+    return roof("hbm", 2 * n, s, "hbm")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,copy (c2 always runs)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported (every GPU box "
+            "here has one GPU and the path has no cross-GPU step in it)" % args.gpus)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        log("bench.py needs a GPU")
+        sys.exit(1)
+    from triton_dist import _lib
+    _lib.check(_lib.load().tdist_init())
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    want = set(x for x in args.only.split(",") if x) or {"c1", "c2", "c3", "c4", "c5", "copy"}
+
+    step_s, gemm_roof, red_roof, cpu, err = bench_c2(dev, args.steps, args.warmup)
+    log("c2 step %.1f us, gemm %s, reduce %s" % (step_s * 1e6, gemm_roof, red_roof))
+    kernels = {"c2_gemm_rs_scatter_gemm_bf16": gemm_roof, "c2_reduce_slices_bf16": red_roof}
+    if "c1" in want:
+        kernels["c1_ag_gemm_bf16_gated"] = bench_c1(dev, args.steps, args.warmup)
+        log("c1", kernels["c1_ag_gemm_bf16_gated"])
+    if "c3" in want:
+        kernels["c3_ag_gemm_fp8_gated"] = bench_c3(dev, args.steps, args.warmup)
+        log("c3", kernels["c3_ag_gemm_fp8_gated"])
+    if "c4" in want:
+        d, c = bench_c4(dev, args.steps, args.warmup)
+        kernels["c4_moe_dispatch_fp8"], kernels["c4_moe_combine"] = d, c
+        log("c4", d, c)
+    if "c5" in want:
+        kernels["c5_decode_split_kv_bf16"] = bench_c5(dev, args.steps, args.warmup)
+        log("c5", kernels["c5_decode_split_kv_bf16"])
+    if "copy" in want:
+        kernels["copy_1GiB_yardstick"] = bench_copy(dev, args.steps, args.warmup)
+        log("copy", kernels["copy_1GiB_yardstick"])
+
+    flops = 2.0 * 8192 * 8192 * 3584
+    line = {
+        "metric": METRIC,
+        "value": round(flops / step_s / 1e12, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "GEMM-RS one-rank share, Llama-70B TP=8 MLP-down: A[8192,3584] x B[3584,8192] bf16 "
+                               "scatter-epilogue GEMM + fp32 sum of 8 partial slices [1024,8192] (BASELINE configs[1])",
+                   "rank": 0, "world_size": 8, "max_rel_err_vs_fp32": float("%.3g" % err)},
+        "roofline": gemm_roof,
+        "cpu_baseline": cpu,
+        "kernels": kernels,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -70,20 +70,23 @@ int tdist_num_cus(void);
  *   spin_limit   > 0: polls per wait before giving up; <= 0: library default (seconds of polling).
  *         On expiry the tile is skipped (its C rows are left untouched) and status[0] is set to
  *         TDIST_ERR_TIMEOUT, status[1] to the chunk index. status may be NULL.
- * Requirements: K % 64 == 0 (bf16/f16) or K % 128 == 0 (fp8), lda/ldb multiples of 8 (16 for fp8)
- * elements, 16-byte aligned bases, m_per_chunk % 256 == 0 when flags != NULL.
+ *   max_workgroups  upper bound on the persistent grid; <= 0: one workgroup per compute unit. A producer
+ *         whose copies run on this same GPU needs compute units of its own while the GEMM spins on a flag:
+ *         leave it 32 (pass tdist_num_cus() - 32). Not needed when the rows arrive from a peer's copy engine.
+ * Requirements: K * element size a multiple of 64 bytes, lda/ldb multiples of 8 (16 for fp8) elements,
+ * 16-byte aligned bases, m_per_chunk % 128 == 0 when flags != NULL (% 256 selects the large tile).
  * ------------------------------------------------------------------------------------------- */
 int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                 int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
                                 int64_t ldc, int M, int N, int K, const int32_t* flags, int m_per_chunk,
                                 int wait_value, const int32_t* chunk_order, int rank, int world_size,
-                                int spin_limit, int32_t* status, void* stream);
+                                int spin_limit, int32_t* status, int max_workgroups, void* stream);
 
 int tdist_gemm_chunk_gated_f16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
                                int64_t ldc, int M, int N, int K, const int32_t* flags, int m_per_chunk,
                                int wait_value, const int32_t* chunk_order, int rank, int world_size,
-                               int spin_limit, int32_t* status, void* stream);
+                               int spin_limit, int32_t* status, int max_workgroups, void* stream);
 
 /* fp8-e4m3 inputs, bf16 output, C = (sum_k A8*B8) * row_scale[m] * col_scale[n].
  * The scale epilogue has no counterpart in the reference (fp8 is a dtype passthrough there,
@@ -93,7 +96,7 @@ int tdist_gemm_chunk_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
                                    void* C, int64_t ldc, int M, int N, int K, const float* row_scale,
                                    const float* col_scale, const int32_t* flags, int m_per_chunk,
                                    int wait_value, const int32_t* chunk_order, int rank, int world_size,
-                                   int spin_limit, int32_t* status, void* stream);
+                                   int spin_limit, int32_t* status, int max_workgroups, void* stream);
 
 /* Producer side of the gate on the same GPU: copy one chunk, then release its flag, both ordered on
  * `stream`.   replaces cp_engine_producer_all_gather_full_mesh_push_multi_stream

@@ -20,6 +20,8 @@
 //  * persistent grid (one workgroup per CU). The tile schedule is chunk-major in arrival order, and
 //    within a round of concurrently running tiles the workgroups of one XCD (workgroup id mod 8) get a
 //    compact block of tiles so they share A rows and B rows in that XCD's L2.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace tdist {
@@ -95,9 +97,12 @@ struct ElemFP8 {
 };
 
 // KB = bytes of K per tile row. Chunk c (16 B) of row r is stored at position c ^ swz(r).
+// A ds_read_b128 is served 16 lanes at a time (16 x 16 B = 256 B = one pass over the 64 banks), and the 16
+// lanes of a pass read the same logical chunk of 16 consecutive rows. Those rows cover 256 B / KB positions
+// "for free" through their row offset; the XOR term has to spread the rest, i.e. change every (256 / KB) rows.
 template <int KB>
 __host__ __device__ constexpr int swz(int r) {
-  return KB >= 128 ? (r & 7) : ((r >> 1) & 3);
+  return KB >= 128 ? ((r >> 1) & 7) : ((r >> 2) & 3);
 }
 
 template <typename E, int BM, int BN, int KB, int WM, int WN, int NST>
@@ -123,8 +128,8 @@ struct GemmCfg {
   static constexpr int kEpiPitch = kWaveN * 2;
   static constexpr int kEpiBytes = kWaveM * kEpiPitch;
   static constexpr int kEpiSwz = (kEpiPitch / 16 < 16 ? kEpiPitch / 16 : 16) - 1;
-  // MFMAs of a K step issued before the next step's operand reads
-  static constexpr int kLeadMfma = (kTM * kTN >= 8) ? 4 : 1;
+  // MFMAs of a tile's last K step issued before the barrier
+  static constexpr int kLeadMfma = (kTM * kTN >= 8) ? 2 : 1;
   static_assert(KB == 64 || KB == 128, "tile rows of 64 or 128 bytes");
   static_assert(BM % (kRowsPerInstr * kWaves) == 0 && BN % (kRowsPerInstr * kWaves) == 0, "tile/wave split");
   static_assert(kP >= 1 && kP <= 3 && kP * kLoadsPerTile < 64, "vmcnt budget");
@@ -132,13 +137,16 @@ struct GemmCfg {
   static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "wave tile");
 };
 
-template <int N>
-__device__ __forceinline__ void wait_tiles_and_barrier(int rem) {
-  // rem = tiles younger than the awaited one that may stay in flight (0..2)
-  if (rem >= 2) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(2 * N < 64 ? 2 * N : 63) : "memory");
-  else if (rem == 1) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
-  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+// Waits until at most `kOutstanding` of this wave's DMA loads are in flight and for its LDS reads, then joins
+// the workgroup barrier.
+template <int kOutstanding>
+__device__ __forceinline__ void wait_tiles_and_barrier() {
+  static_assert(kOutstanding >= 0 && kOutstanding < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
+
+// Instruction classes for __builtin_amdgcn_sched_group_barrier
+constexpr int kSchedMfma = 0x008, kSchedVmem = 0x010, kSchedDsRead = 0x100;  // the LDS-DMA load is VMEM that also stores
 
 // schedule position → chunk id
 __device__ __forceinline__ int chunk_of(const GemmParams& p, int oc) {
@@ -242,40 +250,48 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       b_off[t] = (int64_t)gr * p.ldb_b + ((dma_pos ^ swz<KB>(r)) << 4);
     }
 
-    auto issue_tile = [&](int kt) {
+    // DMA of K tile kt into stage kt % NST, one instruction at a time (kLoadsPerTile of them: A rows first, then
+    // B rows). Past the last tile the last one is fetched again (into a stage nobody reads any more): every trip
+    // of the main loop then issues the same number of loads, which keeps the loop free of branches and the vmcnt
+    // bookkeeping constant.
+    auto issue_dma = [&](int kt, int t) {
       lds_u8 const sa = smem + (kt % NST) * C::kStageBytes;
-      lds_u8 const sb = sa + C::kABytes;
-      const int64_t kb = (int64_t)kt * KB;
-#pragma unroll
-      for (int t = 0; t < C::kAInstr; ++t)
+      const int64_t kb = (int64_t)min(kt, KT - 1) * KB;
+      if (t < C::kAInstr) {
         __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(Arows + a_off[t] + kb),
                                          (TDIST_AS3 void*)(sa + (wave * C::kAInstr + t) * 1024), 16, 0, 0);
+      } else {
+        const int u = t - C::kAInstr;
+        __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(p.B + b_off[u] + kb),
+                                         (TDIST_AS3 void*)(sa + C::kABytes + (wave * C::kBInstr + u) * 1024), 16, 0, 0);
+      }
+    };
+    auto issue_tile = [&](int kt) {
 #pragma unroll
-      for (int t = 0; t < C::kBInstr; ++t)
-        __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(p.B + b_off[t] + kb),
-                                         (TDIST_AS3 void*)(sb + (wave * C::kBInstr + t) * 1024), 16, 0, 0);
+      for (int t = 0; t < C::kLoadsPerTile; ++t) issue_dma(kt, t);
     };
 
-    // operand fragments: row (32*i + l32) of the wave's strip, K bytes [ks*2L + lh*L, +L), L = kLaneBytes
     // operand fragments of the K step being multiplied (cur) and of the one after it (nxt)
     typename E::frag a_cur[C::kTM], b_cur[C::kTN], a_nxt[C::kTM], b_nxt[C::kTN];
-    auto load_frags = [&](int kt, int ks, typename E::frag* af, typename E::frag* bf) {
+    // f-th operand fragment (A fragments first) of K step ks of tile kt
+    auto load_frag = [&](int kt, int ks, int f, typename E::frag* af, typename E::frag* bf) {
       lds_u8 const sa = smem + (kt % NST) * C::kStageBytes;
-      lds_u8 const sb = sa + C::kABytes;
       const int c0 = (ks * 2 + lh) * C::kFragVecs;  // first 16-byte chunk of this lane's K bytes
       const int c1 = c0 + C::kFragVecs - 1;         // last one (== c0 for 16-byte fragments)
-#pragma unroll
-      for (int i = 0; i < C::kTM; ++i) {
-        const int r = wm * C::kWaveM + i * 32 + l32;
+      if (f < C::kTM) {
+        const int r = wm * C::kWaveM + f * 32 + l32;
         lds_u8 const row = sa + r * KB;
-        af[i] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
-      }
-#pragma unroll
-      for (int j = 0; j < C::kTN; ++j) {
+        af[f] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
+      } else {
+        const int j = f - C::kTM;
         const int r = wn * C::kWaveN + j * 32 + l32;
-        lds_u8 const row = sb + r * KB;
+        lds_u8 const row = sa + C::kABytes + r * KB;
         bf[j] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
       }
+    };
+    auto load_frags = [&](int kt, int ks, typename E::frag* af, typename E::frag* bf) {
+#pragma unroll
+      for (int f = 0; f < C::kTM + C::kTN; ++f) load_frag(kt, ks, f, af, bf);
     };
 
     float16v acc[C::kTN][C::kTM];
@@ -288,38 +304,66 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 
     // ---- prologue: P tiles in flight, wait for tile 0 ------------------------------------------
 #pragma unroll
-    for (int t = 0; t < C::kP; ++t)
-      if (t < KT) issue_tile(t);
-    wait_tiles_and_barrier<C::kLoadsPerTile>(min(C::kP - 1, KT - 1));
-    if (C::kP < KT) issue_tile(C::kP);
+    for (int t = 0; t < C::kP; ++t) issue_tile(t);
+    wait_tiles_and_barrier<(C::kP - 1) * C::kLoadsPerTile>();
+    issue_tile(C::kP);
     load_frags(0, 0, a_cur, b_cur);
 
     // ---- main loop over K tiles -----------------------------------------------------------------
+    // Every K step multiplies the fragments read during the previous step while it reads the next ones, one
+    // LDS read slotted behind each of the first MFMAs so that neither pipe waits for the other. The last
+    // step of a tile first joins the barrier (tile kt+1 has landed everywhere, tile kt is no longer read),
+    // then also refills the freed stage.
+    constexpr int kMfmaPerStep = C::kTM * C::kTN;
+    constexpr int kReadsPerStep = (C::kTM + C::kTN) * C::kFragVecs;
     for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
       for (int ks = 0; ks < C::kKSteps; ++ks) {
-        // A few MFMAs of this step go first: the wait the compiler puts in front of them then only covers
-        // operand reads issued a whole step ago, and the reads issued below have the rest of the step's
-        // MFMAs to complete.
-#pragma unroll
-        for (int idx = 0; idx < C::kLeadMfma; ++idx) {
-          const int j = idx / C::kTM, i = idx % C::kTM;
-          acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
         if (ks + 1 < C::kKSteps) {
           load_frags(kt, ks + 1, a_nxt, b_nxt);
-        } else if (kt + 1 < KT) {
-          // tile kt+1 must have landed; tiles kt+2 .. kt+P may stay in flight
-          wait_tiles_and_barrier<C::kLoadsPerTile>(min(C::kP - 1, KT - 2 - kt));
-          if (kt + 1 + C::kP < KT) issue_tile(kt + 1 + C::kP);
-          load_frags(kt + 1, 0, a_nxt, b_nxt);
-        }
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int idx = C::kLeadMfma; idx < C::kTN * C::kTM; ++idx) {
-          const int j = idx / C::kTM, i = idx % C::kTM;
-          acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+          for (int idx = 0; idx < kMfmaPerStep; ++idx) {
+            const int j = idx / C::kTM, i = idx % C::kTM;
+            acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+          }
+#pragma unroll
+          for (int r = 0; r < kReadsPerStep; ++r) {
+            __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(kSchedMfma, kMfmaPerStep - kReadsPerStep, 0);
+        } else {
+#pragma unroll
+          for (int idx = 0; idx < C::kLeadMfma; ++idx) {
+            const int j = idx / C::kTM, i = idx % C::kTM;
+            acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          wait_tiles_and_barrier<(C::kP - 1) * C::kLoadsPerTile>();
+          __builtin_amdgcn_sched_barrier(0);
+          // the rest of the step's MFMAs, each followed by its share of the refill DMA and of the next tile's
+          // first fragment reads; the fences pin this order
+          constexpr int kTail = kMfmaPerStep - C::kLeadMfma;
+          constexpr int kFrags = C::kTM + C::kTN;
+          constexpr int kSlots = kFrags < kTail ? kFrags : kTail;
+          constexpr int kDmaPerSlot = (C::kLoadsPerTile + kSlots - 1) / kSlots;
+          constexpr int kFragPerSlot = (kFrags + kSlots - 1) / kSlots;
+          const int kt_next = min(kt + 1, KT - 1);
+#pragma unroll
+          for (int idx = C::kLeadMfma; idx < kMfmaPerStep; ++idx) {
+            const int j = idx / C::kTM, i = idx % C::kTM;
+            acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+            const int slot = idx - C::kLeadMfma;
+            if (slot < kSlots) {
+#pragma unroll
+              for (int d = 0; d < kDmaPerSlot; ++d)
+                if (slot * kDmaPerSlot + d < C::kLoadsPerTile) issue_dma(kt + 1 + C::kP, slot * kDmaPerSlot + d);
+#pragma unroll
+              for (int f = 0; f < kFragPerSlot; ++f)
+                if (slot * kFragPerSlot + f < kFrags) load_frag(kt_next, 0, slot * kFragPerSlot + f, a_nxt, b_nxt);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
         }
 #pragma unroll
         for (int i = 0; i < C::kTM; ++i) a_cur[i] = a_nxt[i];
@@ -330,7 +374,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 
     // ---- epilogue ---------------------------------------------------------------------------------
     // acc[j][i][e]: output row m = wm*kWaveM + 32i + l32, column n = wn*kWaveN + 32j + 8*(e/4) + 4*lh + e%4
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ring is free
+    wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
     lds_u8 const epi = smem + wave * C::kEpiBytes;
 #pragma unroll
     for (int i = 0; i < C::kTM; ++i) {
@@ -423,6 +467,7 @@ struct GemmCall {
   const int32_t* chunk_order;
   int rank, world_size, spin_limit;
   int32_t* status;
+  int max_workgroups;
   hipStream_t stream;
   const char* who;
 };
@@ -462,7 +507,12 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (c.scatter_bufs && c.world_size > 0 && (c.M % c.world_size != 0 || (c.M / c.world_size) % 256 != 0)) big = false;
   if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) big = false;
   if (c.A_local && (c.local_row_begin % 256 != 0 || c.local_rows % 256 != 0)) big = false;
+  // TDIST_GEMM_VARIANT picks another compiled tiling for the large-tile path (measurement aid); the default,
+  // 2, is 256x256 tiles, 128-byte K rows, 2x4 waves, two stages.
+  int variant = 2;
+  if (const char* v = getenv("TDIST_GEMM_VARIANT")) variant = atoi(v);
   const int BM = big ? 256 : 128;
+  const int BN = big ? (variant == 4 ? 128 : 256) : 128;
 
   GemmParams p;
   p.A = (const unsigned char*)c.A;
@@ -528,19 +578,30 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
     if (c.A_local && (c.local_row_begin % BM != 0 || c.local_rows % BM != 0))
       return fail(TDIST_ERR_UNSUPPORTED, "%s: the local shard must start and end on a %d-row tile", who, BM);
   }
-  const int64_t sched = (int64_t)p.n_chunks * (p.m_per_chunk / BM) * ceil_div(c.N, BM);
+  const int64_t sched = (int64_t)p.n_chunks * (p.m_per_chunk / BM) * ceil_div(c.N, BN);
   if (sched > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many tiles", who);
-  const int grid = (int)(sched < di.num_cus ? sched : di.num_cus);
+  int max_wgs = di.num_cus;
+  if (c.max_workgroups > 0 && c.max_workgroups < max_wgs) max_wgs = c.max_workgroups;
+  const int grid = (int)(sched < max_wgs ? sched : max_wgs);
   const bool scales = elem == kElemFP8 && (c.row_scale || c.col_scale);
 
   if (big) {
-    switch (elem) {
-      case kElemBF16: return launch_gemm_cfg<ElemBF16, 256, 256, 64, 2, 2, 4, false>(p, grid, c.stream, who);
-      case kElemF16: return launch_gemm_cfg<ElemF16, 256, 256, 64, 2, 2, 4, false>(p, grid, c.stream, who);
-      default:
-        return scales ? launch_gemm_cfg<ElemFP8, 256, 256, 64, 2, 2, 4, true>(p, grid, c.stream, who)
-                      : launch_gemm_cfg<ElemFP8, 256, 256, 64, 2, 2, 4, false>(p, grid, c.stream, who);
+#define TDIST_BIG(BN_, KB_, WM_, WN_, NST_)                                                                          \
+  switch (elem) {                                                                                                    \
+    case kElemBF16: return launch_gemm_cfg<ElemBF16, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);  \
+    case kElemF16: return launch_gemm_cfg<ElemF16, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);    \
+    default:                                                                                                         \
+      return scales ? launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, true>(p, grid, c.stream, who)          \
+                    : launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);        \
+  }
+    switch (variant) {
+      case 0: TDIST_BIG(256, 64, 2, 2, 4)
+      case 1: TDIST_BIG(256, 128, 2, 2, 2)
+      case 3: TDIST_BIG(256, 64, 2, 4, 4)
+      case 4: TDIST_BIG(128, 128, 2, 2, 3)
+      default: TDIST_BIG(256, 128, 2, 4, 2)
     }
+#undef TDIST_BIG
   }
   switch (elem) {
     case kElemBF16: return launch_gemm_cfg<ElemBF16, 128, 128, 64, 2, 2, 4, false>(p, grid, c.stream, who);
@@ -562,7 +623,7 @@ using namespace tdist;
   c.B = B; c.ldb = ldb; c.C = C; c.scatter_bufs = nullptr; c.ldc = ldc; c.M = M; c.N = N; c.K = K;                  \
   c.row_scale = RS; c.col_scale = CS; c.flags = flags; c.m_per_chunk = m_per_chunk; c.wait_value = wait_value;      \
   c.chunk_order = chunk_order; c.rank = rank; c.world_size = world_size; c.spin_limit = spin_limit;                 \
-  c.status = status; c.stream = (hipStream_t)stream; c.who = WHO;                                                   \
+  c.status = status; c.max_workgroups = max_workgroups; c.stream = (hipStream_t)stream; c.who = WHO;                                                   \
   return run_gemm(c, ELEM);
 
 extern "C" {
@@ -571,14 +632,14 @@ int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local,
                                 int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C, int64_t ldc,
                                 int M, int N, int K, const int32_t* flags, int m_per_chunk, int wait_value,
                                 const int32_t* chunk_order, int rank, int world_size, int spin_limit, int32_t* status,
-                                void* stream) {
+                                int max_workgroups, void* stream) {
   TDIST_GATED_BODY(kElemBF16, nullptr, nullptr, "tdist_gemm_chunk_gated_bf16")
 }
 
 int tdist_gemm_chunk_gated_f16(const void* A, int64_t lda, const void* A_local, int64_t lda_local, int local_row_begin,
                                int local_rows, const void* B, int64_t ldb, void* C, int64_t ldc, int M, int N, int K,
                                const int32_t* flags, int m_per_chunk, int wait_value, const int32_t* chunk_order,
-                               int rank, int world_size, int spin_limit, int32_t* status, void* stream) {
+                               int rank, int world_size, int spin_limit, int32_t* status, int max_workgroups, void* stream) {
   TDIST_GATED_BODY(kElemF16, nullptr, nullptr, "tdist_gemm_chunk_gated_f16")
 }
 
@@ -586,7 +647,8 @@ int tdist_gemm_chunk_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
                                    int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
                                    int64_t ldc, int M, int N, int K, const float* row_scale, const float* col_scale,
                                    const int32_t* flags, int m_per_chunk, int wait_value, const int32_t* chunk_order,
-                                   int rank, int world_size, int spin_limit, int32_t* status, void* stream) {
+                                   int rank, int world_size, int spin_limit, int32_t* status, int max_workgroups,
+                                   void* stream) {
   TDIST_GATED_BODY(kElemFP8, row_scale, col_scale, "tdist_gemm_chunk_gated_fp8e4m3")
 }
 
@@ -599,6 +661,7 @@ static int gemm_rs_scatter(GemmElem elem, const void* A, int64_t lda, const void
   c.B = B; c.ldb = ldb; c.C = nullptr; c.scatter_bufs = scatter_bufs; c.ldc = ldc; c.M = M; c.N = N; c.K = K;
   c.row_scale = nullptr; c.col_scale = nullptr; c.flags = nullptr; c.m_per_chunk = 0; c.wait_value = 0;
   c.chunk_order = nullptr; c.rank = rank; c.world_size = world_size; c.spin_limit = 0; c.status = nullptr;
+  c.max_workgroups = 0;
   c.stream = (hipStream_t)stream; c.who = who;
   return run_gemm(c, elem);
 }

@@ -30,9 +30,9 @@ PROTOTYPES = {
     "tdist_last_error_string": (c_char_p, []),
     "tdist_init": (_I, []),
     "tdist_num_cus": (_I, []),
-    "tdist_gemm_chunk_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _P]),
-    "tdist_gemm_chunk_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _P]),
-    "tdist_gemm_chunk_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _P]),
+    "tdist_gemm_chunk_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
+    "tdist_gemm_chunk_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
+    "tdist_gemm_chunk_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
     "tdist_producer_push_chunk": (_I, [_P, _P, _L, _P, _P, _I, _P]),
     "tdist_flag_set": (_I, [_P, _I, _P]),
     "tdist_flag_fill": (_I, [_P, _I, _I, _P]),

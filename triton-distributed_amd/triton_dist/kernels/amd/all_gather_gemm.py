@@ -90,6 +90,10 @@ class AllGatherGEMMTensorParallelContext:
     status: Optional[torch.Tensor] = None  # int32[2]: error code, chunk that timed out
     use_sdma: bool = True
     preset_flags: bool = False   # debug: release every flag before the GEMM starts (no overlap)
+    # Compute units the gated GEMM leaves to the producer's copies. On one GPU those copies need compute
+    # units of this GPU; measured on MI355X they make no progress next to a full-chip persistent grid
+    # unless 32 units stay free. A peer's copy engine pushing over xGMI would need none.
+    producer_cus: int = 32
 
     def update(self, rank, num_ranks, BLOCK_M=128, BLOCK_N=256, BLOCK_K=64, stages=3, ag_streams=None, gemm_stream=None,
                serial=False, autotune=False):
@@ -188,9 +192,11 @@ _GEMM_ENTRY = {
 
 
 def gated_gemm(a_ws, a_local, local_row_begin, b, c, flags, m_per_chunk, rank, num_ranks, *, row_scale=None,
-               col_scale=None, chunk_order=None, wait_value=1, spin_limit=0, status=None, stream=None):
+               col_scale=None, chunk_order=None, wait_value=1, spin_limit=0, status=None, max_workgroups=0,
+               stream=None):
     """Thin wrapper over tdist_gemm_chunk_gated_*: C[M,N] = A[M,K] @ B[N,K]^T with per-chunk gating.
-    ``a_ws`` [M,K] gathered rows, ``a_local`` own shard or None, ``b`` [N,K]."""
+    ``a_ws`` [M,K] gathered rows, ``a_local`` own shard or None, ``b`` [N,K]. ``max_workgroups`` > 0 caps the
+    persistent grid (leave compute units to a producer that copies on this same GPU)."""
     _lib.require_cuda(a_ws, b, c)
     M, K = a_ws.shape
     N = b.shape[0]
@@ -210,7 +216,7 @@ def gated_gemm(a_ws, a_local, local_row_begin, b, c, flags, m_per_chunk, rank, n
         raise ValueError("scales are only defined for fp8 inputs")
     args += [
         _lib.ptr(flags), int(m_per_chunk), int(wait_value), _lib.ptr(chunk_order), int(rank), int(num_ranks),
-        int(spin_limit), _lib.ptr(status), _lib.stream_ptr(stream),
+        int(spin_limit), _lib.ptr(status), int(max_workgroups), _lib.stream_ptr(stream),
     ]
     _lib.call(_GEMM_ENTRY[a_ws.dtype], *args)
     return c
@@ -257,11 +263,14 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
         if serial:
             torch.cuda.synchronize()
 
+    max_wgs = 0
+    if ctx is not None and num_ranks > 1 and ctx.producer_cus > 0 and not (serial or ctx.preset_flags):
+        max_wgs = max(1, _lib.load().tdist_num_cus() - ctx.producer_cus)
     with torch.cuda.stream(gemm_stream):
         gated_gemm(workspace[:M], a, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
                    row_scale=row_scale, col_scale=col_scale, wait_value=1,
                    spin_limit=ctx.spin_limit if ctx is not None else 0,
-                   status=ctx.status if ctx is not None else None, stream=gemm_stream)
+                   status=ctx.status if ctx is not None else None, max_workgroups=max_wgs, stream=gemm_stream)
     current_stream.wait_stream(gemm_stream)
     for ag_stream in ag_streams:
         current_stream.wait_stream(ag_stream)
