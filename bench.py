@@ -193,8 +193,8 @@ def bench_c4(dev, steps, warmup):
     ids_d, q_d, s_d = ids.to(dev), q.to(dev), s.to(dev)
     splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids_d, G)
     pre_s = time_launches(lambda: moe_dispatch_preprocess(ids_d, G), steps, warmup)
-    disp_s = time_launches(lambda: fast_all_to_all(ctx, q_d, cumsum, s_d, gather_index=gather), steps, warmup)
-    _, recv, recv_scale = fast_all_to_all(ctx, q_d, cumsum, s_d, gather_index=gather)
+    disp_s = time_launches(lambda: fast_all_to_all(ctx, q_d, cumsum, s_d, scatter_index=scatter), steps, warmup)
+    _, recv, recv_scale = fast_all_to_all(ctx, q_d, cumsum, s_d, scatter_index=scatter)
     comb_s = time_launches(lambda: moe_weighted_combine(ctx, recv, recv_scale, scatter, w, cumsum), steps, warmup)
     n = T * topk
     disp_bytes = T * H + n * H + T * 4 + n * 4 + n * 4          # unique row reads + row writes + scales + gather index

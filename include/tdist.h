@@ -179,6 +179,15 @@ int tdist_moe_dispatch(const void* rows, int64_t row_bytes, const float* scales,
                        const int32_t* cumsum, int64_t n_rows, int world_size, int experts_per_rank,
                        int max_m, void* slot_rows, float* slot_scales, int32_t* splits_out, void* stream);
 
+/* Token-major form of the dispatch, fusing the reference's index_select (test/nvidia/test_all_to_all.py:
+ * 328-329) into it: tokens [n_tokens, row_bytes] unsorted, token_scales fp32[n_tokens] or NULL, scatter_idx
+ * int32[n_tokens*topk]; the row of token t is read once and written to the slot rows of its topk sorted
+ * positions scatter_idx[t*topk + k] (same slot layout and skipping rules as tdist_moe_dispatch). */
+int tdist_moe_dispatch_tokens(const void* tokens, int64_t row_bytes, const float* token_scales,
+                              const int32_t* scatter_idx, int topk, const int32_t* cumsum, int64_t n_tokens,
+                              int world_size, int experts_per_rank, int max_m, void* slot_rows, float* slot_scales,
+                              int32_t* splits_out, void* stream);
+
 /* Compaction of the slots into one [sum, row_bytes] tensor in destination order
  * (all_to_all_post_process, low_latency_all_to_all.py:251-270): output row p comes from slot row
  * d*max_m + (p - start_d) where start_d = sum of splits of destinations < d.

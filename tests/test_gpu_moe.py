@@ -70,8 +70,11 @@ def test_splits_cumsum_entry_point(cuda):
 
 
 @pytest.mark.parametrize("T,topk,G,W,H,max_m,fused", [(4096, 8, 256, 32, 7168, 4096, True), (4096, 8, 256, 32, 7168, 4096, False),
-                                                     (96, 4, 16, 4, 48, 160, True), (50, 3, 6, 2, 24, 40, False),
-                                                     (10, 2, 8, 8, 1024, 8, True)])
+                                                     (4096, 8, 256, 32, 7168, 4096, "tokens"), (96, 4, 16, 4, 48, 160, True),
+                                                     (96, 4, 16, 4, 48, 160, "tokens"), (50, 3, 6, 2, 24, 40, False),
+                                                     (50, 3, 6, 2, 24, 40, "tokens"), (10, 2, 8, 8, 1024, 8, True),
+                                                     (10, 2, 8, 8, 1024, 8, "tokens"), (33, 5, 8, 2, 12000, 128, "tokens"),
+                                                     (21, 3, 4, 4, 52, 64, "tokens")])
 def test_dispatch_bytes_bit_exact_and_round_trip(cuda, T, topk, G, W, H, max_m, fused):
     from triton_dist.kernels.amd import (all_to_all_post_process, create_all_to_all_context, fast_all_to_all,
                                          moe_dispatch_preprocess)
@@ -82,7 +85,9 @@ def test_dispatch_bytes_bit_exact_and_round_trip(cuda, T, topk, G, W, H, max_m, 
     ctx.recv_buf.view(torch.uint8).fill_(0xAB)
     splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids.to(cuda), G)
     dq, ds = q.to(cuda), s.to(cuda)
-    if fused:
+    if fused == "tokens":
+        out_splits, recv, recv_scale = fast_all_to_all(ctx, dq, cumsum, ds, scatter_index=scatter)
+    elif fused:
         out_splits, recv, recv_scale = fast_all_to_all(ctx, dq, cumsum, ds, gather_index=gather)
     else:
         rows = torch.index_select(dq.view(torch.uint8), 0, gather.long()).view(torch.float8_e4m3fn)

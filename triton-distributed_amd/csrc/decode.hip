@@ -9,14 +9,17 @@
 //  * K and V rows go HBM → LDS with asynchronous 16-byte-per-lane LDS-DMA loads into a per-wave ring of
 //    NST stages (P = NST-1 stages in flight), so the only synchronisation is the wave's own vmcnt;
 //    the page-table entries a stage needs travel the same way, two rounds ahead of the rows;
-//  * scores:  S^T[key, head] = K[16 keys, D] . Q^T[D, 16 heads]   v_mfma_f32_16x16x32 (D/32 steps);
-//    the result layout (lane = head, 4 keys per lane) is exactly the B operand of
-//    O^T[dv, head] += V^T[16 dv, 16 keys] . P^T[16 keys, 16 heads]  v_mfma_f32_16x16x16 (D/16 tiles),
-//    so probabilities never leave registers; V^T fragments are 16-bit LDS reads from the swizzled rows;
+//  * scores:  S^T[key, head] = K[16 keys, D] . Q^T[D, 16 heads]   v_mfma_f32_16x16x32 (D/32 steps) per group
+//    of 16 keys; the result layout (lane = head, 4 keys per lane) is exactly the B operand of
+//    O^T[dv, head] += V^T[16 dv, keys] . P^T[keys, 16 heads]  (v_mfma 16x16x32 over two key groups, or
+//    16x16x16 over one), so probabilities never leave registers; the V^T fragments come from the
+//    row-major V rows in LDS with the transposing read ds_read_b64_tr_b16, one instruction per 4 keys;
 //  * probabilities enter the PV product as a hi+lo pair of 16-bit values, which keeps the product at
 //    fp32-level accuracy for the cost of a second (idle anyway) MFMA.
 //
 // HBM traffic per launch: every K and V row of the split once (2 * len * Hkv * D * 2 B per sequence).
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace tdist {
@@ -47,55 +50,63 @@ struct DecodeParams {
 struct MmaBF16 {
   typedef bf16x8v frag8;
   typedef short4v frag4;
-  __device__ static __forceinline__ float4v qk(frag8 a, frag8 b, float4v c) {
+  __device__ static __forceinline__ float4v mma32(frag8 a, frag8 b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
-  __device__ static __forceinline__ float4v pv(frag4 a, frag4 b, float4v c) {
+  __device__ static __forceinline__ float4v mma16(frag4 a, frag4 b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
   }
   // p → (hi, lo) 16-bit patterns with hi + lo ≈ p to ~16 mantissa bits
-  __device__ static __forceinline__ void split(float p, uint32_t& hi, uint32_t& lo) {
-    hi = f32_to_bf16_bits(p);
-    lo = f32_to_bf16_bits(p - bf16_bits_to_f32(hi));
+  __device__ static __forceinline__ void split(float p0, float p1, uint32_t& hi, uint32_t& lo) {
+    hi = pack_bf16x2(p0, p1);
+    lo = pack_bf16x2(p0 - BF16::lo(hi), p1 - BF16::hi(hi));
   }
 };
 struct MmaF16 {
   typedef f16x8v frag8;
   typedef f16x4v frag4;
-  __device__ static __forceinline__ float4v qk(frag8 a, frag8 b, float4v c) {
+  __device__ static __forceinline__ float4v mma32(frag8 a, frag8 b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
-  __device__ static __forceinline__ float4v pv(frag4 a, frag4 b, float4v c) {
+  __device__ static __forceinline__ float4v mma16(frag4 a, frag4 b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
   }
-  __device__ static __forceinline__ void split(float p, uint32_t& hi, uint32_t& lo) {
-    _Float16 h = (_Float16)p;
-    _Float16 l = (_Float16)(p - (float)h);
-    hi = __builtin_bit_cast(unsigned short, h);
-    lo = __builtin_bit_cast(unsigned short, l);
+  __device__ static __forceinline__ void split(float p0, float p1, uint32_t& hi, uint32_t& lo) {
+    hi = pack_f16x2(p0, p1);
+    lo = pack_f16x2(p0 - F16::lo(hi), p1 - F16::hi(hi));
   }
 };
 
-constexpr int kBlockKeys = 16;
-constexpr int kTableSlots = 8;          // ring of page-table rows per wave (>= 2P+2)
-constexpr int kTableSlotBytes = 16 * 4; // 16 entries
+constexpr int kTableSlots = 8;  // ring of page-table rows per wave (>= 2P+2)
 
-template <int D, int NST>
+// KEYS = keys per block (16 or 32): one or two groups of 16 keys, a group being one MFMA tile of scores.
+template <int D, int KEYS, int NST>
 struct DecodeCfg {
+  static constexpr int kGroups = KEYS / 16;
   static constexpr int kRowBytes = D * 2;
   static constexpr int kLanesPerRow = kRowBytes / 16;       // 16-byte chunks per row
   static constexpr int kRowsPerInstr = 64 / kLanesPerRow;   // rows one wave-wide DMA covers
-  static constexpr int kInstrPerTensor = kBlockKeys / kRowsPerInstr;
-  static constexpr int kTensorBytes = kBlockKeys * kRowBytes;
+  static constexpr int kInstrPerTensor = KEYS / kRowsPerInstr;
+  static constexpr int kTensorBytes = KEYS * kRowBytes;
   static constexpr int kStageBytes = 2 * kTensorBytes;
   static constexpr int kLoadsPerGroup = 1 + 2 * kInstrPerTensor;  // table row + K + V
   static constexpr int kP = NST - 1;
-  static constexpr int kSwz = (kLanesPerRow < 16 ? kLanesPerRow : 16) - 1;
+  // LDS position of 16-byte chunk c of a row: K rows c ^ kswz(key), V rows c ^ vswz(key).
+  // K operand reads: 16 lanes = 16 keys, same chunk      → spread over 16 positions: key & 15.
+  // V transposed reads: 32 lanes = 8 keys x 2 adjacent chunks → spread the chunk pairs: (key & 7) << 1.
+  static constexpr int kSwzMask = (kLanesPerRow < 16 ? kLanesPerRow : 16) - 1;
+  static constexpr int kTableSlotBytes = KEYS * 4;
   static constexpr int kWaveBytes = NST * kStageBytes + kTableSlots * kTableSlotBytes;
+  static_assert(KEYS == 16 || KEYS == 32, "one or two key groups");
   static_assert(kP >= 1 && kP <= 3, "1..3 stages in flight");
   static_assert(kP * kLoadsPerGroup < 64, "vmcnt is 6 bits");
   static_assert(2 * kP + 2 <= kTableSlots, "table ring too small");
   static_assert(D % 32 == 0 && D >= 64 && D <= 256, "head dim");
+  // Rows shorter than the 256-byte bank window already differ in their row offset: only every kRowsPerWindow-th
+  // key needs a new XOR term.
+  static constexpr int kRowsPerWindow = kRowBytes >= 256 ? 1 : 256 / kRowBytes;
+  __device__ static __forceinline__ int kswz(int key) { return (key / kRowsPerWindow) & kSwzMask; }
+  __device__ static __forceinline__ int vswz(int key) { return (((key / kRowsPerWindow) & 7) << 1) & kSwzMask; }
 };
 
 template <int N>
@@ -107,16 +118,19 @@ __device__ __forceinline__ void wait_groups(int rem) {
   else wait_vmcnt<0>();
 }
 
-template <typename MMA, int D, int NW, int NST, bool kSoftCap>
+template <typename MMA, int D, int KEYS, int NW, int NST, bool kSoftCap>
 __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodeParams prm) {
-  typedef DecodeCfg<D, NST> C;
+  typedef DecodeCfg<D, KEYS, NST> C;
+  constexpr int G = C::kGroups;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
-  const int split = blockIdx.x;
+  // kv heads vary fastest over the grid: workgroups that run together then read the neighbouring 2*D-byte
+  // pieces of the same token rows
+  const int split = blockIdx.y;
   const int group = prm.Hq / prm.Hkv;
   const int head_blocks = (group + 15) >> 4;
-  const int kvh = blockIdx.y / head_blocks;
-  const int hb = blockIdx.y - kvh * head_blocks;
+  const int kvh = blockIdx.x / head_blocks;
+  const int hb = blockIdx.x - kvh * head_blocks;
   const int b = blockIdx.z;
   const int h0 = kvh * group + hb * 16;
   const int nvalid = min(16, group - hb * 16);
@@ -124,7 +138,7 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform for the compiler too
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;   // lane group 0..3
-  const int x = lane & 15;   // head (QK result column) / dv within tile (V^T row)
+  const int x = lane & 15;   // head (score column) / dv within tile (V^T row) / key (K row)
 
   const int len = prm.lens[b];
   const int per = (len + prm.S - 1) / prm.S;
@@ -149,7 +163,7 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
   lds_u8 const wbase = smem3 + wave * C::kWaveBytes;
   lds_u8 const tbl_base = wbase + NST * C::kStageBytes;
 
-  const int nb_total = (end - start + kBlockKeys - 1) / kBlockKeys;
+  const int nb_total = (end - start + KEYS - 1) / KEYS;
   const int n_w = nb_total > wave ? (nb_total - wave + NW - 1) / NW : 0;  // this wave's blocks
 
   // ---- Q fragments (B operand of the score MFMA): head x, dims 32s + 8g .. +8 -------------------
@@ -173,27 +187,50 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
 #pragma unroll
   for (int d = 0; d < D / 16; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  // first key of the wave's j-th block
-  auto block_key0 = [&](int j) { return start + (wave + j * NW) * kBlockKeys; };
+  // Loop-invariant LDS offsets (relative to the stage) of this lane's operand reads.
+  // K (A operand of the scores): row = key x of group q, logical chunk 4s+g.
+  int koff[G][D / 32];
+#pragma unroll
+  for (int q = 0; q < G; ++q)
+#pragma unroll
+    for (int s = 0; s < D / 32; ++s) {
+      const int key = 16 * q + x;
+      koff[q][s] = key * C::kRowBytes + (((4 * s + g) ^ C::kswz(key)) << 4);
+    }
+  // V^T (A operand of the output MFMA) through the transposing LDS read: within a 16-lane block, lane x ends
+  // up with elements x, 16+x, 32+x, 48+x of the 64 the block loads (lane s loads 4 consecutive ones), so lane s
+  // supplies V[key 4g + s/4 of group q][dv 16d + 4(s%4) .. +3] and lane x receives V[4g+j][16d+x], j = 0..3.
+  int voff[G][D / 16];
+#pragma unroll
+  for (int q = 0; q < G; ++q)
+#pragma unroll
+    for (int d = 0; d < D / 16; ++d) {
+      const int key = 16 * q + 4 * g + (x >> 2);
+      const int chunk = 2 * d + ((x & 3) >> 1);
+      voff[q][d] = C::kTensorBytes + key * C::kRowBytes + ((chunk ^ C::vswz(key)) << 4) + (x & 1) * 8;
+    }
 
-  // page-table row of block j → table ring slot j % kTableSlots (lanes 0..15, one entry per key)
+  // first key of the wave's j-th block
+  auto block_key0 = [&](int j) { return start + (wave + j * NW) * KEYS; };
+
+  // page-table row of block j → table ring slot j % kTableSlots (one entry per key)
   auto issue_table = [&](int j) {
-    if (lane < 16) {
+    if (lane < KEYS) {
       int n = block_key0(j) + lane;
       n = min(n, end - 1);
       n = max(n, start);
       const int e = (int)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift);
       const int32_t* src = prm.table + (int64_t)b * prm.t_s + e;
       __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)src,
-                                       (TDIST_AS3 void*)(tbl_base + (j % kTableSlots) * kTableSlotBytes), 4, 0, 0);
+                                       (TDIST_AS3 void*)(tbl_base + (j % kTableSlots) * C::kTableSlotBytes), 4, 0, 0);
     }
   };
 
-  // K and V rows of block j → stage j % NST. LDS position i of a row holds 16-byte chunk i ^ (key & swz).
+  // K and V rows of block j → stage j % NST
   auto issue_rows = [&](int j) {
     const int key0 = block_key0(j);
     const volatile TDIST_AS3 int32_t* tbl =
-        (const volatile TDIST_AS3 int32_t*)(tbl_base + (j % kTableSlots) * kTableSlotBytes);
+        (const volatile TDIST_AS3 int32_t*)(tbl_base + (j % kTableSlots) * C::kTableSlotBytes);
     lds_u8 const kst = wbase + (j % NST) * C::kStageBytes;
     lds_u8 const vst = kst + C::kTensorBytes;
     const int chunk = lane % C::kLanesPerRow;
@@ -202,13 +239,12 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
       const int key = i * C::kRowsPerInstr + lane / C::kLanesPerRow;
       int n = min(key0 + key, end - 1);
       n = max(n, start);
-      const int page = tbl[key];
-      const int in_page = n - (int)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift) * prm.page_size;
-      const int src_chunk = chunk ^ (key & C::kSwz);
-      const unsigned char* ksrc = prm.k + (int64_t)page * prm.k_sp + (int64_t)in_page * prm.k_st +
-                                  (int64_t)kvh * prm.k_sh + src_chunk * 16;
-      const unsigned char* vsrc = prm.v + (int64_t)page * prm.v_sp + (int64_t)in_page * prm.v_st +
-                                  (int64_t)kvh * prm.v_sh + src_chunk * 16;
+      const uint32_t page = (uint32_t)tbl[key];
+      const uint32_t in_page = (uint32_t)n - (uint32_t)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift) * (uint32_t)prm.page_size;
+      const unsigned char* ksrc = prm.k + (uint64_t)page * (uint64_t)prm.k_sp +
+                                  (in_page * (uint32_t)prm.k_st + (uint32_t)kvh * (uint32_t)prm.k_sh + ((chunk ^ C::kswz(key)) << 4));
+      const unsigned char* vsrc = prm.v + (uint64_t)page * (uint64_t)prm.v_sp +
+                                  (in_page * (uint32_t)prm.v_st + (uint32_t)kvh * (uint32_t)prm.v_sh + ((chunk ^ C::vswz(key)) << 4));
       __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)ksrc, (TDIST_AS3 void*)(kst + i * 1024), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)vsrc, (TDIST_AS3 void*)(vst + i * 1024), 16, 0, 0);
     }
@@ -216,31 +252,34 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
 
   auto compute = [&](int j) {
     const int key0 = block_key0(j);
-    lds_u8 const kst = wbase + (j % NST) * C::kStageBytes;
-    lds_u8 const vst = kst + C::kTensorBytes;
-    // scores: A = K rows (key x, dims 32s+8g..), B = Q
-    float4v sc = {0.f, 0.f, 0.f, 0.f};
+    lds_u8 const st = wbase + (j % NST) * C::kStageBytes;
+    // scores: A = K rows (key x of group q, dims 32s+8g..), B = Q  →  sc[q][i]: key 16q+4g+i, head x
+    float4v sc[G];
 #pragma unroll
-    for (int s = 0; s < D / 32; ++s) {
-      const int c = 4 * s + g;
-      const int4v raw = *(const TDIST_AS3 int4v*)(kst + x * C::kRowBytes + ((c ^ (x & C::kSwz)) << 4));
-      sc = MMA::qk(__builtin_bit_cast(typename MMA::frag8, raw), qf[s], sc);
+    for (int q = 0; q < G; ++q) {
+      sc[q] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < D / 32; ++s) {
+        const int4v raw = *(const TDIST_AS3 int4v*)(st + koff[q][s]);
+        sc[q] = MMA::mma32(__builtin_bit_cast(typename MMA::frag8, raw), qf[s], sc[q]);
+      }
     }
-    // sc[i]: key 4g+i, head x
-    float t[4];
+    float t[G][4];
     float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float v;
-      if (kSoftCap) {
-        v = prm.soft_cap * tanhf(sc[i] * prm.sm_scale / prm.soft_cap) * kLog2e;
-      } else {
-        v = sc[i] * scale_log2;
+    for (int q = 0; q < G; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v;
+        if (kSoftCap) {
+          v = prm.soft_cap * tanhf(sc[q][i] * prm.sm_scale / prm.soft_cap) * kLog2e;
+        } else {
+          v = sc[q][i] * scale_log2;
+        }
+        const bool valid = key0 + 16 * q + 4 * g + i < end;
+        t[q][i] = valid ? v : -INFINITY;
+        mx = fmaxf(mx, t[q][i]);
       }
-      const bool valid = key0 + 4 * g + i < end;
-      t[i] = valid ? v : -INFINITY;
-      mx = fmaxf(mx, t[i]);
-    }
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
@@ -252,31 +291,40 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
       m_run = m_new;
     }
     const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
-    uint32_t hi[4], lo[4];
+    // probabilities as the B operand: k slots 4q..4q+3 of lane group g ↔ keys 16q+4g .. +3
+    uint32_t hi[G][2], lo[G][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float p = __builtin_amdgcn_exp2f(t[i] - m_safe);
-      l_run += p;
-      MMA::split(p, hi[i], lo[i]);
-    }
-    int2v ph = {(int)(hi[0] | (hi[1] << 16)), (int)(hi[2] | (hi[3] << 16))};
-    int2v pl = {(int)(lo[0] | (lo[1] << 16)), (int)(lo[2] | (lo[3] << 16))};
-    const typename MMA::frag4 p_hi = __builtin_bit_cast(typename MMA::frag4, ph);
-    const typename MMA::frag4 p_lo = __builtin_bit_cast(typename MMA::frag4, pl);
-    // O^T tiles: A = V^T (dv 16d+x, keys 4g..4g+3), B = P^T
-#pragma unroll
-    for (int d = 0; d < D / 16; ++d) {
-      const int dv = 16 * d + x;
-      uint32_t e[4];
+    for (int q = 0; q < G; ++q) {
+      float p[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = 4 * g + i;
-        e[i] = *(const TDIST_AS3 unsigned short*)(vst + key * C::kRowBytes + (((dv >> 3) ^ (key & C::kSwz)) << 4) + (dv & 7) * 2);
+        p[i] = __builtin_amdgcn_exp2f(t[q][i] - m_safe);
+        l_run += p[i];
       }
-      int2v vv = {(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16))};
-      const typename MMA::frag4 vt = __builtin_bit_cast(typename MMA::frag4, vv);
-      acc[d] = MMA::pv(vt, p_hi, acc[d]);
-      acc[d] = MMA::pv(vt, p_lo, acc[d]);
+      MMA::split(p[0], p[1], hi[q][0], lo[q][0]);
+      MMA::split(p[2], p[3], hi[q][1], lo[q][1]);
+    }
+    // O^T tiles: A = V^T (dv 16d+x; k slots as above), B = P^T
+#pragma unroll
+    for (int d = 0; d < D / 16; ++d) {
+      if (G == 2) {
+        const short4v v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TDIST_AS3 short4v*)(st + voff[0][d]));
+        const short4v v1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TDIST_AS3 short4v*)(st + voff[G - 1][d]));
+        const int2v a0 = __builtin_bit_cast(int2v, v0), a1 = __builtin_bit_cast(int2v, v1);
+        const int4v vt = {a0[0], a0[1], a1[0], a1[1]};
+        const int4v ph = {(int)hi[0][0], (int)hi[0][1], (int)hi[G - 1][0], (int)hi[G - 1][1]};
+        const int4v pl = {(int)lo[0][0], (int)lo[0][1], (int)lo[G - 1][0], (int)lo[G - 1][1]};
+        const typename MMA::frag8 vf = __builtin_bit_cast(typename MMA::frag8, vt);
+        acc[d] = MMA::mma32(vf, __builtin_bit_cast(typename MMA::frag8, ph), acc[d]);
+        acc[d] = MMA::mma32(vf, __builtin_bit_cast(typename MMA::frag8, pl), acc[d]);
+      } else {
+        const short4v v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TDIST_AS3 short4v*)(st + voff[0][d]));
+        const int2v ph = {(int)hi[0][0], (int)hi[0][1]};
+        const int2v pl = {(int)lo[0][0], (int)lo[0][1]};
+        const typename MMA::frag4 vf = __builtin_bit_cast(typename MMA::frag4, v0);
+        acc[d] = MMA::mma16(vf, __builtin_bit_cast(typename MMA::frag4, ph), acc[d]);
+        acc[d] = MMA::mma16(vf, __builtin_bit_cast(typename MMA::frag4, pl), acc[d]);
+      }
     }
   };
 
@@ -411,26 +459,27 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams
   if (prm.lse_out && lane == 0) prm.lse_out[bh] = L > 0.f ? M + logf(L) : -INFINITY;
 }
 
-template <typename MMA, int D, int NW, int NST, bool kSoftCap>
+template <typename MMA, int D, int KEYS, int NW, int NST, bool kSoftCap>
 static int launch_decode_sc(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
-  typedef DecodeCfg<D, NST> C;
+  typedef DecodeCfg<D, KEYS, NST> C;
+  static_assert((32 + D * 16) * 4 <= C::kWaveBytes, "merge scratch must fit in a wave's ring");
   const size_t lds = (size_t)NW * C::kWaveBytes;
-  auto kern = decode_split_kv_kernel<MMA, D, NW, NST, kSoftCap>;
+  auto kern = decode_split_kv_kernel<MMA, D, KEYS, NW, NST, kSoftCap>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(TDIST_ERR_LAUNCH, "decode: cannot reserve %zu B of LDS: %s", lds, hipGetErrorString(e));
     attr_set = true;
   }
-  dim3 grid(prm.S, prm.Hkv * head_blocks, prm.B);
+  dim3 grid(prm.Hkv * head_blocks, prm.S, prm.B);
   hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, prm);
   return launch_status("tdist_decode_split_kv");
 }
 
-template <typename MMA, int D, int NW, int NST>
+template <typename MMA, int D, int KEYS, int NW, int NST>
 static int launch_decode(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
-  return prm.soft_cap > 0.f ? launch_decode_sc<MMA, D, NW, NST, true>(prm, head_blocks, stream)
-                            : launch_decode_sc<MMA, D, NW, NST, false>(prm, head_blocks, stream);
+  return prm.soft_cap > 0.f ? launch_decode_sc<MMA, D, KEYS, NW, NST, true>(prm, head_blocks, stream)
+                            : launch_decode_sc<MMA, D, KEYS, NW, NST, false>(prm, head_blocks, stream);
 }
 
 }  // namespace tdist
@@ -494,12 +543,24 @@ int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cach
   hipStream_t st = (hipStream_t)stream;
   const bool bf = dtype == TDIST_BF16;
   switch (head_dim) {
+    // <dtype, D, keys per block, waves, stages>: LDS = waves * (stages * keys * D * 4 B + tables) <= 160 KB
     case 64:
-      return bf ? launch_decode<MmaBF16, 64, 4, 4>(prm, head_blocks, st) : launch_decode<MmaF16, 64, 4, 4>(prm, head_blocks, st);
-    case 128:
-      return bf ? launch_decode<MmaBF16, 128, 4, 4>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 4, 4>(prm, head_blocks, st);
+      return bf ? launch_decode<MmaBF16, 64, 32, 4, 4>(prm, head_blocks, st) : launch_decode<MmaF16, 64, 32, 4, 4>(prm, head_blocks, st);
+    case 128: {
+      // TDIST_DECODE_VARIANT picks another compiled shape (measurement aid). Default: 16-key blocks, 4 waves,
+      // 2 stages = 66 KB of LDS, so two workgroups share a CU; measured within 2 % of the best of the others.
+      int variant = 0;
+      if (const char* v = getenv("TDIST_DECODE_VARIANT")) variant = atoi(v);
+      if (variant == 1)
+        return bf ? launch_decode<MmaBF16, 128, 32, 4, 2>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 32, 4, 2>(prm, head_blocks, st);
+      if (variant == 2)
+        return bf ? launch_decode<MmaBF16, 128, 32, 3, 3>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 32, 3, 3>(prm, head_blocks, st);
+      if (variant == 3)
+        return bf ? launch_decode<MmaBF16, 128, 16, 8, 2>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 16, 8, 2>(prm, head_blocks, st);
+      return bf ? launch_decode<MmaBF16, 128, 16, 4, 2>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 16, 4, 2>(prm, head_blocks, st);
+    }
     default:
-      return bf ? launch_decode<MmaBF16, 256, 2, 3>(prm, head_blocks, st) : launch_decode<MmaF16, 256, 2, 3>(prm, head_blocks, st);
+      return bf ? launch_decode<MmaBF16, 256, 16, 2, 3>(prm, head_blocks, st) : launch_decode<MmaF16, 256, 16, 2, 3>(prm, head_blocks, st);
   }
 }
 

@@ -58,11 +58,16 @@ __global__ __launch_bounds__(kScanThreads) void moe_scan_kernel(int32_t* __restr
     const int g = g0 + j;
     if (g < G) {
       int32_t run = 0;
-      for (int b = 0; b < num_blocks; ++b) {
-        const int64_t at = (int64_t)b * G + g;
-        const int32_t h = hist[at];
-        hist[at] = run;
-        run += h;
+      // 16 independent loads at a time, then their exclusive prefix
+      for (int b0 = 0; b0 < num_blocks; b0 += 16) {
+        int32_t h[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) h[u] = (b0 + u < num_blocks) ? hist[(int64_t)(b0 + u) * G + g] : 0;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          if (b0 + u < num_blocks) hist[(int64_t)(b0 + u) * G + g] = run;
+          run += h[u];
+        }
       }
       splits[g] = run;
       local_total += run;
@@ -277,6 +282,72 @@ __global__ __launch_bounds__(256) void moe_rows_kernel(const unsigned char* __re
   }
 }
 
+// Token-major dispatch: the row of token t is read once and written to the slot rows of its topk sorted
+// positions p = scatter_idx[t*topk + k]. One wave per (token, window of 512 16-byte chunks).
+template <bool kVec16>
+__global__ __launch_bounds__(256) void moe_dispatch_tokens_kernel(const unsigned char* __restrict__ tokens,
+                                                                  int64_t row_bytes, const float* __restrict__ scales,
+                                                                  const int32_t* __restrict__ scatter_idx, int topk,
+                                                                  const int32_t* __restrict__ cumsum, int64_t n_tokens,
+                                                                  int W, int Er, int max_m,
+                                                                  unsigned char* __restrict__ slot_rows,
+                                                                  float* __restrict__ slot_scales,
+                                                                  int32_t* __restrict__ splits_out, int windows) {
+  extern __shared__ int32_t s_bound[];  // [W+1]
+  for (int d = threadIdx.x; d <= W; d += 256) s_bound[d] = cumsum[d * Er];
+  if (splits_out && blockIdx.x == 0) {
+    const int G = W * Er;
+    for (int g = threadIdx.x; g < G; g += 256) splits_out[g] = cumsum[g + 1] - cumsum[g];
+  }
+  __syncthreads();
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
+  const int64_t t = unit / windows;
+  const int win = (int)(unit - t * windows);
+  if (t >= n_tokens) return;
+  // lane k < topk resolves the slot row of copy k
+  int32_t my_dst = -1;
+  if (lane < topk) {
+    const int32_t p = scatter_idx[t * topk + lane];
+    if (p >= 0 && p < s_bound[W]) {
+      const int d = find_dest(s_bound, 1, W, p);
+      const int32_t in_slot = p - s_bound[d];
+      if (in_slot < max_m) my_dst = d * max_m + in_slot;
+    }
+    if (win == 0 && my_dst >= 0 && scales) slot_scales[my_dst] = scales[t];
+  }
+  const unsigned char* src = tokens + t * row_bytes;
+  if (kVec16) {
+    const int n16 = (int)(row_bytes >> 4);
+    const int base = win * 512;
+    const int4v* s16 = (const int4v*)src;
+    int4v v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = base + j * 64 + lane;
+      if (c < n16) v[j] = s16[c];
+    }
+    for (int k = 0; k < topk; ++k) {
+      const int32_t dst_row = __shfl(my_dst, k);
+      if (dst_row < 0) continue;
+      int4v* d16 = (int4v*)(slot_rows + (int64_t)dst_row * row_bytes);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int c = base + j * 64 + lane;
+        if (c < n16) __builtin_nontemporal_store(v[j], d16 + c);
+      }
+    }
+  } else {
+    for (int k = 0; k < topk; ++k) {
+      const int32_t dst_row = __shfl(my_dst, k);
+      if (dst_row < 0) continue;
+      unsigned char* dst = slot_rows + (int64_t)dst_row * row_bytes;
+      for (int64_t c = (int64_t)win * 8192 + lane; c < row_bytes && c < (int64_t)(win + 1) * 8192; c += 64) dst[c] = src[c];
+    }
+  }
+}
+
 // Weighted combine: one workgroup per token; thread c owns 16-byte column chunk(s) of the row.
 // kFp8: rows are e4m3 bytes (16 elements per chunk), else bf16 (8 elements per chunk).
 constexpr int kCombineMaxTopk = 32;
@@ -448,6 +519,31 @@ int tdist_moe_dispatch(const void* rows, int64_t row_bytes, const float* scales,
                      (const unsigned char*)rows, row_bytes, scales, gather_idx, cumsum, n_rows, world_size,
                      experts_per_rank, max_m, (unsigned char*)slot_rows, slot_scales, splits_out);
   return launch_status("tdist_moe_dispatch");
+}
+
+int tdist_moe_dispatch_tokens(const void* tokens, int64_t row_bytes, const float* token_scales,
+                              const int32_t* scatter_idx, int topk, const int32_t* cumsum, int64_t n_tokens,
+                              int world_size, int experts_per_rank, int max_m, void* slot_rows, float* slot_scales,
+                              int32_t* splits_out, void* stream) {
+  if (!tokens || !scatter_idx || !cumsum || !slot_rows)
+    return fail(TDIST_ERR_INVALID, "tdist_moe_dispatch_tokens: null pointer");
+  if ((token_scales != nullptr) != (slot_scales != nullptr))
+    return fail(TDIST_ERR_INVALID, "tdist_moe_dispatch_tokens: token_scales and slot_scales go together");
+  if (row_bytes <= 0 || n_tokens < 0 || world_size <= 0 || experts_per_rank <= 0 || max_m <= 0 || topk <= 0)
+    return fail(TDIST_ERR_INVALID, "tdist_moe_dispatch_tokens: bad sizes");
+  if (topk > 64) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_dispatch_tokens: topk > 64");
+  if (world_size > 8192 || (int64_t)world_size * max_m > 0x7fffffff)
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_dispatch_tokens: world_size * max_m too large");
+  const int windows = (int)ceil_div(row_bytes, 8192);
+  const int64_t units = (n_tokens > 0 ? n_tokens : 1) * windows;
+  const int64_t blocks = ceil_div(units, 4);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_dispatch_tokens: too many tokens");
+  const bool vec = (row_bytes % 16 == 0) && aligned16(tokens) && aligned16(slot_rows);
+  auto kern = vec ? moe_dispatch_tokens_kernel<true> : moe_dispatch_tokens_kernel<false>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), (size_t)(world_size + 1) * 4, (hipStream_t)stream,
+                     (const unsigned char*)tokens, row_bytes, token_scales, scatter_idx, topk, cumsum, n_tokens,
+                     world_size, experts_per_rank, max_m, (unsigned char*)slot_rows, slot_scales, splits_out, windows);
+  return launch_status("tdist_moe_dispatch_tokens");
 }
 
 int tdist_moe_post_process(const void* slot_rows, int64_t row_bytes, const float* slot_scales, const int32_t* splits,

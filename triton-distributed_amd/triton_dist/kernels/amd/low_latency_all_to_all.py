@@ -128,6 +128,7 @@ def fast_all_to_all(
     send_split_cumsum: torch.Tensor,
     send_scale: Optional[torch.Tensor],
     gather_index: Optional[torch.Tensor] = None,
+    scatter_index: Optional[torch.Tensor] = None,
 ):
     """
     low-latency all-to-all communication (reference :189-248).
@@ -136,11 +137,13 @@ def fast_all_to_all(
     or None. With ``gather_index`` (int32[n_sorted], an addition) ``send_tensor`` is the unsorted
     [T, hidden] token tensor (``send_scale`` per token) and sorted row p is read from token
     gather_index[p], which fuses the reference's index_select (test_all_to_all.py:328-329) into the copy.
+    With ``scatter_index`` (int32[T, topk], an addition) the same fusion runs token-major: every token row is
+    read once and written to its topk slot rows, which is the faster form.
 
     Returns [splits int32[G], recv [W*max_m, hidden], scales [W*max_m] | None] — views into the context's
     buffers, valid until the call after next.
     """
-    _lib.require_cuda(send_tensor, send_split_cumsum, send_scale, gather_index)
+    _lib.require_cuda(send_tensor, send_split_cumsum, send_scale, gather_index, scatter_index)
     with_scale = send_scale is not None
     act_pos = ctx.call_count % 2
 
@@ -165,10 +168,18 @@ def fast_all_to_all(
     recv = ctx.recv_buf[data_buf_st:data_buf_ed, :]
     scale_recv = ctx.scale_recv_buf[data_buf_st:data_buf_ed]
     splits = ctx.split_recv_buf[split_buf_st:split_buf_ed]
-    _lib.call("tdist_moe_dispatch", send_tensor.data_ptr(), ctx.hidden * ctx.ele_size, _lib.ptr(send_scale),
-              _lib.ptr(gather_index), send_split_cumsum.data_ptr(), n_rows, ctx.WORLD_SIZE, ctx.experts_per_rank,
-              ctx.max_m, recv.data_ptr(), scale_recv.data_ptr() if with_scale else None, splits.data_ptr(),
-              _lib.stream_ptr())
+    if scatter_index is not None:
+        assert scatter_index.dtype == torch.int32 and scatter_index.is_contiguous()
+        assert scatter_index.shape[0] == send_tensor.shape[0]
+        _lib.call("tdist_moe_dispatch_tokens", send_tensor.data_ptr(), ctx.hidden * ctx.ele_size, _lib.ptr(send_scale),
+                  scatter_index.data_ptr(), scatter_index.shape[1], send_split_cumsum.data_ptr(), send_tensor.shape[0],
+                  ctx.WORLD_SIZE, ctx.experts_per_rank, ctx.max_m, recv.data_ptr(),
+                  scale_recv.data_ptr() if with_scale else None, splits.data_ptr(), _lib.stream_ptr())
+    else:
+        _lib.call("tdist_moe_dispatch", send_tensor.data_ptr(), ctx.hidden * ctx.ele_size, _lib.ptr(send_scale),
+                  _lib.ptr(gather_index), send_split_cumsum.data_ptr(), n_rows, ctx.WORLD_SIZE, ctx.experts_per_rank,
+                  ctx.max_m, recv.data_ptr(), scale_recv.data_ptr() if with_scale else None, splits.data_ptr(),
+                  _lib.stream_ptr())
 
     ctx.call_count = (ctx.call_count + 1) % ctx.MOD_VALUE
     out_lis = [splits, recv]
