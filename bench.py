@@ -24,6 +24,7 @@ for p in (ROOT, os.path.join(ROOT, "triton-distributed_amd")):
         sys.path.insert(0, p)
 
 PEAK = {"bf16": 2.5e15, "fp8": 5.0e15, "hbm": 8.0e12}  # MI355X published dense MFMA peaks (FLOP/s) and HBM3E B/s
+LIVE_PRODUCER = True  # --no-live-producer clears it
 METRIC = "AG-GEMM/GEMM-RS TFLOPS (% MFMA peak); decode & A2A GB/s (% HBM peak)"
 
 
@@ -132,18 +133,20 @@ def bench_c1(dev, steps, warmup):
     ctx.set_peer_shards({r: s.to(dev) for r, s in enumerate(shards) if r != rank})
     a_d, b_d = shards[rank].to(dev), b.to(dev)
     flops = 2.0 * world * mpr * N * K
-    live_s = time_launches(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx), steps, warmup)
-    c = ag_gemm_intra_node(a_d, b_d, False, ctx)
-    ctx.check_status()
-    err = golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32(shards, b))
-    assert err <= 1e-2
+    live_s = None
+    if LIVE_PRODUCER:
+        live_s = time_launches(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx), steps, warmup)
+        c = ag_gemm_intra_node(a_d, b_d, False, ctx)
+        ctx.check_status()
+        err = golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32(shards, b))
+        assert err <= 1e-2
     # kernel alone, every flag already released
     full = torch.cat(shards).to(dev)
     flags = torch.ones(world, dtype=torch.int32, device=dev)
     out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 1024, rank, world), steps, warmup)
     r = roof("mfma", flops, pre_s, "bf16")
-    r["with_live_producer_us"] = round(live_s * 1e6, 2)
+    r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
     return r
 
 
@@ -162,20 +165,22 @@ def bench_c3(dev, steps, warmup):
     ctx.set_peer_shards({r: s.to(dev) for r, s in enumerate(shards) if r != rank})
     a_d, b_d = shards[rank].to(dev), b.to(dev)
     flops = 2.0 * world * mpr * N * K
-    live_s = time_launches(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb), steps, warmup)
-    c = ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb)
-    ctx.check_status()
-    rows = slice(5 * mpr + 11, 5 * mpr + 75)
-    ref = golden.fp8_scaled_gemm_fp32(shards[5][11:75], sa.cpu()[rows], b, sb.cpu())
-    err = golden.max_rel_err(c[rows].float().cpu(), ref)
-    assert err <= 1e-2
+    live_s = None
+    if LIVE_PRODUCER:
+        live_s = time_launches(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb), steps, warmup)
+        c = ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb)
+        ctx.check_status()
+        rows = slice(5 * mpr + 11, 5 * mpr + 75)
+        ref = golden.fp8_scaled_gemm_fp32(shards[5][11:75], sa.cpu()[rows], b, sb.cpu())
+        err = golden.max_rel_err(c[rows].float().cpu(), ref)
+        assert err <= 1e-2
     full = torch.cat([s.view(torch.uint8) for s in shards]).to(dev).view(torch.float8_e4m3fn)
     flags = torch.ones(world, dtype=torch.int32, device=dev)
     out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 2048, rank, world, row_scale=sa, col_scale=sb),
                           steps, warmup)
     r = roof("mfma", flops, pre_s, "fp8")
-    r["with_live_producer_us"] = round(live_s * 1e6, 2)
+    r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
     return r
 
 
@@ -248,7 +253,12 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,copy (c2 always runs)")
+    ap.add_argument("--no-live-producer", action="store_true",
+                    help="skip the AG-GEMM legs in which a copy stream releases the flags while the GEMM spins: a "
+                    "counter-collecting profiler serialises dispatches, so the producer could never run beside it")
     args = ap.parse_args()
+    global LIVE_PRODUCER
+    LIVE_PRODUCER = not args.no_live_producer
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported (every GPU box "
             "here has one GPU and the path has no cross-GPU step in it)" % args.gpus)
