@@ -24,6 +24,14 @@ for p in (ROOT, os.path.join(ROOT, "triton-distributed_amd")):
         sys.path.insert(0, p)
 
 PEAK = {"bf16": 2.5e15, "fp8": 5.0e15, "hbm": 8.0e12}  # MI355X published dense MFMA peaks (FLOP/s) and HBM3E B/s
+# HBM-side bytes per launch, read off two rocprofv3 counter passes over this same script (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch, each scaled by what the counter reads for the 1 GiB copy kernel: x2.000 and
+# x1.000). Counters cannot be collected inside a timed run, so the figures are carried here as constants;
+# the summaries are kept under profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "c2_gemm": 839.0e6, "c2_reduce": 151.0e6, "c1_gemm": 163.7e6, "c3_gemm": 1672.1e6, "c4_dispatch": 265.8e6,
+    "c4_combine": 313.9e6, "c5_split_kv": 4315.6e6,
+}
 LIVE_PRODUCER = True  # --no-live-producer clears it
 METRIC = "AG-GEMM/GEMM-RS TFLOPS (% MFMA peak); decode & A2A GB/s (% HBM peak)"
 
@@ -118,7 +126,8 @@ def bench_c2(dev, steps, warmup):
     else:
         cpu = {"value": round(flops / 8 / probe / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                "sample": "1/8 of the rows (1024 of 8192) of the fp32 up-cast golden GEMM, %.2f s" % probe}
-    return step_s, roof("mfma", flops, gemm_s, "bf16"), roof("hbm", red_bytes, red_s, "hbm"), cpu, err
+    return (step_s, roof("mfma", flops, gemm_s, "bf16", MEASURED_TRAFFIC_BYTES["c2_gemm"]),
+            roof("hbm", red_bytes, red_s, "hbm", MEASURED_TRAFFIC_BYTES["c2_reduce"]), cpu, err)
 
 
 def bench_c1(dev, steps, warmup):
@@ -145,7 +154,7 @@ def bench_c1(dev, steps, warmup):
     flags = torch.ones(world, dtype=torch.int32, device=dev)
     out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 1024, rank, world), steps, warmup)
-    r = roof("mfma", flops, pre_s, "bf16")
+    r = roof("mfma", flops, pre_s, "bf16", MEASURED_TRAFFIC_BYTES["c1_gemm"])
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
     return r
 
@@ -179,7 +188,7 @@ def bench_c3(dev, steps, warmup):
     out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 2048, rank, world, row_scale=sa, col_scale=sb),
                           steps, warmup)
-    r = roof("mfma", flops, pre_s, "fp8")
+    r = roof("mfma", flops, pre_s, "fp8", MEASURED_TRAFFIC_BYTES["c3_gemm"])
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
     return r
 
@@ -204,9 +213,9 @@ def bench_c4(dev, steps, warmup):
     n = T * topk
     disp_bytes = T * H + n * H + T * 4 + n * 4 + n * 4          # unique row reads + row writes + scales + gather index
     comb_bytes = n * H + n * 4 + n * 4 + n * 4 + T * H * 2      # row reads + scales + weights + scatter index + bf16 out
-    d = roof("hbm", disp_bytes, disp_s, "hbm")
+    d = roof("hbm", disp_bytes, disp_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_dispatch"])
     d["index_build_us"] = round(pre_s * 1e6, 2)
-    return d, roof("hbm", comb_bytes, comb_s, "hbm")
+    return d, roof("hbm", comb_bytes, comb_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_combine"])
 
 
 def bench_c5(dev, steps, warmup):
@@ -232,7 +241,7 @@ def bench_c5(dev, steps, warmup):
                                (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), merged), steps, warmup)
     kv_bytes = 2 * B * L * Hkv * D * 2
     split_bytes = kv_bytes + q.numel() * 2 + table.numel() * 4 + out_split.numel() * 4 + lse_split.numel() * 4
-    r = roof("hbm", split_bytes, split_s, "hbm")
+    r = roof("hbm", split_bytes, split_s, "hbm", MEASURED_TRAFFIC_BYTES["c5_split_kv"])
     r["combine_us"] = round(comb_s * 1e6, 2)
     return r
 
