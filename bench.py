@@ -10,7 +10,10 @@ algorithmic GEMM work (2*M*N*K) over the whole step time. The same line carries
                 with HIP events on the launch stream,
   cpu_baseline  the oracle's torch golden for the same step timed on the host cores,
   kernels       every other hot-path kernel at its BASELINE config with its own roofline fraction.
-Inputs are synthetic, seeded, and resident in HBM before any timed region.
+Inputs are synthetic, seeded, and resident in HBM before any timed region. Every timed region is preceded by
+``--settle-seconds`` (1.5 s) of the same launches, untimed, and then by the ``--warmup`` launches: after an idle
+gap the GPU spends its first ~0.7 s of work at a lower core clock than the one it then sustains, and it is the
+sustained rate that is reported.
 """
 import argparse
 import json
@@ -40,10 +43,26 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+SETTLE_SECONDS = 1.5  # --settle-seconds
+
+
+def settle(fn, seconds=None):
+    """Keeps the GPU busy with ``fn`` for ``seconds`` so that the timed region starts at the sustained clock: after
+    an idle gap this GPU runs its first ~0.7 s of work at a lower core clock than it then holds for good."""
+    import torch
+    seconds = SETTLE_SECONDS if seconds is None else seconds
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+
+
 def time_launches(fn, steps, warmup):
     """Average duration in seconds of ``fn`` (which launches on torch's current stream), HIP events on that
-    stream around ``steps`` back-to-back calls."""
+    stream around ``steps`` back-to-back calls, after the settle period and ``warmup`` untimed calls."""
     import torch
+    settle(fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -89,7 +108,8 @@ def bench_c2(dev, steps, warmup):
     a_d, b_d = a.to(dev), b.to(dev)
     flops = 2.0 * M * N * K
 
-    # whole step: barrier + sync on both sides of exactly `steps` steps
+    # whole step: settle, `warmup` untimed steps, then sync on both sides of exactly `steps` steps
+    settle(lambda: gemm_rs_intra_node(a_d, b_d, ctx))
     for _ in range(warmup):
         out = gemm_rs_intra_node(a_d, b_d, ctx)
     torch.cuda.synchronize()
@@ -257,17 +277,20 @@ def bench_copy(dev, steps, warmup):
 
 
 def main():
+    global LIVE_PRODUCER, SETTLE_SECONDS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--settle-seconds", type=float, default=SETTLE_SECONDS,
+                    help="untimed period of the same launches before each warm-up, to reach the sustained clock")
     ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,copy (c2 always runs)")
     ap.add_argument("--no-live-producer", action="store_true",
                     help="skip the AG-GEMM legs in which a copy stream releases the flags while the GEMM spins: a "
                     "counter-collecting profiler serialises dispatches, so the producer could never run beside it")
     args = ap.parse_args()
-    global LIVE_PRODUCER
     LIVE_PRODUCER = not args.no_live_producer
+    SETTLE_SECONDS = args.settle_seconds
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported (every GPU box "
             "here has one GPU and the path has no cross-GPU step in it)" % args.gpus)

@@ -122,7 +122,14 @@ struct GemmCfg {
   static constexpr int kFragVecs = E::kLaneBytes / 16;  // 16-byte pieces per operand fragment (1 or 2)
   static constexpr int kWaveM = BM / WM, kWaveN = BN / WN;
   static constexpr int kTM = kWaveM / 32, kTN = kWaveN / 32;
-  static constexpr int kLdsBytes = NST * kStageBytes;
+  // NST == 5 selects the split ring: three stages of A rows and two of B rows (five half stages, exactly the
+  // 160 KB of LDS at 256x256x128). A freed B stage is refilled at once; the A refill then has a whole K tile of
+  // time, so the DMA issue can be spread evenly over the K steps instead of bunching up behind the barrier.
+  static constexpr bool kSplit = NST == 5;
+  static constexpr int kAStages = kSplit ? 3 : NST, kBStages = kSplit ? 2 : NST;
+  static constexpr int kLdsBytes = kSplit ? kAStages * kABytes + kBStages * kBBytes : NST * kStageBytes;
+  // split ring: DMA instructions issued per K step (list of one K tile: the B rows, then the A rows)
+  static constexpr int kDmaPerStep = (kLoadsPerTile + kKSteps - 1) / kKSteps;
   // epilogue staging: per wave kWaveM rows of kWaveN 16-bit outputs; 16-byte chunk c of row r sits at
   // position c ^ (r & kEpiSwz) so that the 32 rows one store instruction touches spread over the banks
   static constexpr int kEpiPitch = kWaveN * 2;
@@ -130,9 +137,28 @@ struct GemmCfg {
   static constexpr int kEpiSwz = (kEpiPitch / 16 < 16 ? kEpiPitch / 16 : 16) - 1;
   // MFMAs of a tile's last K step issued before the barrier
   static constexpr int kLeadMfma = (kTM * kTN >= 8) ? 2 : 1;
+  // n-th operand fragment (A fragments are 0..kTM-1, B fragments kTM..) in the order in which the MFMA sequence
+  // (idx -> B fragment idx / kTM, A fragment idx % kTM) first needs them
+  static constexpr int frag_order(int n) {
+    int c = 0;
+    for (int u = 0; u < kTM * kTN; ++u) {
+      if (u % kTM == 0) {
+        if (c == n) return kTM + u / kTM;
+        ++c;
+      }
+      if (u < kTM) {
+        if (c == n) return u;
+        ++c;
+      }
+    }
+    return -1;
+  }
   static_assert(KB == 64 || KB == 128, "tile rows of 64 or 128 bytes");
   static_assert(BM % (kRowsPerInstr * kWaves) == 0 && BN % (kRowsPerInstr * kWaves) == 0, "tile/wave split");
-  static_assert(kP >= 1 && kP <= 3 && kP * kLoadsPerTile < 64, "vmcnt budget");
+  static_assert(kSplit || (kP >= 1 && kP <= 3 && kP * kLoadsPerTile < 64), "vmcnt budget");
+  static_assert(!kSplit || (kTM + kTN <= kTM * kTN - kLeadMfma && kLoadsPerTile % kKSteps == 0 &&
+                            kBInstr % kDmaPerStep == 0),
+                "split ring: one fragment read per MFMA slot, whole DMA groups per K step");
   static_assert(kEpiBytes * kWaves <= kLdsBytes, "epilogue staging must fit in the stage ring");
   static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "wave tile");
 };
@@ -145,8 +171,12 @@ __device__ __forceinline__ void wait_tiles_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
 
+#ifndef TDIST_DMA_AUX
+#define TDIST_DMA_AUX 0  // cache-policy bits of the LDS-DMA loads
+#endif
+
 // Instruction classes for __builtin_amdgcn_sched_group_barrier
-constexpr int kSchedMfma = 0x008, kSchedVmem = 0x010, kSchedDsRead = 0x100;  // the LDS-DMA load is VMEM that also stores
+constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
 
 // schedule position → chunk id
 __device__ __forceinline__ int chunk_of(const GemmParams& p, int oc) {
@@ -171,7 +201,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   typedef TDIST_AS3 unsigned char* lds_u8;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_generic[];
   lds_u8 const smem = (lds_u8)smem_generic;
-  __shared__ int s_gate;  // 1 = tile may proceed, 0 = wait expired
+  // gate result (1 = tile may proceed, 0 = wait expired) lives in the first word of the ring, which is idle
+  // between tiles
+  TDIST_AS3 int* const s_gate = (TDIST_AS3 int*)smem;
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -222,10 +254,10 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         if (!ok && p.status != nullptr) {
           if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = chunk;
         }
-        s_gate = ok;
+        *s_gate = ok;
       }
       __syncthreads();
-      const int ok = s_gate;
+      const int ok = *s_gate;
       __syncthreads();
       if (!ok) continue;
     }
@@ -254,17 +286,26 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // B rows). Past the last tile the last one is fetched again (into a stage nobody reads any more): every trip
     // of the main loop then issues the same number of loads, which keeps the loop free of branches and the vmcnt
     // bookkeeping constant.
-    auto issue_dma = [&](int kt, int t) {
-      lds_u8 const sa = smem + (kt % NST) * C::kStageBytes;
+    auto a_stage = [&](int kt) -> lds_u8 {
+      return C::kSplit ? smem + (kt % C::kAStages) * C::kABytes : smem + (kt % NST) * C::kStageBytes;
+    };
+    auto b_stage = [&](int kt) -> lds_u8 {
+      return C::kSplit ? smem + C::kAStages * C::kABytes + (kt % C::kBStages) * C::kBBytes
+                       : smem + (kt % NST) * C::kStageBytes + C::kABytes;
+    };
+    auto issue_a = [&](int kt, int t) {
       const int64_t kb = (int64_t)min(kt, KT - 1) * KB;
-      if (t < C::kAInstr) {
-        __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(Arows + a_off[t] + kb),
-                                         (TDIST_AS3 void*)(sa + (wave * C::kAInstr + t) * 1024), 16, 0, 0);
-      } else {
-        const int u = t - C::kAInstr;
-        __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(p.B + b_off[u] + kb),
-                                         (TDIST_AS3 void*)(sa + C::kABytes + (wave * C::kBInstr + u) * 1024), 16, 0, 0);
-      }
+      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(Arows + a_off[t] + kb),
+                                       (TDIST_AS3 void*)(a_stage(kt) + (wave * C::kAInstr + t) * 1024), 16, 0, TDIST_DMA_AUX);
+    };
+    auto issue_b = [&](int kt, int u) {
+      const int64_t kb = (int64_t)min(kt, KT - 1) * KB;
+      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(p.B + b_off[u] + kb),
+                                       (TDIST_AS3 void*)(b_stage(kt) + (wave * C::kBInstr + u) * 1024), 16, 0, TDIST_DMA_AUX);
+    };
+    auto issue_dma = [&](int kt, int t) {
+      if (t < C::kAInstr) issue_a(kt, t);
+      else issue_b(kt, t - C::kAInstr);
     };
     auto issue_tile = [&](int kt) {
 #pragma unroll
@@ -275,17 +316,16 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     typename E::frag a_cur[C::kTM], b_cur[C::kTN], a_nxt[C::kTM], b_nxt[C::kTN];
     // f-th operand fragment (A fragments first) of K step ks of tile kt
     auto load_frag = [&](int kt, int ks, int f, typename E::frag* af, typename E::frag* bf) {
-      lds_u8 const sa = smem + (kt % NST) * C::kStageBytes;
       const int c0 = (ks * 2 + lh) * C::kFragVecs;  // first 16-byte chunk of this lane's K bytes
       const int c1 = c0 + C::kFragVecs - 1;         // last one (== c0 for 16-byte fragments)
       if (f < C::kTM) {
         const int r = wm * C::kWaveM + f * 32 + l32;
-        lds_u8 const row = sa + r * KB;
+        lds_u8 const row = a_stage(kt) + r * KB;
         af[f] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
       } else {
         const int j = f - C::kTM;
         const int r = wn * C::kWaveN + j * 32 + l32;
-        lds_u8 const row = sa + C::kABytes + r * KB;
+        lds_u8 const row = b_stage(kt) + r * KB;
         bf[j] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
       }
     };
@@ -302,6 +342,74 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][i][e] = 0.f;
 
+    constexpr int kMfmaPerStep = C::kTM * C::kTN;
+    if constexpr (C::kSplit) {
+      // ---- split ring ------------------------------------------------------------------------------
+      // The DMA list of one cycle is [B(kt+2) rows..., A(kt+3) rows...]; it starts right after the barrier in the
+      // last K step of tile kt (B stage kt%2 and A stage kt%3 have just been released) and runs, kDmaPerStep
+      // instructions per K step, through the K steps of tile kt+1. At the barrier of tile kt+1 only the A rows
+      // of that list may still be in flight.
+      constexpr int kFrags = C::kTM + C::kTN;
+      // q-th instruction of the list whose cycle started in tile `cyc`
+      auto issue_list = [&](int cyc, int q) {
+        if (q < C::kBInstr) issue_b(cyc + 2, q);
+        else issue_a(cyc + 3, q - C::kBInstr);
+      };
+#pragma unroll
+      for (int t = 0; t < C::kAInstr; ++t) issue_a(0, t);
+#pragma unroll
+      for (int u = 0; u < C::kBInstr; ++u) issue_b(0, u);
+#pragma unroll
+      for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+#pragma unroll
+      for (int q = 0; q < C::kDmaPerStep; ++q) issue_list(-1, q);
+      wait_tiles_and_barrier<C::kAInstr + C::kDmaPerStep>();
+      load_frags(0, 0, a_cur, b_cur);
+      __builtin_amdgcn_sched_barrier(0);
+      for (int kt = 0; kt < KT; ++kt) {
+        const int kt_next = min(kt + 1, KT - 1);
+#pragma unroll
+        for (int ks = 0; ks < C::kKSteps; ++ks) {
+          constexpr int kLast = C::kKSteps - 1;
+          const bool last = ks == kLast;
+          const int first = last ? C::kLeadMfma : 0;
+          const int nslots = kMfmaPerStep - first;
+          const int pos = (ks + 1) % C::kKSteps;  // K steps since the list's cycle began
+          if (last) {
+#pragma unroll
+            for (int idx = 0; idx < C::kLeadMfma; ++idx) {
+              const int j = idx / C::kTM, i = idx % C::kTM;
+              acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            wait_tiles_and_barrier<C::kAInstr>();
+            __builtin_amdgcn_sched_barrier(0);
+          }
+#pragma unroll
+          for (int idx = first; idx < kMfmaPerStep; ++idx) {
+            const int j = idx / C::kTM, i = idx % C::kTM;
+            acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+            const int slot = idx - first;
+            // next K step's fragments in the order of their first use; the shorter last step reads two at once
+            if (last) {
+              if (slot == 0) load_frag(kt_next, 0, C::frag_order(0), a_nxt, b_nxt);
+              if (slot + 1 < kFrags) load_frag(kt_next, 0, C::frag_order(slot + 1), a_nxt, b_nxt);
+            } else if (slot < kFrags) {
+              load_frag(kt, ks + 1, C::frag_order(slot), a_nxt, b_nxt);
+            }
+#pragma unroll
+            for (int d = 0; d < C::kDmaPerStep; ++d)
+              if (slot == (d * nslots) / C::kDmaPerStep)
+                issue_list(last ? kt : kt - 1, pos * C::kDmaPerStep + d);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+#pragma unroll
+          for (int i = 0; i < C::kTM; ++i) a_cur[i] = a_nxt[i];
+#pragma unroll
+          for (int j = 0; j < C::kTN; ++j) b_cur[j] = b_nxt[j];
+        }
+      }
+    } else {
     // ---- prologue: P tiles in flight, wait for tile 0 ------------------------------------------
 #pragma unroll
     for (int t = 0; t < C::kP; ++t) issue_tile(t);
@@ -314,7 +422,6 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // LDS read slotted behind each of the first MFMAs so that neither pipe waits for the other. The last
     // step of a tile first joins the barrier (tile kt+1 has landed everywhere, tile kt is no longer read),
     // then also refills the freed stage.
-    constexpr int kMfmaPerStep = C::kTM * C::kTN;
     constexpr int kReadsPerStep = (C::kTM + C::kTN) * C::kFragVecs;
     for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
@@ -370,6 +477,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 #pragma unroll
         for (int j = 0; j < C::kTN; ++j) b_cur[j] = b_nxt[j];
       }
+    }
+
     }
 
     // ---- epilogue ---------------------------------------------------------------------------------
@@ -508,8 +617,8 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) big = false;
   if (c.A_local && (c.local_row_begin % 256 != 0 || c.local_rows % 256 != 0)) big = false;
   // TDIST_GEMM_VARIANT picks another compiled tiling for the large-tile path (measurement aid); the default,
-  // 2, is 256x256 tiles, 128-byte K rows, 2x4 waves, two stages.
-  int variant = 2;
+  // 6, is 256x256 tiles, 128-byte K rows, 2x2 waves of 128x128, split ring (3 A stages + 2 B stages).
+  int variant = 6;
   if (const char* v = getenv("TDIST_GEMM_VARIANT")) variant = atoi(v);
   const int BM = big ? 256 : 128;
   const int BN = big ? (variant == 4 ? 128 : 256) : 128;
@@ -599,7 +708,9 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       case 1: TDIST_BIG(256, 128, 2, 2, 2)
       case 3: TDIST_BIG(256, 64, 2, 4, 4)
       case 4: TDIST_BIG(128, 128, 2, 2, 3)
-      default: TDIST_BIG(256, 128, 2, 4, 2)
+      case 2: TDIST_BIG(256, 128, 2, 4, 2)
+      case 5: TDIST_BIG(256, 128, 2, 4, 5)
+      default: TDIST_BIG(256, 128, 2, 2, 5)
     }
 #undef TDIST_BIG
   }
