@@ -22,6 +22,12 @@
 
 #include "common.h"
 
+// Cache policy of the K/V stream: non-temporal (every byte is used once; the hint lets it pass through the
+// caches without displacing anything and measurably raises the HBM streaming rate).
+#ifndef TDIST_KV_AUX
+#define TDIST_KV_AUX 2
+#endif
+
 namespace tdist {
 
 struct DecodeParams {
@@ -245,8 +251,8 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
                                   (in_page * (uint32_t)prm.k_st + (uint32_t)kvh * (uint32_t)prm.k_sh + ((chunk ^ C::kswz(key)) << 4));
       const unsigned char* vsrc = prm.v + (uint64_t)page * (uint64_t)prm.v_sp +
                                   (in_page * (uint32_t)prm.v_st + (uint32_t)kvh * (uint32_t)prm.v_sh + ((chunk ^ C::vswz(key)) << 4));
-      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)ksrc, (TDIST_AS3 void*)(kst + i * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)vsrc, (TDIST_AS3 void*)(vst + i * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)ksrc, (TDIST_AS3 void*)(kst + i * 1024), 16, 0, TDIST_KV_AUX);
+      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)vsrc, (TDIST_AS3 void*)(vst + i * 1024), 16, 0, TDIST_KV_AUX);
     }
   };
 
@@ -547,17 +553,20 @@ int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cach
     case 64:
       return bf ? launch_decode<MmaBF16, 64, 32, 4, 4>(prm, head_blocks, st) : launch_decode<MmaF16, 64, 32, 4, 4>(prm, head_blocks, st);
     case 128: {
-      // TDIST_DECODE_VARIANT picks another compiled shape (measurement aid). Default: 16-key blocks, 4 waves,
-      // 2 stages = 66 KB of LDS, so two workgroups share a CU; measured within 2 % of the best of the others.
+      // TDIST_DECODE_VARIANT picks another compiled shape (measurement aid). Default: 16-key blocks, 3 waves,
+      // 3 stages = 72 KB of LDS, so two workgroups share a CU and two thirds of the ring are in flight.
       int variant = 0;
       if (const char* v = getenv("TDIST_DECODE_VARIANT")) variant = atoi(v);
-      if (variant == 1)
-        return bf ? launch_decode<MmaBF16, 128, 32, 4, 2>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 32, 4, 2>(prm, head_blocks, st);
-      if (variant == 2)
-        return bf ? launch_decode<MmaBF16, 128, 32, 3, 3>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 32, 3, 3>(prm, head_blocks, st);
-      if (variant == 3)
-        return bf ? launch_decode<MmaBF16, 128, 16, 8, 2>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 16, 8, 2>(prm, head_blocks, st);
-      return bf ? launch_decode<MmaBF16, 128, 16, 4, 2>(prm, head_blocks, st) : launch_decode<MmaF16, 128, 16, 4, 2>(prm, head_blocks, st);
+#define TDIST_DEC(KEYS_, NW_, NST_) \
+  return bf ? launch_decode<MmaBF16, 128, KEYS_, NW_, NST_>(prm, head_blocks, st) : launch_decode<MmaF16, 128, KEYS_, NW_, NST_>(prm, head_blocks, st);
+      switch (variant) {
+        case 1: TDIST_DEC(32, 4, 2)
+        case 2: TDIST_DEC(32, 3, 3)
+        case 3: TDIST_DEC(16, 8, 2)
+        case 4: TDIST_DEC(16, 4, 2)
+        default: TDIST_DEC(16, 3, 3)
+      }
+#undef TDIST_DEC
     }
     default:
       return bf ? launch_decode<MmaBF16, 256, 16, 2, 3>(prm, head_blocks, st) : launch_decode<MmaF16, 256, 16, 2, 3>(prm, head_blocks, st);

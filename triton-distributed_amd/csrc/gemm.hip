@@ -485,30 +485,41 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // acc[j][i][e]: output row m = wm*kWaveM + 32i + l32, column n = wn*kWaveN + 32j + 8*(e/4) + 4*lh + e%4
     wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
     lds_u8 const epi = smem + wave * C::kEpiBytes;
+    float rs[C::kTM];
 #pragma unroll
     for (int i = 0; i < C::kTM; ++i) {
-      const int mrow = 32 * i + l32;
-      float rs = 1.f;
-      if (kScales && p.row_scale) rs = p.row_scale[min(m0 + wm * C::kWaveM + mrow, p.M - 1)];
+      rs[i] = 1.f;
+      if (kScales && p.row_scale) rs[i] = p.row_scale[min(m0 + wm * C::kWaveM + 32 * i + l32, p.M - 1)];
+    }
 #pragma unroll
-      for (int j = 0; j < C::kTN; ++j) {
+    for (int j = 0; j < C::kTN; ++j) {
+      // the four column scales of each of this lane's four column groups in this 32-column block
+      float4v cs[4];
+      if (kScales) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          cs[q] = float4v{1.f, 1.f, 1.f, 1.f};
+          if (p.col_scale) {
+            const int gn = n0 + wn * C::kWaveN + 32 * j + 8 * q + 4 * lh;
+            if (gn + 3 < p.N) cs[q] = *(const float4v*)(p.col_scale + gn);
+            else
+              for (int e = 0; e < 4; ++e) cs[q][e] = p.col_scale[min(gn + e, p.N - 1)];
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < C::kTM; ++i) {
+        const int mrow = 32 * i + l32;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int ncol = 32 * j + 8 * q + 4 * lh;
           float v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2],
                 v3 = acc[j][i][4 * q + 3];
           if (kScales) {
-            float4v cs = {1.f, 1.f, 1.f, 1.f};
-            if (p.col_scale) {
-              const int gn = n0 + wn * C::kWaveN + ncol;
-              if (gn + 3 < p.N) cs = *(const float4v*)(p.col_scale + gn);
-              else
-                for (int e = 0; e < 4; ++e) cs[e] = p.col_scale[min(gn + e, p.N - 1)];
-            }
-            v0 *= rs * cs[0];
-            v1 *= rs * cs[1];
-            v2 *= rs * cs[2];
-            v3 *= rs * cs[3];
+            v0 *= rs[i] * cs[q][0];
+            v1 *= rs[i] * cs[q][1];
+            v2 *= rs[i] * cs[q][2];
+            v3 *= rs[i] * cs[q][3];
           }
           const int2v w = {(int)E::pack(v0, v1), (int)E::pack(v2, v3)};
           *(TDIST_AS3 int2v*)(epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2) = w;
