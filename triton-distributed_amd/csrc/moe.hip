@@ -293,41 +293,55 @@ __global__ __launch_bounds__(256) void moe_dispatch_tokens_kernel(const unsigned
                                                                   unsigned char* __restrict__ slot_rows,
                                                                   float* __restrict__ slot_scales,
                                                                   int32_t* __restrict__ splits_out, int windows) {
-  extern __shared__ int32_t s_bound[];  // [W+1]
-  for (int d = threadIdx.x; d <= W; d += 256) s_bound[d] = cumsum[d * Er];
   if (splits_out && blockIdx.x == 0) {
     const int G = W * Er;
     for (int g = threadIdx.x; g < G; g += 256) splits_out[g] = cumsum[g + 1] - cumsum[g];
   }
-  __syncthreads();
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
   const int64_t t = unit / windows;
   const int win = (int)(unit - t * windows);
   if (t >= n_tokens) return;
-  // lane k < topk resolves the slot row of copy k
-  int32_t my_dst = -1;
-  if (lane < topk) {
-    const int32_t p = scatter_idx[t * topk + lane];
-    if (p >= 0 && p < s_bound[W]) {
-      const int d = find_dest(s_bound, 1, W, p);
-      const int32_t in_slot = p - s_bound[d];
-      if (in_slot < max_m) my_dst = d * max_m + in_slot;
-    }
-    if (win == 0 && my_dst >= 0 && scales) slot_scales[my_dst] = scales[t];
-  }
   const unsigned char* src = tokens + t * row_bytes;
+  // the row's loads go out first: they do not depend on where the copies land
+  const int n16 = (int)(row_bytes >> 4);
+  const int base = win * 512;
+  int4v v[8];
   if (kVec16) {
-    const int n16 = (int)(row_bytes >> 4);
-    const int base = win * 512;
     const int4v* s16 = (const int4v*)src;
-    int4v v[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int c = base + j * 64 + lane;
       if (c < n16) v[j] = s16[c];
     }
+  }
+  // lane k < topk resolves the slot row of copy k; the W+1 slot boundaries sit one per lane, so the search is
+  // register work behind a single load
+  int32_t my_dst = -1;
+  {
+    const int32_t p = lane < topk ? scatter_idx[t * topk + lane] : -1;
+    if (W < 64) {
+      const int32_t bound = lane <= W ? cumsum[lane * Er] : 0x7fffffff;
+      const int32_t total = __builtin_amdgcn_readlane(bound, W);
+      int d = 0;
+      int32_t first = __builtin_amdgcn_readlane(bound, 0);
+      for (int i = 1; i < W; ++i) {
+        const int32_t b = __builtin_amdgcn_readlane(bound, i);
+        if (b <= p) {
+          d = i;
+          first = b;
+        }
+      }
+      if (p >= 0 && p < total && p - first < max_m) my_dst = d * max_m + (p - first);
+    } else if (p >= 0 && p < cumsum[W * Er]) {
+      const int d = find_dest(cumsum, Er, W, p);
+      const int32_t in_slot = p - cumsum[d * Er];
+      if (in_slot < max_m) my_dst = d * max_m + in_slot;
+    }
+    if (win == 0 && my_dst >= 0 && scales) slot_scales[my_dst] = scales[t];
+  }
+  if (kVec16) {
     for (int k = 0; k < topk; ++k) {
       const int32_t dst_row = __shfl(my_dst, k);
       if (dst_row < 0) continue;
@@ -348,109 +362,121 @@ __global__ __launch_bounds__(256) void moe_dispatch_tokens_kernel(const unsigned
   }
 }
 
-// Weighted combine: one workgroup per token; thread c owns 16-byte column chunk(s) of the row.
+// Weighted combine: one wave per (token, window of 64 16-byte column chunks). Lane k < topk resolves the k-th
+// source row and its coefficient w[t,k] * scale[row]; the wave then reads the rows eight at a time (all loads
+// of a batch in flight before the first add) and accumulates in k order.
 // kFp8: rows are e4m3 bytes (16 elements per chunk), else bf16 (8 elements per chunk).
 constexpr int kCombineMaxTopk = 32;
+constexpr int kCombineWaves = 4;
 
 template <bool kFp8>
-__global__ __launch_bounds__(1024) void moe_combine_kernel(const unsigned char* __restrict__ slot_rows,
-                                                           const float* __restrict__ slot_scales,
-                                                           const int32_t* __restrict__ scatter_idx,
-                                                           const float* __restrict__ topk_w,
-                                                           const int32_t* __restrict__ cumsum, int topk, int hidden,
-                                                           int W, int Er, int max_m,
-                                                           unsigned short* __restrict__ out) {
-  __shared__ int64_t s_row[kCombineMaxTopk];  // source row index, -1 = skip
-  __shared__ float s_coef[kCombineMaxTopk];   // w[t,k] * scale[row]
-  const int64_t t = blockIdx.x;
-  if (threadIdx.x < topk) {
-    const int k = threadIdx.x;
-    const int32_t p = scatter_idx[t * topk + k];
-    int64_t row = -1;
-    if (p >= 0) {
-      if (max_m > 0) {
-        const int32_t total = cumsum[W * Er];
-        if (p < total) {
-          const int d = find_dest(cumsum, Er, W, p);
-          const int64_t in_slot = p - cumsum[d * Er];
-          if (in_slot < max_m) row = (int64_t)d * max_m + in_slot;
+__global__ __launch_bounds__(kCombineWaves * 64) void moe_combine_kernel(
+    const unsigned char* __restrict__ slot_rows, const float* __restrict__ slot_scales,
+    const int32_t* __restrict__ scatter_idx, const float* __restrict__ topk_w, const int32_t* __restrict__ cumsum,
+    int64_t n_tokens, int topk, int hidden, int W, int Er, int max_m, int n_windows, unsigned short* __restrict__ out) {
+  // e4m3 rows: a lane ends up with 32 bytes of output; they go through LDS so that each store instruction of the
+  // wave writes one contiguous KiB (16 bytes per lane) instead of every other 16 bytes of two
+  __shared__ __attribute__((aligned(16))) unsigned char s_tr[kCombineWaves][kFp8 ? 2048 : 16];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int64_t gw = (int64_t)blockIdx.x * kCombineWaves + wave;
+  if (gw >= n_tokens * n_windows) return;
+  const int64_t t = gw / n_windows;
+  const int win = (int)(gw - t * n_windows);
+
+  // Lane k resolves source row k. The W+1 slot boundaries sit one per lane (a single load, issued together with
+  // the index and weight loads), so the search for the destination is register work, not a chain of loads.
+  int64_t row = -1;  // source row of the lane's k, -1 = skip
+  const int32_t p = lane < topk ? scatter_idx[t * topk + lane] : -1;
+  float coef = (lane < topk && topk_w) ? topk_w[t * topk + lane] : 1.0f;
+  if (max_m > 0) {
+    if (W < 64) {
+      const int32_t bound = lane <= W ? cumsum[lane * Er] : 0x7fffffff;
+      const int32_t total = __builtin_amdgcn_readlane(bound, W);
+      int d = 0;
+      int32_t base = __builtin_amdgcn_readlane(bound, 0);
+      for (int i = 1; i < W; ++i) {
+        const int32_t b = __builtin_amdgcn_readlane(bound, i);
+        if (b <= p) {
+          d = i;
+          base = b;
         }
-      } else {
-        row = p;
       }
+      if (p >= 0 && p < total && p - base < max_m) row = (int64_t)d * max_m + (p - base);
+    } else if (p >= 0 && p < cumsum[W * Er]) {
+      const int d = find_dest(cumsum, Er, W, p);
+      const int64_t in_slot = p - cumsum[d * Er];
+      if (in_slot < max_m) row = (int64_t)d * max_m + in_slot;
     }
-    float coef = topk_w ? topk_w[t * topk + k] : 1.0f;
-    if (row >= 0 && slot_scales) coef *= slot_scales[row];
-    s_row[k] = row;
-    s_coef[k] = coef;
+  } else if (p >= 0) {
+    row = p;
   }
-  __syncthreads();
+  if (row >= 0 && slot_scales) coef *= slot_scales[row];
+  if (row < 0) coef = 0.f;
   constexpr int kElems = kFp8 ? 16 : 8;
   const int64_t row_bytes = (int64_t)hidden * (kFp8 ? 1 : 2);
   const int n16 = hidden / kElems;
-  for (int c = threadIdx.x; c < n16; c += blockDim.x) {
-    float acc[kElems];
+  const int c = win * 64 + lane;
+  const bool active = c < n16;
+  float acc[kElems];
 #pragma unroll
-    for (int j = 0; j < kElems; ++j) acc[j] = 0.f;
-    int k = 0;
-    // four rows in flight per step
-    for (; k + 4 <= topk; k += 4) {
-      int4v v[4];
+  for (int j = 0; j < kElems; ++j) acc[j] = 0.f;
+  const int row_lo = (int)(uint32_t)row, row_hi = (int)(row >> 32);
+  for (int k0 = 0; k0 < topk; k0 += 8) {
+    int4v v[8];
+    float cf[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int64_t row = s_row[k + j];
-        v[j] = (row >= 0) ? __builtin_nontemporal_load((const int4v*)(slot_rows + row * row_bytes) + c)
-                          : int4v{0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float coef = (s_row[k + j] >= 0) ? s_coef[k + j] : 0.f;
-        if (kFp8) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            float f[4];
-            e4m3x4_to_f32((uint32_t)v[j][q], f);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[4 * q + r] += coef * f[r];
-          }
-        } else {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            acc[2 * q] += coef * BF16::lo((uint32_t)v[j][q]);
-            acc[2 * q + 1] += coef * BF16::hi((uint32_t)v[j][q]);
-          }
-        }
-      }
+    for (int j = 0; j < 8; ++j) {
+      const int k = min(k0 + j, topk - 1);
+      const int64_t r = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readlane(row_hi, k) << 32) |
+                                  (uint32_t)__builtin_amdgcn_readlane(row_lo, k));
+      const bool use = (k0 + j < topk) && r >= 0;
+      v[j] = (use && active) ? __builtin_nontemporal_load((const int4v*)(slot_rows + r * row_bytes) + c)
+                             : int4v{0, 0, 0, 0};
     }
-    for (; k < topk; ++k) {
-      const int64_t row = s_row[k];
-      if (row < 0) continue;
-      const int4v v = __builtin_nontemporal_load((const int4v*)(slot_rows + row * row_bytes) + c);
-      const float coef = s_coef[k];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = min(k0 + j, topk - 1);
+      cf[j] = (k0 + j < topk) ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, coef), k)) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
       if (kFp8) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           float f[4];
-          e4m3x4_to_f32((uint32_t)v[q], f);
+          e4m3x4_to_f32((uint32_t)v[j][q], f);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) acc[4 * q + r] += coef * f[r];
+          for (int r = 0; r < 4; ++r) acc[4 * q + r] += cf[j] * f[r];
         }
       } else {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          acc[2 * q] += coef * BF16::lo((uint32_t)v[q]);
-          acc[2 * q + 1] += coef * BF16::hi((uint32_t)v[q]);
+          acc[2 * q] += cf[j] * BF16::lo((uint32_t)v[j][q]);
+          acc[2 * q + 1] += cf[j] * BF16::hi((uint32_t)v[j][q]);
         }
       }
     }
-    unsigned short* o = out + t * hidden + (int64_t)c * kElems;
+  }
+  int4v w[kElems / 8];
 #pragma unroll
-    for (int q = 0; q < kElems / 8; ++q) {
-      int4v w;
+  for (int q = 0; q < kElems / 8; ++q)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) w[j] = (int)pack_bf16x2(acc[8 * q + 2 * j], acc[8 * q + 2 * j + 1]);
-      __builtin_nontemporal_store(w, (int4v*)o + q);
+    for (int j = 0; j < 4; ++j) w[q][j] = (int)pack_bf16x2(acc[8 * q + 2 * j], acc[8 * q + 2 * j + 1]);
+  unsigned short* const orow = out + t * hidden + (int64_t)win * 64 * kElems;  // first output element of the window
+  if (kFp8) {
+    TDIST_AS3 unsigned char* tr = (TDIST_AS3 unsigned char*)s_tr[wave];
+    *(TDIST_AS3 int4v*)(tr + lane * 32) = w[0];
+    *(TDIST_AS3 int4v*)(tr + lane * 32 + 16) = w[kElems / 8 - 1];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int piece = h * 64 + lane;  // 16-byte piece of the window's 2 KiB of output
+      const int4v o = *(TDIST_AS3 int4v*)(tr + piece * 16);
+      if (win * 64 + piece / 2 < n16) __builtin_nontemporal_store(o, (int4v*)orow + piece);
     }
+  } else {
+    if (active) __builtin_nontemporal_store(w[0], (int4v*)orow + lane);
   }
 }
 
@@ -540,7 +566,7 @@ int tdist_moe_dispatch_tokens(const void* tokens, int64_t row_bytes, const float
   if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_dispatch_tokens: too many tokens");
   const bool vec = (row_bytes % 16 == 0) && aligned16(tokens) && aligned16(slot_rows);
   auto kern = vec ? moe_dispatch_tokens_kernel<true> : moe_dispatch_tokens_kernel<false>;
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), (size_t)(world_size + 1) * 4, (hipStream_t)stream,
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                      (const unsigned char*)tokens, row_bytes, token_scales, scatter_idx, topk, cumsum, n_tokens,
                      world_size, experts_per_rank, max_m, (unsigned char*)slot_rows, slot_scales, splits_out, windows);
   return launch_status("tdist_moe_dispatch_tokens");
@@ -580,13 +606,14 @@ int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_sc
     return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: hidden must be a multiple of %d and buffers 16-byte aligned", elems);
   if (n_tokens == 0) return TDIST_OK;
   if (n_tokens > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: too many tokens");
-  int threads = ((hidden / elems + 63) / 64) * 64;
-  if (threads > 1024) threads = 1024;
-  if (threads < 64) threads = 64;
+  const int n_windows = (hidden / elems + 63) / 64;
+  const int64_t waves = n_tokens * n_windows;
+  const int64_t blocks = ceil_div(waves, kCombineWaves);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: too many tokens");
   auto kern = row_dtype == TDIST_F8E4M3 ? moe_combine_kernel<true> : moe_combine_kernel<false>;
-  hipLaunchKernelGGL(kern, dim3((unsigned)n_tokens), dim3(threads), 0, (hipStream_t)stream,
-                     (const unsigned char*)slot_rows, slot_scales, scatter_idx, topk_w, cumsum, topk, hidden,
-                     world_size, experts_per_rank, max_m, (unsigned short*)out_bf16);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kCombineWaves * 64), 0, (hipStream_t)stream,
+                     (const unsigned char*)slot_rows, slot_scales, scatter_idx, topk_w, cumsum, n_tokens, topk, hidden,
+                     world_size, experts_per_rank, max_m, n_windows, (unsigned short*)out_bf16);
   return launch_status("tdist_moe_combine");
 }
 
