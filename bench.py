@@ -76,6 +76,25 @@ def time_launches(fn, steps, warmup):
     return start.elapsed_time(stop) * 1e-3 / steps
 
 
+def time_live_ag_gemm(call, ctx, steps, warmup):
+    """Times the AG-GEMM with its producer running: first with the GEMM queued before the chunk copies
+    (ctx.gemm_first), and if the copy streams turn out to share a hardware queue with the GEMM stream in this
+    process (the bounded flag wait reports a timeout), in the reference's order. Returns (seconds, order)."""
+    from triton_dist import _lib
+    ctx.gemm_first = True
+    call()
+    try:
+        ctx.check_status()
+        s = time_launches(call, steps, warmup)
+        ctx.check_status()
+        return s, "gemm_first"
+    except _lib.TdistError:
+        ctx.gemm_first = False
+        s = time_launches(call, steps, warmup)
+        ctx.check_status()
+        return s, "copies_first"
+
+
 def roof(bound, work, seconds, peak_key, traffic=None):
     achieved = work / seconds
     unit = "TFLOP/s" if bound == "mfma" else "GB/s"
@@ -162,9 +181,9 @@ def bench_c1(dev, steps, warmup):
     ctx.set_peer_shards({r: s.to(dev) for r, s in enumerate(shards) if r != rank})
     a_d, b_d = shards[rank].to(dev), b.to(dev)
     flops = 2.0 * world * mpr * N * K
-    live_s = None
+    live_s, live_order = None, None
     if LIVE_PRODUCER:
-        live_s = time_launches(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx), steps, warmup)
+        live_s, live_order = time_live_ag_gemm(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx), ctx, steps, warmup)
         c = ag_gemm_intra_node(a_d, b_d, False, ctx)
         ctx.check_status()
         err = golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32(shards, b))
@@ -176,6 +195,7 @@ def bench_c1(dev, steps, warmup):
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 1024, rank, world), steps, warmup)
     r = roof("mfma", flops, pre_s, "bf16", MEASURED_TRAFFIC_BYTES["c1_gemm"])
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
+    r["live_producer_order"] = live_order
     return r
 
 
@@ -194,9 +214,10 @@ def bench_c3(dev, steps, warmup):
     ctx.set_peer_shards({r: s.to(dev) for r, s in enumerate(shards) if r != rank})
     a_d, b_d = shards[rank].to(dev), b.to(dev)
     flops = 2.0 * world * mpr * N * K
-    live_s = None
+    live_s, live_order = None, None
     if LIVE_PRODUCER:
-        live_s = time_launches(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb), steps, warmup)
+        live_s, live_order = time_live_ag_gemm(lambda: ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb),
+                                               ctx, steps, warmup)
         c = ag_gemm_intra_node(a_d, b_d, False, ctx, row_scale=sa, col_scale=sb)
         ctx.check_status()
         rows = slice(5 * mpr + 11, 5 * mpr + 75)
@@ -210,6 +231,7 @@ def bench_c3(dev, steps, warmup):
                           steps, warmup)
     r = roof("mfma", flops, pre_s, "fp8", MEASURED_TRAFFIC_BYTES["c3_gemm"])
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
+    r["live_producer_order"] = live_order
     return r
 
 

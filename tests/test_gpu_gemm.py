@@ -99,6 +99,34 @@ def test_ag_gemm_config1(cuda):
             assert int(ctx.barrier_tensors[rank].abs().sum()) == 0
 
 
+def test_ag_gemm_gemm_first_and_sdma_options(cuda):
+    """The two producer options: the GEMM queued before the chunk copies, and copies on the copy engines. Queuing
+    the GEMM first needs the copy streams on hardware queues of their own; where this process has too many streams
+    for that, the bounded wait reports a timeout (never a hang) and the default order is checked instead."""
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import ag_gemm_intra_node
+    announce("ag_gemm gemm_first / use_sdma")
+    shards, b = make_ag_case(4, 512, 1024, 768, torch.bfloat16, seed=17)
+    ref = golden.ag_gemm_fp32(shards, b)
+    rank = 1
+    ctx = run_ag_gemm(cuda, shards, b, rank, 256, use_sdma=True)
+    c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx)
+    ctx.check_status()
+    assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
+    ctx = run_ag_gemm(cuda, shards, b, rank, 256, gemm_first=True, spin_limit=1 << 18)
+    c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx)
+    try:
+        ctx.check_status()
+    except _lib.TdistError as e:
+        assert e.code == _lib.TDIST_ERR_TIMEOUT
+        ctx.gemm_first = False
+        c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx)
+        ctx.check_status()
+        assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
+        pytest.skip("a copy stream shares a hardware queue with the GEMM stream in this process")
+    assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
 def test_ag_gemm_any_arrival_order(cuda, dtype):
     """Result independent of the order in which chunks arrive: all 3! orders of the peers of rank 1, two chunks each."""

@@ -88,7 +88,15 @@ class AllGatherGEMMTensorParallelContext:
     held_chunks: Tuple[int, ...] = ()
     spin_limit: int = 0          # 0 = library default (seconds of polling)
     status: Optional[torch.Tensor] = None  # int32[2]: error code, chunk that timed out
-    use_sdma: bool = True
+    # True: chunk copies go to the copy engines (hipMemcpyDeviceToDeviceNoCU), as the reference's cp-engine
+    # producer does across GPUs. On one GPU the engines move ~55 GB/s each, far below a kernel copy inside HBM, so
+    # the default is the blit path.
+    use_sdma: bool = False
+    # True: queue the gated GEMM before the chunk copies, so that it works on the caller's own rows while the host
+    # is still queueing copies. Only safe when the GEMM stream and the copy streams sit on different hardware
+    # queues (a process has 4 by default and streams beyond that share them): a copy queued behind the spinning
+    # GEMM on the same queue can never run, and the bounded wait then reports a timeout.
+    gemm_first: bool = False
     preset_flags: bool = False   # debug: release every flag before the GEMM starts (no overlap)
     # Compute units the gated GEMM leaves to the producer's copies. On one GPU those copies need compute
     # units of this GPU; measured on MI355X they make no progress next to a full-chip persistent grid
@@ -156,7 +164,9 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
 
     current_stream = torch.cuda.current_stream()
     # default priority on purpose (the reference asks for priority -1)
-    _ag_streams = [torch.cuda.Stream() for _ in range(num_ranks)] if ag_streams is None else ag_streams
+    # two copy streams by default (the reference makes one per rank): with the GEMM stream that stays within the 4
+    # hardware queues of a process, so no stream waits behind another one's packets
+    _ag_streams = [torch.cuda.Stream() for _ in range(min(num_ranks, 2))] if ag_streams is None else ag_streams
     _gemm_stream = current_stream if gemm_stream is None else gemm_stream
     one = torch.ones((1024, ), dtype=torch.int32, device=device)
     status = torch.zeros((2, ), dtype=torch.int32, device=device)
@@ -256,21 +266,31 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
                 held_chunks=ctx.held_chunks if ctx is not None else (),
                 use_sdma=ctx.use_sdma if ctx is not None else True)
 
-    call_ag()
+    def call_gemm(max_wgs):
+        with torch.cuda.stream(gemm_stream):
+            gated_gemm(workspace[:M], a, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
+                       row_scale=row_scale, col_scale=col_scale, wait_value=1,
+                       spin_limit=ctx.spin_limit if ctx is not None else 0,
+                       status=ctx.status if ctx is not None else None, max_workgroups=max_wgs, stream=gemm_stream)
+
     if serial or (ctx is not None and ctx.preset_flags):
+        # every chunk delivered before the GEMM starts
+        call_ag()
         for ag_stream in ag_streams:
             gemm_stream.wait_stream(ag_stream)
         if serial:
             torch.cuda.synchronize()
-
-    max_wgs = 0
-    if ctx is not None and num_ranks > 1 and ctx.producer_cus > 0 and not (serial or ctx.preset_flags):
-        max_wgs = max(1, _lib.load().tdist_num_cus() - ctx.producer_cus)
-    with torch.cuda.stream(gemm_stream):
-        gated_gemm(workspace[:M], a, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
-                   row_scale=row_scale, col_scale=col_scale, wait_value=1,
-                   spin_limit=ctx.spin_limit if ctx is not None else 0,
-                   status=ctx.status if ctx is not None else None, max_workgroups=max_wgs, stream=gemm_stream)
+        call_gemm(0)
+    else:
+        max_wgs = 0
+        if ctx is not None and num_ranks > 1 and ctx.producer_cus > 0:
+            max_wgs = max(1, _lib.load().tdist_num_cus() - ctx.producer_cus)
+        if ctx is not None and ctx.gemm_first:
+            call_gemm(max_wgs)
+            call_ag()
+        else:
+            call_ag()  # the reference's order (:300-304)
+            call_gemm(max_wgs)
     current_stream.wait_stream(gemm_stream)
     for ag_stream in ag_streams:
         current_stream.wait_stream(ag_stream)
