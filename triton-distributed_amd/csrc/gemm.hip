@@ -171,10 +171,6 @@ __device__ __forceinline__ void wait_tiles_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
 
-#ifndef TDIST_DMA_AUX
-#define TDIST_DMA_AUX 0  // cache-policy bits of the LDS-DMA loads
-#endif
-
 // Instruction classes for __builtin_amdgcn_sched_group_barrier
 constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
 
@@ -267,19 +263,24 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     const int a_row_off = is_local ? p.local_row_begin : 0;
     const int a_row_max = is_local ? p.local_rows - 1 : p.M - 1;
 
-    // per-lane byte offsets (relative to row 0 / column 0 of the matrix) of this lane's DMA sources
-    int64_t a_off[C::kAInstr], b_off[C::kBInstr];
+    // DMA sources: a wave-uniform base (first row of the tile, advanced along K in scalar registers) plus a
+    // 32-bit per-lane offset, so that the load takes its address as SGPR base + VGPR offset and the K loop
+    // carries no vector address arithmetic for it
+    const int a_g0 = min(m0 - a_row_off, a_row_max), b_g0 = min(n0, p.N - 1);
+    const unsigned char* const a_base = Arows + (int64_t)a_g0 * a_ld;
+    const unsigned char* const b_base = p.B + (int64_t)b_g0 * p.ldb_b;
+    uint32_t a_off[C::kAInstr], b_off[C::kBInstr];
 #pragma unroll
     for (int t = 0; t < C::kAInstr; ++t) {
       const int r = (wave * C::kAInstr + t) * C::kRowsPerInstr + dma_row;  // row within the tile
       const int gr = min(m0 + r - a_row_off, a_row_max);
-      a_off[t] = (int64_t)gr * a_ld + ((dma_pos ^ swz<KB>(r)) << 4);
+      a_off[t] = (uint32_t)(gr - a_g0) * (uint32_t)a_ld + (uint32_t)((dma_pos ^ swz<KB>(r)) << 4);
     }
 #pragma unroll
     for (int t = 0; t < C::kBInstr; ++t) {
       const int r = (wave * C::kBInstr + t) * C::kRowsPerInstr + dma_row;
       const int gr = min(n0 + r, p.N - 1);
-      b_off[t] = (int64_t)gr * p.ldb_b + ((dma_pos ^ swz<KB>(r)) << 4);
+      b_off[t] = (uint32_t)(gr - b_g0) * (uint32_t)p.ldb_b + (uint32_t)((dma_pos ^ swz<KB>(r)) << 4);
     }
 
     // DMA of K tile kt into stage kt % NST, one instruction at a time (kLoadsPerTile of them: A rows first, then
@@ -293,15 +294,20 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       return C::kSplit ? smem + C::kAStages * C::kABytes + (kt % C::kBStages) * C::kBBytes
                        : smem + (kt % NST) * C::kStageBytes + C::kABytes;
     };
+    // global_load_lds_dwordx4 in its SGPR-base + 32-bit-VGPR-offset form (the builtin only produces the 64-bit
+    // VGPR address form, which costs a 64-bit vector add per load, and with one wave per SIMD every vector ALU
+    // instruction in the K loop is time the MFMA pipe stands idle): M0 carries the wave-uniform LDS address.
+    auto dma16 = [&](const unsigned char* sbase, uint32_t voff, lds_u8 dst) {
+      const uint32_t lds_addr = (uint32_t)(uintptr_t)dst;
+      // (M0 is a reserved register the compiler never allocates and nothing else in this kernel uses)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
+                   : "memory");
+    };
     auto issue_a = [&](int kt, int t) {
-      const int64_t kb = (int64_t)min(kt, KT - 1) * KB;
-      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(Arows + a_off[t] + kb),
-                                       (TDIST_AS3 void*)(a_stage(kt) + (wave * C::kAInstr + t) * 1024), 16, 0, TDIST_DMA_AUX);
+      dma16(a_base + (int64_t)min(kt, KT - 1) * KB, a_off[t], a_stage(kt) + (wave * C::kAInstr + t) * 1024);
     };
     auto issue_b = [&](int kt, int u) {
-      const int64_t kb = (int64_t)min(kt, KT - 1) * KB;
-      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)(p.B + b_off[u] + kb),
-                                       (TDIST_AS3 void*)(b_stage(kt) + (wave * C::kBInstr + u) * 1024), 16, 0, TDIST_DMA_AUX);
+      dma16(b_base + (int64_t)min(kt, KT - 1) * KB, b_off[u], b_stage(kt) + (wave * C::kBInstr + u) * 1024);
     };
     auto issue_dma = [&](int kt, int t) {
       if (t < C::kAInstr) issue_a(kt, t);
@@ -513,8 +519,17 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int ncol = 32 * j + 8 * q + 4 * lh;
-          float v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2],
-                v3 = acc[j][i][4 * q + 3];
+          float v0, v1, v2, v3;
+          if constexpr (C::kTM * C::kTN * 16 >= 256) {
+            // 256 accumulators live in AGPRs; read each one here, where it is packed, instead of letting the
+            // compiler copy all of them to VGPRs at the loop exit (which spills)
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v0) : "a"(acc[j][i][4 * q + 0]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v1) : "a"(acc[j][i][4 * q + 1]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v2) : "a"(acc[j][i][4 * q + 2]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v3) : "a"(acc[j][i][4 * q + 3]));
+          } else {
+            v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2], v3 = acc[j][i][4 * q + 3];
+          }
           if (kScales) {
             v0 *= rs[i] * cs[q][0];
             v1 *= rs[i] * cs[q][1];
@@ -553,7 +568,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       if (gm < p.M && gn < p.N) {
         unsigned short* dst = (unsigned short*)Cbase + (crow0 + wm * C::kWaveM + mrow) * p.ldc + gn;
         if (gn + 8 <= p.N && n_vec_ok) {
-          *(int4v*)dst = v;
+          if (p.scatter_bufs == nullptr) __builtin_nontemporal_store(v, (int4v*)dst);  // written once, not read back here
+          else *(int4v*)dst = v;
         } else {
           for (int e = 0; e < 8; ++e)
             if (gn + e < p.N) dst[e] = (unsigned short)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
@@ -617,6 +633,8 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       (c.ldb * esz) % 16 || (c.A_local && (c.lda_local * esz) % 16))
     return fail(TDIST_ERR_UNSUPPORTED, "%s: A/B bases and row strides must be 16-byte aligned", who);
   if (c.lda < c.K || c.ldb < c.K || c.ldc < c.N) return fail(TDIST_ERR_INVALID, "%s: leading dimension smaller than row", who);
+  if (c.lda * esz > (1 << 22) || c.ldb * esz > (1 << 22) || (c.A_local && c.lda_local * esz > (1 << 22)))
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: row strides above 4 MiB are not supported", who);
   const DeviceInfo& di = device_info();
   if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "%s: current device is not gfx950", who);
 
