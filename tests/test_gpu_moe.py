@@ -74,7 +74,8 @@ def test_splits_cumsum_entry_point(cuda):
                                                      (96, 4, 16, 4, 48, 160, "tokens"), (50, 3, 6, 2, 24, 40, False),
                                                      (50, 3, 6, 2, 24, 40, "tokens"), (10, 2, 8, 8, 1024, 8, True),
                                                      (10, 2, 8, 8, 1024, 8, "tokens"), (33, 5, 8, 2, 12000, 128, "tokens"),
-                                                     (21, 3, 4, 4, 52, 64, "tokens")])
+                                                     (21, 3, 4, 4, 52, 64, "tokens"), (300, 4, 128, 64, 64, 48, "tokens"),
+                                                     (300, 4, 126, 63, 64, 48, "tokens"), (300, 4, 160, 80, 64, 48, "tokens")])
 def test_dispatch_bytes_bit_exact_and_round_trip(cuda, T, topk, G, W, H, max_m, fused):
     from triton_dist.kernels.amd import (all_to_all_post_process, create_all_to_all_context, fast_all_to_all,
                                          moe_dispatch_preprocess)
@@ -149,7 +150,9 @@ def test_context_double_buffering(cuda):
     assert float(r2[0, 0]) == 2.0 and float(r3[0, 0]) == 3.0 and float(r3[8, 0]) == 3.0
 
 
-@pytest.mark.parametrize("T,topk,G,W,H,max_m", [(4096, 8, 256, 32, 7168, 4096), (96, 4, 16, 4, 64, 160), (7, 3, 8, 2, 16, 32)])
+@pytest.mark.parametrize("T,topk,G,W,H,max_m", [(4096, 8, 256, 32, 7168, 4096), (96, 4, 16, 4, 64, 160), (7, 3, 8, 2, 16, 32),
+                                                (300, 4, 128, 64, 1040, 48), (300, 4, 126, 63, 1040, 48),
+                                                (300, 4, 160, 80, 1040, 48), (40, 12, 24, 3, 2064, 512)])
 def test_weighted_combine(cuda, T, topk, G, W, H, max_m):
     from triton_dist.kernels.amd import (create_all_to_all_context, fast_all_to_all, moe_dispatch_preprocess,
                                          moe_weighted_combine)
