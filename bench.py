@@ -257,6 +257,11 @@ def bench_c4(dev, steps, warmup):
     comb_bytes = n * H + n * 4 + n * 4 + n * 4 + T * H * 2      # row reads + scales + weights + scatter index + bf16 out
     d = roof("hbm", disp_bytes, disp_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_dispatch"])
     d["index_build_us"] = round(pre_s * 1e6, 2)
+    # the step after the dispatch: align / sort of the same ids for the grouped GEMM (8 rank segments, block 128)
+    from triton_dist.kernels.amd import sort_topk_ids_align_block_size
+    ids64 = ids_d.long()
+    align_s = time_launches(lambda: sort_topk_ids_align_block_size(ids64, G, 8, T // 8, 128), steps, warmup)
+    d["align_sort_us"] = round(align_s * 1e6, 2)
     return d, roof("hbm", comb_bytes, comb_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_combine"])
 
 

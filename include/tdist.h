@@ -207,6 +207,26 @@ int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_sc
                       const float* topk_w, const int32_t* cumsum, int64_t n_tokens, int topk, int hidden,
                       int world_size, int experts_per_rank, int max_m, void* out_bf16, void* stream);
 
+/* Align / sort for the grouped GEMM that follows the dispatch.
+ *   replaces moe_ag_scatter_align_block_size_op / _kernel   csrc/lib/moe_utils.cu:60-186
+ *   as called by sort_topk_ids_align_block_size              kernels/nvidia/allgather_group_gemm.py:54-135
+ * topk_ids: n_total = num_iterations * n_per_iteration flat expert ids (int32, or int64 when ids_int64 != 0, the
+ * reference's dtype), one segment of n_per_iteration entries per rank ("iteration"). Per segment, in order, the
+ * entries are grouped by expert keeping their flat order, every group is padded to a multiple of block_size, and the
+ * padded groups are laid end to end, segment after segment:
+ *   sorted_token_ids[pos] = flat index of the entry (positions of padding keep what the caller pre-filled, the
+ *                           reference fills with n_total); capacity n_total + num_experts*num_iterations*(block_size-1)
+ *   expert_ids[b], block_barrier_ids[b] = expert and segment of block b; at most
+ *                           n_total / block_size + num_experts * num_iterations blocks are written (the reference
+ *                           allocates n_total + num_experts * num_iterations entries)
+ *   rank_block_num[r]     = blocks of segment r;  *total_tokens_post_pad = padded total.
+ * Needs num_experts * num_iterations <= 4096. Workspace: tdist_moe_align_workspace_bytes (0 = unsupported sizes). */
+int64_t tdist_moe_align_workspace_bytes(int64_t n_total, int num_experts, int num_iterations);
+int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_total, int num_experts,
+                               int num_iterations, int64_t n_per_iteration, int block_size, int32_t* sorted_token_ids,
+                               int32_t* expert_ids, int32_t* block_barrier_ids, int32_t* rank_block_num,
+                               int32_t* total_tokens_post_pad, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * (d) split-KV GQA flash decode + LSE combine.
  *   replaces kernel_gqa_fwd_batch_decode_split_kv               kernels/nvidia/flash_decode.py:129-239

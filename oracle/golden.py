@@ -343,3 +343,47 @@ def make_paged_kv(batch: int, kv_len_max: int, kv_heads: int, head_dim: int, pag
     perm = torch.randperm(num_pages, generator=generator)[:batch * pages_per_seq]
     block_table = perm.view(batch, pages_per_seq).to(torch.int32).contiguous()
     return k_cache, v_cache, block_table
+
+
+# ---------------------------------------------------------------------------------------------------
+# MoE align / sort for the grouped GEMM (the step after the dispatch)
+# ---------------------------------------------------------------------------------------------------
+def sort_topk_ids_align_block_size(topk_ids, num_experts, num_ranks, num_tokens_per_rank, block_size):
+    """Restates moe_ag_scatter_align_block_size_kernel (csrc/lib/moe_utils.cu:60-165) as called by
+    sort_topk_ids_align_block_size (kernels/nvidia/allgather_group_gemm.py:54-135).
+
+    topk_ids [num_ranks * num_tokens_per_rank, topk]. Per rank segment (``iter`` in the kernel), in order: the
+    flat entries of the segment are grouped by expert, stably (:144-158); every expert's group is padded to a
+    multiple of ``block_size`` (:115-121); the padded groups are laid end to end, segment after segment (:72-75).
+    Returns (sorted_token_ids int32 [capacity] pre-filled with topk_ids.numel() (:115-116 of the Python),
+    expert_ids int32 [n_blocks], block_barrier_ids int32 [n_blocks], rank_block_num int32 [num_ranks],
+    num_tokens_post_pad int). expert_ids / block_barrier_ids are returned at their valid length (the reference
+    leaves the tail of its torch.empty buffers unwritten)."""
+    topk = topk_ids.shape[1]
+    flat = topk_ids.reshape(-1).to(torch.int64)
+    per = num_tokens_per_rank * topk
+    assert flat.numel() == per * num_ranks
+    capacity = (per + num_experts * (block_size - 1)) * num_ranks
+    sorted_ids = torch.full((capacity, ), flat.numel(), dtype=torch.int32)
+    expert_ids, barrier_ids, rank_block_num = [], [], []
+    base = 0
+    for it in range(num_ranks):
+        seg = flat[it * per:(it + 1) * per]
+        counts = torch.bincount(seg, minlength=num_experts)
+        padded = (counts + block_size - 1) // block_size * block_size
+        cum = torch.zeros(num_experts + 1, dtype=torch.int64)
+        cum[1:] = torch.cumsum(padded, 0)
+        order = torch.argsort(seg, stable=True)              # entries grouped by expert, original order kept
+        sorted_e = seg[order]
+        first = torch.zeros(num_experts + 1, dtype=torch.int64)
+        first[1:] = torch.cumsum(counts, 0)
+        within = torch.arange(per) - first[sorted_e]          # rank of each entry inside its expert's group
+        sorted_ids[base + cum[sorted_e] + within] = (order + it * per).to(torch.int32)
+        for e in range(num_experts):
+            nb = int(padded[e]) // block_size
+            expert_ids += [e] * nb
+            barrier_ids += [it] * nb
+        rank_block_num.append(int(cum[-1]) // block_size)
+        base += int(cum[-1])
+    return (sorted_ids, torch.tensor(expert_ids, dtype=torch.int32), torch.tensor(barrier_ids, dtype=torch.int32),
+            torch.tensor(rank_block_num, dtype=torch.int32), base)

@@ -191,3 +191,37 @@ def test_combine_reference_round_trip_bf16(cuda):
     torch.cuda.synchronize()
     torch.testing.assert_close(y_slots.float().cpu(), x.float() * topk, rtol=1e-2, atol=1e-2)
     assert torch.equal(y_slots, y_compact)
+
+
+@pytest.mark.parametrize("R,T,topk,E,BS,dtype", [(1, 4, 3, 4, 4, torch.int64), (8, 1024, 8, 256, 128, torch.int64),
+                                                 (8, 512, 6, 64, 64, torch.int32), (3, 37, 4, 11, 8, torch.int64),
+                                                 (2, 5, 2, 300, 1, torch.int32), (4, 1, 1, 1, 16, torch.int64),
+                                                 (16, 96, 8, 256, 128, torch.int64), (5, 300, 2, 7, 256, torch.int32)])
+def test_align_sort_bit_exact(cuda, R, T, topk, E, BS, dtype):
+    """sort_topk_ids_align_block_size against the oracle (the reference's align kernel restated)."""
+    from triton_dist.kernels.nvidia import sort_topk_ids_align_block_size
+    announce("moe align R=%d T=%d topk=%d E=%d BS=%d" % (R, T, topk, E, BS))
+    g = torch.Generator().manual_seed(R * 1000 + T + E)
+    if topk <= E:
+        ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(R * T)])
+    else:
+        ids = torch.randint(0, E, (R * T, topk), generator=g)
+    if E > 4:
+        ids[ids == 3] = 2   # leave an expert without tokens
+    want = golden.sort_topk_ids_align_block_size(ids, E, R, T, BS)
+    got = sort_topk_ids_align_block_size(ids.to(dtype).to(cuda), E, R, T, BS)
+    torch.cuda.synchronize()
+    n = want[4]
+    assert int(got[4].item()) == n
+    assert torch.equal(got[0].cpu(), want[0])                 # whole buffer: padding positions included
+    nb = n // BS
+    assert torch.equal(got[1].cpu()[:nb], want[1]) and torch.equal(got[2].cpu()[:nb], want[2])
+    assert torch.equal(got[3].cpu(), want[3])
+
+
+def test_align_sort_rejects_too_many_groups(cuda):
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import sort_topk_ids_align_block_size
+    ids = torch.zeros((64, 2), dtype=torch.int64, device=cuda)
+    with pytest.raises(_lib.TdistError):
+        sort_topk_ids_align_block_size(ids, 1024, 8, 8, 16)

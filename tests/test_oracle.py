@@ -219,3 +219,37 @@ def test_split_partials_merge_to_the_full_result():
     m2, _ = golden.lse_merge(part.permute(2, 0, 1, 3), part_lse.permute(2, 0, 1), skip)
     m3, _ = golden.lse_merge(part.permute(2, 0, 1, 3)[1:], part_lse.permute(2, 0, 1)[1:])
     assert torch.allclose(m2, m3, atol=1e-12)
+
+
+# ---- MoE align / sort ------------------------------------------------------------------------------------
+def test_align_sort_reference_examples():
+    """The two worked examples the reference itself documents."""
+    # kernels/nvidia/allgather_group_gemm.py:82-93 (expert ids 1..4 there; 0-based here)
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]]) - 1
+    s, e, b, r, n = golden.sort_topk_ids_align_block_size(ids, 4, 1, 4, 4)
+    assert n == 16 and s[:n].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert e.tolist() == [0, 1, 2, 3] and b.tolist() == [0, 0, 0, 0] and r.tolist() == [4]
+    # csrc/lib/moe_utils.cu:136-142: [0,1,2,1,2,3,0,3,4], block 4 -> [0,6,*,*,1,3,*,*,2,4,*,*,5,7,*,*,8,*,*,*]
+    ids = torch.tensor([0, 1, 2, 1, 2, 3, 0, 3, 4]).view(-1, 1)
+    s, e, b, r, n = golden.sort_topk_ids_align_block_size(ids, 5, 1, 9, 4)
+    P = 9
+    assert s[:n].tolist() == [0, 6, P, P, 1, 3, P, P, 2, 4, P, P, 5, 7, P, P, 8, P, P, P]
+    assert e.tolist() == [0, 1, 2, 3, 4]
+
+
+def test_align_sort_invariants():
+    g = torch.Generator().manual_seed(5)
+    R, T, topk, E, BS = 3, 37, 4, 11, 8
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(R * T)])
+    s, e, b, r, n = golden.sort_topk_ids_align_block_size(ids, E, R, T, BS)
+    flat = ids.reshape(-1)
+    valid = s[:n][s[:n] < flat.numel()].long()
+    assert sorted(valid.tolist()) == list(range(flat.numel()))           # every entry placed exactly once
+    assert n % BS == 0 and int(r.sum()) * BS == n and e.numel() == n // BS
+    per = T * topk
+    for blk in range(n // BS):                                            # a block holds one expert of one segment
+        ent = s[blk * BS:(blk + 1) * BS]
+        ent = ent[ent < flat.numel()].long()
+        assert torch.all(flat[ent] == e[blk]) and torch.all(ent // per == b[blk])
+        assert torch.all(ent[1:] > ent[:-1])                              # flat order kept inside a group
+    assert torch.all(s[n:] == flat.numel())

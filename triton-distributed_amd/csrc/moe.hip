@@ -480,6 +480,78 @@ __global__ __launch_bounds__(kCombineWaves * 64) void moe_combine_kernel(
   }
 }
 
+// ---- align / sort for the grouped GEMM ------------------------------------------------------------------
+// Follows moe_ag_scatter_align_block_size_kernel (csrc/lib/moe_utils.cu:60-165): per rank segment, entries grouped
+// by expert in flat order, every group padded to a multiple of block_size, groups and segments laid end to end.
+// Built on the stable index of this file with the composite key segment * E + expert: the position of an entry in
+// the padded layout is its position in the unpadded sorted order moved by the padding in front of its group.
+
+// keys[i] = (i / per_iter) * E + ids[i], or -1 for an id outside [0, E)
+__global__ __launch_bounds__(256) void moe_align_keys_kernel(const void* __restrict__ ids, int ids_int64, int64_t n,
+                                                            int64_t per_iter, int E, int32_t* __restrict__ keys) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int64_t id = ids_int64 ? ((const int64_t*)ids)[i] : (int64_t)((const int32_t*)ids)[i];
+  keys[i] = (id >= 0 && id < E) ? (int32_t)((i / per_iter) * E + id) : -1;
+}
+
+// One workgroup: padded exclusive prefix over the G = R * E group sizes, the per-block expert / segment ids, the
+// blocks per segment and the padded total.
+__global__ __launch_bounds__(kScanThreads) void moe_align_pad_kernel(const int32_t* __restrict__ splits, int G, int E,
+                                                                    int R, int block_size,
+                                                                    int32_t* __restrict__ pad_cum,
+                                                                    int32_t* __restrict__ expert_ids,
+                                                                    int32_t* __restrict__ block_barrier_ids,
+                                                                    int32_t* __restrict__ rank_block_num,
+                                                                    int32_t* __restrict__ total_post_pad) {
+  __shared__ int32_t s_part[kScanThreads];
+  const int per = (G + kScanThreads - 1) / kScanThreads;  // consecutive groups per thread
+  const int g0 = threadIdx.x * per;
+  int32_t local_total = 0;
+  for (int j = 0; j < per; ++j) {
+    const int g = g0 + j;
+    if (g < G) local_total += (splits[g] + block_size - 1) / block_size * block_size;
+  }
+  s_part[threadIdx.x] = local_total;
+  __syncthreads();
+  for (int off = 1; off < kScanThreads; off <<= 1) {
+    const int32_t v = (threadIdx.x >= off) ? s_part[threadIdx.x - off] : 0;
+    __syncthreads();
+    s_part[threadIdx.x] += v;
+    __syncthreads();
+  }
+  int32_t run = s_part[threadIdx.x] - local_total;
+  if (threadIdx.x == 0) pad_cum[0] = 0;
+  for (int j = 0; j < per; ++j) {
+    const int g = g0 + j;
+    if (g < G) {
+      const int32_t padded = (splits[g] + block_size - 1) / block_size * block_size;
+      for (int32_t b = run / block_size; b < (run + padded) / block_size; ++b) {
+        expert_ids[b] = g % E;
+        block_barrier_ids[b] = g / E;
+      }
+      run += padded;
+      pad_cum[g + 1] = run;
+    }
+  }
+  __threadfence_block();  // pad_cum was written by this workgroup and is read back below
+  __syncthreads();
+  for (int r = threadIdx.x; r < R; r += kScanThreads)
+    rank_block_num[r] = (pad_cum[(r + 1) * E] - pad_cum[r * E]) / block_size;
+  if (threadIdx.x == 0) *total_post_pad = pad_cum[G];
+}
+
+__global__ __launch_bounds__(256) void moe_align_place_kernel(const int32_t* __restrict__ keys,
+                                                             const int32_t* __restrict__ scatter_idx,
+                                                             const int32_t* __restrict__ cumsum,
+                                                             const int32_t* __restrict__ pad_cum, int64_t n,
+                                                             int32_t* __restrict__ sorted_ids) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int32_t k = keys[i];
+  if (k >= 0) sorted_ids[pad_cum[k] + (scatter_idx[i] - cumsum[k])] = (int32_t)i;
+}
+
 static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, int32_t* splits, int32_t* cumsum,
                             int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx, void* workspace,
                             int64_t workspace_bytes, hipStream_t stream, bool want_index, const char* who) {
@@ -615,6 +687,54 @@ int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_sc
                      (const unsigned char*)slot_rows, slot_scales, scatter_idx, topk_w, cumsum, n_tokens, topk, hidden,
                      world_size, experts_per_rank, max_m, n_windows, (unsigned short*)out_bf16);
   return launch_status("tdist_moe_combine");
+}
+
+int64_t tdist_moe_align_workspace_bytes(int64_t n_total, int num_experts, int num_iterations) {
+  if (n_total < 0 || num_experts <= 0 || num_iterations <= 0) return 0;
+  const int64_t G = (int64_t)num_experts * num_iterations;
+  if (G > kMoeMaxExperts) return 0;
+  // keys, scatter index, gather index; group sizes, two prefix rows; then the index build's own scratch
+  return (3 * n_total + 3 * (G + 1)) * 4 + tdist_moe_workspace_bytes(n_total, (int)G);
+}
+
+int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_total, int num_experts,
+                               int num_iterations, int64_t n_per_iteration, int block_size, int32_t* sorted_token_ids,
+                               int32_t* expert_ids, int32_t* block_barrier_ids, int32_t* rank_block_num,
+                               int32_t* total_tokens_post_pad, void* workspace, int64_t workspace_bytes, void* stream) {
+  const char* who = "tdist_moe_align_block_size";
+  if (!topk_ids || !sorted_token_ids || !expert_ids || !block_barrier_ids || !rank_block_num || !total_tokens_post_pad)
+    return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
+  if (num_experts <= 0 || num_iterations <= 0 || block_size <= 0 || n_per_iteration < 0 ||
+      n_total != n_per_iteration * num_iterations)
+    return fail(TDIST_ERR_INVALID, "%s: bad sizes (n_total must be num_iterations * n_per_iteration)", who);
+  const int64_t G = (int64_t)num_experts * num_iterations;
+  if (G > kMoeMaxExperts)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: num_experts * num_iterations = %lld > %d", who, (long long)G, kMoeMaxExperts);
+  if (n_total + G * (int64_t)(block_size - 1) > 0x7fffffffll) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many entries", who);
+  const int64_t need = tdist_moe_align_workspace_bytes(n_total, num_experts, num_iterations);
+  if (!workspace || workspace_bytes < need)
+    return fail(TDIST_ERR_WORKSPACE, "%s: workspace %lld B < %lld B", who, (long long)workspace_bytes, (long long)need);
+  hipStream_t st = (hipStream_t)stream;
+  int32_t* keys = (int32_t*)workspace;
+  int32_t* scatter = keys + n_total;
+  int32_t* gather = scatter + n_total;
+  int32_t* splits = gather + n_total;
+  int32_t* cumsum = splits + (G + 1);
+  int32_t* pad_cum = cumsum + (G + 1);
+  void* index_ws = pad_cum + (G + 1);
+  const int64_t blocks = ceil_div(n_total > 0 ? n_total : 1, 256);
+  if (n_total > 0)
+    hipLaunchKernelGGL(moe_align_keys_kernel, dim3((unsigned)blocks), dim3(256), 0, st, topk_ids, ids_int64, n_total,
+                       n_per_iteration > 0 ? n_per_iteration : 1, num_experts, keys);
+  int rc = moe_index_common(keys, n_total, 1, (int)G, splits, cumsum, scatter, gather, nullptr, index_ws,
+                            tdist_moe_workspace_bytes(n_total, (int)G), st, true, who);
+  if (rc != TDIST_OK) return rc;
+  hipLaunchKernelGGL(moe_align_pad_kernel, dim3(1), dim3(kScanThreads), 0, st, splits, (int)G, num_experts, num_iterations,
+                     block_size, pad_cum, expert_ids, block_barrier_ids, rank_block_num, total_tokens_post_pad);
+  if (n_total > 0)
+    hipLaunchKernelGGL(moe_align_place_kernel, dim3((unsigned)blocks), dim3(256), 0, st, keys, scatter, cumsum, pad_cum,
+                       n_total, sorted_token_ids);
+  return launch_status(who);
 }
 
 }  // extern "C"
