@@ -279,3 +279,21 @@ def test_fp8_ag_gemm_config3_full_size(cuda):
     c2 = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx, row_scale=sa2.to(cuda), col_scale=sb.to(cuda))
     ctx.check_status()
     assert torch.equal(c2[::2].float(), c[::2].float() * 2) and torch.equal(c2[1::2], c[1::2])
+
+
+@pytest.mark.parametrize("dtype,K", [(torch.bfloat16, 96), (torch.bfloat16, 128), (torch.float8_e4m3fn, 192),
+                                     (torch.float16, 224), (torch.bfloat16, 64)])
+def test_many_tiles_with_short_and_odd_k(cuda, dtype, K):
+    """Enough 256 x 256 tiles for the large-tile path, with K rows of one K tile, of an odd number of 64-byte halves
+    (which must take the small tiles) and of a single 64-byte half."""
+    from triton_dist.kernels.amd import gated_gemm
+    announce("gemm many tiles K=%d %s" % (K, dtype))
+    M, N = 4096, 6144
+    g = torch.Generator().manual_seed(K)
+    a = torch.randint(-3, 4, (M, K), generator=g).float()
+    b = torch.randint(-3, 4, (N, K), generator=g).float()
+    c = torch.empty((M, N), dtype=torch.float16 if dtype == torch.float16 else torch.bfloat16, device=cuda)
+    gated_gemm(a.to(dtype).to(cuda), None, 0, b.to(dtype).to(cuda), c, None, 0, 0, 1)
+    torch.cuda.synchronize()
+    ref = a.to(cuda) @ b.to(cuda).T      # small integers: the fp32 sums are exact, so only the final rounding differs
+    assert torch.equal(c, ref.to(c.dtype))

@@ -645,6 +645,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (c.scatter_bufs && c.world_size > 0 && (c.M % c.world_size != 0 || (c.M / c.world_size) % 256 != 0)) big = false;
   if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) big = false;
   if (c.A_local && (c.local_row_begin % 256 != 0 || c.local_rows % 256 != 0)) big = false;
+  if (((int64_t)c.K * esz) % 128 != 0) big = false;  // the large tiles step through K 128 bytes at a time
   // TDIST_GEMM_VARIANT picks another compiled tiling for the large-tile path (measurement aid); the default,
   // 6, is 256x256 tiles, 128-byte K rows, 2x2 waves of 128x128, split ring (3 A stages + 2 B stages).
   int variant = 6;
