@@ -297,3 +297,22 @@ def test_many_tiles_with_short_and_odd_k(cuda, dtype, K):
     torch.cuda.synchronize()
     ref = a.to(cuda) @ b.to(cuda).T      # small integers: the fp32 sums are exact, so only the final rounding differs
     assert torch.equal(c, ref.to(c.dtype))
+
+
+@pytest.mark.parametrize("M,N,K,pad", [(4100, 6150, 256, 0), (4097, 6408, 384, 64), (5000, 5001, 128, 8)])
+def test_large_tiles_with_ragged_edges_and_padded_rows(cuda, M, N, K, pad):
+    """The 256 x 256 path on shapes that are no multiple of the tile, with padded row strides and an output stride
+    that rules out vector stores."""
+    from triton_dist.kernels.amd import gated_gemm
+    announce("gemm ragged M=%d N=%d K=%d pad=%d" % (M, N, K, pad))
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randint(-3, 4, (M, K + pad), generator=g).float()
+    b = torch.randint(-3, 4, (N, K + pad), generator=g).float()
+    a_d = a.to(torch.bfloat16).to(cuda)[:, :K]
+    b_d = b.to(torch.bfloat16).to(cuda)[:, :K]
+    c = torch.full((M + 1, N), 7.0, dtype=torch.bfloat16, device=cuda)
+    gated_gemm(a_d, None, 0, b_d, c[:M], None, 0, 0, 1)
+    torch.cuda.synchronize()
+    ref = a[:, :K].to(cuda) @ b[:, :K].to(cuda).T
+    assert torch.equal(c[:M], ref.to(torch.bfloat16))
+    assert torch.all(c[M] == 7.0)   # nothing written past the last row
