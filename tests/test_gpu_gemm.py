@@ -316,3 +316,52 @@ def test_large_tiles_with_ragged_edges_and_padded_rows(cuda, M, N, K, pad):
     ref = a[:, :K].to(cuda) @ b[:, :K].to(cuda).T
     assert torch.equal(c[:M], ref.to(torch.bfloat16))
     assert torch.all(c[M] == 7.0)   # nothing written past the last row
+
+
+def test_randomised_shapes_gating_and_layouts(cuda):
+    """Forty seeded random cases over both tile paths: ragged M / N, K in 64-byte steps, padded row strides, the three
+    dtypes, gating with a local shard and pre-released flags in either chunk order, plain calls. Integer-valued inputs,
+    so the only rounding is the final one."""
+    import random
+    from triton_dist.kernels.amd import gated_gemm
+    rnd = random.Random(1234)
+    for case in range(40):
+        dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float8_e4m3fn])
+        esz = 1 if dtype == torch.float8_e4m3fn else 2
+        big = rnd.random() < 0.4
+        gated = rnd.random() < 0.5
+        K = rnd.randrange(1, 9) * 64 // esz
+        pad_a, pad_b = rnd.choice([0, 16, 64]), rnd.choice([0, 16, 128])
+        if gated:
+            world = rnd.choice([2, 4, 8])
+            mpc = rnd.choice([256, 512]) if big else rnd.choice([128, 256, 384])
+            cpr = rnd.choice([1, 2])
+            M = world * cpr * mpc
+            N = rnd.randrange(20, 30) * 256 - rnd.choice([0, 8, 100]) if big else rnd.randrange(1, 700)
+            if big and (M // 256) * ((N + 255) // 256) < 384:
+                N = 256 * (384 * 256 // M + 1)
+            rank = rnd.randrange(world)
+        else:
+            M = rnd.randrange(4000, 5200) if big else rnd.randrange(1, 900)
+            N = rnd.randrange(6000, 6600) if big else rnd.randrange(1, 900)
+            world, rank, mpc, cpr = 1, 0, 0, 1
+        announce("gemm case %d: %s M=%d N=%d K=%d gated=%s world=%d mpc=%d rank=%d pads=%d,%d" %
+                 (case, dtype, M, N, K, gated, world, mpc, rank, pad_a, pad_b))
+        g = torch.Generator().manual_seed(case)
+        a = torch.randint(-2, 3, (M, K + pad_a), generator=g).float()
+        b = torch.randint(-2, 3, (N, K + pad_b), generator=g).float()
+        a_d, b_d = a.to(dtype).to(cuda)[:, :K], b.to(dtype).to(cuda)[:, :K]
+        out_dtype = torch.float16 if dtype == torch.float16 else torch.bfloat16
+        c = torch.empty((M, N), dtype=out_dtype, device=cuda)
+        if gated:
+            mpr = M // world
+            local = a_d[rank * mpr:(rank + 1) * mpr].contiguous()
+            ws = a_d.clone()
+            ws[rank * mpr:(rank + 1) * mpr] = 0      # the own rows must come from the local shard
+            flags = torch.ones(world * cpr, dtype=torch.int32, device=cuda)
+            gated_gemm(ws, local, rank * mpr, b_d, c, flags, mpc, rank, world)
+        else:
+            gated_gemm(a_d, None, 0, b_d, c, None, 0, 0, 1)
+        torch.cuda.synchronize()
+        ref = (a[:, :K].to(cuda) @ b[:, :K].to(cuda).T).to(out_dtype)
+        assert torch.equal(c, ref), "case %d differs" % case
