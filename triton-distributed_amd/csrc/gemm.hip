@@ -491,59 +491,6 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // acc[j][i][e]: output row m = wm*kWaveM + 32i + l32, column n = wn*kWaveN + 32j + 8*(e/4) + 4*lh + e%4
     wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
     lds_u8 const epi = smem + wave * C::kEpiBytes;
-    float rs[C::kTM];
-#pragma unroll
-    for (int i = 0; i < C::kTM; ++i) {
-      rs[i] = 1.f;
-      if (kScales && p.row_scale) rs[i] = p.row_scale[min(m0 + wm * C::kWaveM + 32 * i + l32, p.M - 1)];
-    }
-#pragma unroll
-    for (int j = 0; j < C::kTN; ++j) {
-      // the four column scales of each of this lane's four column groups in this 32-column block
-      float4v cs[4];
-      if (kScales) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          cs[q] = float4v{1.f, 1.f, 1.f, 1.f};
-          if (p.col_scale) {
-            const int gn = n0 + wn * C::kWaveN + 32 * j + 8 * q + 4 * lh;
-            if (gn + 3 < p.N) cs[q] = *(const float4v*)(p.col_scale + gn);
-            else
-              for (int e = 0; e < 4; ++e) cs[q][e] = p.col_scale[min(gn + e, p.N - 1)];
-          }
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < C::kTM; ++i) {
-        const int mrow = 32 * i + l32;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int ncol = 32 * j + 8 * q + 4 * lh;
-          float v0, v1, v2, v3;
-          if constexpr (C::kTM * C::kTN * 16 >= 256) {
-            // 256 accumulators live in AGPRs; read each one here, where it is packed, instead of letting the
-            // compiler copy all of them to VGPRs at the loop exit (which spills)
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v0) : "a"(acc[j][i][4 * q + 0]));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v1) : "a"(acc[j][i][4 * q + 1]));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v2) : "a"(acc[j][i][4 * q + 2]));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v3) : "a"(acc[j][i][4 * q + 3]));
-          } else {
-            v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2], v3 = acc[j][i][4 * q + 3];
-          }
-          if (kScales) {
-            v0 *= rs[i] * cs[q][0];
-            v1 *= rs[i] * cs[q][1];
-            v2 *= rs[i] * cs[q][2];
-            v3 *= rs[i] * cs[q][3];
-          }
-          const int2v w = {(int)E::pack(v0, v1), (int)E::pack(v2, v3)};
-          *(TDIST_AS3 int2v*)(epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2) = w;
-        }
-        __builtin_amdgcn_sched_barrier(0);  // keep the accumulator read-out tile by tile (register pressure)
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     // destination of this tile's rows
     unsigned char* Cbase;
     int64_t crow0;
@@ -559,22 +506,94 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     constexpr int kRowsPerPass = 64 / kLanesPerRow;
     const int er = lane / kLanesPerRow, ec = lane % kLanesPerRow;
     const bool n_vec_ok = (p.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(Cbase) & 15) == 0);
-#pragma unroll 4
-    for (int pass = 0; pass < C::kWaveM / kRowsPerPass; ++pass) {
-      const int mrow = pass * kRowsPerPass + er;
-      const int gm = m0 + wm * C::kWaveM + mrow;
-      const int gn = n0 + wn * C::kWaveN + ec * 8;
-      const int4v v = *(const TDIST_AS3 int4v*)(epi + mrow * C::kEpiPitch + ((ec ^ (mrow & C::kEpiSwz)) << 4));
-      if (gm < p.M && gn < p.N) {
-        unsigned short* dst = (unsigned short*)Cbase + (crow0 + wm * C::kWaveM + mrow) * p.ldc + gn;
-        if (gn + 8 <= p.N && n_vec_ok) {
-          if (p.scatter_bufs == nullptr) __builtin_nontemporal_store(v, (int4v*)dst);  // written once, not read back here
-          else *(int4v*)dst = v;
+
+    // packs the 32 x 32 block (i, j) of the wave tile into its staging rows
+    auto stage_block = [&](int i, int j, float rsi, const float4v* cs) {
+      const int mrow = 32 * i + l32;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int ncol = 32 * j + 8 * q + 4 * lh;
+        float v0, v1, v2, v3;
+        if constexpr (C::kTM * C::kTN * 16 >= 256) {
+          // 256 accumulators live in AGPRs; read each one here, where it is packed, instead of letting the
+          // compiler copy all of them to VGPRs at the loop exit (which spills)
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v0) : "a"(acc[j][i][4 * q + 0]));
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v1) : "a"(acc[j][i][4 * q + 1]));
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v2) : "a"(acc[j][i][4 * q + 2]));
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v3) : "a"(acc[j][i][4 * q + 3]));
         } else {
-          for (int e = 0; e < 8; ++e)
-            if (gn + e < p.N) dst[e] = (unsigned short)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+          v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2], v3 = acc[j][i][4 * q + 3];
+        }
+        if (kScales) {
+          v0 *= rsi * cs[q][0];
+          v1 *= rsi * cs[q][1];
+          v2 *= rsi * cs[q][2];
+          v3 *= rsi * cs[q][3];
+        }
+        const int2v w = {(int)E::pack(v0, v1), (int)E::pack(v2, v3)};
+        *(TDIST_AS3 int2v*)(epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2) = w;
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the accumulator read-out block by block (register pressure)
+    };
+    // staged rows [row0, row0 + nrows) of the wave tile → global memory, 16 bytes per lane
+    auto store_rows = [&](int row0, int nrows) {
+#pragma unroll 4
+      for (int pass = 0; pass < nrows / kRowsPerPass; ++pass) {
+        const int mrow = row0 + pass * kRowsPerPass + er;
+        const int gm = m0 + wm * C::kWaveM + mrow;
+        const int gn = n0 + wn * C::kWaveN + ec * 8;
+        const int4v v = *(const TDIST_AS3 int4v*)(epi + mrow * C::kEpiPitch + ((ec ^ (mrow & C::kEpiSwz)) << 4));
+        if (gm < p.M && gn < p.N) {
+          unsigned short* dst = (unsigned short*)Cbase + (crow0 + wm * C::kWaveM + mrow) * p.ldc + gn;
+          if (gn + 8 <= p.N && n_vec_ok) {
+            if (p.scatter_bufs == nullptr) __builtin_nontemporal_store(v, (int4v*)dst);  // written once, not read back here
+            else *(int4v*)dst = v;
+          } else {
+            for (int e = 0; e < 8; ++e)
+              if (gn + e < p.N) dst[e] = (unsigned short)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+          }
         }
       }
+    };
+    static_assert(32 % kRowsPerPass == 0, "a 32-row block is a whole number of store passes");
+
+    if constexpr (!kScales && C::kTM * C::kTN * 16 >= 256) {
+      // row block by row block: the stores of block i drain while block i+1 is being packed
+#pragma unroll
+      for (int i = 0; i < C::kTM; ++i) {
+#pragma unroll
+        for (int j = 0; j < C::kTN; ++j) stage_block(i, j, 1.f, nullptr);
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        store_rows(32 * i, 32);
+      }
+    } else {
+      float rs[C::kTM];
+#pragma unroll
+      for (int i = 0; i < C::kTM; ++i) {
+        rs[i] = 1.f;
+        if (kScales && p.row_scale) rs[i] = p.row_scale[min(m0 + wm * C::kWaveM + 32 * i + l32, p.M - 1)];
+      }
+#pragma unroll
+      for (int j = 0; j < C::kTN; ++j) {
+        // the four column scales of each of this lane's four column groups in this 32-column block
+        float4v cs[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          cs[q] = float4v{1.f, 1.f, 1.f, 1.f};
+          if (kScales && p.col_scale) {
+            const int gn = n0 + wn * C::kWaveN + 32 * j + 8 * q + 4 * lh;
+            if (gn + 3 < p.N) cs[q] = *(const float4v*)(p.col_scale + gn);
+            else
+              for (int e = 0; e < 4; ++e) cs[q][e] = p.col_scale[min(gn + e, p.N - 1)];
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < C::kTM; ++i) stage_block(i, j, rs[i], cs);
+      }
+      __builtin_amdgcn_wave_barrier();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      store_rows(0, C::kWaveM);
     }
     // the next tile's prologue overwrites the ring: every wave must be done reading its staging area
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
