@@ -286,10 +286,20 @@ def bench_c5(dev, steps, warmup):
         lambda: decode_combine(out_split, lse_split, S, 1, lens, B, Hq, D,
                                (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
                                (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), merged), steps, warmup)
+    # the rank merge of BASELINE config 5: own (out, LSE) + 7 seeded synthetic peer shards -> [32, 64, 128] bf16
+    from triton_dist.kernels.amd import gqa_fwd_batch_decode_inter_rank_combine
+    g2 = torch.Generator(device="cuda").manual_seed(3 + 4 + 100)
+    R = 8
+    all_out = torch.randn((R, B, Hq, D), generator=g2, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    all_lse = torch.randn((R, B, Hq), generator=g2, device=dev, dtype=torch.float32) * 2 + 10.4
+    all_lens = torch.full((R, B), L, dtype=torch.int32, device=dev)
+    final = torch.empty((B, Hq, D), dtype=torch.bfloat16, device=dev)
+    rank_s = time_launches(lambda: gqa_fwd_batch_decode_inter_rank_combine(all_out, all_lse, all_lens, final), steps, warmup)
     kv_bytes = 2 * B * L * Hkv * D * 2
     split_bytes = kv_bytes + q.numel() * 2 + table.numel() * 4 + out_split.numel() * 4 + lse_split.numel() * 4
     r = roof("hbm", split_bytes, split_s, "hbm", MEASURED_TRAFFIC_BYTES["c5_split_kv"])
     r["combine_us"] = round(comb_s * 1e6, 2)
+    r["inter_rank_combine_us"] = round(rank_s * 1e6, 2)
     return r
 
 
