@@ -262,6 +262,14 @@ def bench_c4(dev, steps, warmup):
     ids64 = ids_d.long()
     align_s = time_launches(lambda: sort_topk_ids_align_block_size(ids64, G, 8, T // 8, 128), steps, warmup)
     d["align_sort_us"] = round(align_s * 1e6, 2)
+    # dispatch with the e4m3 quantisation (groups of 128 columns) fused in: bf16 tokens read once, 8 e4m3 copies written
+    ctx_q = create_all_to_all_context(max_m, H, 0, G, W, G // W, dtype=torch.float8_e4m3fn, fp8_group_size=128)
+    xb = torch.randn((T, H), generator=g).to(torch.bfloat16).to(dev)
+    qd_s = time_launches(lambda: fast_all_to_all(ctx_q, xb, cumsum, None, scatter_index=scatter, online_quant_fp8=True),
+                         steps, warmup)
+    qd_bytes = T * H * 2 + n * H + n * (H // 128) * 4 + n * 4
+    d["online_quant_dispatch"] = {"us_per_launch": round(qd_s * 1e6, 2), "achieved_GBps": round(qd_bytes / qd_s / 1e9, 1),
+                                  "frac": round(qd_bytes / qd_s / PEAK["hbm"], 4)}
     return d, roof("hbm", comb_bytes, comb_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_combine"])
 
 

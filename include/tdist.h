@@ -202,10 +202,29 @@ int tdist_moe_post_process(const void* slot_rows, int64_t row_bytes, const float
  * fp32 accumulation in k order, output bf16 [T, hidden]. Rows are read from the slot layout written by
  * tdist_moe_dispatch (max_m > 0) or from a compact sorted [n, hidden] tensor (max_m == 0, cumsum
  * ignored). row_dtype: TDIST_F8E4M3 (scales required unless NULL = 1.0) or TDIST_BF16.
- * topk_w fp32 [T, topk] or NULL (= 1.0, the index_add_ form of test_all_to_all.py:366-367). */
+ * topk_w fp32 [T, topk] or NULL (= 1.0, the index_add_ form of test_all_to_all.py:366-367).
+ * scale_group_size 0: slot_scales holds one scale per row; > 0 (e4m3 rows only): one per group of that many columns,
+ * [rows, hidden/scale_group_size], as tdist_moe_dispatch_tokens_quant writes them. */
 int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_scales, const int32_t* scatter_idx,
                       const float* topk_w, const int32_t* cumsum, int64_t n_tokens, int topk, int hidden,
-                      int world_size, int experts_per_rank, int max_m, void* out_bf16, void* stream);
+                      int world_size, int experts_per_rank, int max_m, int scale_group_size, void* out_bf16,
+                      void* stream);
+
+/* Online e4m3 quantisation in groups of group_size = 128 columns.
+ *   replaces _quant_kernel / quant_bf16_fp8   tutorials/04-deepseek-infer-all2all.py:309-360
+ *   and the fused form in its dispatch kernel  tutorials/04-deepseek-infer-all2all.py:180-200
+ * x bf16 [n_rows, hidden] → q e4m3 [n_rows, hidden], scales fp32 [n_rows, hidden/group_size]:
+ *   scale = max|x| over the group (as fp32) * fp32(1/448),  q = e4m3(float(x) / scale), round to nearest even.
+ * (A group of zeros divides 0 by 0, as the reference does: NaN bytes, scale 0.) */
+int tdist_quant_e4m3_groups(const void* x_bf16, int64_t n_rows, int hidden, int group_size, void* q_out,
+                            float* scales_out, void* stream);
+/* tdist_moe_dispatch_tokens with that quantisation fused in: bf16 token rows [n_tokens, hidden] in, e4m3 slot rows
+ * [world_size*max_m, hidden] and slot_scales fp32 [world_size*max_m, hidden/group_size] out; every token row is read
+ * and quantised once and written to its topk slot rows. */
+int tdist_moe_dispatch_tokens_quant(const void* tokens_bf16, int hidden, int group_size, const int32_t* scatter_idx,
+                                    int topk, const int32_t* cumsum, int64_t n_tokens, int world_size,
+                                    int experts_per_rank, int max_m, void* slot_rows, float* slot_scales,
+                                    int32_t* splits_out, void* stream);
 
 /* Align / sort for the grouped GEMM that follows the dispatch.
  *   replaces moe_ag_scatter_align_block_size_op / _kernel   csrc/lib/moe_utils.cu:60-186

@@ -387,3 +387,24 @@ def sort_topk_ids_align_block_size(topk_ids, num_experts, num_ranks, num_tokens_
         base += int(cum[-1])
     return (sorted_ids, torch.tensor(expert_ids, dtype=torch.int32), torch.tensor(barrier_ids, dtype=torch.int32),
             torch.tensor(rank_block_num, dtype=torch.int32), base)
+
+
+# ---------------------------------------------------------------------------------------------------
+# e4m3 quantisation in groups of 128 columns (the fused form of the dispatch)
+# ---------------------------------------------------------------------------------------------------
+def quantize_groups_e4m3(x, group=128):
+    """Restates _quant_kernel (tutorials/04-deepseek-infer-all2all.py:309-329; fused in the dispatch kernel at
+    :180-200): per group, scale = max|x| as fp32 times fp32(1/448), q = e4m3(float(x) / scale). PARITY UNPINNED by
+    the reference: tutorial code, no test or stored vector holds its outputs; pinned here by the closed form and by
+    dequantise(quantise(x)) staying within half an e4m3 step of x."""
+    m, N = x.shape
+    g = x.float().view(m, N // group, group)
+    scale = g.abs().amax(-1, keepdim=True) * torch.tensor(1.0 / 448.0, dtype=torch.float32)
+    q = (g / scale).to(torch.float8_e4m3fn).view(m, N)
+    return q, scale.view(m, N // group)
+
+
+def dequantize_groups(q, scale, group=128):
+    """_dequant_kernel (tutorials/04-deepseek-infer-all2all.py:333-351): bf16(float(q) * scale)."""
+    m, N = q.shape
+    return (q.float().view(m, N // group, group) * scale[..., None]).view(m, N).to(torch.bfloat16)

@@ -225,3 +225,56 @@ def test_align_sort_rejects_too_many_groups(cuda):
     ids = torch.zeros((64, 2), dtype=torch.int64, device=cuda)
     with pytest.raises(_lib.TdistError):
         sort_topk_ids_align_block_size(ids, 1024, 8, 8, 16)
+
+
+@pytest.mark.parametrize("m,N", [(1, 128), (37, 1024), (64, 7168), (5, 2176)])
+def test_group_quantiser_bit_exact(cuda, m, N):
+    from triton_dist.kernels.amd import quant_bf16_fp8
+    announce("group quant m=%d N=%d" % (m, N))
+    g = torch.Generator().manual_seed(m + N)
+    mags = torch.tensor([1e-4, 1e-2, 1.0, 3.0, 100.0, 3e4])[torch.randint(0, 6, (m, 1), generator=g)]
+    x = (torch.randn((m, N), generator=g) * mags).to(torch.bfloat16)
+    x[0, :8] = torch.tensor([0.0, -0.0, 1.0, -1.0, 0.5, 3.0, 448.0, -448.0]).to(torch.bfloat16)
+    want_q, want_s = golden.quantize_groups_e4m3(x)
+    got_q, got_s = quant_bf16_fp8(x.to(cuda))
+    torch.cuda.synchronize()
+    assert torch.equal(got_s.cpu(), want_s)
+    assert torch.equal(got_q.cpu().view(torch.uint8), want_q.view(torch.uint8))
+
+
+@pytest.mark.parametrize("T,topk,G,W,H,max_m", [(4096, 8, 256, 32, 7168, 4096), (96, 4, 16, 4, 256, 160), (33, 5, 8, 2, 1152, 128),
+                                                (300, 4, 128, 64, 128, 48)])
+def test_dispatch_with_online_quantisation_and_grouped_combine(cuda, T, topk, G, W, H, max_m):
+    """The fused path: bf16 tokens in, e4m3 slot rows + group scales out (bit-exact against quantise-then-dispatch),
+    then the weighted combine reading the group scales."""
+    from triton_dist.kernels.amd import (create_all_to_all_context, fast_all_to_all, moe_dispatch_preprocess,
+                                         moe_weighted_combine)
+    announce("moe online quant T=%d topk=%d G=%d H=%d" % (T, topk, G, H))
+    ids, x, _, _, w = make_case(T, topk, G, H, seed=T + 7)
+    xb = x.to(torch.bfloat16)
+    q, s = golden.quantize_groups_e4m3(xb)
+    ctx = create_all_to_all_context(max_m, H, 0, G, W, G // W, dtype=torch.float8_e4m3fn, fp8_group_size=128)
+    ctx.recv_buf.view(torch.uint8).zero_()
+    ctx.scale_recv_buf.zero_()
+    splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids.to(cuda), G)
+    o_splits, recv, recv_scale = fast_all_to_all(ctx, xb.to(cuda), cumsum, None, scatter_index=scatter, online_quant_fp8=True)
+    torch.cuda.synchronize()
+    # expected slots: sorted row p = token gather[p]; destination d takes rows [cumsum[d*Er], cumsum[(d+1)*Er])
+    w_splits, w_cumsum, w_scatter, w_gather, _ = golden.moe_preprocess(ids, G)
+    Er = G // W
+    exp_rows = torch.zeros((W * max_m, H), dtype=torch.uint8)
+    exp_scale = torch.zeros((W * max_m, H // 128))
+    for d in range(W):
+        lo, hi = int(w_cumsum[d * Er]), int(w_cumsum[(d + 1) * Er])
+        n = min(hi - lo, max_m)
+        tok = w_gather[lo:lo + n].long()
+        exp_rows[d * max_m:d * max_m + n] = q.view(torch.uint8)[tok]
+        exp_scale[d * max_m:d * max_m + n] = s[tok]
+    assert torch.equal(o_splits.cpu(), w_splits)
+    assert torch.equal(recv.view(torch.uint8).cpu(), exp_rows)
+    assert torch.equal(recv_scale.cpu(), exp_scale)
+    y = moe_weighted_combine(ctx, recv, recv_scale, scatter, w.to(cuda), cumsum)
+    torch.cuda.synchronize()
+    deq = q.float().view(T, H // 128, 128) * s[..., None]
+    ref = (deq.view(T, H) * w.sum(-1, keepdim=True))           # every copy of token t carries token t's row
+    assert golden.max_rel_err(y.float().cpu(), ref) <= 1e-2

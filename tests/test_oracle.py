@@ -253,3 +253,25 @@ def test_align_sort_invariants():
         assert torch.all(flat[ent] == e[blk]) and torch.all(ent // per == b[blk])
         assert torch.all(ent[1:] > ent[:-1])                              # flat order kept inside a group
     assert torch.all(s[n:] == flat.numel())
+
+
+# ---- group quantisation ----------------------------------------------------------------------------------
+def test_group_quantisation_closed_form_and_round_trip():
+    g = torch.Generator().manual_seed(8)
+    x = (torch.randn((6, 384), generator=g) * torch.tensor([1e-3, 0.1, 1.0, 7.0, 300.0, 5e4])[:, None]).to(torch.bfloat16)
+    q, s = golden.quantize_groups_e4m3(x)
+    xf = x.float().view(6, 3, 128)
+    amax = xf.abs().amax(-1)
+    # the scale maps the group's largest magnitude onto 448, the largest finite e4m3
+    assert torch.allclose(s, amax / 448, rtol=2e-7, atol=0)
+    qf = q.float().view(6, 3, 128)
+    assert qf.abs().amax(-1).eq(448).all()
+    # round trip: every element within half an e4m3 step (relative 2^-4 of its own size, or half the smallest
+    # subnormal step 2^-10, in units of the scale)
+    d = golden.dequantize_groups(q, s).float().view(6, 3, 128)
+    step = torch.maximum(xf.abs() * 2.0**-4, s[..., None] * 2.0**-10) + xf.abs() * 2.0**-8
+    assert ((d - xf).abs() <= step).all()
+    # exact cases: powers of two times the scale are representable
+    x2 = torch.zeros((1, 128)); x2[0, 0] = 448.0; x2[0, 1] = 1.0; x2[0, 2] = -0.5; x2[0, 3] = 2.0**-9
+    q2, s2 = golden.quantize_groups_e4m3(x2.to(torch.bfloat16))
+    assert s2.item() == 1.0 and q2.float()[0, :4].tolist() == [448.0, 1.0, -0.5, 2.0**-9]

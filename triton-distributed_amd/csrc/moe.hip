@@ -362,6 +362,128 @@ __global__ __launch_bounds__(256) void moe_dispatch_tokens_kernel(const unsigned
   }
 }
 
+// ---- online e4m3 quantisation in groups of 128 columns -----------------------------------------------------
+// Follows _quant_kernel of the reference's tutorials/04-deepseek-infer-all2all.py (:309-329) and its fused form in
+// the dispatch kernel (:180-200): per group, scale = max|x| (as fp32) * fp32(1/448), q = e4m3(float(x) / scale).
+// A group whose values are all zero divides 0 by 0 there and so it does here (NaN bytes, scale 0).
+constexpr int kQuantGroup = 128;
+
+// One lane's 16 consecutive bf16 columns (two 16-byte vectors) → 16 e4m3 bytes; the 8 lanes of a group share the scale.
+__device__ __forceinline__ int4v quant16_bf16_e4m3(const int4v& x0, const int4v& x1, float* scale_out) {
+  float f[16];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f[2 * j] = BF16::lo((uint32_t)x0[j]);
+    f[2 * j + 1] = BF16::hi((uint32_t)x0[j]);
+    f[8 + 2 * j] = BF16::lo((uint32_t)x1[j]);
+    f[8 + 2 * j + 1] = BF16::hi((uint32_t)x1[j]);
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(f[j]));
+  amax = fmaxf(amax, __shfl_xor(amax, 1));
+  amax = fmaxf(amax, __shfl_xor(amax, 2));
+  amax = fmaxf(amax, __shfl_xor(amax, 4));
+  const float scale = amax * (float)(1.0 / 448.0);
+  *scale_out = scale;
+  int4v q;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int w = 0;
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * j] / scale, f[4 * j + 1] / scale, w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * j + 2] / scale, f[4 * j + 3] / scale, w, true);
+    q[j] = w;
+  }
+  return q;
+}
+
+// Stand-alone quantiser: one wave per (row, window of 1024 columns).
+__global__ __launch_bounds__(256) void quant_groups_kernel(const unsigned short* __restrict__ x, int64_t n_rows, int hidden,
+                                                          int windows, unsigned char* __restrict__ q,
+                                                          float* __restrict__ scales) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
+  const int64_t r = unit / windows;
+  const int win = (int)(unit - r * windows);
+  if (r >= n_rows) return;
+  const int col = win * 1024 + lane * 16;
+  const bool active = col < hidden;
+  int4v x0 = {0, 0, 0, 0}, x1 = {0, 0, 0, 0};
+  if (active) {
+    const int4v* src = (const int4v*)(x + r * hidden + col);
+    x0 = src[0];
+    x1 = src[1];
+  }
+  float scale;
+  const int4v v = quant16_bf16_e4m3(x0, x1, &scale);
+  if (active) {
+    *(int4v*)(q + r * hidden + col) = v;
+    if ((lane & 7) == 0) scales[r * (hidden / kQuantGroup) + col / kQuantGroup] = scale;
+  }
+}
+
+// Token-major dispatch with the quantisation fused in: bf16 token rows in, e4m3 slot rows + one fp32 scale per
+// group of 128 columns out. One wave per (token, window of 1024 columns).
+__global__ __launch_bounds__(256) void moe_dispatch_quant_kernel(const unsigned short* __restrict__ tokens, int hidden,
+                                                                const int32_t* __restrict__ scatter_idx, int topk,
+                                                                const int32_t* __restrict__ cumsum, int64_t n_tokens,
+                                                                int W, int Er, int max_m,
+                                                                unsigned char* __restrict__ slot_rows,
+                                                                float* __restrict__ slot_scales,
+                                                                int32_t* __restrict__ splits_out, int windows) {
+  if (splits_out && blockIdx.x == 0) {
+    const int G = W * Er;
+    for (int g = threadIdx.x; g < G; g += 256) splits_out[g] = cumsum[g + 1] - cumsum[g];
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t unit = (int64_t)blockIdx.x * 4 + wave;
+  const int64_t t = unit / windows;
+  const int win = (int)(unit - t * windows);
+  if (t >= n_tokens) return;
+  const int col = win * 1024 + lane * 16;
+  const bool active = col < hidden;
+  int4v x0 = {0, 0, 0, 0}, x1 = {0, 0, 0, 0};
+  if (active) {
+    const int4v* src = (const int4v*)(tokens + t * hidden + col);
+    x0 = src[0];
+    x1 = src[1];
+  }
+  // lane k < topk resolves the slot row of copy k (slot boundaries one per lane, as in the unquantised dispatch)
+  int32_t my_dst = -1;
+  {
+    const int32_t p = lane < topk ? scatter_idx[t * topk + lane] : -1;
+    if (W < 64) {
+      const int32_t bound = lane <= W ? cumsum[lane * Er] : 0x7fffffff;
+      const int32_t total = __builtin_amdgcn_readlane(bound, W);
+      int d = 0;
+      int32_t first = __builtin_amdgcn_readlane(bound, 0);
+      for (int i = 1; i < W; ++i) {
+        const int32_t b = __builtin_amdgcn_readlane(bound, i);
+        if (b <= p) {
+          d = i;
+          first = b;
+        }
+      }
+      if (p >= 0 && p < total && p - first < max_m) my_dst = d * max_m + (p - first);
+    } else if (p >= 0 && p < cumsum[W * Er]) {
+      const int d = find_dest(cumsum, Er, W, p);
+      const int32_t in_slot = p - cumsum[d * Er];
+      if (in_slot < max_m) my_dst = d * max_m + in_slot;
+    }
+  }
+  float scale;
+  const int4v v = quant16_bf16_e4m3(x0, x1, &scale);
+  const int ng = hidden / kQuantGroup;
+  for (int k = 0; k < topk; ++k) {
+    const int32_t dst_row = __builtin_amdgcn_readlane(my_dst, k);
+    if (dst_row < 0) continue;
+    if (active) {
+      __builtin_nontemporal_store(v, (int4v*)(slot_rows + (int64_t)dst_row * hidden + col));
+      if ((lane & 7) == 0) slot_scales[(int64_t)dst_row * ng + col / kQuantGroup] = scale;
+    }
+  }
+}
+
 // Weighted combine: one wave per (token, window of 64 16-byte column chunks). Lane k < topk resolves the k-th
 // source row and its coefficient w[t,k] * scale[row]; the wave then reads the rows eight at a time (all loads
 // of a batch in flight before the first add) and accumulates in k order.
@@ -373,7 +495,8 @@ template <bool kFp8>
 __global__ __launch_bounds__(kCombineWaves * 64) void moe_combine_kernel(
     const unsigned char* __restrict__ slot_rows, const float* __restrict__ slot_scales,
     const int32_t* __restrict__ scatter_idx, const float* __restrict__ topk_w, const int32_t* __restrict__ cumsum,
-    int64_t n_tokens, int topk, int hidden, int W, int Er, int max_m, int n_windows, unsigned short* __restrict__ out) {
+    int64_t n_tokens, int topk, int hidden, int W, int Er, int max_m, int scale_group, int n_windows,
+    unsigned short* __restrict__ out) {
   // e4m3 rows: a lane ends up with 32 bytes of output; they go through LDS so that each store instruction of the
   // wave writes one contiguous KiB (16 bytes per lane) instead of every other 16 bytes of two
   __shared__ __attribute__((aligned(16))) unsigned char s_tr[kCombineWaves][kFp8 ? 2048 : 16];
@@ -411,7 +534,8 @@ __global__ __launch_bounds__(kCombineWaves * 64) void moe_combine_kernel(
   } else if (p >= 0) {
     row = p;
   }
-  if (row >= 0 && slot_scales) coef *= slot_scales[row];
+  // scale_group == 0: one scale per row, folded into the coefficient; else one per 128 columns, read per lane below
+  if (row >= 0 && slot_scales && scale_group == 0) coef *= slot_scales[row];
   if (row < 0) coef = 0.f;
   constexpr int kElems = kFp8 ? 16 : 8;
   const int64_t row_bytes = (int64_t)hidden * (kFp8 ? 1 : 2);
@@ -422,9 +546,12 @@ __global__ __launch_bounds__(kCombineWaves * 64) void moe_combine_kernel(
 #pragma unroll
   for (int j = 0; j < kElems; ++j) acc[j] = 0.f;
   const int row_lo = (int)(uint32_t)row, row_hi = (int)(row >> 32);
+  const bool grouped = kFp8 && slot_scales != nullptr && scale_group > 0;
+  const int ng = grouped ? hidden / scale_group : 0;
+  const int my_group = grouped ? (c * kElems) / scale_group : 0;
   for (int k0 = 0; k0 < topk; k0 += 8) {
     int4v v[8];
-    float cf[8];
+    float cf[8], gs[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int k = min(k0 + j, topk - 1);
@@ -433,11 +560,13 @@ __global__ __launch_bounds__(kCombineWaves * 64) void moe_combine_kernel(
       const bool use = (k0 + j < topk) && r >= 0;
       v[j] = (use && active) ? __builtin_nontemporal_load((const int4v*)(slot_rows + r * row_bytes) + c)
                              : int4v{0, 0, 0, 0};
+      gs[j] = (grouped && use && active) ? slot_scales[r * ng + my_group] : 1.f;
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int k = min(k0 + j, topk - 1);
       cf[j] = (k0 + j < topk) ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, coef), k)) : 0.f;
+      cf[j] *= gs[j];
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -665,7 +794,8 @@ int tdist_moe_post_process(const void* slot_rows, int64_t row_bytes, const float
 
 int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_scales, const int32_t* scatter_idx,
                       const float* topk_w, const int32_t* cumsum, int64_t n_tokens, int topk, int hidden,
-                      int world_size, int experts_per_rank, int max_m, void* out_bf16, void* stream) {
+                      int world_size, int experts_per_rank, int max_m, int scale_group_size, void* out_bf16,
+                      void* stream) {
   if (!slot_rows || !scatter_idx || !out_bf16) return fail(TDIST_ERR_INVALID, "tdist_moe_combine: null pointer");
   if (max_m > 0 && (!cumsum || world_size <= 0 || experts_per_rank <= 0))
     return fail(TDIST_ERR_INVALID, "tdist_moe_combine: slot layout needs cumsum, world_size, experts_per_rank");
@@ -673,6 +803,10 @@ int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_sc
     return fail(TDIST_ERR_INVALID, "tdist_moe_combine: bad sizes (topk <= %d)", kCombineMaxTopk);
   if (row_dtype != TDIST_F8E4M3 && row_dtype != TDIST_BF16)
     return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: row dtype %d (e4m3 and bf16 only)", row_dtype);
+  if (scale_group_size != 0 && (row_dtype != TDIST_F8E4M3 || scale_group_size < 16 || scale_group_size % 16 != 0 ||
+                                hidden % scale_group_size != 0))
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: grouped scales need e4m3 rows and a group size that is a "
+                "multiple of 16 and divides hidden");
   const int elems = row_dtype == TDIST_F8E4M3 ? 16 : 8;
   if (hidden % elems != 0 || !aligned16(slot_rows) || !aligned16(out_bf16))
     return fail(TDIST_ERR_UNSUPPORTED, "tdist_moe_combine: hidden must be a multiple of %d and buffers 16-byte aligned", elems);
@@ -685,8 +819,46 @@ int tdist_moe_combine(const void* slot_rows, int row_dtype, const float* slot_sc
   auto kern = row_dtype == TDIST_F8E4M3 ? moe_combine_kernel<true> : moe_combine_kernel<false>;
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kCombineWaves * 64), 0, (hipStream_t)stream,
                      (const unsigned char*)slot_rows, slot_scales, scatter_idx, topk_w, cumsum, n_tokens, topk, hidden,
-                     world_size, experts_per_rank, max_m, n_windows, (unsigned short*)out_bf16);
+                     world_size, experts_per_rank, max_m, scale_group_size, n_windows, (unsigned short*)out_bf16);
   return launch_status("tdist_moe_combine");
+}
+
+int tdist_quant_e4m3_groups(const void* x_bf16, int64_t n_rows, int hidden, int group_size, void* q_out,
+                            float* scales_out, void* stream) {
+  if (!x_bf16 || !q_out || !scales_out) return fail(TDIST_ERR_INVALID, "tdist_quant_e4m3_groups: null pointer");
+  if (n_rows < 0 || hidden <= 0) return fail(TDIST_ERR_INVALID, "tdist_quant_e4m3_groups: bad sizes");
+  if (group_size != kQuantGroup || hidden % kQuantGroup != 0 || !aligned16(x_bf16) || !aligned16(q_out))
+    return fail(TDIST_ERR_UNSUPPORTED, "tdist_quant_e4m3_groups: group size %d, hidden a multiple of it, 16-byte aligned buffers",
+                kQuantGroup);
+  if (n_rows == 0) return TDIST_OK;
+  const int windows = (hidden + 1023) / 1024;
+  const int64_t blocks = ceil_div(n_rows * windows, 4);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_quant_e4m3_groups: too many rows");
+  hipLaunchKernelGGL(quant_groups_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const unsigned short*)x_bf16, n_rows, hidden, windows, (unsigned char*)q_out, scales_out);
+  return launch_status("tdist_quant_e4m3_groups");
+}
+
+int tdist_moe_dispatch_tokens_quant(const void* tokens_bf16, int hidden, int group_size, const int32_t* scatter_idx,
+                                    int topk, const int32_t* cumsum, int64_t n_tokens, int world_size,
+                                    int experts_per_rank, int max_m, void* slot_rows, float* slot_scales,
+                                    int32_t* splits_out, void* stream) {
+  const char* who = "tdist_moe_dispatch_tokens_quant";
+  if (!tokens_bf16 || !scatter_idx || !cumsum || !slot_rows || !slot_scales) return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
+  if (n_tokens < 0 || hidden <= 0 || world_size <= 0 || experts_per_rank <= 0 || max_m <= 0 || topk <= 0)
+    return fail(TDIST_ERR_INVALID, "%s: bad sizes", who);
+  if (topk > 64) return fail(TDIST_ERR_UNSUPPORTED, "%s: topk > 64", who);
+  if (group_size != kQuantGroup || hidden % kQuantGroup != 0 || !aligned16(tokens_bf16) || !aligned16(slot_rows))
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: group size %d, hidden a multiple of it, 16-byte aligned buffers", who, kQuantGroup);
+  if (world_size > 8192 || (int64_t)world_size * max_m > 0x7fffffff)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: world_size * max_m too large", who);
+  const int windows = (hidden + 1023) / 1024;
+  const int64_t blocks = ceil_div((n_tokens > 0 ? n_tokens : 1) * windows, 4);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many tokens", who);
+  hipLaunchKernelGGL(moe_dispatch_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const unsigned short*)tokens_bf16, hidden, scatter_idx, topk, cumsum, n_tokens, world_size,
+                     experts_per_rank, max_m, (unsigned char*)slot_rows, slot_scales, splits_out, windows);
+  return launch_status(who);
 }
 
 int64_t tdist_moe_align_workspace_bytes(int64_t n_total, int num_experts, int num_iterations) {

@@ -45,7 +45,9 @@ PROTOTYPES = {
     "tdist_moe_dispatch": (_I, [_P, _L, _P, _P, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_dispatch_tokens": (_I, [_P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_post_process": (_I, [_P, _L, _P, _P, _L, _I, _I, _I, _P, _P, _P]),
-    "tdist_moe_combine": (_I, [_P, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P, _P]),
+    "tdist_moe_combine": (_I, [_P, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P, _P]),
+    "tdist_quant_e4m3_groups": (_I, [_P, _L, _I, _I, _P, _P, _P]),
+    "tdist_moe_dispatch_tokens_quant": (_I, [_P, _I, _I, _P, _I, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_align_workspace_bytes": (_L, [_L, _I, _I]),
     "tdist_moe_align_block_size": (_I, [_P, _I, _L, _I, _I, _L, _I, _P, _P, _P, _P, _P, _P, _L, _P]),
     "tdist_decode_split_kv": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I,

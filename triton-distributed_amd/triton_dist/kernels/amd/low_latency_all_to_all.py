@@ -34,9 +34,12 @@ class AllToAllContext:
         experts_per_rank: int,
         dtype=torch.bfloat16,
         scale_dtype=torch.float,
+        fp8_group_size: int = 0,
     ):
         """
         max_m: capacity, in rows, of one destination slot
+        fp8_group_size: 0 = one scale per row (the reference's layout, :143); 128 = one scale per group of 128
+            columns, [rows, hidden/128], the layout of the reference's tutorial 04 (its NUM_GROUPS, :138,175)
         """
         if not torch.cuda.is_available():
             raise RuntimeError("AllToAllContext needs a GPU")
@@ -48,7 +51,14 @@ class AllToAllContext:
         device = torch.device("cuda", torch.cuda.current_device())
         # double-buffered like the reference (:141-147): a call fills half call_count % 2
         self.recv_buf = torch.empty([WORLD_SIZE * max_m * 2, hidden], dtype=dtype, device=device)
-        self.scale_recv_buf = torch.empty([WORLD_SIZE * max_m * 2], dtype=scale_dtype, device=device)
+        if fp8_group_size:
+            if dtype != torch.float8_e4m3fn or hidden % fp8_group_size != 0:
+                raise ValueError("group scales need e4m3 rows and a hidden size that is a multiple of the group size")
+            self.scale_recv_buf = torch.empty([WORLD_SIZE * max_m * 2, hidden // fp8_group_size], dtype=scale_dtype,
+                                              device=device)
+        else:
+            self.scale_recv_buf = torch.empty([WORLD_SIZE * max_m * 2], dtype=scale_dtype, device=device)
+        self.fp8_group_size = fp8_group_size
         self.split_recv_buf = torch.zeros([num_tot_experts * 2], dtype=torch.int32, device=device)
         self.signal_buf = torch.zeros([WORLD_SIZE * 2], dtype=torch.int64, device=device)
 
@@ -79,8 +89,26 @@ def create_all_to_all_context(
     experts_per_rank: int,
     dtype=torch.bfloat16,
     scale_dtype=torch.float,
+    fp8_group_size: int = 0,
 ):
-    return AllToAllContext(max_m, hidden, rank, num_tot_experts, WORLD_SIZE, experts_per_rank, dtype, scale_dtype)
+    return AllToAllContext(max_m, hidden, rank, num_tot_experts, WORLD_SIZE, experts_per_rank, dtype, scale_dtype,
+                           fp8_group_size)
+
+
+def quant_bf16_fp8(tensor: torch.Tensor, gsize: int = 128):
+    """bf16 [m, N] → (e4m3 [m, N], fp32 scales [m, N // gsize]) in groups of ``gsize`` columns: scale = max|x| / 448,
+    q = e4m3(x / scale) (reference tutorials/04-deepseek-infer-all2all.py:309-360; that one returns the e4m3 bytes
+    packed two to a bf16 element)."""
+    _lib.require_cuda(tensor)
+    if tensor.dtype != torch.bfloat16:
+        raise TypeError("quant_bf16_fp8 takes bf16")
+    tensor = tensor.contiguous()
+    m, N = tensor.shape
+    out = torch.empty((m, N), dtype=torch.float8_e4m3fn, device=tensor.device)
+    out_scale = torch.empty((m, N // gsize), dtype=torch.float32, device=tensor.device)
+    _lib.call("tdist_quant_e4m3_groups", tensor.data_ptr(), m, N, gsize, out.data_ptr(), out_scale.data_ptr(),
+              _lib.stream_ptr())
+    return out, out_scale
 
 
 def splits_to_cumsum(splits: torch.Tensor):
@@ -129,6 +157,7 @@ def fast_all_to_all(
     send_scale: Optional[torch.Tensor],
     gather_index: Optional[torch.Tensor] = None,
     scatter_index: Optional[torch.Tensor] = None,
+    online_quant_fp8: bool = False,
 ):
     """
     low-latency all-to-all communication (reference :189-248).
@@ -140,10 +169,19 @@ def fast_all_to_all(
     With ``scatter_index`` (int32[T, topk], an addition) the same fusion runs token-major: every token row is
     read once and written to its topk slot rows, which is the faster form.
 
+    With ``online_quant_fp8`` (the reference's tutorial 04, ONLINE_QUANT_FP8 :180-200; needs ``scatter_index`` and a
+    context made with ``fp8_group_size=128``) ``send_tensor`` is the unsorted bf16 [T, hidden] token tensor: every
+    row is quantised to e4m3 in groups of 128 columns while it is dispatched, ``send_scale`` must be None and the
+    scales returned are [W*max_m, hidden/128].
+
     Returns [splits int32[G], recv [W*max_m, hidden], scales [W*max_m] | None] — views into the context's
     buffers, valid until the call after next.
     """
     _lib.require_cuda(send_tensor, send_split_cumsum, send_scale, gather_index, scatter_index)
+    if online_quant_fp8:
+        return _fast_all_to_all_online_quant(ctx, send_tensor, send_split_cumsum, send_scale, scatter_index)
+    if ctx.fp8_group_size:
+        raise ValueError("a context with group scales takes its rows through online_quant_fp8=True")
     with_scale = send_scale is not None
     act_pos = ctx.call_count % 2
 
@@ -185,6 +223,31 @@ def fast_all_to_all(
     out_lis = [splits, recv]
     out_lis.append(scale_recv if with_scale else None)
     return out_lis
+
+
+def _fast_all_to_all_online_quant(ctx, send_tensor, send_split_cumsum, send_scale, scatter_index):
+    if scatter_index is None or send_scale is not None:
+        raise ValueError("online_quant_fp8 takes the unsorted bf16 tokens with scatter_index and no send_scale")
+    if not ctx.fp8_group_size or ctx.dtype != torch.float8_e4m3fn:
+        raise ValueError("online_quant_fp8 needs a context created with dtype=float8_e4m3fn, fp8_group_size=128")
+    if send_tensor.dtype != torch.bfloat16:
+        raise TypeError("online_quant_fp8 quantises bf16 tokens")
+    assert send_tensor.dim() == 2 and send_tensor.shape[1] == ctx.hidden
+    assert send_split_cumsum.dtype == torch.int32 and send_split_cumsum.numel() == ctx.num_tot_experts + 1
+    assert scatter_index.dtype == torch.int32 and scatter_index.is_contiguous()
+    assert scatter_index.shape[0] == send_tensor.shape[0]
+    send_tensor = send_tensor.contiguous()
+    act_pos = ctx.call_count % 2
+    rows = ctx.WORLD_SIZE * ctx.max_m
+    recv = ctx.recv_buf[act_pos * rows:(act_pos + 1) * rows, :]
+    scale_recv = ctx.scale_recv_buf[act_pos * rows:(act_pos + 1) * rows, :]
+    splits = ctx.split_recv_buf[act_pos * ctx.num_tot_experts:(act_pos + 1) * ctx.num_tot_experts]
+    _lib.call("tdist_moe_dispatch_tokens_quant", send_tensor.data_ptr(), ctx.hidden, ctx.fp8_group_size,
+              scatter_index.data_ptr(), scatter_index.shape[1], send_split_cumsum.data_ptr(), send_tensor.shape[0],
+              ctx.WORLD_SIZE, ctx.experts_per_rank, ctx.max_m, recv.data_ptr(), scale_recv.data_ptr(), splits.data_ptr(),
+              _lib.stream_ptr())
+    ctx.call_count = (ctx.call_count + 1) % ctx.MOD_VALUE
+    return [splits, recv, scale_recv]
 
 
 def all_to_all_post_process(
@@ -236,7 +299,11 @@ def moe_weighted_combine(ctx: Optional[AllToAllContext], rows: torch.Tensor, row
         W, Er, max_m = ctx.WORLD_SIZE, ctx.experts_per_rank, ctx.max_m
     else:
         W, Er, max_m = 1, 1, 0
+    scale_group = 0
+    if row_scale is not None and row_scale.dim() == 2:   # one scale per group of columns
+        assert row_scale.is_contiguous() and hidden % row_scale.shape[1] == 0
+        scale_group = hidden // row_scale.shape[1]
     _lib.call("tdist_moe_combine", rows.data_ptr(), code, _lib.ptr(row_scale), scatter_idx.data_ptr(),
-              _lib.ptr(topk_weight), _lib.ptr(split_cumsum), T, topk, hidden, W, Er, max_m, out.data_ptr(),
+              _lib.ptr(topk_weight), _lib.ptr(split_cumsum), T, topk, hidden, W, Er, max_m, scale_group, out.data_ptr(),
               _lib.stream_ptr())
     return out
