@@ -321,6 +321,23 @@ def bench_copy(dev, steps, warmup):
     return roof("hbm", 2 * n, s, "hbm")
 
 
+def bench_mfma_ceiling(dev, steps, warmup):
+    """The MFMA rate the chip sustains with no memory traffic, on constant and on random register operands."""
+    import torch
+    from triton_dist import _lib
+    cus = _lib.load().tdist_num_cus()
+    sink = torch.empty(cus * 256, dtype=torch.float32, device=dev)
+    iters = 2000
+    out = {}
+    for name, code, per in (("bf16", _lib.TDIST_BF16, 32768.0), ("fp8", _lib.TDIST_F8E4M3, 131072.0)):
+        for rnd in (0, 1):
+            s = time_launches(lambda: _lib.call("tdist_mfma_rate_probe", code, rnd, iters, sink.data_ptr(), _lib.stream_ptr()),
+                              max(steps // 4, 5), warmup)
+            tf = cus * 4 * iters * 8 * per / s / 1e12
+            out["%s_%s_operands_TFLOPs" % (name, "random" if rnd else "constant")] = round(tf, 1)
+    return out
+
+
 def main():
     global LIVE_PRODUCER, SETTLE_SECONDS
     ap = argparse.ArgumentParser()
@@ -329,7 +346,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle-seconds", type=float, default=SETTLE_SECONDS,
                     help="untimed period of the same launches before each warm-up, to reach the sustained clock")
-    ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,copy (c2 always runs)")
+    ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,copy,mfma (c2 always runs)")
     ap.add_argument("--no-live-producer", action="store_true",
                     help="skip the AG-GEMM legs in which a copy stream releases the flags while the GEMM spins: a "
                     "counter-collecting profiler serialises dispatches, so the producer could never run beside it")
@@ -348,7 +365,7 @@ def main():
     _lib.check(_lib.load().tdist_init())
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    want = set(x for x in args.only.split(",") if x) or {"c1", "c2", "c3", "c4", "c5", "copy"}
+    want = set(x for x in args.only.split(",") if x) or {"c1", "c2", "c3", "c4", "c5", "copy", "mfma"}
 
     step_s, gemm_roof, red_roof, cpu, err = bench_c2(dev, args.steps, args.warmup)
     log("c2 step %.1f us, gemm %s, reduce %s" % (step_s * 1e6, gemm_roof, red_roof))
@@ -369,6 +386,10 @@ def main():
     if "copy" in want:
         kernels["copy_1GiB_yardstick"] = bench_copy(dev, args.steps, args.warmup)
         log("copy", kernels["copy_1GiB_yardstick"])
+
+    if "mfma" in want:
+        kernels["mfma_only_rate_yardstick"] = bench_mfma_ceiling(dev, args.steps, args.warmup)
+        log("mfma", kernels["mfma_only_rate_yardstick"])
 
     flops = 2.0 * 8192 * 8192 * 3584
     line = {

@@ -293,6 +293,14 @@ int tdist_decode_combine(const void* part, int part_dtype, const float* lse, int
  * ------------------------------------------------------------------------------------------- */
 int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
 
+/* Measurement helper: the MFMA rate this chip sustains with no memory traffic at all. One workgroup of four waves per
+ * compute unit runs iters (a multiple of 4) rounds of eight independent 32x32 MFMAs (bf16: 32x32x16, 32 768 FLOP each;
+ * e4m3: 32x32x64, 131 072 FLOP each) on register operands that change from one MFMA to the next; random_operands != 0
+ * fills them with random bit patterns, else with 1.0. FLOP per launch = tdist_num_cus() * 4 * iters * 8 * FLOP per MFMA.
+ * sink: tdist_num_cus() * 256 floats. With random operands the chip is power-limited well below its nominal rate: this
+ * is the ceiling any GEMM on random data sits under. Not on the hot path. */
+int tdist_mfma_rate_probe(int dtype, int random_operands, int iters, float* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -75,3 +75,21 @@ def test_copy_bytes_helper(cuda):
     _lib.call("tdist_copy_bytes", dst.data_ptr(), src.data_ptr(), src.numel(), _lib.stream_ptr())
     torch.cuda.synchronize()
     assert torch.equal(src, dst)
+
+
+def test_mfma_rate_probe_runs(cuda):
+    from triton_dist import _lib
+    announce("mfma rate probe")
+    cus = _lib.load().tdist_num_cus()
+    sink = torch.full((cus * 256, ), float("nan"), dtype=torch.float32, device=cuda)
+    for code in (_lib.TDIST_BF16, _lib.TDIST_F8E4M3):
+        for rnd in (0, 1):
+            _lib.call("tdist_mfma_rate_probe", code, rnd, 8, sink.data_ptr(), _lib.stream_ptr())
+            torch.cuda.synchronize()
+            assert torch.isfinite(sink).all()
+    # constant operands: 1.0 x 1.0 summed over K (16 per bf16 MFMA), 8 rounds of the lane's first accumulator
+    _lib.call("tdist_mfma_rate_probe", _lib.TDIST_BF16, 0, 8, sink.data_ptr(), _lib.stream_ptr())
+    torch.cuda.synchronize()
+    assert torch.all(sink == 8 * 8 * 16.0)
+    with pytest.raises(_lib.TdistError):
+        _lib.call("tdist_mfma_rate_probe", _lib.TDIST_BF16, 0, 7, sink.data_ptr(), _lib.stream_ptr())

@@ -62,6 +62,62 @@ __global__ __launch_bounds__(256) void copy_bytes_kernel(int4v* __restrict__ dst
   }
 }
 
+// MFMA-only loop for the rate yardstick: no memory traffic at all, eight independent accumulators, and operand
+// fragments that change from one MFMA to the next (eight A and eight B fragments in registers, paired differently
+// every time). kRandom fills them with hashed bit patterns (random sign, mantissa and low exponent bits), else with 1.0.
+__device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7feb352dU;
+  x ^= x >> 15;
+  x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return x;
+}
+
+template <bool kFp8, bool kRandom>
+__global__ __launch_bounds__(256, 1) void mfma_rate_kernel(float* __restrict__ sink, int iters) {
+  typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
+  typedef int int8v_ __attribute__((ext_vector_type(8)));
+  int8v_ a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t h1 = probe_hash(threadIdx.x * 131u + i * 17u + e), h2 = probe_hash(threadIdx.x * 71u + i * 29u + e + 1000u);
+      if (kFp8) {  // e4m3 bytes: random sign, exponent 4..7, random mantissa
+        a[i][e] = kRandom ? (int)((h1 & 0x9f9f9f9fu) | 0x20202020u) : 0x38383838;
+        b[i][e] = kRandom ? (int)((h2 & 0x9f9f9f9fu) | 0x20202020u) : 0x38383838;
+      } else {     // bf16 pairs: random sign, exponent 124..127, random mantissa
+        a[i][e] = kRandom ? (int)((h1 & 0x81ff81ffu) | 0x3e003e00u) : 0x3f803f80;
+        b[i][e] = kRandom ? (int)((h2 & 0x81ff81ffu) | 0x3e003e00u) : 0x3f803f80;
+      }
+    }
+  float16v acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+  for (int it = 0; it < iters; it += 4) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int8v_ av = a[(i + u) & 7], bv = b[(i * 3 + u) & 7];
+        if (kFp8) {
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i], 0, 0, 0, 0, 0, 0);
+        } else {
+          const int4v a4 = __builtin_shufflevector(av, av, 0, 1, 2, 3), b4 = __builtin_shufflevector(bv, bv, 0, 1, 2, 3);
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8v, a4), __builtin_bit_cast(bf16x8v, b4),
+                                                           acc[i], 0, 0, 0);
+        }
+      }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s += acc[i][0];
+  sink[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
 }  // namespace tdist
 
 using namespace tdist;
@@ -122,6 +178,23 @@ int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
   hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (int4v*)dst,
                      (const int4v*)src, n16);
   return launch_status("tdist_copy_bytes");
+}
+
+int tdist_mfma_rate_probe(int dtype, int random_operands, int iters, float* sink, void* stream) {
+  if (!sink || iters <= 0 || iters % 4 != 0) return fail(TDIST_ERR_INVALID, "tdist_mfma_rate_probe: sink, iters (multiple of 4)");
+  if (dtype != TDIST_BF16 && dtype != TDIST_F8E4M3) return fail(TDIST_ERR_UNSUPPORTED, "tdist_mfma_rate_probe: bf16 or e4m3");
+  const DeviceInfo& di = device_info();
+  if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "tdist_mfma_rate_probe: current device is not gfx950");
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(di.num_cus), block(256);
+  if (dtype == TDIST_BF16) {
+    if (random_operands) hipLaunchKernelGGL((mfma_rate_kernel<false, true>), grid, block, 0, st, sink, iters);
+    else hipLaunchKernelGGL((mfma_rate_kernel<false, false>), grid, block, 0, st, sink, iters);
+  } else {
+    if (random_operands) hipLaunchKernelGGL((mfma_rate_kernel<true, true>), grid, block, 0, st, sink, iters);
+    else hipLaunchKernelGGL((mfma_rate_kernel<true, false>), grid, block, 0, st, sink, iters);
+  }
+  return launch_status("tdist_mfma_rate_probe");
 }
 
 }  // extern "C"

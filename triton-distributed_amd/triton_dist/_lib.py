@@ -54,6 +54,7 @@ PROTOTYPES = {
                                    _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
     "tdist_decode_combine": (_I, [_P, _I, _P, _I, _I, _P, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P, _I, _L, _L, _P, _P]),
     "tdist_copy_bytes": (_I, [_P, _P, _L, _P]),
+    "tdist_mfma_rate_probe": (_I, [_I, _I, _I, _P, _P]),
 }
 
 
