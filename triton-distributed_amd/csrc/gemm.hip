@@ -665,12 +665,13 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) big = false;
   if (c.A_local && (c.local_row_begin % 256 != 0 || c.local_rows % 256 != 0)) big = false;
   if (((int64_t)c.K * esz) % 128 != 0) big = false;  // the large tiles step through K 128 bytes at a time
-  // TDIST_GEMM_VARIANT picks another compiled tiling for the large-tile path (measurement aid); the default,
-  // 6, is 256x256 tiles, 128-byte K rows, 2x2 waves of 128x128, split ring (3 A stages + 2 B stages).
+  // TDIST_GEMM_VARIANT picks another compiled schedule of the large-tile path (measurement aid): 2 = 2x4 waves on a
+  // two-stage ring, 5 = 2x4 waves on the split ring. The default is 2x2 waves of 128x128 on the split ring
+  // (3 A stages + 2 B stages).
   int variant = 6;
   if (const char* v = getenv("TDIST_GEMM_VARIANT")) variant = atoi(v);
   const int BM = big ? 256 : 128;
-  const int BN = big ? (variant == 4 ? 128 : 256) : 128;
+  const int BN = big ? 256 : 128;
 
   GemmParams p;
   p.A = (const unsigned char*)c.A;
@@ -753,10 +754,6 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
                     : launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);        \
   }
     switch (variant) {
-      case 0: TDIST_BIG(256, 64, 2, 2, 4)
-      case 1: TDIST_BIG(256, 128, 2, 2, 2)
-      case 3: TDIST_BIG(256, 64, 2, 4, 4)
-      case 4: TDIST_BIG(128, 128, 2, 2, 3)
       case 2: TDIST_BIG(256, 128, 2, 4, 2)
       case 5: TDIST_BIG(256, 128, 2, 4, 5)
       default: TDIST_BIG(256, 128, 2, 2, 5)
