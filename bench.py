@@ -95,6 +95,14 @@ def time_live_ag_gemm(call, ctx, steps, warmup):
         return s, "copies_first"
 
 
+def cpu_time(fn):
+    """Wall time of one call of ``fn`` on the host cores (torch's thread pool at its default width)."""
+    import torch
+    t0 = time.perf_counter()
+    fn()
+    return time.perf_counter() - t0, torch.get_num_threads()
+
+
 def roof(bound, work, seconds, peak_key, traffic=None):
     achieved = work / seconds
     unit = "TFLOP/s" if bound == "mfma" else "GB/s"
@@ -194,6 +202,9 @@ def bench_c1(dev, steps, warmup):
     out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 1024, rank, world), steps, warmup)
     r = roof("mfma", flops, pre_s, "bf16", MEASURED_TRAFFIC_BYTES["c1_gemm"])
+    cs, cores = cpu_time(lambda: golden.torch_ag_gemm(shards, b))
+    r["cpu_baseline"] = {"value": round(flops / cs / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                         "sample": "the whole config once (torch golden: cat + matmul), %.2f s" % cs}
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
     r["live_producer_order"] = live_order
     return r
@@ -230,6 +241,10 @@ def bench_c3(dev, steps, warmup):
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 2048, rank, world, row_scale=sa, col_scale=sb),
                           steps, warmup)
     r = roof("mfma", flops, pre_s, "fp8", MEASURED_TRAFFIC_BYTES["c3_gemm"])
+    sa_c, sb_c = sa.cpu(), sb.cpu()
+    cs, cores = cpu_time(lambda: golden.fp8_scaled_gemm_fp32(shards[0][:1024], sa_c[:1024], b, sb_c))
+    r["cpu_baseline"] = {"value": round(flops / 16 / cs / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                         "sample": "1024 of the 16384 rows (fp32 up-cast golden with scales), %.2f s" % cs}
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
     r["live_producer_order"] = live_order
     return r
@@ -256,6 +271,14 @@ def bench_c4(dev, steps, warmup):
     disp_bytes = T * H + n * H + T * 4 + n * 4 + n * 4          # unique row reads + row writes + scales + gather index
     comb_bytes = n * H + n * 4 + n * 4 + n * 4 + T * H * 2      # row reads + scales + weights + scatter index + bf16 out
     d = roof("hbm", disp_bytes, disp_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_dispatch"])
+
+    def cpu_dispatch():
+        _, c_cumsum, _, c_gather, _ = golden.moe_preprocess(ids, G)
+        rows = q.view(torch.uint8)[c_gather.long()]
+        golden.dispatch_slots(rows, s[c_gather.long()], c_cumsum, W, G // W, max_m)
+    cs, cores = cpu_time(cpu_dispatch)
+    d["cpu_baseline"] = {"value": round(disp_bytes / cs / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                         "sample": "the whole config once (bincount, stable argsort, index_select, slot copies), %.2f s" % cs}
     d["index_build_us"] = round(pre_s * 1e6, 2)
     # the step after the dispatch: align / sort of the same ids for the grouped GEMM (8 rank segments, block 128)
     from triton_dist.kernels.amd import sort_topk_ids_align_block_size
@@ -270,7 +293,13 @@ def bench_c4(dev, steps, warmup):
     qd_bytes = T * H * 2 + n * H + n * (H // 128) * 4 + n * 4
     d["online_quant_dispatch"] = {"us_per_launch": round(qd_s * 1e6, 2), "achieved_GBps": round(qd_bytes / qd_s / 1e9, 1),
                                   "frac": round(qd_bytes / qd_s / PEAK["hbm"], 4)}
-    return d, roof("hbm", comb_bytes, comb_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_combine"])
+    c = roof("hbm", comb_bytes, comb_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_combine"])
+    _, _, c_scatter, c_gather, _ = golden.moe_preprocess(ids, G)
+    rows_f32 = q[c_gather.long()].float()
+    cs, cores = cpu_time(lambda: golden.weighted_combine(rows_f32, s[c_gather.long()], c_scatter, w.cpu()))
+    c["cpu_baseline"] = {"value": round(comb_bytes / cs / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                         "sample": "the whole config once (scale, gather by scatter index, weighted sum over k), %.2f s" % cs}
+    return d, c
 
 
 def bench_c5(dev, steps, warmup):
@@ -306,6 +335,13 @@ def bench_c5(dev, steps, warmup):
     kv_bytes = 2 * B * L * Hkv * D * 2
     split_bytes = kv_bytes + q.numel() * 2 + table.numel() * 4 + out_split.numel() * 4 + lse_split.numel() * 4
     r = roof("hbm", split_bytes, split_s, "hbm", MEASURED_TRAFFIC_BYTES["c5_split_kv"])
+    from oracle import golden
+    pages1 = table[0].long()
+    k1, v1, q1 = k[pages1].cpu(), v[pages1].cpu(), q[:1].cpu()
+    t1 = torch.arange(pages_per_seq, dtype=torch.int32).view(1, -1)
+    cs, cores = cpu_time(lambda: golden.ref_paged_attn(q1, k1, v1, [1], [L], t1, scale))
+    r["cpu_baseline"] = {"value": round(split_bytes / B / cs / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                         "sample": "one of the 32 sequences (torch golden ref_paged_attn, 32768 keys), %.2f s" % cs}
     r["combine_us"] = round(comb_s * 1e6, 2)
     r["inter_rank_combine_us"] = round(rank_s * 1e6, 2)
     return r
