@@ -12,6 +12,10 @@ namespace tdist {
 
 constexpr int kReduceThreads = 256;
 constexpr int kReduceUnroll = 2;
+#ifndef TDIST_REDUCE_RESIDENT
+#define TDIST_REDUCE_RESIDENT 6
+#endif
+constexpr int kReduceResident = TDIST_REDUCE_RESIDENT;
 
 template <typename T>
 __device__ __forceinline__ void accumulate8(float* acc, const int4v& v) {
@@ -27,7 +31,8 @@ template <typename T, int R>
 __global__ __launch_bounds__(kReduceThreads) void reduce_slices_fixed_kernel(const int4v* __restrict__ c,
                                                                               int64_t stride16, int first,
                                                                               int64_t n16, int4v* __restrict__ out) {
-  const int64_t base = (int64_t)blockIdx.x * (kReduceThreads * kReduceUnroll) + threadIdx.x;
+  for (int64_t blk = blockIdx.x; blk * (kReduceThreads * kReduceUnroll) < n16; blk += gridDim.x) {
+  const int64_t base = blk * (kReduceThreads * kReduceUnroll) + threadIdx.x;
   int4v v[kReduceUnroll][R];
 #pragma unroll
   for (int u = 0; u < kReduceUnroll; ++u) {
@@ -53,6 +58,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_slices_fixed_kernel(con
       for (int j = 0; j < 4; ++j) o[j] = (int)T::pack(acc[2 * j], acc[2 * j + 1]);
       __builtin_nontemporal_store(o, out + e);
     }
+  }
   }
 }
 
@@ -80,10 +86,15 @@ static int launch_reduce(const void* c, int64_t slice_stride, int n_slices, int 
   const int64_t n16 = n_elems / 8;
   const int64_t per_block = kReduceThreads * kReduceUnroll;
   const int64_t blocks = ceil_div(n16, per_block);
+  // at most six workgroups per compute unit (what the kernel's registers allow to be resident), each looping over
+  // its share, so that the last round is not a third-full one
+  const DeviceInfo& di = device_info();
+  const int64_t resident = (int64_t)(di.ok == 1 ? di.num_cus : 256) * kReduceResident;
+  const int64_t grid = blocks < resident ? blocks : resident;
   if (vec_ok && blocks <= 0x7fffffff) {
 #define TDIST_REDUCE_CASE(R)                                                                                   \
   case R:                                                                                                      \
-    hipLaunchKernelGGL((reduce_slices_fixed_kernel<T, R>), dim3((unsigned)blocks), dim3(kReduceThreads), 0,    \
+    hipLaunchKernelGGL((reduce_slices_fixed_kernel<T, R>), dim3((unsigned)grid), dim3(kReduceThreads), 0,      \
                        stream, (const int4v*)c, slice_stride / 8, first_slice, n16, (int4v*)out);              \
     return launch_status("tdist_reduce_slices");
     switch (n_slices) {
