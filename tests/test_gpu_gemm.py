@@ -365,3 +365,41 @@ def test_randomised_shapes_gating_and_layouts(cuda):
         torch.cuda.synchronize()
         ref = (a[:, :K].to(cuda) @ b[:, :K].to(cuda).T).to(out_dtype)
         assert torch.equal(c, ref), "case %d differs" % case
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
+def test_each_tile_configuration_forced(cuda, monkeypatch, tile, dtype):
+    """Every compiled tile (256x256, 256x128, 128x128) forced through the library's measurement switch on the same
+    ragged, padded, gated and scaled cases; integer-valued inputs, so only the final rounding remains."""
+    from triton_dist.kernels.amd import gated_gemm
+    monkeypatch.setenv("TDIST_GEMM_TILE", str(tile))
+    esz = 1 if dtype == torch.float8_e4m3fn else 2
+    out_dtype = torch.float16 if dtype == torch.float16 else torch.bfloat16
+    for case, (M, N, K, pad, gated) in enumerate([(1030, 1290, 256 // esz, 16, False), (2048, 1536, 640 // esz, 0, True),
+                                                   (512, 200, 128 // esz, 64, True), (300, 2100, 1152 // esz, 0, False)]):
+        announce("gemm forced tile %d %s M=%d N=%d K=%d gated=%s" % (tile, dtype, M, N, K, gated))
+        g = torch.Generator().manual_seed(100 * tile + case)
+        a = torch.randint(-2, 3, (M, K + pad), generator=g).float()
+        b = torch.randint(-2, 3, (N, K + pad), generator=g).float()
+        a_d, b_d = a.to(dtype).to(cuda)[:, :K], b.to(dtype).to(cuda)[:, :K]
+        c = torch.full((M, N), float("nan"), dtype=out_dtype, device=cuda)
+        sa = sb = None
+        if dtype == torch.float8_e4m3fn and case % 2 == 1:   # power-of-two scales keep the result exact
+            sa = (2.0 ** torch.randint(-3, 3, (M,), generator=g).float()).to(cuda)
+            sb = (2.0 ** torch.randint(-3, 3, (N,), generator=g).float()).to(cuda)
+        if gated:
+            world, rank = 2, 1
+            mpr = M // world
+            local = a_d[rank * mpr:(rank + 1) * mpr].contiguous()
+            ws = a_d.clone()
+            ws[rank * mpr:(rank + 1) * mpr] = 0
+            flags = torch.ones(world, dtype=torch.int32, device=cuda)
+            gated_gemm(ws, local, rank * mpr, b_d, c, flags, mpr, rank, world, row_scale=sa, col_scale=sb)
+        else:
+            gated_gemm(a_d, None, 0, b_d, c, None, 0, 0, 1, row_scale=sa, col_scale=sb)
+        torch.cuda.synchronize()
+        ref = a[:, :K].to(cuda) @ b[:, :K].to(cuda).T
+        if sa is not None:
+            ref = ref * sa[:, None] * sb[None, :]
+        assert torch.equal(c, ref.to(out_dtype)), "tile %d case %d differs" % (tile, case)

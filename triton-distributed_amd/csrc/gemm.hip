@@ -156,8 +156,7 @@ struct GemmCfg {
   static_assert(KB == 64 || KB == 128, "tile rows of 64 or 128 bytes");
   static_assert(BM % (kRowsPerInstr * kWaves) == 0 && BN % (kRowsPerInstr * kWaves) == 0, "tile/wave split");
   static_assert(kSplit || (kP >= 1 && kP <= 3 && kP * kLoadsPerTile < 64), "vmcnt budget");
-  static_assert(!kSplit || (kTM + kTN <= kTM * kTN - kLeadMfma && kLoadsPerTile % kKSteps == 0 &&
-                            kBInstr % kDmaPerStep == 0),
+  static_assert(!kSplit || (kTM + kTN <= kTM * kTN - kLeadMfma && kLoadsPerTile % kKSteps == 0),
                 "split ring: one fragment read per MFMA slot, whole DMA groups per K step");
   static_assert(kEpiBytes * kWaves <= kLdsBytes, "epilogue staging must fit in the stage ring");
   static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "wave tile");
@@ -657,21 +656,41 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   const DeviceInfo& di = device_info();
   if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "%s: current device is not gfx950", who);
 
-  // tile configuration: 256x256 when that fills the chip at least ~1.5 times and the row-block
-  // constraints of the call allow it, else 128x128
-  const int64_t big_tiles = ceil_div(c.M, 256) * ceil_div(c.N, 256);
-  bool big = big_tiles >= (int64_t)di.num_cus * 3 / 2;
-  if (c.scatter_bufs && c.world_size > 0 && (c.M % c.world_size != 0 || (c.M / c.world_size) % 256 != 0)) big = false;
-  if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) big = false;
-  if (c.A_local && (c.local_row_begin % 256 != 0 || c.local_rows % 256 != 0)) big = false;
-  if (((int64_t)c.K * esz) % 128 != 0) big = false;  // the large tiles step through K 128 bytes at a time
-  // TDIST_GEMM_VARIANT picks another compiled schedule of the large-tile path (measurement aid): 2 = 2x4 waves on a
+  // Tile configuration. The 256-row tiles (256x256 and 256x128, both on the split ring) need the call's row blocks
+  // (chunks, rank slices, the local shard) to be multiples of 256 rows and K to be a multiple of 128 bytes; the
+  // 128x128 tile takes everything else. Among the admissible ones the cheapest estimate wins: rounds of the grid
+  // times the tile's work over its measured relative efficiency.
+  bool rows256 = true;
+  if (c.scatter_bufs && c.world_size > 0 && (c.M % c.world_size != 0 || (c.M / c.world_size) % 256 != 0)) rows256 = false;
+  if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) rows256 = false;
+  if (c.A_local && (c.local_row_begin % 256 != 0 || c.local_rows % 256 != 0)) rows256 = false;
+  if (((int64_t)c.K * esz) % 128 != 0) rows256 = false;  // the split ring steps through K 128 bytes at a time
+  int cap_wgs = di.num_cus;
+  if (c.max_workgroups > 0 && c.max_workgroups < cap_wgs) cap_wgs = c.max_workgroups;
+  struct TileChoice { int bm, bn; double eff; };
+  static const TileChoice kChoices[3] = {{256, 256, 1.0}, {256, 128, 0.9}, {128, 128, 0.6}};
+  int pick = 2;
+  double best = 0;
+  for (int t = 0; t < 3; ++t) {
+    if (kChoices[t].bm == 256 && !rows256) continue;
+    const int64_t tiles = ceil_div(c.M, kChoices[t].bm) * ceil_div(c.N, kChoices[t].bn);
+    const double cost = (double)ceil_div(tiles, cap_wgs) * kChoices[t].bm * kChoices[t].bn / kChoices[t].eff;
+    if (best == 0 || cost < best) best = cost, pick = t;
+  }
+  // TDIST_GEMM_TILE forces a tile (measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128; a 256-row tile that the
+  // call's row blocks do not admit is not taken.
+  if (const char* v = getenv("TDIST_GEMM_TILE")) {
+    const int t = atoi(v);
+    if (t >= 0 && t < 3 && (kChoices[t].bm != 256 || rows256)) pick = t;
+  }
+  // TDIST_GEMM_VARIANT picks another compiled schedule of the 256x256 tile (measurement aid): 2 = 2x4 waves on a
   // two-stage ring, 5 = 2x4 waves on the split ring. The default is 2x2 waves of 128x128 on the split ring
   // (3 A stages + 2 B stages).
   int variant = 6;
   if (const char* v = getenv("TDIST_GEMM_VARIANT")) variant = atoi(v);
-  const int BM = big ? 256 : 128;
-  const int BN = big ? 256 : 128;
+  const int BM = kChoices[pick].bm;
+  const int BN = kChoices[pick].bn;
+  const bool big = pick == 0;
 
   GemmParams p;
   p.A = (const unsigned char*)c.A;
@@ -739,9 +758,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   }
   const int64_t sched = (int64_t)p.n_chunks * (p.m_per_chunk / BM) * ceil_div(c.N, BN);
   if (sched > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many tiles", who);
-  int max_wgs = di.num_cus;
-  if (c.max_workgroups > 0 && c.max_workgroups < max_wgs) max_wgs = c.max_workgroups;
-  const int grid = (int)(sched < max_wgs ? sched : max_wgs);
+  const int grid = (int)(sched < cap_wgs ? sched : cap_wgs);
   const bool scales = elem == kElemFP8 && (c.row_scale || c.col_scale);
 
   if (big) {
@@ -758,8 +775,9 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       case 5: TDIST_BIG(256, 128, 2, 4, 5)
       default: TDIST_BIG(256, 128, 2, 2, 5)
     }
-#undef TDIST_BIG
   }
+  if (pick == 1) { TDIST_BIG(128, 128, 2, 2, 5) }
+#undef TDIST_BIG
   switch (elem) {
     case kElemBF16: return launch_gemm_cfg<ElemBF16, 128, 128, 64, 2, 2, 4, false>(p, grid, c.stream, who);
     case kElemF16: return launch_gemm_cfg<ElemF16, 128, 128, 64, 2, 2, 4, false>(p, grid, c.stream, who);
