@@ -304,7 +304,7 @@ def bench_c4(dev, steps, warmup):
 
 def bench_c5(dev, steps, warmup):
     import torch
-    from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine
+    from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine, decode_fused
     B, Hq, Hkv, D, L, S, page = 32, 64, 8, 128, 32768, 16, 16
     g = torch.Generator(device="cuda").manual_seed(3 + 4)
     pages_per_seq = L // page
@@ -323,6 +323,20 @@ def bench_c5(dev, steps, warmup):
         lambda: decode_combine(out_split, lse_split, S, 1, lens, B, Hq, D,
                                (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
                                (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), merged), steps, warmup)
+
+    def two_launches():
+        _split_kv(q, k, v, lens, table, scale, 0.0, S, out_split, lse_split)
+        decode_combine(out_split, lse_split, S, 1, lens, B, Hq, D,
+                       (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
+                       (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), merged)
+
+    both_s = time_launches(two_launches, steps, warmup)
+    # the same in one launch: the last workgroup of a (sequence, head block) merges its splits
+    fused_out = torch.empty_like(merged)
+    fused_s = time_launches(lambda: decode_fused(q, k, v, lens, table, scale, 0.0, S, fused_out, None,
+                                                 out_split=out_split, lse_split=lse_split), steps, warmup)
+    if not torch.equal(fused_out.view(torch.int16), merged.view(torch.int16)):
+        raise RuntimeError("fused decode differs from split + combine")
     # the rank merge of BASELINE config 5: own (out, LSE) + 7 seeded synthetic peer shards -> [32, 64, 128] bf16
     from triton_dist.kernels.amd import gqa_fwd_batch_decode_inter_rank_combine
     g2 = torch.Generator(device="cuda").manual_seed(3 + 4 + 100)
@@ -343,6 +357,8 @@ def bench_c5(dev, steps, warmup):
     r["cpu_baseline"] = {"value": round(split_bytes / B / cs / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
                          "sample": "one of the 32 sequences (torch golden ref_paged_attn, 32768 keys), %.2f s" % cs}
     r["combine_us"] = round(comb_s * 1e6, 2)
+    r["split_then_combine_us"] = round(both_s * 1e6, 2)
+    r["fused_split_and_combine_us"] = round(fused_s * 1e6, 2)
     r["inter_rank_combine_us"] = round(rank_s * 1e6, 2)
     return r
 

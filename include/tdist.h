@@ -251,24 +251,46 @@ int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_to
  *   replaces kernel_gqa_fwd_batch_decode_split_kv               kernels/nvidia/flash_decode.py:129-239
  *            kernel_intra_rank_gqa_fwd_batch_decode_combine_kv  kernels/nvidia/flash_decode.py:392-449
  *            kernel_inter_rank_gqa_fwd_batch_decode_combine_kv  kernels/nvidia/flash_decode.py:481-532
+ *            kernel_gqa_fwd_batch_decode_split_kv_persistent    kernels/nvidia/flash_decode.py:586-760
  * ------------------------------------------------------------------------------------------- */
 /* One query token per sequence. For split s of sequence b (keys [s*per, min((s+1)*per, len)),
  * per = ceil(len/num_splits), flash_decode.py:193-195) and every query head h:
  *   out_split[b,h,s,:] = softmax(q.k*sm_scale [soft-capped]) . v   over the split's keys (fp32)
  *   lse_split[b,h,s]   = log(sum exp(scores))  (natural log, fp32; -inf for an empty split)
- * q [B,Hq,D] (strides q_stride_b, q_stride_h, last dim contiguous); k_cache / v_cache
- * [num_pages, page_size, Hkv, D] with element strides kv_stride_page (between pages),
- * kv_stride_token, kv_stride_head; block_table int32 [B, table_stride]; kv_lens int32 [B].
+ * q [B,Hq,D] (strides q_stride_b, q_stride_h, last dim contiguous); k_cache [num_pages, page_size, Hkv, D] and
+ * v_cache [num_pages, page_size, Hkv, Dv] with element strides k_/v_stride_page (between pages), _token, _head;
+ * block_table int32 [B, table_stride]; kv_lens int32 [B].
  * out_split fp32 [B,Hq,S,Dv] contiguous; lse_split fp32 [B,Hq,S] contiguous.
  * The reference keeps LSE in-band in the q dtype (column Dv of its [.., Dv+1] buffer, :235-239);
- * here it is a separate fp32 tensor. Supported: D == Dv in {64,128,256}, dtype bf16 / f16. */
+ * here it is a separate fp32 tensor. Supported (head_dim, head_dim_v): (64,64), (128,128), (256,256) and the
+ * heads with extra key dimensions (BLOCK_DPE = D - 2^floor(log2 D), flash_decode.py:771-772): (192,128), (576,512);
+ * dtype bf16 / f16. */
 int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cache, float* out_split,
                           float* lse_split, float sm_scale, float soft_cap, const int32_t* block_table,
                           const int32_t* kv_lens, int batch, int q_heads, int kv_heads, int head_dim,
-                          int page_size, int num_splits, int64_t q_stride_b, int64_t q_stride_h,
+                          int head_dim_v, int page_size, int num_splits, int64_t q_stride_b, int64_t q_stride_h,
                           int64_t k_stride_page, int64_t k_stride_token, int64_t k_stride_head,
                           int64_t v_stride_page, int64_t v_stride_token, int64_t v_stride_head,
                           int64_t table_stride, int dtype, void* stream);
+
+/* Split-KV decode and the merge of the splits in ONE launch.
+ *   replaces kernel_gqa_fwd_batch_decode_split_kv_persistent + barrier_on_this_grid
+ *            kernels/nvidia/flash_decode.py:586-760, kernels/nvidia/common_ops.py:62-85
+ * Same arguments and partial outputs as tdist_decode_split_kv, plus the merged result of
+ * tdist_decode_combine(mode 1): out [B,Hq,Dv] of out_dtype (strides out_stride_b, out_stride_h) and lse_out fp32
+ * [B,Hq] or NULL, bit-identical to the two-launch path. Instead of the reference's grid-wide barrier, the last
+ * workgroup to finish a (sequence, block of 16 query heads) merges its S partials, so no workgroup waits.
+ * counters: int32 [n_counters >= tdist_decode_fused_counters(batch, q_heads, kv_heads)], ALL ZERO on entry; the
+ * kernel leaves them zero again, so one zero-initialised buffer serves every later call (calls that share it
+ * must not overlap). out_split / lse_split are still written (they are the exchange buffer of the merge). */
+int64_t tdist_decode_fused_counters(int batch, int q_heads, int kv_heads);
+int tdist_decode_fused(const void* q, const void* k_cache, const void* v_cache, float* out_split, float* lse_split,
+                       float sm_scale, float soft_cap, const int32_t* block_table, const int32_t* kv_lens, int batch,
+                       int q_heads, int kv_heads, int head_dim, int head_dim_v, int page_size, int num_splits,
+                       int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_token,
+                       int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_token, int64_t v_stride_head,
+                       int64_t table_stride, int dtype, int32_t* counters, int64_t n_counters, void* out,
+                       int out_dtype, int64_t out_stride_b, int64_t out_stride_h, float* lse_out, void* stream);
 
 /* LSE-weighted merge of P partial results per (b,h) — used for the splits of one shard and for the
  * shards of several ranks:

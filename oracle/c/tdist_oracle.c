@@ -155,14 +155,14 @@ void oc_combine_e4m3(const uint8_t* sorted_rows, const float* sorted_scales, con
  * q [B,Hq,D]; caches [pages, page_size, Hkv, D] (float copies of the 16-bit data); table [B, table_stride]. */
 void oc_decode_range(const float* q, const float* k_cache, const float* v_cache, const int32_t* table,
                      int64_t table_stride, const int32_t* lo, const int32_t* hi, int B, int Hq, int Hkv, int D,
-                     int page_size, double scale, double soft_cap, double* out, double* lse) {
+                     int Dv, int page_size, double scale, double soft_cap, double* out, double* lse) {
   int group = Hq / Hkv;
   for (int b = 0; b < B; ++b)
     for (int h = 0; h < Hq; ++h) {
       int kvh = h / group;
       int n0 = lo[b], n1 = hi[b];
-      double* o = out + ((int64_t)b * Hq + h) * D;
-      for (int d = 0; d < D; ++d) o[d] = 0.0;
+      double* o = out + ((int64_t)b * Hq + h) * Dv;
+      for (int d = 0; d < Dv; ++d) o[d] = 0.0;
       if (n1 <= n0) {
         lse[(int64_t)b * Hq + h] = -INFINITY;
         continue;
@@ -183,9 +183,9 @@ void oc_decode_range(const float* q, const float* k_cache, const float* v_cache,
       for (int n = n0; n < n1; ++n) denom += exp(s[n - n0] - mx);
       for (int n = n0; n < n1; ++n) {
         int64_t page = table[(int64_t)b * table_stride + n / page_size];
-        const float* vr = v_cache + ((page * page_size + n % page_size) * Hkv + kvh) * D;
+        const float* vr = v_cache + ((page * page_size + n % page_size) * Hkv + kvh) * Dv;
         double p = exp(s[n - n0] - mx) / denom;
-        for (int d = 0; d < D; ++d) o[d] += p * (double)vr[d];
+        for (int d = 0; d < Dv; ++d) o[d] += p * (double)vr[d];
       }
       lse[(int64_t)b * Hq + h] = mx + log(denom);
       free(s);

@@ -132,9 +132,10 @@ def decode_range(q_f32, k_cache_f32, v_cache_f32, table_i32, lo, hi, scale, soft
     lo, hi = _c(lo, np.int32), _c(hi, np.int32)
     B, Hq, D = q.shape
     _, page_size, Hkv, _ = k.shape
-    out = np.empty((B, Hq, D), dtype=np.float64)
+    Dv = v.shape[-1]
+    out = np.empty((B, Hq, Dv), dtype=np.float64)
     lse = np.empty((B, Hq), dtype=np.float64)
     load().oc_decode_range(_p(q), _p(k), _p(v), _p(tb), ctypes.c_int64(tb.shape[1]), _p(lo), _p(hi), ctypes.c_int(B),
-                           ctypes.c_int(Hq), ctypes.c_int(Hkv), ctypes.c_int(D), ctypes.c_int(page_size),
+                           ctypes.c_int(Hq), ctypes.c_int(Hkv), ctypes.c_int(D), ctypes.c_int(Dv), ctypes.c_int(page_size),
                            ctypes.c_double(scale), ctypes.c_double(soft_cap), _p(out), _p(lse))
     return out, lse

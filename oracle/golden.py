@@ -234,7 +234,7 @@ def ref_paged_attn(query: torch.Tensor, key_cache: torch.Tensor, value_cache: to
         num_kv_blocks = (kv_len + block_size - 1) // block_size
         block_indices = block_tables[i, :num_kv_blocks]
         k = key_cache[block_indices].view(-1, num_kv_heads, head_size)[:kv_len]
-        v = value_cache[block_indices].view(-1, num_kv_heads, head_size)[:kv_len]
+        v = value_cache[block_indices].view(-1, num_kv_heads, value_cache.shape[-1])[:kv_len]   # (the reference: head_size)
         if q.shape[1] != k.shape[1]:
             k = torch.repeat_interleave(k, q.shape[1] // k.shape[1], dim=1)
             v = torch.repeat_interleave(v, q.shape[1] // v.shape[1], dim=1)
@@ -332,14 +332,14 @@ def lse_merge(parts: torch.Tensor, lses: torch.Tensor, skip: Optional[torch.Tens
 
 
 def make_paged_kv(batch: int, kv_len_max: int, kv_heads: int, head_dim: int, page_size: int, dtype,
-                  generator: torch.Generator, extra_pages: int = 3):
+                  generator: torch.Generator, extra_pages: int = 3, v_head_dim: Optional[int] = None):
     """Random K/V caches [num_pages, page_size, Hkv, D] and a block table that maps every sequence to a random,
     disjoint set of pages (the data layout of test/nvidia/test_decode_attn.py:148-156, with a permutation
     instead of randint so that no two sequences alias)."""
     pages_per_seq = (kv_len_max + page_size - 1) // page_size
     num_pages = batch * pages_per_seq + extra_pages
     k_cache = torch.randn((num_pages, page_size, kv_heads, head_dim), generator=generator).to(dtype)
-    v_cache = torch.randn((num_pages, page_size, kv_heads, head_dim), generator=generator).to(dtype)
+    v_cache = torch.randn((num_pages, page_size, kv_heads, v_head_dim or head_dim), generator=generator).to(dtype)
     perm = torch.randperm(num_pages, generator=generator)[:batch * pages_per_seq]
     block_table = perm.view(batch, pages_per_seq).to(torch.int32).contiguous()
     return k_cache, v_cache, block_table

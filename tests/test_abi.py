@@ -64,10 +64,20 @@ def test_null_pointers_are_rejected_without_touching_the_gpu():
     assert lib.tdist_reduce_slices(p, 0, 0, 0, 16, p, _lib.TDIST_BF16, None) == _lib.TDIST_ERR_INVALID
     assert lib.tdist_reduce_slices(p, 0, 4, 7, 16, p, _lib.TDIST_BF16, None) == _lib.TDIST_ERR_INVALID
     assert lib.tdist_reduce_slices(p, 0, 4, 0, 16, p, _lib.TDIST_F8E4M3, None) == _lib.TDIST_ERR_UNSUPPORTED
-    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 6, 4, 128, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 6, 4, 128, 128, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
                                      _lib.TDIST_BF16, None) == _lib.TDIST_ERR_INVALID  # 6 % 4 != 0
-    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 96, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 96, 96, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
                                      _lib.TDIST_BF16, None) == _lib.TDIST_ERR_UNSUPPORTED  # head_dim 96
+    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 192, 192, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                     _lib.TDIST_BF16, None) == _lib.TDIST_ERR_UNSUPPORTED  # 192 goes with Dv = 128
+    # the fused launch: 40 query heads over 2 kv heads = 2 blocks of 16 heads per kv head and sequence
+    assert lib.tdist_decode_fused_counters(3, 40, 2) == 3 * 2 * 2
+    assert lib.tdist_decode_fused_counters(3, 40, 3) == -1
+    fused = lambda n_counters, out: lib.tdist_decode_fused(
+        p, p, p, p, p, 1.0, 0.0, p, p, 3, 40, 2, 128, 128, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0, _lib.TDIST_BF16,
+        p, n_counters, out, _lib.TDIST_BF16, 0, 0, None, None)
+    assert fused(11, p) == _lib.TDIST_ERR_WORKSPACE and "counters" in _lib.last_error()
+    assert fused(12, None) == _lib.TDIST_ERR_INVALID
     assert lib.tdist_moe_workspace_bytes(32768, 256) == (32 + 1) * 256 * 4
 
 

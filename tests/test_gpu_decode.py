@@ -15,12 +15,13 @@ pytestmark = pytest.mark.gpu
 ATOL = 2e-3
 
 
-def build_case(kv_lens, heads, head_size, block_size, dtype, seed, num_pages=None):
+def build_case(kv_lens, heads, head_size, block_size, dtype, seed, num_pages=None, v_head_size=None):
     g = torch.Generator().manual_seed(seed)
     Hq, Hkv = heads
     B = len(kv_lens)
     q = torch.randn((B, Hq, head_size), generator=g).to(dtype)
-    k_cache, v_cache, table = golden.make_paged_kv(B, max(max(kv_lens), 1), Hkv, head_size, block_size, dtype, g)
+    k_cache, v_cache, table = golden.make_paged_kv(B, max(max(kv_lens), 1), Hkv, head_size, block_size, dtype, g,
+                                                   v_head_dim=v_head_size)
     return q, k_cache, v_cache, table
 
 
@@ -68,6 +69,83 @@ def test_split_partials_and_lse(cuda, kv_lens, S, dtype):
     assert (got_lse[~empty] - w_lse[~empty]).abs().max() <= ATOL
     assert (out_split.cpu().double() - w_out).abs().max() <= ATOL
     assert (out_split.cpu()[empty] == 0).all()
+
+
+@pytest.mark.parametrize("dims", [(192, 128), (576, 512)])
+@pytest.mark.parametrize("num_heads,kv_lens,S", [((16, 16), [1320, 18, 463], 4), ((32, 8), [1, 54, 293, 70], 8),
+                                                  ((6, 1), [777, 16, 5], 3), ((128, 1), [300, 33], 2)])
+@pytest.mark.parametrize("block_size", [1, 16])
+@pytest.mark.parametrize("dtype,soft_cap", [(torch.bfloat16, 0), (torch.float16, 30)])
+def test_heads_with_extra_key_dimensions(cuda, dims, num_heads, kv_lens, S, block_size, dtype, soft_cap):
+    """Key dimension 192 = 128 + 64 and 576 = 512 + 64 with value dimension 128 / 512 (the reference's BLOCK_DPE
+    heads, flash_decode.py:771-772,186-190,209-213): per-split partials and LSE, then the merged output."""
+    from triton_dist.kernels.amd.flash_decode import _split_kv
+    from triton_dist.kernels.nvidia import gqa_fwd_batch_decode
+    dk, dv = dims
+    announce("decode dims=%s heads=%s kv_lens=%s S=%d page=%d %s cap=%s" % (dims, num_heads, kv_lens, S, block_size, dtype, soft_cap))
+    q, k_cache, v_cache, table = build_case(kv_lens, num_heads, dk, block_size, dtype, seed=dk + S, v_head_size=dv)
+    scale = dk**-0.5
+    B = len(kv_lens)
+    lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
+    qd, kd, vd, td = q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), table.to(cuda)
+    out_split, lse_split, _ = _split_kv(qd, kd, vd, lens_dev, td, scale, soft_cap, S)
+    torch.cuda.synchronize()
+    w_out, w_lse = golden.decode_split_exact(q, k_cache, v_cache, kv_lens, table, scale, S, soft_cap)
+    got_lse = lse_split.cpu().double()
+    empty = torch.isinf(w_lse)
+    assert torch.equal(torch.isinf(got_lse), empty)
+    assert (got_lse[~empty] - w_lse[~empty]).abs().max() <= ATOL
+    assert (out_split.cpu().double() - w_out).abs().max() <= ATOL
+    out = gqa_fwd_batch_decode(qd, kd, vd, None, [1] * B, lens_dev, td, scale, soft_cap, kv_split=S)
+    torch.cuda.synchronize()
+    assert out.shape == (B, num_heads[0], dv)
+    exact, _ = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, scale, soft_cap)
+    eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    assert ((out.cpu().double() - exact).abs() <= ATOL + eps * exact.abs()).all()
+
+
+@pytest.mark.parametrize("num_heads,dims", [((64, 8), (128, 128)), ((6, 1), (128, 128)), ((40, 2), (64, 64)),
+                                            ((16, 16), (192, 128)), ((32, 2), (256, 256)), ((16, 1), (576, 512))])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_decode_is_the_two_launch_result(cuda, num_heads, dims, dtype):
+    """One launch (the last workgroup of a sequence and head block merges the splits) against split-KV followed by
+    the combine: bit-identical outputs and LSE, three calls in a row on the same counters with different lengths
+    (empty splits, a sequence of length 0), counters back at zero after each; and the oracle's bar."""
+    from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine, decode_fused, gqa_fwd_batch_decode_persistent
+    dk, dv = dims
+    Hq, Hkv = num_heads
+    page = 16
+    counters = torch.zeros(4096, dtype=torch.int32, device=cuda)
+    for call, (kv_lens, S) in enumerate([([1320, 18, 463, 5], 32), ([40, 0, 7, 2047], 16), ([100, 3, 64, 1], 1)]):
+        announce("fused decode heads=%s dims=%s %s kv_lens=%s S=%d" % (num_heads, dims, dtype, kv_lens, S))
+        q, k_cache, v_cache, table = build_case(kv_lens, num_heads, dk, page, dtype, seed=call + dk, v_head_size=dv)
+        scale = dk**-0.5
+        B = len(kv_lens)
+        lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
+        qd, kd, vd, td = q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), table.to(cuda)
+        out_split, lse_split, _ = _split_kv(qd, kd, vd, lens_dev, td, scale, 0.0, S)
+        want = torch.empty((B, Hq, dv), dtype=dtype, device=cuda)
+        want_lse = torch.empty((B, Hq), dtype=torch.float32, device=cuda)
+        decode_combine(out_split, lse_split, S, 1, lens_dev, B, Hq, dv,
+                       (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
+                       (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), want, want_lse)
+        got = torch.full((B, Hq, dv), float("nan"), dtype=dtype, device=cuda)
+        got_lse = torch.full((B, Hq), float("nan"), dtype=torch.float32, device=cuda)
+        decode_fused(qd, kd, vd, lens_dev, td, scale, 0.0, S, got, got_lse, workspace=counters)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), "fused output differs from split + combine"
+        assert torch.equal(got_lse.view(torch.int32), want_lse.view(torch.int32))
+        assert int(counters.abs().sum()) == 0, "the arrival counters must be left at zero"
+        exact, exact_lse = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, scale)
+        eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+        assert ((got.cpu().double() - exact).abs() <= ATOL + eps * exact.abs()).all()
+        live = ~torch.isinf(exact_lse)
+        assert torch.equal(torch.isinf(got_lse.cpu()), ~live)
+        assert (got_lse.cpu().double()[live] - exact_lse[live]).abs().max() <= ATOL
+    # the launcher with the reference's signature (cached counters, default output)
+    out = gqa_fwd_batch_decode_persistent(qd, kd, vd, None, [1] * B, lens_dev, td, scale, kv_split=S)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
 
 
 def test_page_indices_beyond_2_31_bytes(cuda):

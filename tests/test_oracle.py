@@ -179,14 +179,16 @@ def test_weighted_combine_vs_c_and_reference_round_trip():
 
 
 # ---- (d) decode ---------------------------------------------------------------------------------------
-@pytest.mark.parametrize("heads,page,soft_cap", [((8, 2), 1, 0.0), ((4, 4), 16, 0.0), ((6, 1), 4, 30.0)])
-def test_decode_exact_vs_c_and_reference_golden(heads, page, soft_cap):
+@pytest.mark.parametrize("heads,page,soft_cap,dims", [((8, 2), 1, 0.0, (64, 64)), ((4, 4), 16, 0.0, (64, 64)),
+                                                      ((6, 1), 4, 30.0, (64, 64)), ((4, 2), 4, 0.0, (96, 64)),
+                                                      ((2, 1), 16, 20.0, (192, 128))])
+def test_decode_exact_vs_c_and_reference_golden(heads, page, soft_cap, dims):
     g = torch.Generator().manual_seed(9)
     Hq, Hkv = heads
-    D, kv_lens = 64, [37, 1, 130]
+    (D, Dv), kv_lens = dims, [37, 1, 130]
     B = len(kv_lens)
     q = torch.randn((B, Hq, D), generator=g).to(torch.bfloat16)
-    k_cache, v_cache, table = golden.make_paged_kv(B, max(kv_lens), Hkv, D, page, torch.bfloat16, g)
+    k_cache, v_cache, table = golden.make_paged_kv(B, max(kv_lens), Hkv, D, page, torch.bfloat16, g, v_head_dim=Dv)
     scale = D**-0.5
     out, lse = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, scale, soft_cap)
     c_out, c_lse = cref.decode_range(q.float().numpy(), k_cache.float().numpy(), v_cache.float().numpy(), table.numpy(),
@@ -196,8 +198,12 @@ def test_decode_exact_vs_c_and_reference_golden(heads, page, soft_cap):
     assert torch.allclose(ref.float(), out.float(), atol=1e-2, rtol=1e-2)   # the reference test's own tolerance
     # kv_len == 1: softmax is 1, the output is that key's value row and LSE its score
     n0 = int(table[1, 0]) * page
-    v_row = v_cache.view(-1, Hkv, D)[n0]
+    v_row = v_cache.view(-1, Hkv, Dv)[n0]
     assert torch.allclose(out[1].float(), torch.repeat_interleave(v_row, Hq // Hkv, dim=0).float(), atol=1e-6)
+    # the extra key dimensions take part in the scores: dropping them changes the LSE
+    if D != Dv:
+        _, lse_cut = golden.decode_exact(q[..., :Dv], k_cache[..., :Dv].contiguous(), v_cache, kv_lens, table, scale, soft_cap)
+        assert not torch.allclose(lse_cut, lse, atol=1e-3)
 
 
 def test_split_partials_merge_to_the_full_result():

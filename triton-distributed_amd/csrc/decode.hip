@@ -17,7 +17,15 @@
 //  * probabilities enter the PV product as a hi+lo pair of 16-bit values, which keeps the product at
 //    fp32-level accuracy for the cost of a second (idle anyway) MFMA.
 //
-// HBM traffic per launch: every K and V row of the split once (2 * len * Hkv * D * 2 B per sequence).
+//  * heads whose key dimension is not a power of two (192 = 128 + 64, 576 = 512 + 64: flash_decode.py:771-772,
+//    BLOCK_DPE) are handled as the reference does: the power-of-two part DM (= the value dimension) and the
+//    extra DPE key dimensions are two row sets of the stage, each with its own DMA layout and swizzle;
+//  * the fused entry point replaces the reference's persistent kernel (split-KV, grid barrier, combine:
+//    flash_decode.py:586-760) by "the last workgroup to arrive merges": every workgroup publishes its partial
+//    result, bumps a counter of its (sequence, head block), and the one that finds the counter at S-1 merges the S
+//    partials. No workgroup ever waits for another, so nothing depends on the grid being co-resident.
+//
+// HBM traffic per launch: every K and V row of the split once (len * Hkv * (Dk + Dv) * 2 B per sequence).
 #include <stdlib.h>
 
 #include "common.h"
@@ -51,6 +59,12 @@ struct DecodeParams {
   int64_t k_sp, k_st, k_sh;
   int64_t v_sp, v_st, v_sh;
   int64_t t_s;  // table stride in entries
+  // fused merge (null counters = plain split-KV launch)
+  int32_t* counters;         // one per (sequence, head block), zero on entry, left zero on exit
+  unsigned char* final_out;  // [B,Hq,Dv] of final_dtype
+  float* final_lse;          // [B,Hq] or null
+  int final_dtype;
+  int64_t fo_sb, fo_sh;      // element strides of final_out
 };
 
 struct MmaBF16 {
@@ -86,33 +100,50 @@ struct MmaF16 {
 constexpr int kTableSlots = 8;  // ring of page-table rows per wave (>= 2P+2)
 
 // KEYS = keys per block (16 or 32): one or two groups of 16 keys, a group being one MFMA tile of scores.
-template <int D, int KEYS, int NST>
+// DM = value dimension = power-of-two part of the key dimension; DPE = the extra key dimensions (0 or 64).
+template <int DM, int DPE, int KEYS, int NST>
 struct DecodeCfg {
   static constexpr int kGroups = KEYS / 16;
-  static constexpr int kRowBytes = D * 2;
+  static constexpr int kRowBytes = DM * 2;
   static constexpr int kLanesPerRow = kRowBytes / 16;       // 16-byte chunks per row
   static constexpr int kRowsPerInstr = 64 / kLanesPerRow;   // rows one wave-wide DMA covers
   static constexpr int kInstrPerTensor = KEYS / kRowsPerInstr;
   static constexpr int kTensorBytes = KEYS * kRowBytes;
-  static constexpr int kStageBytes = 2 * kTensorBytes;
-  static constexpr int kLoadsPerGroup = 1 + 2 * kInstrPerTensor;  // table row + K + V
+  // the extra key dimensions: rows of DPE * 2 bytes behind the K and V rows of the stage
+  static constexpr int kPeRowBytes = DPE * 2;
+  static constexpr int kPeLanesPerRow = DPE > 0 ? kPeRowBytes / 16 : 1;
+  static constexpr int kPeRowsPerInstr = 64 / kPeLanesPerRow;
+  static constexpr int kPeInstr = DPE > 0 ? KEYS / kPeRowsPerInstr : 0;
+  static constexpr int kPeBytes = KEYS * kPeRowBytes;
+  static constexpr int kPeBase = 2 * kTensorBytes;
+  static constexpr int kStageBytes = 2 * kTensorBytes + kPeBytes;
+  static constexpr int kLoadsPerGroup = 1 + 2 * kInstrPerTensor + kPeInstr;  // table row + K + V (+ extra K)
   static constexpr int kP = NST - 1;
   // LDS position of 16-byte chunk c of a row: K rows c ^ kswz(key), V rows c ^ vswz(key).
   // K operand reads: 16 lanes = 16 keys, same chunk      → spread over 16 positions: key & 15.
   // V transposed reads: 32 lanes = 8 keys x 2 adjacent chunks → spread the chunk pairs: (key & 7) << 1.
   static constexpr int kSwzMask = (kLanesPerRow < 16 ? kLanesPerRow : 16) - 1;
+  static constexpr int kPeSwzMask = kPeLanesPerRow - 1;
   static constexpr int kTableSlotBytes = KEYS * 4;
   static constexpr int kWaveBytes = NST * kStageBytes + kTableSlots * kTableSlotBytes;
   static_assert(KEYS == 16 || KEYS == 32, "one or two key groups");
   static_assert(kP >= 1 && kP <= 3, "1..3 stages in flight");
-  static_assert(kP * kLoadsPerGroup < 64, "vmcnt is 6 bits");
+  // vmcnt is a 6-bit counter. When a new group is issued, up to kP older ones may still be in flight; where
+  // kP + 1 groups do not fit the counter (the 576-dimension heads: 35 loads per group), the loop waits for the
+  // block it is about to use BEFORE it issues the next one, so only one group is ever outstanding.
+  static constexpr bool kWaitFirst = (kP + 1) * kLoadsPerGroup >= 64;
+  static_assert(kLoadsPerGroup < 64 && (!kWaitFirst || kP == 1), "vmcnt is 6 bits");
   static_assert(2 * kP + 2 <= kTableSlots, "table ring too small");
-  static_assert(D % 32 == 0 && D >= 64 && D <= 256, "head dim");
+  static_assert(DM % 32 == 0 && DM >= 64 && DM <= 512, "head dim");
+  static_assert(DPE == 0 || DPE == 64, "extra key dimensions: none or 64");
+  static_assert(DPE == 0 || KEYS % kPeRowsPerInstr == 0, "whole DMA instructions for the extra key rows");
   // Rows shorter than the 256-byte bank window already differ in their row offset: only every kRowsPerWindow-th
   // key needs a new XOR term.
   static constexpr int kRowsPerWindow = kRowBytes >= 256 ? 1 : 256 / kRowBytes;
+  static constexpr int kPeRowsPerWindow = DPE > 0 ? 256 / kPeRowBytes : 1;
   __device__ static __forceinline__ int kswz(int key) { return (key / kRowsPerWindow) & kSwzMask; }
   __device__ static __forceinline__ int vswz(int key) { return (((key / kRowsPerWindow) & 7) << 1) & kSwzMask; }
+  __device__ static __forceinline__ int peswz(int key) { return (key / kPeRowsPerWindow) & kPeSwzMask; }
 };
 
 template <int N>
@@ -124,10 +155,21 @@ __device__ __forceinline__ void wait_groups(int rem) {
   else wait_vmcnt<0>();
 }
 
-template <typename MMA, int D, int KEYS, int NW, int NST, bool kSoftCap>
-__global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodeParams prm) {
-  typedef DecodeCfg<D, KEYS, NST> C;
+// One workgroup's split: streams its keys and writes the partial result and LSE of its 16 heads.
+// Partial results that another workgroup of the same launch will read (fused merge) are written through to where
+// every XCD sees them (agent-scope store: the L2 caches of the 8 XCDs are not coherent with each other); with that,
+// publishing them needs no cache write-back, only the wait for the stores themselves.
+template <bool kCoherent>
+__device__ __forceinline__ void store_partial(float* p, float v) {
+  if constexpr (kCoherent) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *p = v;
+}
+
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse>
+__device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
+  typedef DecodeCfg<D, DPE, KEYS, NST> C;
   constexpr int G = C::kGroups;
+  constexpr int DK = D + DPE;  // key (and query) dimensions; D is the value dimension
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   // kv heads vary fastest over the grid: workgroups that run together then read the neighbouring 2*D-byte
@@ -157,9 +199,9 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
     // empty split: zeros and LSE = -inf so that any merge gives it weight 0
     for (int i = threadIdx.x; i < nvalid * D; i += NW * 64) {
       const int h = i / D, d = i - h * D;
-      out_base[(int64_t)h * prm.S * D + d] = 0.f;
+      store_partial<kFuse>(out_base + (int64_t)h * prm.S * D + d, 0.f);
     }
-    if (threadIdx.x < nvalid) lse_base[(int64_t)threadIdx.x * prm.S] = -INFINITY;
+    if (threadIdx.x < nvalid) store_partial<kFuse>(lse_base + (int64_t)threadIdx.x * prm.S, -INFINITY);
     return;
   }
 
@@ -173,11 +215,11 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
   const int n_w = nb_total > wave ? (nb_total - wave + NW - 1) / NW : 0;  // this wave's blocks
 
   // ---- Q fragments (B operand of the score MFMA): head x, dims 32s + 8g .. +8 -------------------
-  typename MMA::frag8 qf[D / 32];
+  typename MMA::frag8 qf[DK / 32];
   {
     const unsigned char* qrow = prm.q + (int64_t)b * prm.q_sb + (int64_t)(h0 + x) * prm.q_sh;
 #pragma unroll
-    for (int s = 0; s < D / 32; ++s) {
+    for (int s = 0; s < DK / 32; ++s) {
       int4v raw = {0, 0, 0, 0};
       if (x < nvalid) raw = *(const int4v*)(qrow + (32 * s + 8 * g) * 2);
       qf[s] = __builtin_bit_cast(typename MMA::frag8, raw);
@@ -195,13 +237,15 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
 
   // Loop-invariant LDS offsets (relative to the stage) of this lane's operand reads.
   // K (A operand of the scores): row = key x of group q, logical chunk 4s+g.
-  int koff[G][D / 32];
+  // The extra key dimensions D + 32s' + 8g live in their own rows behind the K and V rows.
+  int koff[G][DK / 32];
 #pragma unroll
   for (int q = 0; q < G; ++q)
 #pragma unroll
-    for (int s = 0; s < D / 32; ++s) {
+    for (int s = 0; s < DK / 32; ++s) {
       const int key = 16 * q + x;
-      koff[q][s] = key * C::kRowBytes + (((4 * s + g) ^ C::kswz(key)) << 4);
+      if (s < D / 32) koff[q][s] = key * C::kRowBytes + (((4 * s + g) ^ C::kswz(key)) << 4);
+      else koff[q][s] = C::kPeBase + key * C::kPeRowBytes + (((4 * (s - D / 32) + g) ^ C::peswz(key)) << 4);
     }
   // V^T (A operand of the output MFMA) through the transposing LDS read: within a 16-lane block, lane x ends
   // up with elements x, 16+x, 32+x, 48+x of the 64 the block loads (lane s loads 4 consecutive ones), so lane s
@@ -254,6 +298,22 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
       __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)ksrc, (TDIST_AS3 void*)(kst + i * 1024), 16, 0, TDIST_KV_AUX);
       __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)vsrc, (TDIST_AS3 void*)(vst + i * 1024), 16, 0, TDIST_KV_AUX);
     }
+    if constexpr (DPE > 0) {
+      lds_u8 const pst = kst + C::kPeBase;
+      const int pchunk = lane % C::kPeLanesPerRow;
+#pragma unroll
+      for (int i = 0; i < C::kPeInstr; ++i) {
+        const int key = i * C::kPeRowsPerInstr + lane / C::kPeLanesPerRow;
+        int n = min(key0 + key, end - 1);
+        n = max(n, start);
+        const uint32_t page = (uint32_t)tbl[key];
+        const uint32_t in_page = (uint32_t)n - (uint32_t)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift) * (uint32_t)prm.page_size;
+        const unsigned char* psrc = prm.k + (uint64_t)page * (uint64_t)prm.k_sp +
+                                    (in_page * (uint32_t)prm.k_st + (uint32_t)kvh * (uint32_t)prm.k_sh +
+                                     (uint32_t)(C::kRowBytes + ((pchunk ^ C::peswz(key)) << 4)));
+        __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)psrc, (TDIST_AS3 void*)(pst + i * 1024), 16, 0, TDIST_KV_AUX);
+      }
+    }
   };
 
   auto compute = [&](int j) {
@@ -265,7 +325,7 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
     for (int q = 0; q < G; ++q) {
       sc[q] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < D / 32; ++s) {
+      for (int s = 0; s < DK / 32; ++s) {
         const int4v raw = *(const TDIST_AS3 int4v*)(st + koff[q][s]);
         sc[q] = MMA::mma32(__builtin_bit_cast(typename MMA::frag8, raw), qf[s], sc[q]);
       }
@@ -345,11 +405,12 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
       }
     }
     for (int i = 0; i < n_w; ++i) {
+      if constexpr (C::kWaitFirst) wait_vmcnt<0>();
       if (i + C::kP < n_w) {
         issue_table(i + 2 * C::kP + 1);
         issue_rows(i + C::kP);
       }
-      wait_groups<C::kLoadsPerGroup>(min(C::kP, n_w - 1 - i));
+      if constexpr (!C::kWaitFirst) wait_groups<C::kLoadsPerGroup>(min(C::kP, n_w - 1 - i));
       compute(i);
     }
   }
@@ -386,8 +447,8 @@ __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodePa
       L += wm[16 + h] * sc;
       O += wm[32 + dv * 16 + h] * sc;
     }
-    out_base[(int64_t)h * prm.S * D + dv] = O / L;
-    if (dv == 0) lse_base[(int64_t)h * prm.S] = (M + log2f(L)) * kLn2;
+    store_partial<kFuse>(out_base + (int64_t)h * prm.S * D + dv, O / L);
+    if (dv == 0) store_partial<kFuse>(lse_base + (int64_t)h * prm.S, (M + log2f(L)) * kLn2);
   }
 }
 
@@ -439,8 +500,8 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams
   for (int j = 0; j < prm.P; ++j)
     if (!skipped(j)) M = fmaxf(M, lse[(int64_t)j * prm.l_sp]);
   float L = 0.f;
-  constexpr int kMaxPerLane = 4;  // Dv <= 256
-  float acc[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f};
+  constexpr int kMaxPerLane = 8;  // Dv <= 512
+  float acc[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (M != -INFINITY) {
     for (int j = 0; j < prm.P; ++j) {
       if (skipped(j)) continue;
@@ -465,12 +526,81 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams
   if (prm.lse_out && lane == 0) prm.lse_out[bh] = L > 0.f ? M + logf(L) : -INFINITY;
 }
 
-template <typename MMA, int D, int KEYS, int NW, int NST, bool kSoftCap>
-static int launch_decode_sc(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
-  typedef DecodeCfg<D, KEYS, NST> C;
+// Fused tail: publishes this workgroup's partial result; the last of the S workgroups of a (sequence, head block)
+// to get here merges their partials (same arithmetic, in the same order, as decode_combine_kernel in mode 1) and
+// puts the counter back to zero for the next launch.
+template <int D, int NW>
+__device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  TDIST_AS3 int* const s_last = (TDIST_AS3 int*)smem;
+  const int group = prm.Hq / prm.Hkv;
+  const int head_blocks = (group + 15) >> 4;
+  const int kvh = blockIdx.x / head_blocks;
+  const int hb = blockIdx.x - kvh * head_blocks;
+  const int b = blockIdx.z;
+  const int h0 = kvh * group + hb * 16;
+  const int nvalid = min(16, group - hb * 16);
+
+  // This thread's partial results were stored write-through (store_partial): once the stores have completed they
+  // are visible to every XCD. The barrier then orders all of the workgroup's stores before thread 0's counter
+  // update. (A release fence here would write back the whole L2 once per wave: measured at 2x the kernel time.)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();   // (also: every wave is done with the merge scratch that s_last overlays)
+  if (threadIdx.x == 0) {
+    int32_t* ctr = prm.counters + (int64_t)b * gridDim.x + blockIdx.x;
+    const int old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = old == prm.S - 1;
+    if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *s_last = last;
+  }
+  __syncthreads();
+  if (!*s_last) return;
+  // The counter said S-1: every other workgroup's stores completed before its increment. Only the merging
+  // workgroup pays for an acquire (it drops this CU's and this XCD's possibly stale lines; the K/V stream is
+  // non-temporal and loses nothing by it), after which plain vector loads may read the partial results.
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+
+  const float* lse_p = prm.lse + ((int64_t)b * prm.Hq + h0) * prm.S;
+  const float* out_p = prm.out + ((int64_t)b * prm.Hq + h0) * prm.S * D;
+  constexpr int kVecs = D / 4;
+  for (int idx = threadIdx.x; idx < nvalid * kVecs; idx += NW * 64) {
+    const int h = idx / kVecs, dv = (idx - h * kVecs) * 4;
+    const float* l = lse_p + (int64_t)h * prm.S;
+    float M = -INFINITY;
+    for (int j = 0; j < prm.S; ++j) M = fmaxf(M, l[j]);
+    float L = 0.f;
+    float4v acc = {0.f, 0.f, 0.f, 0.f};
+    if (M != -INFINITY) {
+      // an empty split has LSE = -inf and zeros: weight exp(-inf) = 0 adds nothing, as skipping it would
+#pragma unroll 4
+      for (int j = 0; j < prm.S; ++j) {
+        const float w = __expf(l[j] - M);
+        L += w;
+        const float4v x = *(const float4v*)(out_p + ((int64_t)h * prm.S + j) * D + dv);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += w * x[e];
+      }
+    }
+    const int64_t o = (int64_t)b * prm.fo_sb + (int64_t)(h0 + h) * prm.fo_sh + dv;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) store_elem(prm.final_out, o + e, prm.final_dtype, L > 0.f ? acc[e] / L : 0.f);
+    if (dv == 0 && prm.final_lse) prm.final_lse[(int64_t)b * prm.Hq + h0 + h] = L > 0.f ? M + logf(L) : -INFINITY;
+  }
+}
+
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse>
+__global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodeParams prm) {
+  decode_split_body<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse>(prm);
+  if constexpr (kFuse) decode_fused_merge<D, NW>(prm);
+}
+
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse>
+static int launch_decode_cfg(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
+  typedef DecodeCfg<D, DPE, KEYS, NST> C;
   static_assert((32 + D * 16) * 4 <= C::kWaveBytes, "merge scratch must fit in a wave's ring");
   const size_t lds = (size_t)NW * C::kWaveBytes;
-  auto kern = decode_split_kv_kernel<MMA, D, KEYS, NW, NST, kSoftCap>;
+  static_assert((size_t)NW * C::kWaveBytes <= 160 * 1024, "LDS of one CU");
+  auto kern = decode_split_kv_kernel<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -479,98 +609,186 @@ static int launch_decode_sc(const DecodeParams& prm, int head_blocks, hipStream_
   }
   dim3 grid(prm.Hkv * head_blocks, prm.S, prm.B);
   hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, prm);
-  return launch_status("tdist_decode_split_kv");
+  return launch_status(kFuse ? "tdist_decode_fused" : "tdist_decode_split_kv");
 }
 
-template <typename MMA, int D, int KEYS, int NW, int NST>
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST>
 static int launch_decode(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
-  return prm.soft_cap > 0.f ? launch_decode_sc<MMA, D, KEYS, NW, NST, true>(prm, head_blocks, stream)
-                            : launch_decode_sc<MMA, D, KEYS, NW, NST, false>(prm, head_blocks, stream);
+  const bool fuse = prm.counters != nullptr;
+  if (prm.soft_cap > 0.f)
+    return fuse ? launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, true, true>(prm, head_blocks, stream)
+                : launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, true, false>(prm, head_blocks, stream);
+  return fuse ? launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, false, true>(prm, head_blocks, stream)
+              : launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, false, false>(prm, head_blocks, stream);
 }
 
 }  // namespace tdist
 
 using namespace tdist;
 
-extern "C" {
+namespace tdist {
 
-int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cache, float* out_split, float* lse_split,
-                          float sm_scale, float soft_cap, const int32_t* block_table, const int32_t* kv_lens, int batch,
-                          int q_heads, int kv_heads, int head_dim, int page_size, int num_splits, int64_t q_stride_b,
-                          int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_token, int64_t k_stride_head,
-                          int64_t v_stride_page, int64_t v_stride_token, int64_t v_stride_head, int64_t table_stride,
-                          int dtype, void* stream) {
-  if (!q || !k_cache || !v_cache || !out_split || !lse_split || !block_table || !kv_lens)
-    return fail(TDIST_ERR_INVALID, "tdist_decode_split_kv: null pointer");
-  if (batch <= 0 || q_heads <= 0 || kv_heads <= 0 || page_size <= 0 || num_splits <= 0)
-    return fail(TDIST_ERR_INVALID, "tdist_decode_split_kv: sizes must be positive");
-  if (q_heads % kv_heads != 0)
-    return fail(TDIST_ERR_INVALID, "tdist_decode_split_kv: q_heads %d not a multiple of kv_heads %d", q_heads, kv_heads);
-  if (dtype != TDIST_BF16 && dtype != TDIST_F16)
-    return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: dtype %d (bf16 and f16 only)", dtype);
-  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
-    return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: head_dim %d (64, 128, 256 only)", head_dim);
-  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (q_stride_b % 8) || (q_stride_h % 8) ||
-      (k_stride_page % 8) || (k_stride_token % 8) || (k_stride_head % 8) || (v_stride_page % 8) ||
-      (v_stride_token % 8) || (v_stride_head % 8))
-    return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: q/k/v rows must be 16-byte aligned");
-  if (num_splits > 65535 || batch > 65535) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: grid too large");
-  DecodeParams prm;
-  prm.q = (const unsigned char*)q;
-  prm.k = (const unsigned char*)k_cache;
-  prm.v = (const unsigned char*)v_cache;
-  prm.out = out_split;
-  prm.lse = lse_split;
-  prm.table = block_table;
-  prm.lens = kv_lens;
-  prm.sm_scale = sm_scale;
-  prm.soft_cap = soft_cap;
-  prm.B = batch;
-  prm.Hq = q_heads;
-  prm.Hkv = kv_heads;
-  prm.S = num_splits;
-  prm.page_size = page_size;
-  int lg = 0;
-  while ((1ll << lg) < page_size) ++lg;
-  prm.page_shift = 31 + lg;
-  prm.page_magic = ((1ull << prm.page_shift) + (uint64_t)page_size - 1) / (uint64_t)page_size;
-  prm.q_sb = q_stride_b * 2;
-  prm.q_sh = q_stride_h * 2;
-  prm.k_sp = k_stride_page * 2;
-  prm.k_st = k_stride_token * 2;
-  prm.k_sh = k_stride_head * 2;
-  prm.v_sp = v_stride_page * 2;
-  prm.v_st = v_stride_token * 2;
-  prm.v_sh = v_stride_head * 2;
-  prm.t_s = table_stride;
+struct DecodeCall {
+  const void *q, *k_cache, *v_cache;
+  float *out_split, *lse_split;
+  float sm_scale, soft_cap;
+  const int32_t *block_table, *kv_lens;
+  int batch, q_heads, kv_heads, head_dim, head_dim_v, page_size, num_splits;
+  int64_t q_stride_b, q_stride_h, k_stride_page, k_stride_token, k_stride_head, v_stride_page, v_stride_token,
+      v_stride_head, table_stride;
+  int dtype;
+  // fused merge
+  int32_t* counters;
+  int64_t n_counters;
+  void* out;
+  int out_dtype;
+  int64_t out_stride_b, out_stride_h;
+  float* lse_out;
+  void* stream;
+  const char* who;
+};
+
+static int64_t decode_fused_counters(int batch, int q_heads, int kv_heads) {
+  if (batch <= 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return -1;
   const int group = q_heads / kv_heads;
+  return (int64_t)batch * kv_heads * ((group + 15) / 16);
+}
+
+static int run_decode(const DecodeCall& c, bool fuse) {
+  const char* who = c.who;
+  if (!c.q || !c.k_cache || !c.v_cache || !c.out_split || !c.lse_split || !c.block_table || !c.kv_lens)
+    return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
+  if (c.batch <= 0 || c.q_heads <= 0 || c.kv_heads <= 0 || c.page_size <= 0 || c.num_splits <= 0)
+    return fail(TDIST_ERR_INVALID, "%s: sizes must be positive", who);
+  if (c.q_heads % c.kv_heads != 0)
+    return fail(TDIST_ERR_INVALID, "%s: q_heads %d not a multiple of kv_heads %d", who, c.q_heads, c.kv_heads);
+  if (c.dtype != TDIST_BF16 && c.dtype != TDIST_F16)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: dtype %d (bf16 and f16 only)", who, c.dtype);
+  const int dk = c.head_dim, dv = c.head_dim_v;
+  const bool dims_ok = (dk == dv && (dk == 64 || dk == 128 || dk == 256)) || (dk == 192 && dv == 128) ||
+                       (dk == 576 && dv == 512);
+  if (!dims_ok)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: head dims (%d, %d): (64,64), (128,128), (256,256), (192,128), (576,512) only",
+                who, dk, dv);
+  if (!aligned16(c.q) || !aligned16(c.k_cache) || !aligned16(c.v_cache) || (c.q_stride_b % 8) || (c.q_stride_h % 8) ||
+      (c.k_stride_page % 8) || (c.k_stride_token % 8) || (c.k_stride_head % 8) || (c.v_stride_page % 8) ||
+      (c.v_stride_token % 8) || (c.v_stride_head % 8))
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: q/k/v rows must be 16-byte aligned", who);
+  if (c.num_splits > 65535 || c.batch > 65535) return fail(TDIST_ERR_UNSUPPORTED, "%s: grid too large", who);
+  DecodeParams prm;
+  prm.q = (const unsigned char*)c.q;
+  prm.k = (const unsigned char*)c.k_cache;
+  prm.v = (const unsigned char*)c.v_cache;
+  prm.out = c.out_split;
+  prm.lse = c.lse_split;
+  prm.table = c.block_table;
+  prm.lens = c.kv_lens;
+  prm.sm_scale = c.sm_scale;
+  prm.soft_cap = c.soft_cap;
+  prm.B = c.batch;
+  prm.Hq = c.q_heads;
+  prm.Hkv = c.kv_heads;
+  prm.S = c.num_splits;
+  prm.page_size = c.page_size;
+  int lg = 0;
+  while ((1ll << lg) < c.page_size) ++lg;
+  prm.page_shift = 31 + lg;
+  prm.page_magic = ((1ull << prm.page_shift) + (uint64_t)c.page_size - 1) / (uint64_t)c.page_size;
+  prm.q_sb = c.q_stride_b * 2;
+  prm.q_sh = c.q_stride_h * 2;
+  prm.k_sp = c.k_stride_page * 2;
+  prm.k_st = c.k_stride_token * 2;
+  prm.k_sh = c.k_stride_head * 2;
+  prm.v_sp = c.v_stride_page * 2;
+  prm.v_st = c.v_stride_token * 2;
+  prm.v_sh = c.v_stride_head * 2;
+  prm.t_s = c.table_stride;
+  prm.counters = nullptr;
+  prm.final_out = nullptr;
+  prm.final_lse = nullptr;
+  prm.final_dtype = TDIST_F32;
+  prm.fo_sb = prm.fo_sh = 0;
+  if (fuse) {
+    if (!c.counters || !c.out) return fail(TDIST_ERR_INVALID, "%s: null counters or output", who);
+    if (!aligned16(c.out_split)) return fail(TDIST_ERR_UNSUPPORTED, "%s: out_split must be 16-byte aligned", who);
+    if (c.out_dtype != TDIST_F32 && c.out_dtype != TDIST_BF16 && c.out_dtype != TDIST_F16)
+      return fail(TDIST_ERR_UNSUPPORTED, "%s: output dtype %d", who, c.out_dtype);
+    const int64_t need = decode_fused_counters(c.batch, c.q_heads, c.kv_heads);
+    if (c.n_counters < need)
+      return fail(TDIST_ERR_WORKSPACE, "%s: %lld counters given, %lld needed", who, (long long)c.n_counters, (long long)need);
+    prm.counters = c.counters;
+    prm.final_out = (unsigned char*)c.out;
+    prm.final_lse = c.lse_out;
+    prm.final_dtype = c.out_dtype;
+    prm.fo_sb = c.out_stride_b;
+    prm.fo_sh = c.out_stride_h;
+  }
+  const int group = c.q_heads / c.kv_heads;
   const int head_blocks = (group + 15) / 16;
-  if ((int64_t)kv_heads * head_blocks > 65535) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_split_kv: too many heads");
-  hipStream_t st = (hipStream_t)stream;
-  const bool bf = dtype == TDIST_BF16;
-  switch (head_dim) {
-    // <dtype, D, keys per block, waves, stages>: LDS = waves * (stages * keys * D * 4 B + tables) <= 160 KB
-    case 64:
-      return bf ? launch_decode<MmaBF16, 64, 32, 4, 4>(prm, head_blocks, st) : launch_decode<MmaF16, 64, 32, 4, 4>(prm, head_blocks, st);
+  if ((int64_t)c.kv_heads * head_blocks > 65535) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many heads", who);
+  hipStream_t st = (hipStream_t)c.stream;
+  const bool bf = c.dtype == TDIST_BF16;
+  // <dtype, Dv, extra key dims, keys per block, waves, stages>:
+  // LDS = waves * (stages * keys * (Dk + Dv) * 2 B + tables) <= 160 KB
+#define TDIST_DEC(D_, DPE_, KEYS_, NW_, NST_)                                             \
+  return bf ? launch_decode<MmaBF16, D_, DPE_, KEYS_, NW_, NST_>(prm, head_blocks, st)   \
+            : launch_decode<MmaF16, D_, DPE_, KEYS_, NW_, NST_>(prm, head_blocks, st);
+  switch (dk) {
+    case 64: TDIST_DEC(64, 0, 32, 4, 4)
     case 128: {
       // TDIST_DECODE_VARIANT picks another compiled shape (measurement aid). Default: 16-key blocks, 3 waves,
       // 3 stages = 72 KB of LDS, so two workgroups share a CU and two thirds of the ring are in flight.
       int variant = 0;
       if (const char* v = getenv("TDIST_DECODE_VARIANT")) variant = atoi(v);
-#define TDIST_DEC(KEYS_, NW_, NST_) \
-  return bf ? launch_decode<MmaBF16, 128, KEYS_, NW_, NST_>(prm, head_blocks, st) : launch_decode<MmaF16, 128, KEYS_, NW_, NST_>(prm, head_blocks, st);
       switch (variant) {
-        case 1: TDIST_DEC(32, 4, 2)
-        case 2: TDIST_DEC(32, 3, 3)
-        case 3: TDIST_DEC(16, 8, 2)
-        case 4: TDIST_DEC(16, 4, 2)
-        default: TDIST_DEC(16, 3, 3)
+        case 1: TDIST_DEC(128, 0, 32, 4, 2)
+        case 2: TDIST_DEC(128, 0, 32, 3, 3)
+        case 3: TDIST_DEC(128, 0, 16, 8, 2)
+        case 4: TDIST_DEC(128, 0, 16, 4, 2)
+        default: TDIST_DEC(128, 0, 16, 3, 3)
       }
-#undef TDIST_DEC
     }
-    default:
-      return bf ? launch_decode<MmaBF16, 256, 16, 2, 3>(prm, head_blocks, st) : launch_decode<MmaF16, 256, 16, 2, 3>(prm, head_blocks, st);
+    case 192: TDIST_DEC(128, 64, 16, 2, 3)   // 61 KB: two workgroups per CU
+    case 256: TDIST_DEC(256, 0, 16, 2, 3)
+    default: TDIST_DEC(512, 64, 16, 2, 2)    // 576 = 512 + 64: 136 KB
   }
+#undef TDIST_DEC
+}
+
+}  // namespace tdist
+
+extern "C" {
+
+int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cache, float* out_split, float* lse_split,
+                          float sm_scale, float soft_cap, const int32_t* block_table, const int32_t* kv_lens, int batch,
+                          int q_heads, int kv_heads, int head_dim, int head_dim_v, int page_size, int num_splits,
+                          int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_token,
+                          int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_token, int64_t v_stride_head,
+                          int64_t table_stride, int dtype, void* stream) {
+  DecodeCall c = {q, k_cache, v_cache, out_split, lse_split, sm_scale, soft_cap, block_table, kv_lens, batch, q_heads,
+                  kv_heads, head_dim, head_dim_v, page_size, num_splits, q_stride_b, q_stride_h, k_stride_page,
+                  k_stride_token, k_stride_head, v_stride_page, v_stride_token, v_stride_head, table_stride, dtype,
+                  nullptr, 0, nullptr, TDIST_F32, 0, 0, nullptr, stream, "tdist_decode_split_kv"};
+  return run_decode(c, false);
+}
+
+int64_t tdist_decode_fused_counters(int batch, int q_heads, int kv_heads) {
+  return decode_fused_counters(batch, q_heads, kv_heads);
+}
+
+int tdist_decode_fused(const void* q, const void* k_cache, const void* v_cache, float* out_split, float* lse_split,
+                       float sm_scale, float soft_cap, const int32_t* block_table, const int32_t* kv_lens, int batch,
+                       int q_heads, int kv_heads, int head_dim, int head_dim_v, int page_size, int num_splits,
+                       int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_token,
+                       int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_token, int64_t v_stride_head,
+                       int64_t table_stride, int dtype, int32_t* counters, int64_t n_counters, void* out, int out_dtype,
+                       int64_t out_stride_b, int64_t out_stride_h, float* lse_out, void* stream) {
+  DecodeCall c = {q, k_cache, v_cache, out_split, lse_split, sm_scale, soft_cap, block_table, kv_lens, batch, q_heads,
+                  kv_heads, head_dim, head_dim_v, page_size, num_splits, q_stride_b, q_stride_h, k_stride_page,
+                  k_stride_token, k_stride_head, v_stride_page, v_stride_token, v_stride_head, table_stride, dtype,
+                  counters, n_counters, out, out_dtype, out_stride_b, out_stride_h, lse_out, stream,
+                  "tdist_decode_fused"};
+  return run_decode(c, true);
 }
 
 int tdist_decode_combine(const void* part, int part_dtype, const float* lse, int num_partials, int mode,
@@ -581,7 +799,7 @@ int tdist_decode_combine(const void* part, int part_dtype, const float* lse, int
   if (!part || !lse || !out) return fail(TDIST_ERR_INVALID, "tdist_decode_combine: null pointer");
   if (num_partials <= 0 || batch <= 0 || q_heads <= 0 || head_dim_v <= 0)
     return fail(TDIST_ERR_INVALID, "tdist_decode_combine: sizes must be positive");
-  if (head_dim_v > 256) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_combine: head_dim_v %d > 256", head_dim_v);
+  if (head_dim_v > 512) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_combine: head_dim_v %d > 512", head_dim_v);
   if (mode < 0 || mode > 2 || (mode != 0 && !lens))
     return fail(TDIST_ERR_INVALID, "tdist_decode_combine: mode %d needs lens", mode);
   if ((part_dtype != TDIST_F32 && part_dtype != TDIST_BF16 && part_dtype != TDIST_F16) ||

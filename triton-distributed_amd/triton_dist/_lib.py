@@ -50,8 +50,11 @@ PROTOTYPES = {
     "tdist_moe_dispatch_tokens_quant": (_I, [_P, _I, _I, _P, _I, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_align_workspace_bytes": (_L, [_L, _I, _I]),
     "tdist_moe_align_block_size": (_I, [_P, _I, _L, _I, _I, _L, _I, _P, _P, _P, _P, _P, _P, _L, _P]),
-    "tdist_decode_split_kv": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I,
+    "tdist_decode_split_kv": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                    _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
+    "tdist_decode_fused_counters": (_L, [_I, _I, _I]),
+    "tdist_decode_fused": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I,
+                                _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P, _L, _P, _I, _L, _L, _P, _P]),
     "tdist_decode_combine": (_I, [_P, _I, _P, _I, _I, _P, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P, _I, _L, _L, _P, _P]),
     "tdist_copy_bytes": (_I, [_P, _P, _L, _P]),
     "tdist_mfma_rate_probe": (_I, [_I, _I, _I, _P, _P]),

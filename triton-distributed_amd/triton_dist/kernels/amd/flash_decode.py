@@ -15,15 +15,18 @@ from triton_dist import _lib
 DEFAULT_KV_SPLITS = 32  # reference :777, :861
 
 
-def _split_kv(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, out_split=None, lse_split=None):
+SUPPORTED_HEAD_DIMS = ((64, 64), (128, 128), (256, 256), (192, 128), (576, 512))  # (q/k head dim, v head dim)
+
+
+def _check_inputs(q, k_cache, v_cache, kv_lens, block_table):
     _lib.require_cuda(q, k_cache, v_cache, kv_lens, block_table)
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
     v_head_dim = v_cache.shape[-1]
     assert q_heads % kv_heads == 0
-    if v_head_dim != q_head_dim:
-        raise NotImplementedError("v_head_dim != q_head_dim")
+    if (q_head_dim, v_head_dim) not in SUPPORTED_HEAD_DIMS:
+        raise NotImplementedError("head dims (%d, %d); supported: %s" % (q_head_dim, v_head_dim, SUPPORTED_HEAD_DIMS))
     if q.dtype != k_cache.dtype or q.dtype != v_cache.dtype:
         raise TypeError("q, k_cache and v_cache must share one dtype")
     if q.stride(-1) != 1 or k_cache.stride(-1) != 1 or v_cache.stride(-1) != 1:
@@ -33,17 +36,68 @@ def _split_kv(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_sp
     if block_table.dtype != torch.int32:
         block_table = block_table.to(torch.int32)
     assert block_table.stride(-1) == 1
-    dev = q.device
+    return kv_lens, block_table
+
+
+def _decode_args(q, k_cache, v_cache, out_split, lse_split, scale, soft_cap, block_table, kv_lens, num_splits):
+    batch, q_heads, q_head_dim = q.shape
+    _, page_size, kv_heads, _ = k_cache.shape
+    return [q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out_split.data_ptr(), lse_split.data_ptr(),
+            float(scale), float(soft_cap), block_table.data_ptr(), kv_lens.data_ptr(), batch, q_heads, kv_heads,
+            q_head_dim, v_cache.shape[-1], page_size, num_splits, q.stride(0), q.stride(1), k_cache.stride(0),
+            k_cache.stride(1), k_cache.stride(2), v_cache.stride(0), v_cache.stride(1), v_cache.stride(2),
+            block_table.stride(0), _lib.dtype_code(q.dtype)]
+
+
+def _split_buffers(q, v_cache, num_splits, out_split, lse_split):
+    batch, q_heads, _ = q.shape
     if out_split is None:
-        out_split = torch.empty((batch, q_heads, num_splits, v_head_dim), dtype=torch.float32, device=dev)
+        out_split = torch.empty((batch, q_heads, num_splits, v_cache.shape[-1]), dtype=torch.float32, device=q.device)
     if lse_split is None:
-        lse_split = torch.empty((batch, q_heads, num_splits), dtype=torch.float32, device=dev)
-    _lib.call("tdist_decode_split_kv", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out_split.data_ptr(),
-              lse_split.data_ptr(), float(scale), float(soft_cap), block_table.data_ptr(), kv_lens.data_ptr(), batch,
-              q_heads, kv_heads, q_head_dim, page_size, num_splits, q.stride(0), q.stride(1), k_cache.stride(0),
-              k_cache.stride(1), k_cache.stride(2), v_cache.stride(0), v_cache.stride(1), v_cache.stride(2),
-              block_table.stride(0), _lib.dtype_code(q.dtype), _lib.stream_ptr())
+        lse_split = torch.empty((batch, q_heads, num_splits), dtype=torch.float32, device=q.device)
+    return out_split, lse_split
+
+
+def _split_kv(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, out_split=None, lse_split=None):
+    kv_lens, block_table = _check_inputs(q, k_cache, v_cache, kv_lens, block_table)
+    out_split, lse_split = _split_buffers(q, v_cache, num_splits, out_split, lse_split)
+    _lib.call("tdist_decode_split_kv",
+              *_decode_args(q, k_cache, v_cache, out_split, lse_split, scale, soft_cap, block_table, kv_lens, num_splits),
+              _lib.stream_ptr())
     return out_split, lse_split, kv_lens
+
+
+_fused_counters = {}   # device index -> zero-initialised int32 counters (the kernel leaves them zero)
+
+
+def _counters_for(q, kv_heads, workspace):
+    """Arrival counters of the fused launch: a caller's ``workspace`` when it is a contiguous int32 tensor on the
+    device that is large enough (it must be ALL ZERO; the kernel leaves it zero), else a cached per-device buffer."""
+    batch, q_heads, _ = q.shape
+    need = _lib.load().tdist_decode_fused_counters(batch, q_heads, kv_heads)
+    if (isinstance(workspace, torch.Tensor) and workspace.is_cuda and workspace.dtype == torch.int32
+            and workspace.is_contiguous() and workspace.numel() >= need):
+        return workspace, workspace.numel()
+    buf = _fused_counters.get(q.device.index)
+    if buf is None or buf.numel() < need:
+        buf = torch.zeros(max(int(need), 4096), dtype=torch.int32, device=q.device)
+        _fused_counters[q.device.index] = buf
+    return buf, buf.numel()
+
+
+def decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, out, lse_out=None,
+                 workspace=None, out_split=None, lse_split=None):
+    """tdist_decode_fused: split-KV decode and the merge of the splits in one launch. ``out`` [B,Hq,Dv]
+    (bf16 / f16 / fp32), ``lse_out`` fp32 [B,Hq] or None. Returns (out, out_split, lse_split)."""
+    kv_lens, block_table = _check_inputs(q, k_cache, v_cache, kv_lens, block_table)
+    out_split, lse_split = _split_buffers(q, v_cache, num_splits, out_split, lse_split)
+    assert out.stride(-1) == 1 and (lse_out is None or (lse_out.dtype == torch.float32 and lse_out.is_contiguous()))
+    counters, n_counters = _counters_for(q, k_cache.shape[2], workspace)
+    _lib.call("tdist_decode_fused",
+              *_decode_args(q, k_cache, v_cache, out_split, lse_split, scale, soft_cap, block_table, kv_lens, num_splits),
+              counters.data_ptr(), n_counters, out.data_ptr(), _lib.dtype_code(out.dtype), out.stride(0), out.stride(1),
+              _lib.ptr(lse_out), _lib.stream_ptr())
+    return out, out_split, lse_split
 
 
 def decode_combine(part, lse, num_partials, mode, lens, batch, q_heads, dv, part_strides, lse_strides, out,
@@ -79,10 +133,17 @@ def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_
 
 def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
                                     output_split=None, output_combine=None, kv_split=-1):
-    """Same result as gqa_fwd_batch_decode (reference :931-1004 fuses split and combine into one persistent
-    launch; here the two kernels run back to back)."""
-    return gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap,
-                                output_split, output_combine, kv_split)
+    """Same result as gqa_fwd_batch_decode in one launch (reference :931-1004: split-KV, a grid barrier on
+    ``workspace``, then the combine). Here the last workgroup to finish a (sequence, head block) merges its splits;
+    the arrival counters are a cached per-device buffer that the kernel leaves at zero (``workspace`` is accepted
+    and unused: nothing here depends on what a caller left in it). ``output_split`` is ignored (partials are fp32
+    internally). Calls on different streams of one device share the counters and must not overlap."""
+    num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
+    batch, q_heads, _ = q.shape
+    if output_combine is None:
+        output_combine = torch.empty((batch, q_heads, v_cache.shape[-1]), dtype=q.dtype, device=q.device)
+    decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, output_combine)
+    return output_combine
 
 
 def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
@@ -92,16 +153,14 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
     passes a buffer of another dtype (the reference uses q's dtype). With ``return_lse`` also returns the
     fp32 (out [B,Hq,Dv], lse [B,Hq]) pair the merge produced."""
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
-    out_split, lse_split, kv_lens = _split_kv(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits)
     batch, q_heads, _ = q.shape
     dv = v_cache.shape[-1]
     if output_combine is None:
         output_combine = torch.empty((batch, q_heads, dv + 1), dtype=torch.float32, device=q.device)
     out32 = torch.empty((batch, q_heads, dv), dtype=torch.float32, device=q.device)
     lse32 = torch.empty((batch, q_heads), dtype=torch.float32, device=q.device)
-    decode_combine(out_split, lse_split, num_splits, 1, kv_lens, batch, q_heads, dv,
-                   (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
-                   (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), out32, lse32)
+    # split-KV and the merge of the splits (keeping the LSE) in one launch
+    decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, out32, lse32)
     output_combine[..., :dv].copy_(out32)
     output_combine[..., dv].copy_(lse32)
     if return_lse:
