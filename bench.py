@@ -95,6 +95,31 @@ def time_live_ag_gemm(call, ctx, steps, warmup):
         return s, "copies_first"
 
 
+XGMI_LINK_GBPS = 153.0   # one xGMI link of MI355X: the rate at which one peer's rows arrive
+
+
+def paced_ag_gemm(make_call, world, rank, mpr, N, K, in_dtype, peer_shards, chunk_rows, pre_s, steps, warmup):
+    """AG-GEMM with every peer's chunks held back to the pace of one xGMI link per peer (the one-GPU producer kernel
+    copies chunk c of every peer no earlier than (c+1) chunk times of a link after the call started), for several
+    chunk sizes. Overlap efficiency = time with every flag pre-set / time with paced arrivals; the time includes
+    the host's queueing of the call (three streams, their events), which is what bounds the small config."""
+    import torch
+    from triton_dist.kernels.amd import create_ag_gemm_intra_node_context
+    out = {}
+    for rows in chunk_rows:
+        ctx = create_ag_gemm_intra_node_context(world * mpr, N, K, in_dtype, torch.bfloat16, rank, world, None,
+                                                M_PER_CHUNK=rows)
+        ctx.set_peer_shards(peer_shards)
+        ctx.link_gbps = XGMI_LINK_GBPS
+        ctx.producer_kernel, ctx.producer_workgroups = True, 16   # every peer in one launch, pacing inside the kernel
+        s, order = time_live_ag_gemm(make_call(ctx), ctx, max(steps // 2, 1), warmup)
+        arrive_us = mpr * K * peer_shards[(rank + 1) % world].element_size() / XGMI_LINK_GBPS / 1e3
+        out["m_per_chunk_%d" % rows] = {"us": round(s * 1e6, 2), "order": order,
+                                        "overlap_efficiency": round(pre_s / s, 4),
+                                        "last_chunk_arrives_us": round(arrive_us, 1)}
+    return out
+
+
 def cpu_time(fn):
     """Wall time of one call of ``fn`` on the host cores (torch's thread pool at its default width)."""
     import torch
@@ -207,6 +232,10 @@ def bench_c1(dev, steps, warmup):
                          "sample": "the whole config once (torch golden: cat + matmul), %.2f s" % cs}
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
     r["live_producer_order"] = live_order
+    if LIVE_PRODUCER:
+        r["paced_xgmi_%dGBps" % XGMI_LINK_GBPS] = paced_ag_gemm(
+            lambda c: (lambda: ag_gemm_intra_node(a_d, b_d, False, c)), world, rank, mpr, N, K, torch.bfloat16,
+            ctx.peer_shards, (1024, 256), pre_s, steps, warmup)
     return r
 
 
@@ -247,6 +276,10 @@ def bench_c3(dev, steps, warmup):
                          "sample": "1024 of the 16384 rows (fp32 up-cast golden with scales), %.2f s" % cs}
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
     r["live_producer_order"] = live_order
+    if LIVE_PRODUCER:
+        r["paced_xgmi_%dGBps" % XGMI_LINK_GBPS] = paced_ag_gemm(
+            lambda c: (lambda: ag_gemm_intra_node(a_d, b_d, False, c, row_scale=sa, col_scale=sb)), world, rank, mpr, N, K,
+            torch.float8_e4m3fn, ctx.peer_shards, (2048, 512), pre_s, steps, warmup)
     return r
 
 

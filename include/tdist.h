@@ -107,6 +107,31 @@ int tdist_gemm_chunk_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
 int tdist_producer_push_chunk(void* dst, const void* src, int64_t nbytes, int32_t* flag, const int32_t* one,
                               int use_sdma, void* stream);
 
+/* All peers of an all-gather in ONE launch (no counterpart in the reference, where every peer's copy engine pushes
+ * its own rows: this stands for those engines on a box with one GPU). Block row y plays peer
+ * (rank + 1 + y) % world_size: it copies that peer's rows peer_src[r][0 .. rank_bytes) into
+ * workspace + r*rank_bytes chunk by chunk (chunk_bytes each) with workgroups_per_peer workgroups, and when the
+ * last of them has stored its part of chunk c it stores flag_value into flags[r*chunks_per_rank + c] (release,
+ * system scope) — the data-then-flag protocol of kernels/amd/all_gather_gemm.py:80-100.
+ * peer_src: device array of world_size device pointers (entry `rank` unused). counters: int32
+ * [world_size*chunks_per_rank], zero on entry, left zero. held: optional int32 mask of chunks never to deliver
+ * (test hook for the consumer's bounded wait). stamp + ns_per_chunk > 0: chunk c of every peer is held back
+ * until (c+1)*ns_per_chunk after the stamp (tdist_producer_mark), the pace of one link per peer; the total must
+ * stay within 100 ms. The kernel needs 32 registers per lane and no LDS, so its waves fit on a SIMD beside a
+ * resident wave of the consumer GEMM; nothing in it waits for another workgroup. */
+int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int world_size, int rank,
+                              int64_t rank_bytes, int64_t chunk_bytes, int32_t* flags, int flag_value,
+                              int32_t* counters, const int32_t* held, const uint64_t* stamp, int64_t ns_per_chunk,
+                              int workgroups_per_peer, void* stream);
+
+/* Link pacing for the one-GPU producer (no counterpart in the reference, whose chunks arrive over xGMI at the
+ * link's rate: ~153 GB/s per peer). tdist_producer_mark stores the device's constant-rate wall clock into *stamp
+ * (device uint64); tdist_producer_wait_until holds `stream` until that clock is offset_ns (0 .. 100 ms) past the
+ * stamp, with one idle wave. Queued before a chunk's copy, it makes the chunk arrive no earlier than a link of
+ * the given rate would have delivered it. */
+int tdist_producer_mark(uint64_t* stamp, void* stream);
+int tdist_producer_wait_until(const uint64_t* stamp, int64_t offset_ns, void* stream);
+
 /* Stream-ordered store of `value` into *flag by a one-thread kernel (release, system scope).
  *   replaces set_signal  kernels/amd/common_ops.py:97-112 */
 int tdist_flag_set(int32_t* flag, int value, void* stream);

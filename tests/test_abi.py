@@ -78,6 +78,10 @@ def test_null_pointers_are_rejected_without_touching_the_gpu():
         p, n_counters, out, _lib.TDIST_BF16, 0, 0, None, None)
     assert fused(11, p) == _lib.TDIST_ERR_WORKSPACE and "counters" in _lib.last_error()
     assert fused(12, None) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_producer_mark(None, None) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_producer_wait_until(None, 1000, None) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_producer_wait_until(p, -1, None) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_producer_wait_until(p, 100000001, None) == _lib.TDIST_ERR_INVALID and "100 ms" in _lib.last_error()
     assert lib.tdist_moe_workspace_bytes(32768, 256) == (32 + 1) * 256 * 4
 
 

@@ -403,3 +403,69 @@ def test_each_tile_configuration_forced(cuda, monkeypatch, tile, dtype):
         if sa is not None:
             ref = ref * sa[:, None] * sb[None, :]
         assert torch.equal(c, ref.to(out_dtype)), "tile %d case %d differs" % (tile, case)
+
+
+def test_paced_arrivals_hold_the_chunks_back(cuda):
+    """Link pacing of the one-GPU producer: with a slow emulated link the call cannot finish before the last chunk's
+    link time has passed, and the result is the unpaced one."""
+    from triton_dist.kernels.amd import ag_gemm_intra_node, create_ag_gemm_intra_node_context
+    announce("ag-gemm with paced arrivals")
+    world, rank, mpr, K, N = 4, 1, 256, 512, 384
+    shards, b = make_ag_case(world, mpr, K, N, torch.bfloat16, seed=77)
+    ctx = create_ag_gemm_intra_node_context(world * mpr, N, K, torch.bfloat16, torch.bfloat16, rank, world, None, M_PER_CHUNK=128)
+    ctx.set_peer_shards({r: s.to(cuda) for r, s in enumerate(shards) if r != rank})
+    a_d, b_d = shards[rank].to(cuda), b.to(cuda)
+    want = ag_gemm_intra_node(a_d, b_d, False, ctx)
+    ctx.check_status()
+    chunk_bytes = 128 * K * 2
+    ctx.link_gbps = chunk_bytes / 1.5e6          # 1.5 ms per chunk, two chunks per peer: the last one is due at 3 ms
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    got = ag_gemm_intra_node(a_d, b_d, False, ctx)
+    stop.record()
+    ctx.check_status()
+    assert torch.equal(got, want)
+    assert golden.max_rel_err(got.float().cpu(), golden.ag_gemm_fp32(shards, b)) <= 1e-2
+    assert start.elapsed_time(stop) >= 2.9, "the last chunk was released before its link time"
+    assert start.elapsed_time(stop) < 200
+
+
+@pytest.mark.parametrize("producer_kernel,link_gbps", [(False, 0.0), (True, 0.0), (True, 50.0)])
+def test_ag_gemm_kernel_producer_and_graph_replay(cuda, producer_kernel, link_gbps):
+    """The whole op (producer on its stream, gated GEMM, flag reset) captured into a HIP graph and replayed three
+    times with eager work in between: every replay must reproduce the eager result from a poisoned workspace. Runs
+    with the copy producer and with the one-launch kernel producer (unpaced and paced)."""
+    from triton_dist.kernels.amd import ag_gemm_intra_node, create_ag_gemm_intra_node_context
+    announce("ag-gemm graph replay, kernel producer %s, link %s" % (producer_kernel, link_gbps))
+    world, rank, mpr, K, N = 4, 2, 512, 1024, 640
+    shards, b = make_ag_case(world, mpr, K, N, torch.bfloat16, seed=91)
+    # capture needs streams other than the default one
+    ctx = create_ag_gemm_intra_node_context(world * mpr, N, K, torch.bfloat16, torch.bfloat16, rank, world, None,
+                                            M_PER_CHUNK=256, gemm_stream=torch.cuda.Stream(),
+                                            ag_streams=[torch.cuda.Stream(), torch.cuda.Stream()])
+    ctx.set_peer_shards({r: s.to(cuda) for r, s in enumerate(shards) if r != rank})
+    ctx.producer_kernel, ctx.link_gbps = producer_kernel, link_gbps
+    a_d, b_d = shards[rank].to(cuda), b.to(cuda)
+    want = ag_gemm_intra_node(a_d, b_d, False, ctx).clone()
+    ctx.check_status()
+    assert golden.max_rel_err(want.float().cpu(), golden.ag_gemm_fp32(shards, b)) <= 1e-2
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ag_gemm_intra_node(a_d, b_d, False, ctx)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = ag_gemm_intra_node(a_d, b_d, False, ctx)
+    torch.cuda.synchronize()
+    for replay in range(3):
+        ctx.workspace_tensors[rank].view(torch.uint8).fill_(0x7B)   # eager work between the replays
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), "replay %d differs from the eager result" % replay
+    ctx.check_status()
+    if producer_kernel:
+        assert int(ctx.producer_counters.abs().sum()) == 0

@@ -239,13 +239,16 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         int ok = 0;
         int limit = p.spin_limit;
         if (p.status != nullptr && __hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) limit = 1;
+        // poll with plain coherent loads and acquire once, after the flag has been seen: an acquiring load
+        // invalidates this CU's and this XCD's caches every time it is executed
         for (int it = 0; it < limit; ++it) {
-          if (__hip_atomic_load(f, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) == p.wait_value) {
+          if (__hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == p.wait_value) {
             ok = 1;
             break;
           }
           __builtin_amdgcn_s_sleep(4);
         }
+        if (ok) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
         if (!ok && p.status != nullptr) {
           if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = chunk;
         }

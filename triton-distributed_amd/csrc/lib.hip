@@ -47,9 +47,118 @@ const DeviceInfo& device_info() {
   return g_info;
 }
 
+static int wall_clock_khz() {
+  static int rate_khz = 0;   // constant-rate wall clock of the device (100 MHz on gfx950)
+  if (rate_khz == 0) {
+    int dev = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess ||
+        khz <= 0) {
+      (void)hipGetLastError();
+      return 0;
+    }
+    rate_khz = khz;
+  }
+  return rate_khz;
+}
+
 __global__ void flag_fill_kernel(int32_t* flags, int n, int value) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) __hip_atomic_store(flags + i, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Link pacing of the one-GPU producer: a time stamp of the constant-rate wall clock, and a one-wave kernel that
+// holds its stream until that clock has moved `ticks` past the stamp. The loop ends by itself: the clock only
+// moves forward, a stamp from the future makes the unsigned difference huge, and `ticks` is capped by the host.
+__global__ void producer_mark_kernel(unsigned long long* stamp) {
+  if (threadIdx.x == 0) *stamp = wall_clock64();
+}
+__global__ void producer_wait_until_kernel(const unsigned long long* stamp, unsigned long long ticks) {
+  if (threadIdx.x != 0) return;
+  const unsigned long long t0 = *stamp;
+  const unsigned long long begin = wall_clock64();
+  while (true) {
+    const unsigned long long now = wall_clock64();
+    if (now - t0 >= ticks || now - begin >= ticks) break;
+    __builtin_amdgcn_s_sleep(16);
+  }
+}
+
+// The peers' copy engines of an all-gather, played by one small kernel on the GPU that consumes the rows: block
+// row y stands for peer (rank + 1 + y) % world and pushes that peer's chunks into the workspace one after the
+// other, each no earlier than its link time, and releases the chunk's flag when the last of its workgroups has
+// stored its part. Nothing in it waits for another workgroup, and the pacing wait is bounded by the clock.
+// It is written to need few registers and no LDS so that its waves fit beside a resident GEMM wave on the same
+// SIMD: the consumer then needs no compute units set aside for the producer.
+struct PushParams {
+  unsigned char* workspace;
+  const unsigned char* const* peer_src;  // [world] device pointers; the entry of `rank` is not read
+  int32_t* flags;
+  int32_t* counters;                     // [world * chunks_per_rank], zero on entry, left zero
+  const int32_t* held;                   // optional [world * chunks_per_rank]: non-zero = never deliver (test hook)
+  const unsigned long long* stamp;       // optional: wall-clock stamp of the op's start
+  unsigned long long ticks_per_chunk;
+  long long chunk_bytes, rank_bytes;
+  int world, rank, chunks_per_rank, flag_value;
+};
+
+__global__ __launch_bounds__(256) void producer_push_kernel(const PushParams p) {
+  const int r = (p.rank + 1 + (int)blockIdx.y) % p.world;
+  const unsigned char* src = p.peer_src[r];
+  unsigned char* dst = p.workspace + (long long)r * p.rank_bytes;
+  unsigned long long t0 = 0, begin = 0;
+  if (p.stamp != nullptr && threadIdx.x == 0) {
+    t0 = *p.stamp;
+    begin = wall_clock64();
+  }
+  for (int c = 0; c < p.chunks_per_rank; ++c) {
+    const int chunk_pos = r * p.chunks_per_rank + c;
+    if (p.held != nullptr && p.held[chunk_pos] != 0) continue;
+    if (p.stamp != nullptr) {
+      if (threadIdx.x == 0) {
+        const unsigned long long due = (unsigned long long)(c + 1) * p.ticks_per_chunk;
+        while (true) {
+          const unsigned long long now = wall_clock64();
+          if (now - t0 >= due || now - begin >= due) break;
+          __builtin_amdgcn_s_sleep(16);
+        }
+      }
+      __syncthreads();
+    }
+    // Four loads in flight per lane: more would cost the registers that let these waves sit beside a GEMM wave.
+    // Addresses are a wave-uniform chunk base plus a 32-bit byte offset (chunks are below 4 GiB): one register
+    // per lane instead of a 64-bit pointer per load.
+    const unsigned char* const sbase = (const unsigned char*)src + (long long)c * p.chunk_bytes;
+    unsigned char* const dbase = (unsigned char*)dst + (long long)c * p.chunk_bytes;
+    const uint32_t nbytes = (uint32_t)p.chunk_bytes;
+    const uint32_t stride = gridDim.x * 256u * 16u;
+    auto put = [&](uint32_t off, const int4v v) { __builtin_nontemporal_store(v, (int4v*)(dbase + off)); };
+    uint32_t off = (blockIdx.x * 256u + threadIdx.x) * 16u;
+    // (the host keeps chunk_bytes + 4 * stride below 2^32, so the offsets cannot wrap)
+    for (; off + 3 * stride < nbytes; off += 4 * stride) {
+      const int4v v0 = __builtin_nontemporal_load((const int4v*)(sbase + off));
+      const int4v v1 = __builtin_nontemporal_load((const int4v*)(sbase + off + stride));
+      const int4v v2 = __builtin_nontemporal_load((const int4v*)(sbase + off + 2 * stride));
+      const int4v v3 = __builtin_nontemporal_load((const int4v*)(sbase + off + 3 * stride));
+      put(off, v0);
+      put(off + stride, v1);
+      put(off + 2 * stride, v2);
+      put(off + 3 * stride, v3);
+    }
+    for (; off < nbytes; off += stride) put(off, __builtin_nontemporal_load((const int4v*)(sbase + off)));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      // one release per workgroup and chunk: writes this XCD's dirty lines (the workgroup's rows among them) back
+      // to memory before the counter says that this part is in place
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+      int32_t* ctr = p.counters + chunk_pos;
+      const int old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (old == (int)gridDim.x - 1) {
+        __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(p.flags + chunk_pos, p.flag_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+    }
+  }
 }
 
 __global__ __launch_bounds__(256) void copy_bytes_kernel(int4v* __restrict__ dst, const int4v* __restrict__ src,
@@ -166,6 +275,67 @@ int tdist_producer_push_chunk(void* dst, const void* src, int64_t nbytes, int32_
   hipError_t e = hipMemcpyAsync(flag, one, sizeof(int32_t), kind, s);
   if (e != hipSuccess) return fail(TDIST_ERR_LAUNCH, "tdist_producer_push_chunk(flag): %s", hipGetErrorString(e));
   return TDIST_OK;
+}
+
+int tdist_producer_mark(uint64_t* stamp, void* stream) {
+  if (!stamp) return fail(TDIST_ERR_INVALID, "tdist_producer_mark: null stamp");
+  hipLaunchKernelGGL(producer_mark_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)stamp);
+  return launch_status("tdist_producer_mark");
+}
+
+int tdist_producer_wait_until(const uint64_t* stamp, int64_t offset_ns, void* stream) {
+  if (!stamp) return fail(TDIST_ERR_INVALID, "tdist_producer_wait_until: null stamp");
+  if (offset_ns < 0 || offset_ns > 100000000)
+    return fail(TDIST_ERR_INVALID, "tdist_producer_wait_until: offset %lld ns outside [0, 100 ms]", (long long)offset_ns);
+  const int rate_khz = wall_clock_khz();
+  if (rate_khz <= 0) return fail(TDIST_ERR_DEVICE, "tdist_producer_wait_until: cannot read the wall clock rate");
+  const unsigned long long ticks = (unsigned long long)((double)offset_ns * 1e-6 * (double)rate_khz);
+  hipLaunchKernelGGL(producer_wait_until_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream,
+                     (const unsigned long long*)stamp, ticks);
+  return launch_status("tdist_producer_wait_until");
+}
+
+int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int world_size, int rank,
+                              int64_t rank_bytes, int64_t chunk_bytes, int32_t* flags, int flag_value,
+                              int32_t* counters, const int32_t* held, const uint64_t* stamp, int64_t ns_per_chunk,
+                              int workgroups_per_peer, void* stream) {
+  const char* who = "tdist_producer_push_peers";
+  if (!workspace || !peer_src || !flags || !counters) return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
+  if (world_size < 1 || rank < 0 || rank >= world_size) return fail(TDIST_ERR_INVALID, "%s: rank %d / world_size %d", who, rank, world_size);
+  if (chunk_bytes <= 0 || rank_bytes <= 0 || rank_bytes % chunk_bytes != 0 || chunk_bytes % 16 != 0)
+    return fail(TDIST_ERR_INVALID, "%s: rank_bytes %lld must be a multiple of chunk_bytes %lld, itself a multiple of 16",
+                who, (long long)rank_bytes, (long long)chunk_bytes);
+  if (!aligned16(workspace)) return fail(TDIST_ERR_UNSUPPORTED, "%s: workspace must be 16-byte aligned", who);
+  if (workgroups_per_peer < 1 || workgroups_per_peer > 64) return fail(TDIST_ERR_INVALID, "%s: workgroups_per_peer in 1..64", who);
+  const int64_t cpr = rank_bytes / chunk_bytes;
+  if (cpr > 65535) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many chunks per rank", who);
+  if (chunk_bytes > (1ll << 31)) return fail(TDIST_ERR_UNSUPPORTED, "%s: chunks above 2 GiB are not supported", who);
+  if (world_size == 1) return TDIST_OK;
+  PushParams p;
+  p.workspace = (unsigned char*)workspace;
+  p.peer_src = (const unsigned char* const*)peer_src;
+  p.flags = flags;
+  p.counters = counters;
+  p.held = held;
+  p.stamp = nullptr;
+  p.ticks_per_chunk = 0;
+  if (stamp != nullptr && ns_per_chunk > 0) {
+    if (ns_per_chunk * cpr > 100000000)
+      return fail(TDIST_ERR_INVALID, "%s: %lld ns per chunk x %lld chunks is beyond the 100 ms the pacing may hold a kernel", who,
+                  (long long)ns_per_chunk, (long long)cpr);
+    const int khz = wall_clock_khz();
+    if (khz <= 0) return fail(TDIST_ERR_DEVICE, "%s: cannot read the wall clock rate", who);
+    p.stamp = (const unsigned long long*)stamp;
+    p.ticks_per_chunk = (unsigned long long)((double)ns_per_chunk * 1e-6 * (double)khz);
+  }
+  p.chunk_bytes = chunk_bytes;
+  p.rank_bytes = rank_bytes;
+  p.world = world_size;
+  p.rank = rank;
+  p.chunks_per_rank = (int)cpr;
+  p.flag_value = flag_value;
+  hipLaunchKernelGGL(producer_push_kernel, dim3(workgroups_per_peer, world_size - 1), dim3(256), 0, (hipStream_t)stream, p);
+  return launch_status(who);
 }
 
 int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {

@@ -34,6 +34,9 @@ PROTOTYPES = {
     "tdist_gemm_chunk_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
     "tdist_gemm_chunk_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
     "tdist_producer_push_chunk": (_I, [_P, _P, _L, _P, _P, _I, _P]),
+    "tdist_producer_push_peers": (_I, [_P, _P, _I, _I, _L, _L, _P, _I, _P, _P, _P, _L, _I, _P]),
+    "tdist_producer_mark": (_I, [_P, _P]),
+    "tdist_producer_wait_until": (_I, [_P, _L, _P]),
     "tdist_flag_set": (_I, [_P, _I, _P]),
     "tdist_flag_fill": (_I, [_P, _I, _I, _P]),
     "tdist_gemm_rs_scatter_bf16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P]),

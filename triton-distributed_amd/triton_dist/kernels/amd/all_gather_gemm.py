@@ -30,12 +30,16 @@ def cp_engine_producer_all_gather_full_mesh_push_multi_stream(
     arrival_order: Optional[Sequence[Tuple[int, int]]] = None,
     held_chunks: Sequence[int] = (),
     use_sdma: bool = True,
+    link_gbps: float = 0.0,
+    start_stamp: Optional[torch.Tensor] = None,
 ):
     """Delivers the peers' shards into ``workspace`` chunk by chunk: data copy, then a 4-byte copy of
     ``one`` into the chunk's flag on the same stream (reference :80-100). ``arrival_order`` is a list of
     (peer_rank, chunk_in_rank); the default is the reference's (:54-66): peers rank+1, rank+2, ... each
     on its own stream, chunks in order. Chunks listed in ``held_chunks`` (global chunk ids) are never
-    delivered — a test hook for the bounded wait."""
+    delivered — a test hook for the bounded wait. With ``link_gbps`` > 0 every peer's n-th chunk is held back
+    until n * chunk_bytes / link rate after ``start_stamp`` (a device time stamp taken when the op started): the
+    pace at which a peer's copy engine would deliver it over one xGMI link."""
     some = next(iter(peer_shards.values()))
     M_per_rank, K = some.shape
     chunk_num_per_rank = M_per_rank // M_PER_CHUNK
@@ -48,6 +52,7 @@ def cp_engine_producer_all_gather_full_mesh_push_multi_stream(
             arrival_order += [(r, c) for c in range(chunk_num_per_rank)]
     held = set(int(c) for c in held_chunks)
     n_streams = len(ag_stream_pool)
+    sent: Dict[int, int] = {}
     for r, c in arrival_order:
         if r == rank:
             continue
@@ -59,8 +64,38 @@ def cp_engine_producer_all_gather_full_mesh_push_multi_stream(
         src_ptr = src.data_ptr() + c * M_PER_CHUNK * K * esz
         dst_ptr = workspace.data_ptr() + (r * M_per_rank + c * M_PER_CHUNK) * K * esz
         flag_ptr = barrier.data_ptr() + chunk_pos * 4
+        if link_gbps > 0:
+            sent[r] = sent.get(r, 0) + 1
+            _lib.call("tdist_producer_wait_until", start_stamp.data_ptr(), int(sent[r] * nbytes / link_gbps),
+                      stream.cuda_stream)
         _lib.call("tdist_producer_push_chunk", dst_ptr, src_ptr, nbytes, flag_ptr, one.data_ptr(),
                   1 if use_sdma else 0, stream.cuda_stream)
+
+
+def kernel_producer_all_gather_push(rank, num_ranks, ctx, workspace, M_PER_CHUNK, stream, barrier):
+    """The peers' pushes as ONE launch of tdist_producer_push_peers (a block row per peer, pacing inside the kernel):
+    the same data-then-flag protocol as the copy-engine producer above with a single host call, and light enough
+    on registers to share compute units with the GEMM."""
+    some = next(iter(ctx.peer_shards.values()))
+    M_per_rank, K = some.shape
+    esz = some.element_size()
+    n_chunks = num_ranks * (M_per_rank // M_PER_CHUNK)
+    if ctx.arrival_order is not None:
+        raise ValueError("the kernel producer delivers every peer's chunks in order; arrival_order needs the copy producer")
+    if ctx.producer_counters is None or ctx.producer_counters.numel() < n_chunks:
+        ctx.producer_counters = torch.zeros(n_chunks, dtype=torch.int32, device=some.device)
+    held = None
+    if ctx.held_chunks:
+        held = torch.zeros(n_chunks, dtype=torch.int32)
+        held[list(int(c) for c in ctx.held_chunks)] = 1
+        held = held.to(some.device)
+    ctx.held_mask = held   # stays alive until the next call replaces it
+    paced = ctx.link_gbps > 0
+    nbytes = M_PER_CHUNK * K * esz
+    _lib.call("tdist_producer_push_peers", workspace.data_ptr(), ctx.peer_ptrs.data_ptr(), num_ranks, rank,
+              M_per_rank * K * esz, nbytes, barrier.data_ptr(), 1, ctx.producer_counters.data_ptr(), _lib.ptr(held),
+              ctx.start_stamp.data_ptr() if paced else None, int(nbytes / ctx.link_gbps) if paced else 0,
+              int(ctx.producer_workgroups), stream.cuda_stream)
 
 
 @dataclasses.dataclass
@@ -98,6 +133,18 @@ class AllGatherGEMMTensorParallelContext:
     # GEMM on the same queue can never run, and the bounded wait then reports a timeout.
     gemm_first: bool = False
     preset_flags: bool = False   # debug: release every flag before the GEMM starts (no overlap)
+    # > 0: pace the arrivals like one xGMI link per peer (GB/s; a link of MI355X moves ~153): a peer's n-th chunk is
+    # copied no earlier than n * chunk_bytes / rate after the op started. 0: chunks are copied as fast as this GPU can.
+    link_gbps: float = 0.0
+    start_stamp: Optional[torch.Tensor] = None   # int64[1], device wall-clock stamp of the current call
+    # True: the peers' pushes are one launch of a small kernel (a block row per peer) instead of two async copies
+    # per chunk on the copy streams. Its waves fit beside the GEMM's on a SIMD, so no compute units are set aside
+    # (producer_cus is ignored) and the host queues three launches per call, however many chunks there are.
+    producer_kernel: bool = False
+    producer_workgroups: int = 8   # workgroups per peer of that kernel
+    producer_counters: Optional[torch.Tensor] = None
+    peer_ptrs: Optional[torch.Tensor] = None   # int64[num_ranks] device array of the peer shards' addresses
+    held_mask: Optional[torch.Tensor] = None
     # Compute units the gated GEMM leaves to the producer's copies. On one GPU those copies need compute
     # units of this GPU; measured on MI355X they make no progress next to a full-chip persistent grid
     # unless 32 units stay free. A peer's copy engine pushing over xGMI would need none.
@@ -128,6 +175,8 @@ class AllGatherGEMMTensorParallelContext:
             if not t.is_contiguous():
                 raise ValueError("peer shard of rank %d must be contiguous" % r)
         self.peer_shards = {r: t for r, t in shards.items() if r != self.rank}
+        ptrs = [self.peer_shards[r].data_ptr() if r in self.peer_shards else 0 for r in range(self.num_ranks)]
+        self.peer_ptrs = torch.tensor(ptrs, dtype=torch.int64).to(self.one.device)
 
     def check_status(self):
         """Synchronises and raises TdistError if a bounded flag wait expired in an earlier call."""
@@ -170,6 +219,7 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
     _gemm_stream = current_stream if gemm_stream is None else gemm_stream
     one = torch.ones((1024, ), dtype=torch.int32, device=device)
     status = torch.zeros((2, ), dtype=torch.int32, device=device)
+    start_stamp = torch.zeros((1, ), dtype=torch.int64, device=device)
     torch.cuda.synchronize()
 
     return AllGatherGEMMTensorParallelContext(
@@ -191,6 +241,7 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
         autotune=autotune,
         output_dtype=output_dtype,
         status=status,
+        start_stamp=start_stamp,
     )
 
 
@@ -254,17 +305,25 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
                 "(ctx.set_peer_shards); missing ranks %s" % missing)
 
     current_stream = torch.cuda.current_stream()
+    paced = ctx is not None and ctx.link_gbps > 0 and num_ranks > 1
+    if paced:
+        _lib.call("tdist_producer_mark", ctx.start_stamp.data_ptr(), current_stream.cuda_stream)
     gemm_stream.wait_stream(current_stream)
     for ag_stream in ag_streams:
         ag_stream.wait_stream(current_stream)
 
+    use_kernel = ctx is not None and ctx.producer_kernel
+
     def call_ag():
-        if num_ranks > 1:
+        if num_ranks > 1 and use_kernel:
+            kernel_producer_all_gather_push(rank, num_ranks, ctx, workspace, M_PER_CHUNK, ag_streams[0], barrier)
+        elif num_ranks > 1:
             cp_engine_producer_all_gather_full_mesh_push_multi_stream(
                 rank, num_ranks, peer_shards, workspace, one, M_PER_CHUNK, ag_streams, barrier,
                 arrival_order=ctx.arrival_order if ctx is not None else None,
                 held_chunks=ctx.held_chunks if ctx is not None else (),
-                use_sdma=ctx.use_sdma if ctx is not None else True)
+                use_sdma=ctx.use_sdma if ctx is not None else True,
+                link_gbps=ctx.link_gbps if paced else 0.0, start_stamp=ctx.start_stamp if paced else None)
 
     def call_gemm(max_wgs):
         with torch.cuda.stream(gemm_stream):
@@ -283,7 +342,7 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
         call_gemm(0)
     else:
         max_wgs = 0
-        if ctx is not None and num_ranks > 1 and ctx.producer_cus > 0:
+        if ctx is not None and num_ranks > 1 and ctx.producer_cus > 0 and not use_kernel:
             max_wgs = max(1, _lib.load().tdist_num_cus() - ctx.producer_cus)
         if ctx is not None and ctx.gemm_first:
             call_gemm(max_wgs)
