@@ -502,18 +502,31 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams
   float L = 0.f;
   constexpr int kMaxPerLane = 8;  // Dv <= 512
   float acc[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const int per_lane = (prm.Dv + 63) >> 6;
   if (M != -INFINITY) {
-    for (int j = 0; j < prm.P; ++j) {
-      if (skipped(j)) continue;
-      const float lj = lse[(int64_t)j * prm.l_sp];
-      if (lj == -INFINITY) continue;
-      const float w = __expf(lj - M);
-      L += w;
-      const int64_t base = (int64_t)j * prm.p_sp + (int64_t)b * prm.p_sb + (int64_t)h * prm.p_sh;
+    // four partials at a time: their loads are issued together, the sums stay in partial order
+    constexpr int kBatch = 4;
+    for (int j0 = 0; j0 < prm.P; j0 += kBatch) {
+      float w[kBatch];
+      float x[kBatch][kMaxPerLane];
 #pragma unroll
-      for (int u = 0; u < kMaxPerLane; ++u) {
-        const int d = lane + u * 64;
-        if (d < prm.Dv) acc[u] += w * load_elem(prm.part, base + d, prm.part_dtype);
+      for (int u = 0; u < kBatch; ++u) {
+        const int j = j0 + u;
+        float lj = -INFINITY;
+        if (j < prm.P && !skipped(j)) lj = lse[(int64_t)j * prm.l_sp];
+        w[u] = lj == -INFINITY ? 0.f : __expf(lj - M);
+        const int64_t base = (int64_t)min(j, prm.P - 1) * prm.p_sp + (int64_t)b * prm.p_sb + (int64_t)h * prm.p_sh;
+#pragma unroll
+        for (int q = 0; q < kMaxPerLane; ++q) {
+          const int d = lane + q * 64;
+          x[u][q] = (q < per_lane && d < prm.Dv && lj != -INFINITY) ? load_elem(prm.part, base + d, prm.part_dtype) : 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        L += w[u];   // a skipped, empty or out-of-range partial has w = 0 and x = 0: it adds nothing
+#pragma unroll
+        for (int q = 0; q < kMaxPerLane; ++q) acc[q] += w[u] * x[u][q];
       }
     }
   }
