@@ -76,6 +76,40 @@ def main():
     np.savez_compressed(os.path.join(HERE, "decode_2seq.npz"), q=bits16(qd), k_cache=bits16(k_cache), v_cache=bits16(v_cache),
                         block_table=table.numpy(), kv_lens=np.array(kv_lens, dtype=np.int32), out=out.numpy(), lse=lse.numpy(),
                         part=part.numpy(), part_lse=part_lse.numpy(), meta=np.array([Hq, Hkv, D, page, S]))
+
+    # decode with extra key dimensions: 2 sequences (100 and 37 keys), 4 query heads over 1 kv head, key dim 192,
+    # value dim 128, page 4, 3 splits, f16, soft cap 30
+    g = torch.Generator().manual_seed(105)
+    kv_lens, Hq, Hkv, Dk, Dv, page, S, cap = [100, 37], 4, 1, 192, 128, 4, 3, 30.0
+    qd = torch.randn((2, Hq, Dk), generator=g).to(torch.float16)
+    k_cache, v_cache, table = golden.make_paged_kv(2, max(kv_lens), Hkv, Dk, page, torch.float16, g, v_head_dim=Dv)
+    scale = Dk**-0.5
+    out, lse = golden.decode_exact(qd, k_cache, v_cache, kv_lens, table, scale, cap)
+    part, part_lse = golden.decode_split_exact(qd, k_cache, v_cache, kv_lens, table, scale, S, cap)
+    np.savez_compressed(os.path.join(HERE, "decode_dk192_dv128.npz"), q=bits16(qd), k_cache=bits16(k_cache),
+                        v_cache=bits16(v_cache), block_table=table.numpy(), kv_lens=np.array(kv_lens, dtype=np.int32),
+                        out=out.numpy(), lse=lse.numpy(), part=part.numpy(), part_lse=part_lse.numpy(),
+                        meta=np.array([Hq, Hkv, Dk, Dv, page, S, int(cap)]))
+
+    # align / sort for the grouped GEMM: 4 rank segments x 24 tokens x top-3 over 10 experts, block 8
+    g = torch.Generator().manual_seed(106)
+    R, Tr, topk, E, block = 4, 24, 3, 10, 8
+    ids = golden.random_distinct_experts(R * Tr, E, topk, g)
+    sorted_ids, expert_ids, barrier_ids, rank_blocks, post_pad = golden.sort_topk_ids_align_block_size(ids, E, R, Tr, block)
+    np.savez_compressed(os.path.join(HERE, "moe_align_4x24x3.npz"), ids=ids.numpy(), sorted_token_ids=sorted_ids.numpy(),
+                        expert_ids=expert_ids.numpy(), block_barrier_ids=barrier_ids.numpy(),
+                        rank_block_num=rank_blocks.numpy(), meta=np.array([R, Tr, topk, E, block, int(post_pad)]))
+
+    # e4m3 quantisation in groups of 128 columns: 6 rows x 384 columns bf16 (one all-zero group, one with a huge entry)
+    g = torch.Generator().manual_seed(107)
+    x = torch.randn((6, 384), generator=g)
+    x[1, 128:256] = 0.0
+    x[2, 5] = 3.0e4
+    x = x.to(torch.bfloat16)
+    qx, sx = golden.quantize_groups_e4m3(x)
+    np.savez_compressed(os.path.join(HERE, "quant_groups_6x384.npz"), x=bits16(x), q_u8=qx.view(torch.uint8).numpy(),
+                        scales=sx.numpy())
+
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

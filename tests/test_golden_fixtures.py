@@ -59,6 +59,63 @@ def test_decode_fixture():
     assert np.allclose(out, f["out"], atol=1e-10) and np.allclose(lse, f["lse"], atol=1e-10)
 
 
+def f16(bits):
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.float16)
+
+
+def test_decode_fixture_with_extra_key_dimensions():
+    f = load("decode_dk192_dv128.npz")
+    Hq, Hkv, Dk, Dv, page, S, cap = f["meta"].tolist()
+    q, k, v = f16(f["q"]), f16(f["k_cache"]), f16(f["v_cache"])
+    assert q.shape[-1] == Dk and k.shape[-1] == Dk and v.shape[-1] == Dv
+    out, lse = cref.decode_range(q.float().numpy(), k.float().numpy(), v.float().numpy(), f["block_table"], [0, 0],
+                                 f["kv_lens"], Dk**-0.5, float(cap))
+    assert np.allclose(out, f["out"], atol=1e-10) and np.allclose(lse, f["lse"], atol=1e-10)
+    # the frozen per-split partials merge to the frozen full result
+    merged, merged_lse = golden.lse_merge(torch.from_numpy(f["part"]).permute(2, 0, 1, 3), torch.from_numpy(f["part_lse"]).permute(2, 0, 1))
+    assert np.allclose(merged.numpy(), f["out"], atol=1e-12) and np.allclose(merged_lse.numpy(), f["lse"], atol=1e-12)
+
+
+def test_align_sort_fixture_invariants():
+    """The frozen align / sort output against what the layout fixes, without calling the oracle: every block holds one
+    expert's entries of one rank segment in ascending flat order, padding carries the fill value, every entry
+    appears exactly once."""
+    f = load("moe_align_4x24x3.npz")
+    R, Tr, topk, E, block, post_pad = f["meta"].tolist()
+    ids = f["ids"].reshape(-1)
+    n = ids.size
+    sorted_ids, expert_ids, barrier_ids, rank_blocks = f["sorted_token_ids"], f["expert_ids"], f["block_barrier_ids"], f["rank_block_num"]
+    assert post_pad % block == 0 and expert_ids.size == post_pad // block == barrier_ids.size == rank_blocks.sum()
+    assert np.array_equal(barrier_ids, np.repeat(np.arange(R), rank_blocks))
+    seen = []
+    for blk in range(post_pad // block):
+        entries = sorted_ids[blk * block:(blk + 1) * block]
+        real = entries[entries < n]
+        assert (entries[len(real):] == n).all(), "padding sits at the end of a block"
+        assert (np.diff(real) > 0).all() and (ids[real] == expert_ids[blk]).all()
+        assert (real // (Tr * topk) == barrier_ids[blk]).all()
+        seen.append(real)
+    assert np.array_equal(np.sort(np.concatenate(seen)), np.arange(n))
+    assert (sorted_ids[post_pad:] == n).all()
+    got = golden.sort_topk_ids_align_block_size(torch.from_numpy(f["ids"]), E, R, Tr, block)
+    assert np.array_equal(got[0].numpy(), sorted_ids) and np.array_equal(got[1].numpy(), expert_ids)
+
+
+def test_group_quant_fixture_closed_form():
+    f = load("quant_groups_6x384.npz")
+    x = bf16(f["x"]).float().view(6, 3, 128)
+    scales = torch.from_numpy(f["scales"])
+    assert torch.equal(scales, x.abs().amax(-1) * torch.tensor(1.0 / 448.0))
+    q = torch.from_numpy(f["q_u8"]).view(torch.float8_e4m3fn).float().view(6, 3, 128)
+    assert (q[1, 1] == 0).all() or torch.isnan(q[1, 1]).all()          # an all-zero group: 0 / 0
+    live = scales > 0
+    assert (q.abs().amax(-1)[live] == 448).all()                       # the largest element of a group maps to 448
+    deq = q * scales[..., None]
+    # half an e4m3 step (3 mantissa bits) of the magnitude, or half the smallest subnormal step (2^-9) times the scale
+    bound = torch.maximum(2.0**-4 * x.abs(), 2.0**-10 * scales[..., None].expand_as(x))
+    assert ((deq - x).abs()[live] <= bound[live] * 1.0001).all()
+
+
 # ---- GPU: the HIP path against the frozen vectors ------------------------------------------------------
 @pytest.mark.gpu
 def test_gpu_against_fixtures(cuda):
@@ -111,3 +168,31 @@ def test_gpu_against_fixtures(cuda):
     finite = np.isfinite(d["part_lse"])
     assert np.array_equal(np.isfinite(lse_split.cpu().numpy()), finite)
     assert np.abs(lse_split.cpu().numpy()[finite] - d["part_lse"][finite]).max() <= 2e-3
+    announce("fixtures: decode with extra key dimensions, align / sort, group quantiser")
+    d = load("decode_dk192_dv128.npz")
+    Hq, Hkv, Dk, Dv, page, S, cap = d["meta"].tolist()
+    out_split, lse_split, _ = _split_kv(f16(d["q"]).to(cuda), f16(d["k_cache"]).to(cuda), f16(d["v_cache"]).to(cuda),
+                                        torch.from_numpy(d["kv_lens"]).to(cuda), torch.from_numpy(d["block_table"]).to(cuda),
+                                        Dk**-0.5, float(cap), S)
+    torch.cuda.synchronize()
+    assert np.abs(out_split.cpu().numpy() - d["part"]).max() <= 2e-3
+    finite = np.isfinite(d["part_lse"])
+    assert np.array_equal(np.isfinite(lse_split.cpu().numpy()), finite)
+    assert np.abs(lse_split.cpu().numpy()[finite] - d["part_lse"][finite]).max() <= 2e-3
+    from triton_dist.kernels.amd import quant_bf16_fp8, sort_topk_ids_align_block_size
+    a = load("moe_align_4x24x3.npz")
+    R, Tr, topk, E, block, post_pad = a["meta"].tolist()
+    got = sort_topk_ids_align_block_size(torch.from_numpy(a["ids"]).to(cuda), E, R, Tr, block)
+    torch.cuda.synchronize()
+    assert int(got[4]) == post_pad
+    assert np.array_equal(got[0].cpu().numpy()[:a["sorted_token_ids"].size], a["sorted_token_ids"])
+    nb = post_pad // block
+    assert np.array_equal(got[1].cpu().numpy()[:nb], a["expert_ids"]) and np.array_equal(got[2].cpu().numpy()[:nb], a["block_barrier_ids"])
+    assert np.array_equal(got[3].cpu().numpy(), a["rank_block_num"])
+    qf = load("quant_groups_6x384.npz")
+    qx, sx = quant_bf16_fp8(bf16(qf["x"]).to(cuda))
+    torch.cuda.synchronize()
+    assert np.array_equal(sx.cpu().numpy(), qf["scales"])
+    want_q, got_q = qf["q_u8"].reshape(6, 3, 128), qx.view(torch.uint8).cpu().numpy().reshape(6, 3, 128)
+    live = qf["scales"] > 0
+    assert np.array_equal(got_q[live], want_q[live])      # (an all-zero group is 0 / 0: NaN on both sides, payload free)
