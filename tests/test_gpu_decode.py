@@ -246,3 +246,23 @@ def test_full_size_shard_sampled(cuda):
         exact, exact_lse = golden.decode_exact(q_dev[b:b + 1].cpu(), k_b, v_b, [L], t_b, scale)
         assert (merged[b].cpu().double() - exact[0]).abs().max() <= ATOL
         assert (merged_lse[b].cpu().double() - exact_lse[0]).abs().max() <= ATOL
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+def test_alternative_block_shapes(cuda, monkeypatch, variant):
+    """The other compiled block shapes for D = 128 (keys per block, waves, stages), selectable for measurements:
+    same partials and LSE within the bar."""
+    from triton_dist.kernels.amd.flash_decode import _split_kv
+    monkeypatch.setenv("TDIST_DECODE_VARIANT", str(variant))
+    kv_lens, S, heads, D, page = [1320, 18, 463, 5], 8, (32, 8), 128, 16
+    announce("decode block shape variant %d" % variant)
+    q, k_cache, v_cache, table = build_case(kv_lens, heads, D, page, torch.bfloat16, seed=40 + variant)
+    lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
+    out_split, lse_split, _ = _split_kv(q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), lens_dev, table.to(cuda), D**-0.5, 0.0, S)
+    torch.cuda.synchronize()
+    w_out, w_lse = golden.decode_split_exact(q, k_cache, v_cache, kv_lens, table, D**-0.5, S)
+    empty = torch.isinf(w_lse)
+    got_lse = lse_split.cpu().double()
+    assert torch.equal(torch.isinf(got_lse), empty)
+    assert (got_lse[~empty] - w_lse[~empty]).abs().max() <= ATOL
+    assert (out_split.cpu().double() - w_out).abs().max() <= ATOL

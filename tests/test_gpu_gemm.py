@@ -469,3 +469,30 @@ def test_ag_gemm_kernel_producer_and_graph_replay(cuda, producer_kernel, link_gb
     ctx.check_status()
     if producer_kernel:
         assert int(ctx.producer_counters.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("variant", [2, 5])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
+def test_alternative_schedules_of_the_large_tile(cuda, monkeypatch, variant, dtype):
+    """The two other compiled schedules of the 256 x 256 tile (eight waves on a two-stage ring and on the split
+    ring), selectable for measurements, give the same exact result on integer-valued inputs."""
+    from triton_dist.kernels.amd import gated_gemm
+    monkeypatch.setenv("TDIST_GEMM_VARIANT", str(variant))
+    monkeypatch.setenv("TDIST_GEMM_TILE", "0")
+    esz = 1 if dtype == torch.float8_e4m3fn else 2
+    M, N, K = 1100, 780, 640 // esz
+    announce("gemm schedule variant %d %s" % (variant, dtype))
+    g = torch.Generator().manual_seed(variant)
+    a = torch.randint(-2, 3, (M, K), generator=g).float()
+    b = torch.randint(-2, 3, (N, K), generator=g).float()
+    c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+    sa = sb = None
+    if dtype == torch.float8_e4m3fn:
+        sa = (2.0 ** torch.randint(-3, 3, (M,), generator=g).float()).to(cuda)
+        sb = (2.0 ** torch.randint(-3, 3, (N,), generator=g).float()).to(cuda)
+    gated_gemm(a.to(dtype).to(cuda), None, 0, b.to(dtype).to(cuda), c, None, 0, 0, 1, row_scale=sa, col_scale=sb)
+    torch.cuda.synchronize()
+    ref = a.to(cuda) @ b.to(cuda).T
+    if sa is not None:
+        ref = ref * sa[:, None] * sb[None, :]
+    assert torch.equal(c, ref.to(torch.bfloat16))
