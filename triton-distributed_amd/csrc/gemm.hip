@@ -538,24 +538,41 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       __builtin_amdgcn_sched_barrier(0);  // keep the accumulator read-out block by block (register pressure)
     };
     // staged rows [row0, row0 + nrows) of the wave tile → global memory, 16 bytes per lane
+    // one staged 16-byte piece → global memory
+    auto store_piece = [&](int mrow, const int4v v) {
+      const int gm = m0 + wm * C::kWaveM + mrow;
+      const int gn = n0 + wn * C::kWaveN + ec * 8;
+      if (gm < p.M && gn < p.N) {
+        unsigned short* dst = (unsigned short*)Cbase + (crow0 + wm * C::kWaveM + mrow) * p.ldc + gn;
+        if (gn + 8 <= p.N && n_vec_ok) {
+          if (p.scatter_bufs == nullptr) __builtin_nontemporal_store(v, (int4v*)dst);  // written once, not read back here
+          else *(int4v*)dst = v;
+        } else {
+          for (int e = 0; e < 8; ++e)
+            if (gn + e < p.N) dst[e] = (unsigned short)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+        }
+      }
+    };
+    auto staged_piece = [&](int mrow) -> int4v {
+      return *(const TDIST_AS3 int4v*)(epi + mrow * C::kEpiPitch + ((ec ^ (mrow & C::kEpiSwz)) << 4));
+    };
+    // staged rows [row0, row0 + nrows) of the wave tile → global memory, 16 bytes per lane
     auto store_rows = [&](int row0, int nrows) {
 #pragma unroll 4
       for (int pass = 0; pass < nrows / kRowsPerPass; ++pass) {
         const int mrow = row0 + pass * kRowsPerPass + er;
-        const int gm = m0 + wm * C::kWaveM + mrow;
-        const int gn = n0 + wn * C::kWaveN + ec * 8;
-        const int4v v = *(const TDIST_AS3 int4v*)(epi + mrow * C::kEpiPitch + ((ec ^ (mrow & C::kEpiSwz)) << 4));
-        if (gm < p.M && gn < p.N) {
-          unsigned short* dst = (unsigned short*)Cbase + (crow0 + wm * C::kWaveM + mrow) * p.ldc + gn;
-          if (gn + 8 <= p.N && n_vec_ok) {
-            if (p.scatter_bufs == nullptr) __builtin_nontemporal_store(v, (int4v*)dst);  // written once, not read back here
-            else *(int4v*)dst = v;
-          } else {
-            for (int e = 0; e < 8; ++e)
-              if (gn + e < p.N) dst[e] = (unsigned short)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
-          }
-        }
+        store_piece(mrow, staged_piece(mrow));
       }
+    };
+    // the same for one 32-row block with all its LDS reads issued before the first store, so that no store waits for
+    // the LDS round trip of its own read (costs 32 registers: used where the instance has them)
+    auto store_block32 = [&](int row0) {
+      constexpr int kPasses = 32 / kRowsPerPass;
+      int4v v[kPasses];
+#pragma unroll
+      for (int u = 0; u < kPasses; ++u) v[u] = staged_piece(row0 + u * kRowsPerPass + er);
+#pragma unroll
+      for (int u = 0; u < kPasses; ++u) store_piece(row0 + u * kRowsPerPass + er, v[u]);
     };
     static_assert(32 % kRowsPerPass == 0, "a 32-row block is a whole number of store passes");
 
@@ -567,7 +584,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         for (int j = 0; j < C::kTN; ++j) stage_block(i, j, 1.f, nullptr);
         __builtin_amdgcn_wave_barrier();
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        store_rows(32 * i, 32);
+        if constexpr (C::kWaves <= 4 && C::kFragVecs == 1) store_block32(32 * i);
+        else store_rows(32 * i, 32);
       }
     } else {
       float rs[C::kTM];
