@@ -396,6 +396,47 @@ def bench_c5(dev, steps, warmup):
     return r
 
 
+def bench_group_gemm(dev, steps, warmup):
+    """AG + grouped GEMM of the MoE tensor-parallel path at the reference's Mixtral-8x7B layer shape
+    (test/nvidia/test_ag_moe.py:160-171: K 14336, N 4096 over 8 ranks, 8 experts, top-2) with 8192 tokens: the step
+    that consumes the align / sort output. Not a BASELINE config; reported beside them."""
+    import torch
+    from oracle import golden
+    from triton_dist.kernels.amd import (ag_group_gemm_intra_node, create_ag_group_gemm_intra_node_context,
+                                         group_gemm_gated)
+    world, rank, mpr, K, N, E, topk, block = 8, 0, 1024, 14336, 512, 8, 2, 128
+    g = torch.Generator().manual_seed(3 + 7)
+    shards = [torch.randn((mpr, K), generator=g).to(torch.bfloat16) for _ in range(world)]
+    w_nk = (torch.randn((E, N, K), generator=g) * 0.02).to(torch.bfloat16).to(dev)
+    w = w_nk.transpose(1, 2)                       # [E, K, N] as the reference takes it, K-contiguous underneath
+    ids = golden.random_distinct_experts(world * mpr, E, topk, g).to(dev)
+    a_d = shards[rank].to(dev)
+    ctx = create_ag_group_gemm_intra_node_context(None, a_d, w, ids, E, max_M=world * mpr, BLOCK_M=block, rank=rank,
+                                                  num_ranks=world)
+    ctx.set_peer_shards({r: s.to(dev) for r, s in enumerate(shards) if r != rank})
+    flops = 2.0 * world * mpr * topk * K * N
+    live_s = None
+    if LIVE_PRODUCER:
+        c = ag_group_gemm_intra_node(a_d, w, ctx)
+        ctx.check_status()
+        rows = torch.arange(5 * mpr * topk + 3, 5 * mpr * topk + 67)
+        ref = golden.ag_group_gemm_fp32(shards, w.cpu(), ids.cpu())[rows]
+        assert golden.max_rel_err(c[rows.to(dev)].float().cpu(), ref) <= 1e-2
+        live_s = time_launches(lambda: ag_group_gemm_intra_node(a_d, w, ctx), steps, warmup)
+        ctx.check_status()
+    full = torch.cat(shards).to(dev)
+    flags = torch.ones(world, dtype=torch.int32, device=dev)
+    out = torch.empty((world * mpr * topk, N), dtype=torch.bfloat16, device=dev)
+    pre_s = time_launches(
+        lambda: group_gemm_gated(full, None, 0, w_nk, out, ctx.sorted_topk_ids, ctx.aligned_expert_ids,
+                                 ctx.aligned_barrier_ids, ctx.aligned_num_tokens, block, ctx.full_num_tokens, topk, mpr,
+                                 ctx.first_block, flags, rank), steps, warmup)
+    r = roof("mfma", flops, pre_s, "bf16")
+    r["workload"] = "8192 tokens x top-2 of 8 experts, K 14336, N 512 per rank, row blocks of 128 (128 x 256 tiles)"
+    r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
+    return r
+
+
 def bench_copy(dev, steps, warmup):
     import torch
     from triton_dist import _lib
@@ -431,7 +472,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle-seconds", type=float, default=SETTLE_SECONDS,
                     help="untimed period of the same launches before each warm-up, to reach the sustained clock")
-    ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,copy,mfma (c2 always runs)")
+    ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,moe_gemm,copy,mfma (c2 always runs)")
     ap.add_argument("--no-live-producer", action="store_true",
                     help="skip the AG-GEMM legs in which a copy stream releases the flags while the GEMM spins: a "
                     "counter-collecting profiler serialises dispatches, so the producer could never run beside it")
@@ -450,7 +491,7 @@ def main():
     _lib.check(_lib.load().tdist_init())
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    want = set(x for x in args.only.split(",") if x) or {"c1", "c2", "c3", "c4", "c5", "copy", "mfma"}
+    want = set(x for x in args.only.split(",") if x) or {"c1", "c2", "c3", "c4", "c5", "moe_gemm", "copy", "mfma"}
 
     step_s, gemm_roof, red_roof, cpu, err = bench_c2(dev, args.steps, args.warmup)
     log("c2 step %.1f us, gemm %s, reduce %s" % (step_s * 1e6, gemm_roof, red_roof))
@@ -468,6 +509,9 @@ def main():
     if "c5" in want:
         kernels["c5_decode_split_kv_bf16"] = bench_c5(dev, args.steps, args.warmup)
         log("c5", kernels["c5_decode_split_kv_bf16"])
+    if "moe_gemm" in want:
+        kernels["ag_group_gemm_bf16_mixtral_8x7b_tp8"] = bench_group_gemm(dev, args.steps, args.warmup)
+        log("moe_gemm", kernels["ag_group_gemm_bf16_mixtral_8x7b_tp8"])
     if "copy" in want:
         kernels["copy_1GiB_yardstick"] = bench_copy(dev, args.steps, args.warmup)
         log("copy", kernels["copy_1GiB_yardstick"])

@@ -271,6 +271,45 @@ int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_to
                                int32_t* expert_ids, int32_t* block_barrier_ids, int32_t* rank_block_num,
                                int32_t* total_tokens_post_pad, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Chunk-gated grouped GEMM of the MoE tensor-parallel path: the consumer of the align / sort step.
+ *   replaces kernel_consumer_m_parallel_scatter_group_gemm   kernels/nvidia/allgather_group_gemm.py:238-314
+ *   as launched by rowise_intranode_ag_scatter_group_gemm    kernels/nvidia/allgather_group_gemm.py:317-403
+ * Row block m (block_size rows of the sorted space, one expert, one rank segment):
+ *   C[sorted_token_ids[m*bs + r], :] = A[sorted_token_ids[m*bs + r] / topk, :] . B[expert_ids[m]]^T
+ * for the rows whose id is < num_valid_tokens (the rest is padding: read as some valid row, never stored), after
+ * flags[block_barrier_ids[m]] == wait_value (dl.wait on block_barrier_ptr, :285-287); blocks at or beyond
+ * *num_tokens_post_padded (device int32) are skipped (:274-277). Blocks are taken from first_block on, wrapping
+ * (the reference rotates by rank, :263-270): pass the own segment's first block.
+ * A [a_rows, K] gathered tokens (lda), A_local optional own shard (tokens [local_row_begin, +local_rows), never
+ * waited for); B: expert e's weights at B + e*expert_stride, [N, K] with K contiguous and row stride ldb (the
+ * reference takes [E, K, N] with explicit strides: pass a K-contiguous copy or view); C [num_valid_tokens, N]
+ * (ldc), of the input dtype (bf16 for e4m3). block_size 128 or 256 = the block_size given to the align / sort;
+ * num_blocks = capacity of expert_ids / block_barrier_ids (sorted_token_ids holds num_blocks*block_size ids).
+ * tokens_per_rank: tokens of one rank segment. spin_limit / status / max_workgroups as for the gated GEMM;
+ * status[1] is the rank segment whose flag did not arrive. */
+int tdist_group_gemm_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local, int local_row_begin,
+                                int local_rows, const void* B, int64_t ldb, int64_t expert_stride, void* C, int64_t ldc,
+                                int a_rows, int N, int K, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                const int32_t* block_barrier_ids, const int32_t* num_tokens_post_padded, int num_blocks,
+                                int block_size, int num_valid_tokens, int topk, int tokens_per_rank, int first_block,
+                                const int32_t* flags, int wait_value, int rank, int spin_limit, int32_t* status,
+                                int max_workgroups, void* stream);
+int tdist_group_gemm_gated_f16(const void* A, int64_t lda, const void* A_local, int64_t lda_local, int local_row_begin,
+                               int local_rows, const void* B, int64_t ldb, int64_t expert_stride, void* C, int64_t ldc,
+                               int a_rows, int N, int K, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                               const int32_t* block_barrier_ids, const int32_t* num_tokens_post_padded, int num_blocks,
+                               int block_size, int num_valid_tokens, int topk, int tokens_per_rank, int first_block,
+                               const int32_t* flags, int wait_value, int rank, int spin_limit, int32_t* status,
+                               int max_workgroups, void* stream);
+int tdist_group_gemm_gated_fp8e4m3(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
+                                   int local_row_begin, int local_rows, const void* B, int64_t ldb,
+                                   int64_t expert_stride, void* C, int64_t ldc, int a_rows, int N, int K,
+                                   const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                   const int32_t* block_barrier_ids, const int32_t* num_tokens_post_padded,
+                                   int num_blocks, int block_size, int num_valid_tokens, int topk, int tokens_per_rank,
+                                   int first_block, const int32_t* flags, int wait_value, int rank, int spin_limit,
+                                   int32_t* status, int max_workgroups, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * (d) split-KV GQA flash decode + LSE combine.
  *   replaces kernel_gqa_fwd_batch_decode_split_kv               kernels/nvidia/flash_decode.py:129-239

@@ -392,6 +392,28 @@ def sort_topk_ids_align_block_size(topk_ids, num_experts, num_ranks, num_tokens_
 # ---------------------------------------------------------------------------------------------------
 # e4m3 quantisation in groups of 128 columns (the fused form of the dispatch)
 # ---------------------------------------------------------------------------------------------------
+def torch_moe_scatter_group_gemm(in_features, expert_weights, topk_ids):
+    """test/nvidia/test_ag_moe.py:20-38: every (token, k) row is the token's features times the weights of its k-th
+    expert. in_features [M, K], expert_weights [E, K, N], topk_ids [M, topk] → [M * topk, N] in the input dtype."""
+    M, K = in_features.shape
+    in_features = in_features.view(M, -1, K).repeat(1, topk_ids.shape[1], 1).reshape(-1, K)
+    out = torch.zeros(M * topk_ids.shape[1], expert_weights.shape[2], dtype=in_features.dtype, device=in_features.device)
+    topk_ids = topk_ids.reshape(-1)
+    for i in range(expert_weights.shape[0]):
+        mask = topk_ids == i
+        if mask.sum():
+            out[mask] = in_features[mask] @ expert_weights[i]
+    return out
+
+
+def ag_group_gemm_fp32(shards, expert_weights, full_topk_ids):
+    """Closed form of the AG + grouped GEMM (test/nvidia/test_ag_moe.py:41-56: all-gather of the ranks' token rows,
+    then torch_moe_scatter_group_gemm) with fp32 operands and result: the reference the 1e-2 bar is taken against.
+    Pinned by: row (t, k) of the result equals (cat(shards)[t].float() @ W[ids[t, k]].float()) by definition."""
+    a = torch.cat([s.float() for s in shards], dim=0)
+    return torch_moe_scatter_group_gemm(a, expert_weights.float(), full_topk_ids)
+
+
 def quantize_groups_e4m3(x, group=128):
     """Restates _quant_kernel (tutorials/04-deepseek-infer-all2all.py:309-329; fused in the dispatch kernel at
     :180-200): per group, scale = max|x| as fp32 times fp32(1/448), q = e4m3(float(x) / scale). PARITY UNPINNED by

@@ -281,3 +281,22 @@ def test_group_quantisation_closed_form_and_round_trip():
     x2 = torch.zeros((1, 128)); x2[0, 0] = 448.0; x2[0, 1] = 1.0; x2[0, 2] = -0.5; x2[0, 3] = 2.0**-9
     q2, s2 = golden.quantize_groups_e4m3(x2.to(torch.bfloat16))
     assert s2.item() == 1.0 and q2.float()[0, :4].tolist() == [448.0, 1.0, -0.5, 2.0**-9]
+
+
+def test_group_gemm_golden_is_the_per_row_product():
+    """torch_moe_scatter_group_gemm (the reference's golden) against its definition, row by row, and against the
+    dense product when every token goes to one expert."""
+    g = torch.Generator().manual_seed(21)
+    M, K, N, E, topk = 12, 16, 8, 5, 3
+    x = torch.randint(-3, 4, (M, K), generator=g).float()
+    w = torch.randint(-3, 4, (E, K, N), generator=g).float()
+    ids = golden.random_distinct_experts(M, E, topk, g)
+    out = golden.torch_moe_scatter_group_gemm(x, w, ids)
+    assert out.shape == (M * topk, N)
+    for t in range(M):
+        for k in range(topk):
+            assert torch.equal(out[t * topk + k], x[t] @ w[int(ids[t, k])])
+    one = golden.torch_moe_scatter_group_gemm(x, w, torch.full((M, 1), 2))
+    assert torch.equal(one, x @ w[2])
+    halves = golden.ag_group_gemm_fp32([x[:6].bfloat16(), x[6:].bfloat16()], w, ids)
+    assert torch.equal(halves, out)

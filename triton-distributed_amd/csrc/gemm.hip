@@ -48,8 +48,17 @@ struct GemmParams {
   int rank, world_size;
   int order_mode;    // 0 identity, 1 reference AG order, 2 reference RS order (owner = oc+rank+1), 3 explicit
   int spin_limit;
-  int m_per_rank;    // GEMM-RS
+  int m_per_rank;    // GEMM-RS: rows per owner; grouped mode: token rows per rank segment
   int num_xcds;
+  // Grouped (MoE) mode, kernel instances with kGrouped: row r of row block m is the token sorted_ids[m*BM + r] / topk
+  // (an id >= num_valid is padding), the block multiplies by the weights of expert block_expert[m], waits for the
+  // flag of rank segment block_segment[m], and writes its rows to C at row sorted_ids[m*BM + r].
+  const int32_t* sorted_ids;
+  const int32_t* block_expert;
+  const int32_t* block_segment;
+  const int32_t* post_pad;       // device scalar: rows of the sorted space in use (a multiple of BM)
+  int64_t b_expert_stride_b;     // bytes between the experts' weight matrices
+  int num_valid, topk, first_block, a_rows;
 };
 
 // Operand fragment of one lane: K bytes [0, kLaneBytes) of one row; chunk0 / chunk1 are LDS addresses of its
@@ -185,12 +194,14 @@ __device__ __forceinline__ int chunk_of(const GemmParams& p, int oc) {
       return (oc + p.rank + 1) % p.world_size;
     case 3:
       return p.chunk_order[oc];
+    case 4:  // grouped: row blocks starting at the own rank segment's first one
+      return (oc + p.first_block) % p.n_chunks;
     default:
       return oc;
   }
 }
 
-template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales>
+template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales, bool kGrouped = false>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams p) {
   typedef GemmCfg<E, BM, BN, KB, WM, WN, NST> C;
   typedef TDIST_AS3 unsigned char* lds_u8;
@@ -230,12 +241,18 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     const int pid_n = within / cm;
     if (pid_m >= num_pid_m) continue;
     const int m0 = pid_m * BM, n0 = pid_n * BN;
+    int segment = 0;  // grouped: rank segment of this row block
+    if constexpr (kGrouped) {
+      if (m0 >= __builtin_nontemporal_load(p.post_pad)) continue;  // (written by an earlier kernel of the stream)
+      segment = p.block_segment[pid_m];
+    }
 
     // ---- gate ---------------------------------------------------------------------------------
-    const bool is_local = p.A_local != nullptr && m0 >= p.local_row_begin && m0 < p.local_row_begin + p.local_rows;
+    const bool is_local = kGrouped ? (p.A_local != nullptr && segment == p.rank)
+                                   : (p.A_local != nullptr && m0 >= p.local_row_begin && m0 < p.local_row_begin + p.local_rows);
     if (p.flags != nullptr && !is_local) {
       if (threadIdx.x == 0) {
-        const int32_t* f = p.flags + chunk;
+        const int32_t* f = p.flags + (kGrouped ? segment : chunk);
         int ok = 0;
         int limit = p.spin_limit;
         if (p.status != nullptr && __hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) limit = 1;
@@ -250,7 +267,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         }
         if (ok) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
         if (!ok && p.status != nullptr) {
-          if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = chunk;
+          if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = kGrouped ? segment : chunk;
         }
         *s_gate = ok;
       }
@@ -268,14 +285,24 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // DMA sources: a wave-uniform base (first row of the tile, advanced along K in scalar registers) plus a
     // 32-bit per-lane offset, so that the load takes its address as SGPR base + VGPR offset and the K loop
     // carries no vector address arithmetic for it
-    const int a_g0 = min(m0 - a_row_off, a_row_max), b_g0 = min(n0, p.N - 1);
+    const int a_g0 = kGrouped ? 0 : min(m0 - a_row_off, a_row_max), b_g0 = min(n0, p.N - 1);
     const unsigned char* const a_base = Arows + (int64_t)a_g0 * a_ld;
-    const unsigned char* const b_base = p.B + (int64_t)b_g0 * p.ldb_b;
+    const unsigned char* b_base_ = p.B + (int64_t)b_g0 * p.ldb_b;
+    if constexpr (kGrouped) b_base_ += (int64_t)p.block_expert[pid_m] * p.b_expert_stride_b;
+    const unsigned char* const b_base = b_base_;
     uint32_t a_off[C::kAInstr], b_off[C::kBInstr];
 #pragma unroll
     for (int t = 0; t < C::kAInstr; ++t) {
       const int r = (wave * C::kAInstr + t) * C::kRowsPerInstr + dma_row;  // row within the tile
-      const int gr = min(m0 + r - a_row_off, a_row_max);
+      int gr;
+      if constexpr (kGrouped) {
+        // the token this row stands for; padding reads the first token of the block's segment (never stored)
+        const int sid = p.sorted_ids[m0 + r];
+        const int tok = sid < p.num_valid ? sid / p.topk : segment * p.m_per_rank;
+        gr = min(max(tok - a_row_off, 0), is_local ? p.local_rows - 1 : p.a_rows - 1);
+      } else {
+        gr = min(m0 + r - a_row_off, a_row_max);
+      }
       a_off[t] = (uint32_t)(gr - a_g0) * (uint32_t)a_ld + (uint32_t)((dma_pos ^ swz<KB>(r)) << 4);
     }
 #pragma unroll
@@ -542,8 +569,15 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     auto store_piece = [&](int mrow, const int4v v) {
       const int gm = m0 + wm * C::kWaveM + mrow;
       const int gn = n0 + wn * C::kWaveN + ec * 8;
-      if (gm < p.M && gn < p.N) {
-        unsigned short* dst = (unsigned short*)Cbase + (crow0 + wm * C::kWaveM + mrow) * p.ldc + gn;
+      int64_t crow = crow0 + wm * C::kWaveM + mrow;
+      bool row_ok = gm < p.M;
+      if constexpr (kGrouped) {
+        const int sid = p.sorted_ids[gm];  // the row's place in C; padding is dropped
+        crow = sid;
+        row_ok = sid < p.num_valid;
+      }
+      if (row_ok && gn < p.N) {
+        unsigned short* dst = (unsigned short*)Cbase + crow * p.ldc + gn;
         if (gn + 8 <= p.N && n_vec_ok) {
           if (p.scatter_bufs == nullptr) __builtin_nontemporal_store(v, (int4v*)dst);  // written once, not read back here
           else *(int4v*)dst = v;
@@ -647,10 +681,10 @@ struct GemmCall {
   const char* who;
 };
 
-template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales>
+template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales, bool kGrouped = false>
 static int launch_gemm_cfg(const GemmParams& prm, int grid, hipStream_t stream, const char* who) {
   typedef GemmCfg<E, BM, BN, KB, WM, WN, NST> C;
-  auto kern = gemm_kernel<E, BM, BN, KB, WM, WN, NST, kScales>;
+  auto kern = gemm_kernel<E, BM, BN, KB, WM, WN, NST, kScales, kGrouped>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes);
@@ -740,6 +774,9 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   p.num_xcds = di.num_xcds;
   p.m_per_rank = 0;
   p.chunks_per_rank = 1;
+  p.sorted_ids = p.block_expert = p.block_segment = p.post_pad = nullptr;
+  p.b_expert_stride_b = 0;
+  p.num_valid = p.topk = p.first_block = p.a_rows = 0;
 
   if (c.scatter_bufs) {
     if (c.world_size <= 0 || c.rank < 0 || c.rank >= c.world_size)
@@ -808,6 +845,114 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   }
 }
 
+struct GroupGemmCall {
+  const void* A;
+  int64_t lda;
+  const void* A_local;
+  int64_t lda_local;
+  int local_row_begin, local_rows;
+  const void* B;
+  int64_t ldb, expert_stride;
+  void* C;
+  int64_t ldc;
+  int a_rows, N, K;
+  const int32_t *sorted_ids, *expert_ids, *block_segment, *post_pad;
+  int num_blocks, block_size, num_valid, topk, tokens_per_rank, first_block;
+  const int32_t* flags;
+  int wait_value, rank, spin_limit;
+  int32_t* status;
+  int max_workgroups;
+  hipStream_t stream;
+  const char* who;
+};
+
+static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
+  const char* who = c.who;
+  const int esz = elem == kElemFP8 ? 1 : 2;
+  if (!c.A || !c.B || !c.C || !c.sorted_ids || !c.expert_ids || !c.block_segment || !c.post_pad)
+    return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
+  if (c.a_rows <= 0 || c.N <= 0 || c.K <= 0 || c.num_blocks <= 0 || c.topk <= 0 || c.num_valid < 0 || c.tokens_per_rank <= 0)
+    return fail(TDIST_ERR_INVALID, "%s: sizes must be positive", who);
+  if (c.block_size != 128 && c.block_size != 256)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: block_size %d (the row blocks of the align / sort step must be 128 or 256 rows)", who, c.block_size);
+  if (((int64_t)c.K * esz) % 64 != 0)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: K*elem_size = %lld must be a multiple of 64 bytes", who, (long long)c.K * esz);
+  if (!aligned16(c.A) || !aligned16(c.B) || (c.A_local && !aligned16(c.A_local)) || (c.lda * esz) % 16 || (c.ldb * esz) % 16 ||
+      (c.expert_stride * esz) % 16 || (c.A_local && (c.lda_local * esz) % 16))
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: A/B bases and strides must be 16-byte aligned", who);
+  if (c.lda < c.K || c.ldb < c.K || c.ldc < c.N) return fail(TDIST_ERR_INVALID, "%s: leading dimension smaller than row", who);
+  // rows are addressed as a scalar base plus a 32-bit byte offset: the gathered A (and the own shard) must stay
+  // below 4 GiB, as must one expert's B panel
+  if ((int64_t)c.a_rows * c.lda * esz >= (1ll << 32) || (c.A_local && (int64_t)c.local_rows * c.lda_local * esz >= (1ll << 32)) ||
+      c.ldb * esz > (1 << 22))
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: A above 4 GiB or B row stride above 4 MiB", who);
+  if ((int64_t)c.num_blocks * c.block_size > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many rows", who);
+  if (c.first_block < 0 || c.first_block >= c.num_blocks) return fail(TDIST_ERR_INVALID, "%s: first_block %d", who, c.first_block);
+  if (c.A_local && (c.rank < 0 || c.local_rows <= 0)) return fail(TDIST_ERR_INVALID, "%s: local shard without rank / rows", who);
+  const DeviceInfo& di = device_info();
+  if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "%s: current device is not gfx950", who);
+
+  GemmParams p;
+  p.A = (const unsigned char*)c.A;
+  p.A_local = (const unsigned char*)c.A_local;
+  p.B = (const unsigned char*)c.B;
+  p.C = (unsigned char*)c.C;
+  p.scatter_bufs = nullptr;
+  p.row_scale = p.col_scale = nullptr;
+  p.flags = c.flags;
+  p.chunk_order = nullptr;
+  p.status = c.status;
+  p.lda_b = c.lda * esz;
+  p.lda_local_b = c.lda_local * esz;
+  p.ldb_b = c.ldb * esz;
+  p.ldc = c.ldc;
+  p.M = c.num_blocks * c.block_size;  // rows of the sorted space
+  p.N = c.N;
+  p.K = c.K;
+  p.local_row_begin = c.A_local ? c.local_row_begin : 0;
+  p.local_rows = c.A_local ? c.local_rows : 0;
+  p.m_per_chunk = c.block_size;
+  p.n_chunks = c.num_blocks;
+  p.chunks_per_rank = 1;
+  p.wait_value = c.wait_value;
+  p.rank = c.rank;
+  p.world_size = 1;
+  p.order_mode = 4;
+  p.spin_limit = c.spin_limit > 0 ? c.spin_limit : (1 << 22);
+  p.m_per_rank = c.tokens_per_rank;
+  p.num_xcds = di.num_xcds;
+  p.sorted_ids = c.sorted_ids;
+  p.block_expert = c.expert_ids;
+  p.block_segment = c.block_segment;
+  p.post_pad = c.post_pad;
+  p.b_expert_stride_b = c.expert_stride * esz;
+  p.num_valid = c.num_valid;
+  p.topk = c.topk;
+  p.first_block = c.first_block;
+  p.a_rows = c.a_rows;
+
+  const bool k128 = ((int64_t)c.K * esz) % 128 == 0;
+  const int BN = (c.block_size == 256 || k128) ? 256 : 128;
+  const int64_t sched = (int64_t)c.num_blocks * ceil_div(c.N, BN);
+  if (sched > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many tiles", who);
+  int cap_wgs = di.num_cus;
+  if (c.max_workgroups > 0 && c.max_workgroups < cap_wgs) cap_wgs = c.max_workgroups;
+  const int grid = (int)(sched < cap_wgs ? sched : cap_wgs);
+#define TDIST_GROUPED(BM_, BN_, KB_, NST_)                                                                            \
+  switch (elem) {                                                                                                    \
+    case kElemBF16: return launch_gemm_cfg<ElemBF16, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who); \
+    case kElemF16: return launch_gemm_cfg<ElemF16, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);   \
+    default: return launch_gemm_cfg<ElemFP8, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);         \
+  }
+  if (c.block_size == 256) {
+    if (!k128) return fail(TDIST_ERR_UNSUPPORTED, "%s: 256-row blocks need K*elem_size to be a multiple of 128 bytes", who);
+    TDIST_GROUPED(256, 256, 128, 5)
+  }
+  if (k128) { TDIST_GROUPED(128, 256, 128, 5) }   // 64 x 128 per wave on the split ring
+  TDIST_GROUPED(128, 128, 64, 4)
+#undef TDIST_GROUPED
+}
+
 }  // namespace tdist
 
 using namespace tdist;
@@ -872,6 +1017,31 @@ int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t
                               int64_t ldc, int M, int N, int K, int rank, int world_size, void* stream) {
   return gemm_rs_scatter(kElemF16, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, stream,
                          "tdist_gemm_rs_scatter_f16");
+}
+
+#define TDIST_GROUP_GEMM_BODY(ELEM, WHO)                                                                              \
+  GroupGemmCall c;                                                                                                    \
+  c.A = A; c.lda = lda; c.A_local = A_local; c.lda_local = lda_local; c.local_row_begin = local_row_begin;            \
+  c.local_rows = local_rows; c.B = B; c.ldb = ldb; c.expert_stride = expert_stride; c.C = C; c.ldc = ldc;             \
+  c.a_rows = a_rows; c.N = N; c.K = K; c.sorted_ids = sorted_token_ids; c.expert_ids = expert_ids;                    \
+  c.block_segment = block_barrier_ids; c.post_pad = num_tokens_post_padded; c.num_blocks = num_blocks;                \
+  c.block_size = block_size; c.num_valid = num_valid_tokens; c.topk = topk; c.tokens_per_rank = tokens_per_rank;      \
+  c.first_block = first_block; c.flags = flags; c.wait_value = wait_value; c.rank = rank; c.spin_limit = spin_limit;  \
+  c.status = status; c.max_workgroups = max_workgroups; c.stream = (hipStream_t)stream; c.who = WHO;                  \
+  return run_group_gemm(c, ELEM);
+
+#define TDIST_GROUP_GEMM_ARGS                                                                                         \
+  const void *A, int64_t lda, const void *A_local, int64_t lda_local, int local_row_begin, int local_rows,            \
+      const void *B, int64_t ldb, int64_t expert_stride, void *C, int64_t ldc, int a_rows, int N, int K,              \
+      const int32_t *sorted_token_ids, const int32_t *expert_ids, const int32_t *block_barrier_ids,                   \
+      const int32_t *num_tokens_post_padded, int num_blocks, int block_size, int num_valid_tokens, int topk,          \
+      int tokens_per_rank, int first_block, const int32_t *flags, int wait_value, int rank, int spin_limit,           \
+      int32_t *status, int max_workgroups, void *stream
+
+int tdist_group_gemm_gated_bf16(TDIST_GROUP_GEMM_ARGS) { TDIST_GROUP_GEMM_BODY(kElemBF16, "tdist_group_gemm_gated_bf16") }
+int tdist_group_gemm_gated_f16(TDIST_GROUP_GEMM_ARGS) { TDIST_GROUP_GEMM_BODY(kElemF16, "tdist_group_gemm_gated_f16") }
+int tdist_group_gemm_gated_fp8e4m3(TDIST_GROUP_GEMM_ARGS) {
+  TDIST_GROUP_GEMM_BODY(kElemFP8, "tdist_group_gemm_gated_fp8e4m3")
 }
 
 }  // extern "C"

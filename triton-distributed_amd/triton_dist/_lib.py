@@ -53,6 +53,9 @@ PROTOTYPES = {
     "tdist_moe_dispatch_tokens_quant": (_I, [_P, _I, _I, _P, _I, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_align_workspace_bytes": (_L, [_L, _I, _I]),
     "tdist_moe_align_block_size": (_I, [_P, _I, _L, _I, _I, _L, _I, _P, _P, _P, _P, _P, _P, _L, _P]),
+    "tdist_group_gemm_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
+    "tdist_group_gemm_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
+    "tdist_group_gemm_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
     "tdist_decode_split_kv": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                    _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
     "tdist_decode_fused_counters": (_L, [_I, _I, _I]),

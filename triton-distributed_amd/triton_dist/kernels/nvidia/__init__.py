@@ -3,11 +3,14 @@ triton_dist.kernels.nvidia (kernels/nvidia/__init__.py:25-89). The names resolve
 implementations as triton_dist.kernels.amd; nothing here is CUDA."""
 from triton_dist.kernels.amd.low_latency_all_to_all import (create_all_to_all_context, fast_all_to_all,
                                                             all_to_all_post_process)
-from triton_dist.kernels.amd.allgather_group_gemm import sort_topk_ids_align_block_size
+from triton_dist.kernels.amd.allgather_group_gemm import (sort_topk_ids_align_block_size,
+                                                          create_ag_group_gemm_intra_node_context,
+                                                          ag_group_gemm_intra_node)
 from triton_dist.kernels.amd.flash_decode import (gqa_fwd_batch_decode, gqa_fwd_batch_decode_intra_rank,
                                                   gqa_fwd_batch_decode_persistent)
 
 __all__ = [
     "create_all_to_all_context", "fast_all_to_all", "all_to_all_post_process", "gqa_fwd_batch_decode",
     "gqa_fwd_batch_decode_intra_rank", "gqa_fwd_batch_decode_persistent", "sort_topk_ids_align_block_size",
+    "create_ag_group_gemm_intra_node_context", "ag_group_gemm_intra_node",
 ]
