@@ -496,3 +496,38 @@ def test_alternative_schedules_of_the_large_tile(cuda, monkeypatch, variant, dty
     if sa is not None:
         ref = ref * sa[:, None] * sb[None, :]
     assert torch.equal(c, ref.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("m_per,K", [(256, 256), (200, 320), (72, 96)])
+def test_nvidia_side_signatures(cuda, m_per, K):
+    """The NVIDIA-side entry points of the reference (kernels/nvidia/allgather_gemm.py:785-882,
+    gemm_reduce_scatter.py:77-88, 468-538): context from the local tensors, one flag per rank segment, M_per_rank padded
+    to BLOCK_M for the reduce-scatter."""
+    from triton_dist.kernels.nvidia import (ag_gemm_intra_node, create_ag_gemm_intra_node_context, create_gemm_rs_context,
+                                            gemm_rs)
+    announce("nvidia-side signatures m_per=%d K=%d" % (m_per, K))
+    W, rank, N = 4, 1, 384
+    g = torch.Generator().manual_seed(m_per)
+    # GEMM-RS with padded rows
+    a = torch.randn((W * m_per, K), generator=g).to(torch.bfloat16)
+    b = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    peers = [None if r == rank else torch.randn((m_per, N), generator=g).to(torch.bfloat16) for r in range(W)]
+    ctx = create_gemm_rs_context(W * m_per, N, rank, W, W, torch.bfloat16, torch.cuda.current_stream())
+    ctx.set_peer_partials(peers)
+    out = gemm_rs(a.to(cuda), b.to(cuda), ctx)
+    torch.cuda.synchronize()
+    assert out.shape == (m_per, N)
+    assert golden.max_rel_err(out.float().cpu(), golden.gemm_rs_fp32(a, b, peers, rank, W)) <= 1e-2
+    # AG-GEMM gated per rank segment
+    if m_per % 128 == 0:
+        shards, bb = make_ag_case(W, m_per, K, N, torch.bfloat16, seed=K)
+        actx = create_ag_gemm_intra_node_context(shards[rank].to(cuda), bb.to(cuda), rank, W)
+        assert actx.barrier_tensors[rank].numel() == W and actx.M_PER_CHUNK == m_per
+        actx.set_peer_shards({r: s.to(cuda) for r, s in enumerate(shards) if r != rank})
+        c = ag_gemm_intra_node(shards[rank].to(cuda), bb.to(cuda), actx)
+        actx.check_status()
+        assert golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32(shards, bb)) <= 1e-2
+    else:
+        with pytest.raises(NotImplementedError):
+            create_ag_gemm_intra_node_context(torch.zeros((m_per, K), dtype=torch.bfloat16, device=cuda),
+                                              torch.zeros((N, K), dtype=torch.bfloat16, device=cuda), rank, W)

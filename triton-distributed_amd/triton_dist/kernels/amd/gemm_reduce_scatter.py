@@ -26,6 +26,9 @@ class GEMMReduceScatterTensorParallelContext:
     output_dtype: torch.dtype
     fuse_scatter: bool
     transpose_weight: bool
+    # rows every rank's slice is padded to in the scatter buffer (the NVIDIA-side entry point pads M_per_rank to its
+    # BLOCK_M, kernels/nvidia/gemm_reduce_scatter.py:468-479); None = no padding
+    block_m: Optional[int] = None
 
     def set_peer_partials(self, partials):
         """``partials``: dict rank -> [M_per_rank, N] tensor, or a list of num_ranks entries (the entry of
@@ -38,7 +41,8 @@ class GEMMReduceScatterTensorParallelContext:
             if r == self.rank:
                 continue
             m_per_rank = t.shape[0]
-            buf[r * m_per_rank:(r + 1) * m_per_rank, :t.shape[1]].copy_(t)
+            stride = m_per_rank if self.block_m is None else -(-m_per_rank // self.block_m) * self.block_m
+            buf[r * stride:r * stride + m_per_rank, :t.shape[1]].copy_(t)
 
 
 def create_gemm_rs_intra_node_context(max_M, N, output_dtype, rank, num_ranks, tp_group, fuse_scatter=True,
@@ -71,8 +75,11 @@ def create_gemm_rs_intra_node_context(max_M, N, output_dtype, rank, num_ranks, t
 _SCATTER_ENTRY = {torch.bfloat16: "tdist_gemm_rs_scatter_bf16", torch.float16: "tdist_gemm_rs_scatter_f16"}
 
 
-def matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weight, ldc=None, stream=None):
-    """GEMM with the scatter epilogue (reference :289-314). ``b`` is [N, K]."""
+def matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weight, ldc=None, stream=None,
+                        strict_alignment=True):
+    """GEMM with the scatter epilogue (reference :289-314). ``b`` is [N, K]. ``strict_alignment`` keeps the
+    reference's assertion (M, N, K multiples of 256); without it the library's own limits apply (M / num_ranks a
+    multiple of 128, K rows a multiple of 64 bytes)."""
     if transpose_weight:
         raise NotImplementedError()
     assert a.shape[1] == b.shape[1], "Incompatible dimensions"
@@ -80,7 +87,7 @@ def matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weigh
     M, K = a.shape
     N = b.shape[0]
     alignment = 256
-    assert M % alignment == 0 and N % alignment == 0 and K % alignment == 0
+    assert not strict_alignment or (M % alignment == 0 and N % alignment == 0 and K % alignment == 0)
     if a.dtype not in _SCATTER_ENTRY:
         raise TypeError("unsupported GEMM-RS dtype %s" % a.dtype)
     _lib.call(_SCATTER_ENTRY[a.dtype], a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
