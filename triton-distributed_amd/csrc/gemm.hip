@@ -1,16 +1,19 @@
 // (a)/(b1) Persistent MFMA tile GEMM for gfx950: C[M,N] = A[M,K] * B[N,K]^T with
 //   - per-chunk gating of A rows on HBM flag words (the AG-GEMM consumer), and/or
-//   - an epilogue that scatters row blocks to per-rank buffers (the GEMM-RS producer).
+//   - an epilogue that scatters row blocks to per-rank buffers (the GEMM-RS producer), or
+//   - the grouped form of the MoE tensor-parallel path: gathered A rows, per-block expert weights, scattered C rows.
 //
 // Restates kernel_consumer_gemm_persistent (kernels/amd/all_gather_gemm.py:140-254), wait_eq_sys
-// (kernels/amd/common_ops.py:39-46) and kernel_gemm_rs_producer_fuse_scatter
-// (kernels/amd/gemm_reduce_scatter.py:125-229) as one hand-scheduled kernel:
+// (kernels/amd/common_ops.py:39-46), kernel_gemm_rs_producer_fuse_scatter
+// (kernels/amd/gemm_reduce_scatter.py:125-229) and kernel_consumer_m_parallel_scatter_group_gemm
+// (kernels/nvidia/allgather_group_gemm.py:238-314) as one hand-scheduled kernel:
 //
 //  * workgroup = WM x WN waves, macro tile BM x BN, each wave owns (BM/WM) x (BN/WN) of it as 32x32
 //    MFMA tiles: v_mfma_f32_32x32x16_{bf16,f16} (16 B of K per lane) or v_mfma_f32_32x32x64_f8f6f4
 //    (32 B of K per lane) with fp32 accumulators;
 //  * A and B tiles go HBM/L2 → LDS with asynchronous 16-byte-per-lane LDS-DMA loads into a ring of NST
-//    stages, P = NST-1 tiles in flight; rows are stored with an XOR swizzle of the 16-byte chunk index
+//    stages, P = NST-1 tiles in flight (NST == 5: a split ring of three A and two B half stages whose refill is
+//    spread over the K steps); rows are stored with an XOR swizzle of the 16-byte chunk index
 //    so that the ds_read_b128 operand reads are bank-conflict free; the swizzle is applied on the global
 //    side (which chunk a lane fetches) because the DMA writes lanes to consecutive LDS addresses;
 //  * one s_barrier per K tile, placed before the MFMAs of the tile's last K step, so the first operand
