@@ -54,23 +54,41 @@ __global__ __launch_bounds__(kScanThreads) void moe_scan_kernel(int32_t* __restr
   const int per = (G + kScanThreads - 1) / kScanThreads;  // consecutive experts per thread
   const int g0 = threadIdx.x * per;
   int32_t local_total = 0;
-  for (int j = 0; j < per; ++j) {
-    const int g = g0 + j;
-    if (g < G) {
-      int32_t run = 0;
-      // 16 independent loads at a time, then their exclusive prefix
-      for (int b0 = 0; b0 < num_blocks; b0 += 16) {
-        int32_t h[16];
+  // two experts and 32 blocks at a time: 64 independent loads in flight per thread, then their exclusive prefixes
+  // (the kernel is one workgroup and all latency, so the depth of each round of loads is what it costs)
+  constexpr int kCols = 2, kDepth = 32;
+  for (int j0 = 0; j0 < per; j0 += kCols) {
+    int32_t run[kCols];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) h[u] = (b0 + u < num_blocks) ? hist[(int64_t)(b0 + u) * G + g] : 0;
+    for (int c = 0; c < kCols; ++c) run[c] = 0;
+    for (int b0 = 0; b0 < num_blocks; b0 += kDepth) {
+      int32_t h[kCols][kDepth];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) {
-          if (b0 + u < num_blocks) hist[(int64_t)(b0 + u) * G + g] = run;
-          run += h[u];
+      for (int c = 0; c < kCols; ++c) {
+        const int g = g0 + j0 + c;
+        const bool col_ok = j0 + c < per && g < G;
+#pragma unroll
+        for (int u = 0; u < kDepth; ++u)
+          h[c][u] = (col_ok && b0 + u < num_blocks) ? hist[(int64_t)(b0 + u) * G + g] : 0;
+      }
+#pragma unroll
+      for (int c = 0; c < kCols; ++c) {
+        const int g = g0 + j0 + c;
+        const bool col_ok = j0 + c < per && g < G;
+#pragma unroll
+        for (int u = 0; u < kDepth; ++u) {
+          if (col_ok && b0 + u < num_blocks) hist[(int64_t)(b0 + u) * G + g] = run[c];
+          run[c] += h[c][u];
         }
       }
-      splits[g] = run;
-      local_total += run;
+    }
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+      const int g = g0 + j0 + c;
+      if (j0 + c < per && g < G) {
+        splits[g] = run[c];
+        local_total += run[c];
+      }
     }
   }
   s_part[threadIdx.x] = local_total;

@@ -56,15 +56,21 @@ def sort_topk_ids_align_block_size(
         raise _lib.TdistError(_lib.TDIST_ERR_UNSUPPORTED,
                               "num_experts * num_ranks = %d is above what the align kernel handles" % (num_experts * num_ranks))
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    moe_stream = torch.cuda.current_stream() if moe_stream is None else moe_stream
-    with torch.cuda.stream(moe_stream):
+
+    def launch(stream):
         sorted_ids.fill_(n_total)
         _lib.call("tdist_moe_align_block_size", topk_ids.data_ptr(), 1 if topk_ids.dtype == torch.int64 else 0, n_total,
                   num_experts, num_ranks, n_per, block_size, sorted_ids.data_ptr(), expert_ids.data_ptr(),
                   block_barrier_ids.data_ptr(), rank_block_num.data_ptr(), num_tokens_post_pad.data_ptr(),
-                  workspace.data_ptr(), ws_bytes, moe_stream.cuda_stream)
-    torch.cuda.current_stream().wait_stream(moe_stream)
-    workspace.record_stream(moe_stream)
+                  workspace.data_ptr(), ws_bytes, stream.cuda_stream)
+
+    if moe_stream is None:
+        launch(torch.cuda.current_stream())      # no stream switch, event or allocator bookkeeping to pay for
+    else:
+        with torch.cuda.stream(moe_stream):
+            launch(moe_stream)
+        torch.cuda.current_stream().wait_stream(moe_stream)
+        workspace.record_stream(moe_stream)
     return (
         sorted_ids,
         expert_ids,
