@@ -414,6 +414,33 @@ def ag_group_gemm_fp32(shards, expert_weights, full_topk_ids):
     return torch_moe_scatter_group_gemm(a, expert_weights.float(), full_topk_ids)
 
 
+def torch_group_gemm_reduce_rs(intermediate_states, w, topk_ids, topk_weight, peer_partials, rank, world_size):
+    """TorchGroupGemmReduceRS.forward (test/nvidia/test_moe_reduce_rs.py:103-133) in fp32, with its
+    reduce_scatter_tensor written out: intermediate_states [M * topk, K] (row t*topk + k), w [E, K, hidden], topk_ids /
+    topk_weight [M, topk]; out[t] = sum_k weight[t,k] * (states[t*topk+k] @ w[ids[t,k]]); this rank keeps rows
+    [rank*M/W, (rank+1)*M/W) and adds the other ranks' partial results for them (``peer_partials``: list with one
+    [M/W, hidden] tensor per rank, the own entry ignored), in the order rank+1, rank+2, ... Returns fp32.
+    Pinned by: the per-row definition (brute force in tests/test_oracle.py)."""
+    n_rows, _ = intermediate_states.shape
+    topk = topk_ids.shape[1]
+    M = n_rows // topk
+    ids = topk_ids.reshape(-1)
+    wt = topk_weight.reshape(-1).float()
+    out = torch.zeros(n_rows, w.shape[2], dtype=torch.float32)
+    for i in range(w.shape[0]):
+        mask = ids == i
+        if mask.sum():
+            out[mask] = (intermediate_states[mask].float() @ w[i].float()) * wt[mask, None]
+    out = out.reshape(M, topk, -1).sum(dim=1)
+    m_per = M // world_size
+    acc = None
+    for step in range(world_size):
+        r = (rank + 1 + step) % world_size
+        part = out[rank * m_per:(rank + 1) * m_per] if r == rank else peer_partials[r].float()
+        acc = part.clone() if acc is None else acc + part
+    return acc
+
+
 def quantize_groups_e4m3(x, group=128):
     """Restates _quant_kernel (tutorials/04-deepseek-infer-all2all.py:309-329; fused in the dispatch kernel at
     :180-200): per group, scale = max|x| as fp32 times fp32(1/448), q = e4m3(float(x) / scale). PARITY UNPINNED by

@@ -300,3 +300,17 @@ def test_group_gemm_golden_is_the_per_row_product():
     assert torch.equal(one, x @ w[2])
     halves = golden.ag_group_gemm_fp32([x[:6].bfloat16(), x[6:].bfloat16()], w, ids)
     assert torch.equal(halves, out)
+
+
+def test_group_gemm_reduce_rs_golden_by_brute_force():
+    g = torch.Generator().manual_seed(33)
+    M, K, H, E, topk, W, rank = 8, 6, 5, 4, 2, 2, 1
+    states = torch.randint(-3, 4, (M * topk, K), generator=g).float()
+    w = torch.randint(-3, 4, (E, K, H), generator=g).float()
+    ids = golden.random_distinct_experts(M, E, topk, g)
+    wt = torch.randint(1, 4, (M, topk), generator=g).float()
+    peers = [torch.randint(-5, 6, (M // W, H), generator=g).float() for _ in range(W)]
+    got = golden.torch_group_gemm_reduce_rs(states, w, ids, wt, peers, rank, W)
+    for i, t in enumerate(range(rank * M // W, (rank + 1) * M // W)):
+        want = sum(wt[t, k] * (states[t * topk + k] @ w[int(ids[t, k])]) for k in range(topk)) + peers[0][i]
+        assert torch.equal(got[i], want)

@@ -7,6 +7,7 @@ from triton_dist.kernels.amd.low_latency_all_to_all import (create_all_to_all_co
 from triton_dist.kernels.amd.allgather_group_gemm import (sort_topk_ids_align_block_size,
                                                           create_ag_group_gemm_intra_node_context,
                                                           ag_group_gemm_intra_node)
+from triton_dist.kernels.amd.moe_reduce_rs import create_moe_rs_context, moe_reduce_rs, select_experts
 from triton_dist.kernels.amd.flash_decode import (gqa_fwd_batch_decode, gqa_fwd_batch_decode_intra_rank,
                                                   gqa_fwd_batch_decode_persistent)
 
@@ -17,5 +18,5 @@ __all__ = [
     "ag_gemm_intra_node", "create_ag_gemm_intra_node_context", "create_gemm_rs_context", "gemm_rs",
     "create_all_to_all_context", "fast_all_to_all", "all_to_all_post_process", "gqa_fwd_batch_decode",
     "gqa_fwd_batch_decode_intra_rank", "gqa_fwd_batch_decode_persistent", "sort_topk_ids_align_block_size",
-    "create_ag_group_gemm_intra_node_context", "ag_group_gemm_intra_node",
+    "create_ag_group_gemm_intra_node_context", "ag_group_gemm_intra_node", "create_moe_rs_context", "moe_reduce_rs", "select_experts",
 ]
