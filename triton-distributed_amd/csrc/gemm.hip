@@ -523,6 +523,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // acc[j][i][e]: output row m = wm*kWaveM + 32i + l32, column n = wn*kWaveN + 32j + 8*(e/4) + 4*lh + e%4
     wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
     lds_u8 const epi = smem + wave * C::kEpiBytes;
+    // The epilogue's lane-dependent addresses are the same for every tile; computed from these opaque copies they are
+    // rebuilt per tile (a few dozen instructions) instead of being held in ~100 registers across the K loop.
+    int e_lane = lane;
+    asm volatile("" : "+v"(e_lane));
+    const int e_l32 = e_lane & 31, e_lh = e_lane >> 5;
     // destination of this tile's rows
     unsigned char* Cbase;
     int64_t crow0;
@@ -536,35 +541,42 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     }
     constexpr int kLanesPerRow = C::kWaveN * 2 / 16;  // 16-byte vectors per staged row
     constexpr int kRowsPerPass = 64 / kLanesPerRow;
-    const int er = lane / kLanesPerRow, ec = lane % kLanesPerRow;
+    const int er = e_lane / kLanesPerRow, ec = e_lane % kLanesPerRow;
     const bool n_vec_ok = (p.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(Cbase) & 15) == 0);
 
     // packs the 32 x 32 block (i, j) of the wave tile into its staging rows
-    auto stage_block = [&](int i, int j, float rsi, const float4v* cs) {
-      const int mrow = 32 * i + l32;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int ncol = 32 * j + 8 * q + 4 * lh;
-        float v0, v1, v2, v3;
-        if constexpr (C::kTM * C::kTN * 16 >= 256) {
-          // 256 accumulators live in AGPRs; read each one here, where it is packed, instead of letting the
-          // compiler copy all of them to VGPRs at the loop exit (which spills)
-          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v0) : "a"(acc[j][i][4 * q + 0]));
-          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v1) : "a"(acc[j][i][4 * q + 1]));
-          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v2) : "a"(acc[j][i][4 * q + 2]));
-          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v3) : "a"(acc[j][i][4 * q + 3]));
-        } else {
-          v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2], v3 = acc[j][i][4 * q + 3];
-        }
-        if (kScales) {
-          v0 *= rsi * cs[q][0];
-          v1 *= rsi * cs[q][1];
-          v2 *= rsi * cs[q][2];
-          v3 *= rsi * cs[q][3];
-        }
-        const int2v w = {(int)E::pack(v0, v1), (int)E::pack(v2, v3)};
-        *(TDIST_AS3 int2v*)(epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2) = w;
+    // packs four columns x 32 rows (column group q of block (i, j)) into the staging rows
+    auto stage_group_at = [&](int i, int j, int q, float rsi, const float4v* cs, lds_u8 where) {
+      float v0, v1, v2, v3;
+      if constexpr (C::kTM * C::kTN * 16 >= 256) {
+        // 256 accumulators live in AGPRs; read each one here, where it is packed, instead of letting the
+        // compiler copy all of them to VGPRs at the loop exit (which spills)
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v0) : "a"(acc[j][i][4 * q + 0]));
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v1) : "a"(acc[j][i][4 * q + 1]));
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v2) : "a"(acc[j][i][4 * q + 2]));
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v3) : "a"(acc[j][i][4 * q + 3]));
+      } else {
+        v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2], v3 = acc[j][i][4 * q + 3];
       }
+      if (kScales) {
+        v0 *= rsi * cs[q][0];
+        v1 *= rsi * cs[q][1];
+        v2 *= rsi * cs[q][2];
+        v3 *= rsi * cs[q][3];
+      }
+      const int2v w = {(int)E::pack(v0, v1), (int)E::pack(v2, v3)};
+      *(TDIST_AS3 int2v*)where = w;
+    };
+    auto stage_group = [&](int i, int j, int q, float rsi, const float4v* cs) {
+      const int mrow = 32 * i + e_l32;
+      const int ncol = 32 * j + 8 * q + 4 * e_lh;
+      stage_group_at(i, j, q, rsi, cs,
+                     epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2);
+    };
+    // the same for the 32 x 32 block (i, j)
+    auto stage_block = [&](int i, int j, float rsi, const float4v* cs) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) stage_group(i, j, q, rsi, cs);
       __builtin_amdgcn_sched_barrier(0);  // keep the accumulator read-out block by block (register pressure)
     };
     // staged rows [row0, row0 + nrows) of the wave tile → global memory, 16 bytes per lane
@@ -580,10 +592,10 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         row_ok = sid < p.num_valid;
       }
       if (row_ok && gn < p.N) {
-        unsigned short* dst = (unsigned short*)Cbase + crow * p.ldc + gn;
+        TDIST_AS1 unsigned short* dst = (TDIST_AS1 unsigned short*)Cbase + crow * p.ldc + gn;  // device memory: global stores
         if (gn + 8 <= p.N && n_vec_ok) {
-          if (p.scatter_bufs == nullptr) __builtin_nontemporal_store(v, (int4v*)dst);  // written once, not read back here
-          else *(int4v*)dst = v;
+          if (p.scatter_bufs == nullptr) __builtin_nontemporal_store(v, (TDIST_AS1 int4v*)dst);  // written once, not read back here
+          else *(TDIST_AS1 int4v*)dst = v;
         } else {
           for (int e = 0; e < 8; ++e)
             if (gn + e < p.N) dst[e] = (unsigned short)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
@@ -601,19 +613,109 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         store_piece(mrow, staged_piece(mrow));
       }
     };
-    // the same for one 32-row block with all its LDS reads issued before the first store, so that no store waits for
-    // the LDS round trip of its own read (costs 32 registers: used where the instance has them)
-    auto store_block32 = [&](int row0) {
-      constexpr int kPasses = 32 / kRowsPerPass;
-      int4v v[kPasses];
-#pragma unroll
-      for (int u = 0; u < kPasses; ++u) v[u] = staged_piece(row0 + u * kRowsPerPass + er);
-#pragma unroll
-      for (int u = 0; u < kPasses; ++u) store_piece(row0 + u * kRowsPerPass + er, v[u]);
-    };
     static_assert(32 % kRowsPerPass == 0, "a 32-row block is a whole number of store passes");
 
-    if constexpr (!kScales && C::kTM * C::kTN * 16 >= 256) {
+    // A tile that lies inside C with 16-byte-aligned rows. Row block by row block, software-pipelined: the staged rows
+    // of block i are read back (LDS serves one wave's instructions in order, so the reads see the writes before them
+    // without a wait), block i+1 is packed while those reads are in flight, then block i is stored, with one address
+    // per lane for the whole tile (uniform base + constant row step) and no per-store bounds arithmetic. The scales
+    // of the whole wave tile are fetched up front, in one round trip.
+    bool stored = false;
+    if constexpr (C::kWaves <= 4 && !kGrouped) {
+      if (m0 + BM <= p.M && n0 + BN <= p.N && n_vec_ok) {
+        stored = true;
+        constexpr int kPasses = 32 / kRowsPerPass;
+        static_assert(2 * kPasses == 4 * C::kTN, "one read or store per column group of a row block");
+        const int64_t row_bytes = p.ldc * 2;
+        unsigned char* const tile_dst = Cbase + ((crow0 + wm * C::kWaveM) * p.ldc + n0 + wn * C::kWaveN) * 2;
+        const uint32_t lane_off = (uint32_t)er * (uint32_t)row_bytes + (uint32_t)ec * 16u;
+        const bool streaming = p.scatter_bufs == nullptr;
+        float rs[C::kTM];
+        float4v cs[kScales ? C::kTN : 1][4];
+#pragma unroll
+        for (int i = 0; i < C::kTM; ++i) {
+          rs[i] = 1.f;
+          if (kScales && p.row_scale) rs[i] = p.row_scale[m0 + wm * C::kWaveM + 32 * i + e_l32];
+        }
+        if constexpr (kScales) {
+#pragma unroll
+          for (int j = 0; j < C::kTN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {  // the four column scales of each of this lane's four column groups in block j
+              cs[j][q] = float4v{1.f, 1.f, 1.f, 1.f};
+              if (p.col_scale) cs[j][q] = *(const float4v*)(p.col_scale + n0 + wn * C::kWaveN + 32 * j + 8 * q + 4 * e_lh);
+            }
+          }
+        }
+        // Staging addresses: a row block adds a constant to them (32 rows leave the swizzle term alone), so one
+        // address per column group and one per swizzle phase of the read-back serve the whole tile, with the row
+        // block in the instruction's offset field.
+        constexpr int kGroups = 4 * C::kTN;
+        constexpr int kReadPhases = (C::kEpiSwz + 1) / kRowsPerPass > 1 ? (C::kEpiSwz + 1) / kRowsPerPass : 1;
+        static_assert(kPasses % kReadPhases == 0 && (C::kEpiSwz + 1) <= 32, "swizzle period within a row block");
+        lds_u8 wbase[kGroups], rbase[kReadPhases];
+#pragma unroll
+        for (int c = 0; c < kGroups; ++c)
+          wbase[c] = epi + e_l32 * C::kEpiPitch + ((c ^ (e_l32 & C::kEpiSwz)) << 4) + 8 * e_lh;
+#pragma unroll
+        for (int ph = 0; ph < kReadPhases; ++ph)
+          rbase[ph] = epi + er * C::kEpiPitch + ((ec ^ ((ph * kRowsPerPass + er) & C::kEpiSwz)) << 4);
+        auto stage_fast = [&](int i, int g) {
+          stage_group_at(i, g / 4, g % 4, rs[i], cs[kScales ? g / 4 : 0], wbase[g] + i * 32 * C::kEpiPitch);
+        };
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) stage_fast(0, g);
+        __builtin_amdgcn_sched_barrier(0);
+        int4v v[kPasses];
+        auto read_piece = [&](int i, int u) {
+          v[u] = *(const TDIST_AS3 int4v*)(rbase[u % kReadPhases] + (32 * i + u * kRowsPerPass) * C::kEpiPitch);
+        };
+        auto store_fast = [&](int i, int u) {
+          TDIST_AS1 int4v* dst = (TDIST_AS1 int4v*)(tile_dst + (int64_t)(32 * i + u * kRowsPerPass) * row_bytes + lane_off);
+          if (streaming) __builtin_nontemporal_store(v[u], dst);
+          else *dst = v[u];
+        };
+        // One LDS read or one store behind every column group of the next block's packing, so that the three pipes
+        // (vector ALU, LDS, vector memory) work at the same time. A wave issues in order and the four waves share one
+        // path to memory, so a burst of stores would hold each wave for the whole burst: spread out, a store costs
+        // its wave one issue. Piece u of block i is read behind group 2u and stored kLag reads later; the last
+        // kLag stores of a block go behind the first groups of the next one.
+        constexpr int kLag = 2;
+        static_assert(kPasses >= 2 * kLag, "the store of a piece follows its read by kLag reads");
+#pragma unroll
+        for (int i = 0; i + 1 < C::kTM; ++i) {
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int g = 0; g < 4 * C::kTN; ++g) {
+            stage_fast(i + 1 < C::kTM ? i + 1 : 0, g);
+            if (g % 2 == 0) {
+              read_piece(i, g / 2);
+            } else {
+              const int u = (g - 1) / 2 - kLag;
+              if (u >= 0) store_fast(i, u);
+              else if (i > 0) store_fast(i - 1, u + kPasses);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        {
+          constexpr int i = C::kTM - 1;  // nothing left to pack behind the last block
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int u = 0; u < kPasses - kLag; ++u) read_piece(i, u);
+          if (i > 0) {
+#pragma unroll
+            for (int u = kPasses - kLag; u < kPasses; ++u) store_fast(i - 1, u);
+          }
+#pragma unroll
+          for (int u = kPasses - kLag; u < kPasses; ++u) read_piece(i, u);
+#pragma unroll
+          for (int u = 0; u < kPasses; ++u) store_fast(i, u);
+        }
+      }
+    }
+    if (stored) {
+    } else if constexpr (!kScales && C::kTM * C::kTN * 16 >= 256) {
       // row block by row block: the stores of block i drain while block i+1 is being packed
 #pragma unroll
       for (int i = 0; i < C::kTM; ++i) {
@@ -621,15 +723,14 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         for (int j = 0; j < C::kTN; ++j) stage_block(i, j, 1.f, nullptr);
         __builtin_amdgcn_wave_barrier();
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if constexpr (C::kWaves <= 4 && C::kFragVecs == 1) store_block32(32 * i);
-        else store_rows(32 * i, 32);
+        store_rows(32 * i, 32);
       }
     } else {
       float rs[C::kTM];
 #pragma unroll
       for (int i = 0; i < C::kTM; ++i) {
         rs[i] = 1.f;
-        if (kScales && p.row_scale) rs[i] = p.row_scale[min(m0 + wm * C::kWaveM + 32 * i + l32, p.M - 1)];
+        if (kScales && p.row_scale) rs[i] = p.row_scale[min(m0 + wm * C::kWaveM + 32 * i + e_l32, p.M - 1)];
       }
 #pragma unroll
       for (int j = 0; j < C::kTN; ++j) {
@@ -639,7 +740,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         for (int q = 0; q < 4; ++q) {
           cs[q] = float4v{1.f, 1.f, 1.f, 1.f};
           if (kScales && p.col_scale) {
-            const int gn = n0 + wn * C::kWaveN + 32 * j + 8 * q + 4 * lh;
+            const int gn = n0 + wn * C::kWaveN + 32 * j + 8 * q + 4 * e_lh;
             if (gn + 3 < p.N) cs[q] = *(const float4v*)(p.col_scale + gn);
             else
               for (int e = 0; e < 4; ++e) cs[q][e] = p.col_scale[min(gn + e, p.N - 1)];
