@@ -311,6 +311,27 @@ int tdist_group_gemm_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
                                    int32_t* status, int max_workgroups, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Split-K workspace for the GEMM entry points above (tdist_gemm_chunk_gated_*, tdist_gemm_rs_scatter_*,
+ * tdist_group_gemm_gated_*). Optional. The reference's kernels run whole tiles per program and leave a last round
+ * that does not fill the grid to its autotuner's tile choice (kernels/amd/all_gather_gemm.py:151-246 persistent
+ * loop; kernels/nvidia/allgather_group_gemm.py:238-314). Here, with a workspace registered for the current device,
+ * a last round that fills at most half of the grid is cut along K: each of its tiles goes to s = grid / tiles
+ * workgroups (at most 8, pieces of at least 4 K tiles), which add their fp32 accumulators through the workspace
+ * before the usual epilogue (same products, other order of the sums: results stay within the stated tolerance
+ * and are exact on integer-valued inputs). Whole rounds run as before. Bounded waits as for the chunk flags: a
+ * piece that never arrives sets status to {TDIST_ERR_TIMEOUT, -1 - workgroup}.
+ *   tdist_gemm_split_k_workspace_bytes(): size that serves every call on the current device (one fp32 256 x 256
+ *     tile per compute unit + 4096 bytes of flags: 64 MiB + 4 KiB on MI355X); 0 if the device is not gfx950.
+ *   tdist_gemm_split_k_set_workspace(workspace, bytes, stream): registers (workspace != NULL; 256-byte aligned
+ *     device memory; the call clears the flag words on `stream`) or unregisters (NULL) the current device's
+ *     workspace. The caller keeps the memory alive until it unregisters. One GEMM launch at a time may use it:
+ *     launches of these entry points that can overlap on the device (different streams without an ordering) must
+ *     not both find a workspace registered.
+ * TDIST_GEMM_SPLIT_K=0 in the environment turns the path off, =1 takes it wherever a round can be split. */
+int64_t tdist_gemm_split_k_workspace_bytes(void);
+int tdist_gemm_split_k_set_workspace(void* workspace, int64_t bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * (d) split-KV GQA flash decode + LSE combine.
  *   replaces kernel_gqa_fwd_batch_decode_split_kv               kernels/nvidia/flash_decode.py:129-239
  *            kernel_intra_rank_gqa_fwd_batch_decode_combine_kv  kernels/nvidia/flash_decode.py:392-449

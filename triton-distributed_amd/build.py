@@ -62,12 +62,47 @@ def is_stale():
     return any(os.path.getmtime(f) > t for f in _inputs())
 
 
+# The four-wave GEMM instances (one wave per SIMD, 256 accumulators in AGPRs) are only fast while the compiler keeps
+# their loops free of spills, and they must leave registers for a copy kernel's wave beside them on the SIMD (the
+# register file holds 512 per lane). Small edits far from the K loop have tipped the allocation over, so every build
+# checks the compiler's own resource report.
+GEMM_REGISTER_BUDGET = 480   # architectural + accumulation registers per lane
+_RESOURCE_FLAG = "-Rpass-analysis=kernel-resource-usage"
+
+
+def _check_gemm_resources(report):
+    import re
+    name, vgprs, agprs, offenders = None, 0, 0, []
+    for line in report.splitlines():
+        m = re.search(r"remark: (?:Function Name: (\S+)|\s+(VGPRs|AGPRs|ScratchSize \[bytes/lane\]): (\d+))", line)
+        if not m:
+            continue
+        if m.group(1):
+            name, vgprs, agprs = m.group(1), 0, 0
+        elif m.group(2) == "VGPRs":
+            vgprs = int(m.group(3))
+        elif m.group(2) == "AGPRs":
+            agprs = int(m.group(3))
+        elif name and "gemm_kernel" in name and re.search(r"ELi2ELi2ELi\d+ELb", name):   # WM = WN = 2
+            total = (vgprs + 7) // 8 * 8 + agprs
+            if int(m.group(3)) != 0 or total > GEMM_REGISTER_BUDGET:
+                offenders.append("%s: %d + %d registers, %s bytes of scratch" % (name, vgprs, agprs, m.group(3)))
+    if offenders:
+        raise RuntimeError("gemm.hip: four-wave instances over the register budget (%d, no scratch):\n  %s"
+                           % (GEMM_REGISTER_BUDGET, "\n  ".join(offenders)))
+
+
 def _compile_one(hipcc, src):
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
     cmd = [hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    if src == "gemm.hip":
+        cmd += [_RESOURCE_FLAG, "-fno-caret-diagnostics"]   # (no source excerpt under each of the report's lines)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    # the host pass does not know the device-only target feature; that line is noise
-    log = "\n".join(l for l in res.stdout.splitlines() if "is not a recognized feature for this target" not in l)
+    if src == "gemm.hip" and res.returncode == 0:
+        _check_gemm_resources(res.stdout)
+    # the host pass does not know the device-only target feature; that line is noise, and so is the resource report
+    log = "\n".join(l for l in res.stdout.splitlines()
+                    if "is not a recognized feature for this target" not in l and "-Rpass-analysis" not in l)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed on %s:\n%s" % (src, log))
     return obj, log

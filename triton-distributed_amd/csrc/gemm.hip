@@ -25,6 +25,8 @@
 //    compact block of tiles so they share A rows and B rows in that XCD's L2.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace tdist {
@@ -62,6 +64,17 @@ struct GemmParams {
   const int32_t* post_pad;       // device scalar: rows of the sorted space in use (a multiple of BM)
   int64_t b_expert_stride_b;     // bytes between the experts' weight matrices
   int num_valid, topk, first_block, a_rows;
+  // Split last round (sk_on != 0): whole rounds of the grid run tile by tile as always; the tiles of a last round
+  // that fills at most half of the grid are cut along K into s = grid / tiles equal pieces (at most kSkMaxSplit, at
+  // least kSkMinPiece K tiles each), one per workgroup, so that the round takes 1/s of a tile's time. Workgroups
+  // s*t .. s*t+s-1 share tile t: each but the last adds the next one's accumulators (fp32, in register order,
+  // through slot [workgroup] of sk_partials, announced by sk_flags[workgroup] == sk_epoch) to its own, and the
+  // first runs the epilogue. (Cutting every tile of the schedule into equal shares of K tiles, "stream-K",
+  // was measured slower than whole tiles: workgroups that share an operand panel are then at different K
+  // positions, and the panel is fetched once per workgroup instead of once per XCD.)
+  float* sk_partials;
+  int32_t* sk_flags;
+  int sk_on, sk_epoch;
 };
 
 // Operand fragment of one lane: K bytes [0, kLaneBytes) of one row; chunk0 / chunk1 are LDS addresses of its
@@ -182,6 +195,9 @@ __device__ __forceinline__ void wait_tiles_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
 
+// Split last round: most pieces per tile, fewest K tiles per piece
+constexpr int kSkMaxSplit = 8, kSkMinPiece = 4;
+
 // Instruction classes for __builtin_amdgcn_sched_group_barrier
 constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
 
@@ -223,7 +239,10 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   const int num_pid_n = (p.N + BN - 1) / BN;
   const int cm = p.m_per_chunk / BM;                 // row tiles per chunk
   const int tiles_per_chunk = cm * num_pid_n;
-  const int total_sched = p.n_chunks * tiles_per_chunk;
+  // grouped: only the row blocks in use are scheduled (their count is written by an earlier kernel of the stream)
+  int n_chunks = p.n_chunks;
+  if constexpr (kGrouped) n_chunks = min(n_chunks, __builtin_nontemporal_load(p.post_pad) / BM);
+  const int total_sched = n_chunks * tiles_per_chunk;
   const int G = gridDim.x;
   const int KT = p.K * E::kBytes / KB;
 
@@ -231,15 +250,33 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   const int dma_row = lane / C::kChunksPerRow;
   const int dma_pos = lane % C::kChunksPerRow;
 
-  for (int sbase = 0; sbase < total_sched; sbase += G) {
-    // XCD-aware position within the round: workgroups of XCD x take a contiguous range
-    int u = blockIdx.x;
-    if (p.num_xcds > 1 && G % p.num_xcds == 0) u = (u % p.num_xcds) * (G / p.num_xcds) + u / p.num_xcds;
-    const int sidx = sbase + u;
-    if (sidx >= total_sched) continue;
+  // XCD-aware position within a round: workgroups of XCD x take a contiguous range
+  int wg_pos = blockIdx.x;
+  if (p.num_xcds > 1 && G % p.num_xcds == 0) wg_pos = (wg_pos % p.num_xcds) * (G / p.num_xcds) + wg_pos / p.num_xcds;
+  // split last round: s pieces per tile (1 = not split)
+  const int sk_tail_tiles = total_sched % G;
+  int sk_split = 1;
+  if (p.sk_on && sk_tail_tiles > 0) sk_split = min(min(G / sk_tail_tiles, kSkMaxSplit), KT / kSkMinPiece);
+  if (sk_split < 2) sk_split = 1;
+
+  for (int sbase = 0;; sbase += G) {
+    int sidx, ka = 0, kb = KT;  // the piece: K tiles [ka, kb) of scheduled tile sidx
+    if (sbase >= total_sched) break;
+    if (sk_split > 1 && sbase + G > total_sched) {
+      // the last round, split: workgroup s*t + j takes piece j of the round's tile t
+      const int t = wg_pos / sk_split, j = wg_pos - t * sk_split;
+      if (t >= sk_tail_tiles) break;
+      sidx = __builtin_amdgcn_readfirstlane(sbase + t);
+      ka = __builtin_amdgcn_readfirstlane(KT * j / sk_split);  // (KT < 2^20 and j < 8: 32-bit scalar arithmetic)
+      kb = __builtin_amdgcn_readfirstlane(KT * (j + 1) / sk_split);
+    } else {
+      sidx = sbase + wg_pos;
+      if (sidx >= total_sched) continue;
+    }
+    const int KTp = kb - ka;
     const int oc = sidx / tiles_per_chunk;
     const int within = sidx - oc * tiles_per_chunk;
-    const int chunk = chunk_of(p, oc);
+    const int chunk = kGrouped ? (oc + p.first_block) % n_chunks : chunk_of(p, oc);
     const int pid_m = chunk * cm + within % cm;
     const int pid_n = within / cm;
     if (pid_m >= num_pid_m) continue;
@@ -289,8 +326,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // 32-bit per-lane offset, so that the load takes its address as SGPR base + VGPR offset and the K loop
     // carries no vector address arithmetic for it
     const int a_g0 = kGrouped ? 0 : min(m0 - a_row_off, a_row_max), b_g0 = min(n0, p.N - 1);
-    const unsigned char* const a_base = Arows + (int64_t)a_g0 * a_ld;
-    const unsigned char* b_base_ = p.B + (int64_t)b_g0 * p.ldb_b;
+    const unsigned char* const a_base = Arows + (int64_t)a_g0 * a_ld + (int64_t)ka * KB;
+    const unsigned char* b_base_ = p.B + (int64_t)b_g0 * p.ldb_b + (int64_t)ka * KB;
     if constexpr (kGrouped) b_base_ += (int64_t)p.block_expert[pid_m] * p.b_expert_stride_b;
     const unsigned char* const b_base = b_base_;
     uint32_t a_off[C::kAInstr], b_off[C::kBInstr];
@@ -336,10 +373,10 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
                    : "memory");
     };
     auto issue_a = [&](int kt, int t) {
-      dma16(a_base + (int64_t)min(kt, KT - 1) * KB, a_off[t], a_stage(kt) + (wave * C::kAInstr + t) * 1024);
+      dma16(a_base + (int64_t)min(kt, KTp - 1) * KB, a_off[t], a_stage(kt) + (wave * C::kAInstr + t) * 1024);
     };
     auto issue_b = [&](int kt, int u) {
-      dma16(b_base + (int64_t)min(kt, KT - 1) * KB, b_off[u], b_stage(kt) + (wave * C::kBInstr + u) * 1024);
+      dma16(b_base + (int64_t)min(kt, KTp - 1) * KB, b_off[u], b_stage(kt) + (wave * C::kBInstr + u) * 1024);
     };
     auto issue_dma = [&](int kt, int t) {
       if (t < C::kAInstr) issue_a(kt, t);
@@ -404,8 +441,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       wait_tiles_and_barrier<C::kAInstr + C::kDmaPerStep>();
       load_frags(0, 0, a_cur, b_cur);
       __builtin_amdgcn_sched_barrier(0);
-      for (int kt = 0; kt < KT; ++kt) {
-        const int kt_next = min(kt + 1, KT - 1);
+      for (int kt = 0; kt < KTp; ++kt) {
+        const int kt_next = min(kt + 1, KTp - 1);
 #pragma unroll
         for (int ks = 0; ks < C::kKSteps; ++ks) {
           constexpr int kLast = C::kKSteps - 1;
@@ -461,7 +498,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // step of a tile first joins the barrier (tile kt+1 has landed everywhere, tile kt is no longer read),
     // then also refills the freed stage.
     constexpr int kReadsPerStep = (C::kTM + C::kTN) * C::kFragVecs;
-    for (int kt = 0; kt < KT; ++kt) {
+    for (int kt = 0; kt < KTp; ++kt) {
 #pragma unroll
       for (int ks = 0; ks < C::kKSteps; ++ks) {
         if (ks + 1 < C::kKSteps) {
@@ -493,7 +530,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
           constexpr int kSlots = kFrags < kTail ? kFrags : kTail;
           constexpr int kDmaPerSlot = (C::kLoadsPerTile + kSlots - 1) / kSlots;
           constexpr int kFragPerSlot = (kFrags + kSlots - 1) / kSlots;
-          const int kt_next = min(kt + 1, KT - 1);
+          const int kt_next = min(kt + 1, KTp - 1);
 #pragma unroll
           for (int idx = C::kLeadMfma; idx < kMfmaPerStep; ++idx) {
             const int j = idx / C::kTM, i = idx % C::kTM;
@@ -522,6 +559,99 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // ---- epilogue ---------------------------------------------------------------------------------
     // acc[j][i][e]: output row m = wm*kWaveM + 32i + l32, column n = wn*kWaveN + 32j + 8*(e/4) + 4*lh + e%4
     wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
+    if (p.sk_on && KTp < KT) {
+      // ---- split last round: this piece is not the whole K range -------------------------------
+      // The pieces of a tile form a chain along the workgroup order: a piece that does not reach the tile's last K
+      // tile waits for the next workgroup's piece and adds it; a piece that does not start at the tile's first K
+      // tile then hands its sum on through its slot; the piece that does start there runs the epilogue. (The pieces
+      // are equally long and start together, so the chain costs its length times one hand-over.)
+      constexpr int kThreads = C::kWaves * 64;
+      constexpr int kQuads = C::kTM * C::kTN * 4;  // float4 groups of accumulators per lane
+      constexpr bool kAgpr = C::kTM * C::kTN * 16 >= 256;
+      // slot addresses: a uniform base per float4 group plus one 32-bit lane offset (from an opaque copy of the
+      // thread id, so that nothing of this is computed ahead and held across the K loop)
+      uint32_t sk_voff = threadIdx.x;
+      asm volatile("" : "+v"(sk_voff));
+      sk_voff *= 16u;
+      if (kb < KT) {
+        const int w = wg_pos + 1;  // the workgroup with the next piece of this tile
+        if (threadIdx.x == 0) {
+          int ok = 0;
+          // (the full limit even after an error elsewhere: this piece is being computed, not awaited from outside;
+          // if its workgroup gave it up at a chunk flag, the wait runs out and the tile is not stored)
+          for (int it = 0; it < p.spin_limit; ++it) {
+            if (__hip_atomic_load(p.sk_flags + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.sk_epoch) {
+              ok = 1;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(4);
+          }
+          if (!ok && p.status != nullptr) {
+            if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = -1 - w;
+          }
+          *s_gate = ok;
+        }
+        __syncthreads();
+        const int ok = *s_gate;
+        __syncthreads();
+        if (!ok) continue;  // (a piece further up the chain then runs out of its wait as well: the tile is not stored)
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const TDIST_AS1 unsigned char* src = (const TDIST_AS1 unsigned char*)(p.sk_partials + (int64_t)w * (BM * BN));
+        constexpr int kLoadBatch = 16;
+#pragma unroll
+        for (int r0 = 0; r0 < kQuads; r0 += kLoadBatch) {
+          float4v t[kLoadBatch];
+#pragma unroll
+          for (int r = 0; r < kLoadBatch; ++r) t[r] = *(const TDIST_AS1 float4v*)(src + (size_t)(r0 + r) * (kThreads * 16) + sk_voff);
+#pragma unroll
+          for (int r = 0; r < kLoadBatch; ++r) {
+            const int j = (r0 + r) / (C::kTM * 4), i = ((r0 + r) / 4) % C::kTM, q = (r0 + r) % 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if constexpr (kAgpr) {
+                // in place, so that the accumulators stay where they are on both sides of this branch
+                float tmp;
+                asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_add_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+                             : "+a"(acc[j][i][4 * q + e]), "=&v"(tmp)
+                             : "v"(t[r][e]));
+              } else {
+                acc[j][i][4 * q + e] += t[r][e];
+              }
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (ka != 0) {
+        // hand the sum on: coherent at device scope, every store instruction a contiguous KiB
+        // The store sits in inline assembly (the cache-policy bit has no builtin), where the compiler sees neither
+        // a memory instruction nor its hazards. Hence: a vector address (a scalar base that the compiler happened
+        // to reload from a spill lane with v_readlane would need five wait states before the store), and a wait
+        // state after the store before anything may overwrite its data registers.
+        unsigned char* slot = (unsigned char*)(p.sk_partials + (int64_t)wg_pos * (BM * BN)) + sk_voff;
+#pragma unroll
+        for (int r = 0; r < kQuads; ++r) {
+          const int j = r / (C::kTM * 4), i = (r / 4) % C::kTM, q = r % 4;
+          float4v t;
+          if constexpr (kAgpr) {
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[0]) : "a"(acc[j][i][4 * q + 0]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[1]) : "a"(acc[j][i][4 * q + 1]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[2]) : "a"(acc[j][i][4 * q + 2]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[3]) : "a"(acc[j][i][4 * q + 3]));
+          } else {
+            t = float4v{acc[j][i][4 * q + 0], acc[j][i][4 * q + 1], acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]};
+          }
+          asm volatile("s_nop 1\n\tglobal_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(slot), "v"(t) : "memory");
+          slot += kThreads * 16;
+          asm volatile("" : "+v"(slot));  // one running address, not sixty-four precomputed ones
+          if (r % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0) __hip_atomic_store(p.sk_flags + wg_pos, p.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        continue;
+      }
+    }
     lds_u8 const epi = smem + wave * C::kEpiBytes;
     // The epilogue's lane-dependent addresses are the same for every tile; computed from these opaque copies they are
     // rebuilt per tile (a few dozen instructions) instead of being held in ~100 registers across the K loop.
@@ -799,6 +929,45 @@ static int launch_gemm_cfg(const GemmParams& prm, int grid, hipStream_t stream, 
   return launch_status(who);
 }
 
+// ---- split-K workspace (one per device, handed in by the caller) -------------------------------------------
+// [0, kSkFlagBytes): one flag word per workgroup; then one fp32 tile per workgroup. A launch that uses it gets a
+// fresh epoch: its flags count as raised when they hold that value, so nothing is cleared between launches.
+constexpr int64_t kSkFlagBytes = 4096;
+constexpr int kSkMaxDevices = 64;
+struct SkWorkspace {
+  unsigned char* base = nullptr;
+  int64_t bytes = 0;
+  int epoch = 0;
+};
+static SkWorkspace g_sk[kSkMaxDevices];
+static std::mutex g_sk_mutex;
+
+// 0 = off, 1 = on wherever the workspace allows, -1 = by the cost estimate
+static int sk_env() {
+  if (const char* v = getenv("TDIST_GEMM_SPLIT_K")) return atoi(v) != 0 ? 1 : 0;
+  return -1;
+}
+
+static bool sk_workspace_fits(int workgroups, int bm, int bn) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSkMaxDevices) return false;
+  std::lock_guard<std::mutex> lock(g_sk_mutex);
+  const SkWorkspace& w = g_sk[dev];
+  return w.base != nullptr && workgroups * 4 <= kSkFlagBytes && w.bytes >= kSkFlagBytes + (int64_t)workgroups * bm * bn * 4;
+}
+
+static void sk_attach(GemmParams& p) {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  std::lock_guard<std::mutex> lock(g_sk_mutex);
+  SkWorkspace& w = g_sk[dev];
+  w.epoch = w.epoch == 0x7fffffff ? 1 : w.epoch + 1;
+  p.sk_on = 1;
+  p.sk_epoch = w.epoch;
+  p.sk_flags = (int32_t*)w.base;
+  p.sk_partials = (float*)(w.base + kSkFlagBytes);
+}
+
 static int run_gemm(const GemmCall& c, GemmElem elem) {
   const char* who = c.who;
   const int esz = elem == kElemFP8 ? 1 : 2;
@@ -828,19 +997,43 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (c.max_workgroups > 0 && c.max_workgroups < cap_wgs) cap_wgs = c.max_workgroups;
   struct TileChoice { int bm, bn; double eff; };
   static const TileChoice kChoices[3] = {{256, 256, 1.0}, {256, 128, 0.9}, {128, 128, 0.6}};
+  // With a workspace registered, a last round that fills at most half of the grid is split along K (see GemmParams):
+  // it then costs 1/s of a round plus s-1 hand-overs of a tile's accumulators (priced at 2 + 2 * tile/64Ki K tiles
+  // of work each), and that form is taken where it beats whole tiles by a margin.
+  const int sk_mode = sk_env();
   int pick = 2;
+  bool use_sk = false;
   double best = 0;
   for (int t = 0; t < 3; ++t) {
     if (kChoices[t].bm == 256 && !rows256) continue;
-    const int64_t tiles = ceil_div(c.M, kChoices[t].bm) * ceil_div(c.N, kChoices[t].bn);
-    const double cost = (double)ceil_div(tiles, cap_wgs) * kChoices[t].bm * kChoices[t].bn / kChoices[t].eff;
-    if (best == 0 || cost < best) best = cost, pick = t;
+    const int bm = kChoices[t].bm, bn = kChoices[t].bn;
+    const int64_t tiles = ceil_div(c.M, bm) * ceil_div(c.N, bn);
+    const int64_t kt = (int64_t)c.K * esz / (bm == 256 ? 128 : 64);
+    const double per_k_tile = (double)bm * bn / kChoices[t].eff;
+    const double cost = (double)ceil_div(tiles, cap_wgs) * kt * per_k_tile;
+    if (best == 0 || cost < best) best = cost, pick = t, use_sk = false;
+    const int64_t tail = tiles % cap_wgs;
+    int64_t split = tail > 0 ? cap_wgs / tail : 1;
+    if (split > kSkMaxSplit) split = kSkMaxSplit;
+    if (split > kt / kSkMinPiece) split = kt / kSkMinPiece;
+    if (sk_mode != 0 && split >= 2 && sk_workspace_fits(cap_wgs, bm, bn)) {
+      const double cost_sk = ((double)(tiles / cap_wgs) * kt + (double)kt / split + (split - 1) * (2.0 + 2.0 * bm * bn / 65536.0)) * per_k_tile;
+      if (cost_sk < 0.95 * best || (sk_mode == 1 && (!use_sk || cost_sk < best))) best = cost_sk, pick = t, use_sk = true;
+    }
   }
   // TDIST_GEMM_TILE forces a tile (measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128; a 256-row tile that the
   // call's row blocks do not admit is not taken.
   if (const char* v = getenv("TDIST_GEMM_TILE")) {
     const int t = atoi(v);
-    if (t >= 0 && t < 3 && (kChoices[t].bm != 256 || rows256)) pick = t;
+    if (t >= 0 && t < 3 && (kChoices[t].bm != 256 || rows256)) {
+      pick = t;
+      // (the split is re-derived for the forced tile)
+      const int64_t tiles = ceil_div(c.M, kChoices[t].bm) * ceil_div(c.N, kChoices[t].bn);
+      const int64_t kt = (int64_t)c.K * esz / (kChoices[t].bm == 256 ? 128 : 64);
+      const int64_t tail = tiles % cap_wgs;
+      use_sk = sk_mode != 0 && use_sk && tail > 0 && cap_wgs / tail >= 2 && kt / kSkMinPiece >= 2 &&
+               sk_workspace_fits(cap_wgs, kChoices[t].bm, kChoices[t].bn);
+    }
   }
   // TDIST_GEMM_VARIANT picks another compiled schedule of the 256x256 tile (measurement aid): 2 = 2x4 waves on a
   // two-stage ring, 5 = 2x4 waves on the split ring. The default is 2x2 waves of 128x128 on the split ring
@@ -881,6 +1074,9 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   p.sorted_ids = p.block_expert = p.block_segment = p.post_pad = nullptr;
   p.b_expert_stride_b = 0;
   p.num_valid = p.topk = p.first_block = p.a_rows = 0;
+  p.sk_partials = nullptr;
+  p.sk_flags = nullptr;
+  p.sk_on = p.sk_epoch = 0;
 
   if (c.scatter_bufs) {
     if (c.world_size <= 0 || c.rank < 0 || c.rank >= c.world_size)
@@ -920,7 +1116,11 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   }
   const int64_t sched = (int64_t)p.n_chunks * (p.m_per_chunk / BM) * ceil_div(c.N, BN);
   if (sched > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many tiles", who);
-  const int grid = (int)(sched < cap_wgs ? sched : cap_wgs);
+  int grid = (int)(sched < cap_wgs ? sched : cap_wgs);
+  if (use_sk) {
+    grid = cap_wgs;
+    sk_attach(p);
+  }
   const bool scales = elem == kElemFP8 && (c.row_scale || c.col_scale);
 
   if (big) {
@@ -1034,6 +1234,9 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   p.topk = c.topk;
   p.first_block = c.first_block;
   p.a_rows = c.a_rows;
+  p.sk_partials = nullptr;
+  p.sk_flags = nullptr;
+  p.sk_on = p.sk_epoch = 0;
 
   const bool k128 = ((int64_t)c.K * esz) % 128 == 0;
   const int BN = (c.block_size == 256 || k128) ? 256 : 128;
@@ -1041,7 +1244,17 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   if (sched > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many tiles", who);
   int cap_wgs = di.num_cus;
   if (c.max_workgroups > 0 && c.max_workgroups < cap_wgs) cap_wgs = c.max_workgroups;
-  const int grid = (int)(sched < cap_wgs ? sched : cap_wgs);
+  int grid = (int)(sched < cap_wgs ? sched : cap_wgs);
+  // The number of row blocks in use is only known on the device and is seldom a multiple of the grid: with a
+  // workspace at hand the kernel splits the last round along K whenever it fills at most half of the grid.
+  {
+    const int bm = c.block_size == 256 ? 256 : 128;
+    const int64_t kt = (int64_t)c.K * esz / (c.block_size == 256 || k128 ? 128 : 64);
+    if (sk_env() != 0 && kt >= 2 * kSkMinPiece && sk_workspace_fits(cap_wgs, bm, BN)) {
+      grid = cap_wgs;
+      sk_attach(p);
+    }
+  }
 #define TDIST_GROUPED(BM_, BN_, KB_, NST_)                                                                            \
   switch (elem) {                                                                                                    \
     case kElemBF16: return launch_gemm_cfg<ElemBF16, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who); \
@@ -1072,6 +1285,32 @@ using namespace tdist;
   return run_gemm(c, ELEM);
 
 extern "C" {
+
+int64_t tdist_gemm_split_k_workspace_bytes(void) {
+  const tdist::DeviceInfo& di = tdist::device_info();
+  if (di.ok != 1) return 0;
+  return tdist::kSkFlagBytes + (int64_t)di.num_cus * 256 * 256 * 4;
+}
+
+int tdist_gemm_split_k_set_workspace(void* workspace, int64_t bytes, void* stream) {
+  using namespace tdist;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSkMaxDevices)
+    return fail(TDIST_ERR_DEVICE, "tdist_gemm_split_k_set_workspace: no current device");
+  if (workspace != nullptr) {
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || bytes < kSkFlagBytes + 128 * 128 * 4)
+      return fail(TDIST_ERR_WORKSPACE, "tdist_gemm_split_k_set_workspace: %lld bytes at %p (256-byte aligned, see "
+                  "tdist_gemm_split_k_workspace_bytes)", (long long)bytes, workspace);
+    // flags start below every epoch
+    if (hipMemsetAsync(workspace, 0, kSkFlagBytes, (hipStream_t)stream) != hipSuccess)
+      return fail(TDIST_ERR_LAUNCH, "tdist_gemm_split_k_set_workspace: clearing the flags failed");
+  }
+  std::lock_guard<std::mutex> lock(g_sk_mutex);
+  g_sk[dev].base = (unsigned char*)workspace;
+  g_sk[dev].bytes = workspace ? bytes : 0;
+  g_sk[dev].epoch = 0;
+  return TDIST_OK;
+}
 
 int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                 int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C, int64_t ldc,

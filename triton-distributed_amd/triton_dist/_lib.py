@@ -56,6 +56,8 @@ PROTOTYPES = {
     "tdist_group_gemm_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
     "tdist_group_gemm_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
     "tdist_group_gemm_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
+    "tdist_gemm_split_k_workspace_bytes": (_L, []),
+    "tdist_gemm_split_k_set_workspace": (_I, [_P, _L, _P]),
     "tdist_decode_split_kv": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                    _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
     "tdist_decode_fused_counters": (_L, [_I, _I, _I]),
@@ -131,6 +133,37 @@ def dtype_code(dtype):
     if dtype == torch.float32:
         return TDIST_F32
     raise TypeError("unsupported dtype %s" % dtype)
+
+
+_split_k_workspaces = {}   # device index -> uint8 tensor registered with the library (kept alive here)
+
+
+def enable_split_k(device=None):
+    """Allocates and registers the current (or given) device's split-K workspace once; the GEMM entry points then
+    cut the tiles of a last round that fills at most half of the grid along K. Returns the workspace tensor."""
+    import torch
+    dev = torch.cuda.current_device() if device is None else torch.device(device).index
+    if dev in _split_k_workspaces:
+        return _split_k_workspaces[dev]
+    with torch.cuda.device(dev):
+        nbytes = load().tdist_gemm_split_k_workspace_bytes()
+        if nbytes <= 0:
+            raise TdistError(TDIST_ERR_DEVICE, "split-K workspace: device %d is not gfx950" % dev)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda:%d" % dev)
+        call("tdist_gemm_split_k_set_workspace", ws.data_ptr(), nbytes, stream_ptr())
+        torch.cuda.current_stream().synchronize()
+    _split_k_workspaces[dev] = ws
+    return ws
+
+
+def disable_split_k(device=None):
+    import torch
+    dev = torch.cuda.current_device() if device is None else torch.device(device).index
+    if dev in _split_k_workspaces:
+        with torch.cuda.device(dev):
+            torch.cuda.synchronize()
+            call("tdist_gemm_split_k_set_workspace", None, 0, stream_ptr())
+        del _split_k_workspaces[dev]
 
 
 def require_cuda(*tensors):

@@ -189,11 +189,13 @@ class AllGatherGEMMTensorParallelContext:
 
 def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, rank, num_ranks, tp_group,
                                       ag_streams=None, gemm_stream=None, M_PER_CHUNK=1024, BLOCK_M=128, BLOCK_N=256,
-                                      BLOCK_K=64, stages=3, serial=False, autotune=False):
+                                      BLOCK_K=64, stages=3, serial=False, autotune=False, split_k=True):
     """create context for allgather gemm intra-node (reference :360-429).
 
     ``tp_group`` may be None: one GPU holds the only real rank. BLOCK_*/stages/autotune are accepted for
-    signature compatibility; the HIP kernel picks its own tiling.
+    signature compatibility; the HIP kernel picks its own tiling. ``split_k``: register the device's split-K
+    workspace (64 MiB, once per device), with which a last round of tiles that fills at most half of the grid is cut
+    along K (one GEMM launch at a time per device may use it).
     """
     assert M_PER_CHUNK % BLOCK_M == 0
     assert max_M % num_ranks == 0
@@ -202,6 +204,8 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
     if not torch.cuda.is_available():
         raise RuntimeError("create_ag_gemm_intra_node_context needs a GPU")
     _lib.check(_lib.load().tdist_init())
+    if split_k:
+        _lib.enable_split_k()
     device = torch.device("cuda", torch.cuda.current_device())
     workspace = torch.empty([max_M, K], dtype=input_dtype, device=device)
     m_chunk_num = (max_M + M_PER_CHUNK - 1) // M_PER_CHUNK

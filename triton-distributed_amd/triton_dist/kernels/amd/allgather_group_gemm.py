@@ -167,16 +167,20 @@ class MoE_AllGatherGroupGEMMTensorParallelContext:
 
 def create_ag_group_gemm_intra_node_context(tp_pg, tensor_A, tensor_B, full_topk_ids, num_experts, max_M=2**14, BLOCK_M=128,
                                             BLOCK_N=256, BLOCK_K=64, GROUP_SIZE_M=8, stages=3, warps=8, ag_stream=None,
-                                            group_gemm_stream=None, rank=None, num_ranks=None):
+                                            group_gemm_stream=None, rank=None, num_ranks=None, split_k=True):
     """create context for allgather group gemm intra-node (reference :555-638).
 
     tensor_A [M_per_rank, K] local tokens, tensor_B [E, K, N_per_rank] local expert weights, full_topk_ids
     [M_per_rank * num_ranks, topk]. ``tp_pg`` may be None on one GPU: pass ``rank`` / ``num_ranks``. BLOCK_M is the
     row block of the align / sort and of the GEMM tile (128 or 256); the other tiling arguments are accepted for
-    signature compatibility."""
+    signature compatibility. ``split_k``: register the device's split-K workspace (64 MiB, once per device): the
+    number of row blocks in use is seldom a multiple of the grid, and with the workspace the grouped GEMM cuts the tiles
+    of a last round that fills at most half of the grid along K (one GEMM launch at a time per device may use it)."""
     if not torch.cuda.is_available():
         raise RuntimeError("create_ag_group_gemm_intra_node_context needs a GPU")
     _lib.check(_lib.load().tdist_init())
+    if split_k:
+        _lib.enable_split_k()
     M_per_rank, K = tensor_A.shape
     _, topk = full_topk_ids.shape
     assert tensor_B.shape[1] == K, "tensor_B should have shape [E, %d, N_per_rank], got %s" % (K, tuple(tensor_B.shape))

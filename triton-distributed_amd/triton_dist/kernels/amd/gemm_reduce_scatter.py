@@ -46,8 +46,9 @@ class GEMMReduceScatterTensorParallelContext:
 
 
 def create_gemm_rs_intra_node_context(max_M, N, output_dtype, rank, num_ranks, tp_group, fuse_scatter=True,
-                                      transpose_weight=False):
-    """create context for gemm reduce-scatter intra-node (reference :381-426). ``tp_group`` may be None."""
+                                      transpose_weight=False, split_k=True):
+    """create context for gemm reduce-scatter intra-node (reference :381-426). ``tp_group`` may be None.
+    ``split_k``: register the device's split-K workspace (see create_ag_gemm_intra_node_context)."""
     if not fuse_scatter:
         raise NotImplementedError()
     if transpose_weight:
@@ -55,6 +56,8 @@ def create_gemm_rs_intra_node_context(max_M, N, output_dtype, rank, num_ranks, t
     if not torch.cuda.is_available():
         raise RuntimeError("create_gemm_rs_intra_node_context needs a GPU")
     _lib.check(_lib.load().tdist_init())
+    if split_k:
+        _lib.enable_split_k()
     device = torch.device("cuda", torch.cuda.current_device())
     scatter_bufs = [torch.zeros([max_M, N], dtype=output_dtype, device=device) for _ in range(num_ranks)]
     scatter_bufs_ptr = torch.tensor([t.data_ptr() for t in scatter_bufs], dtype=torch.int64, device=device)

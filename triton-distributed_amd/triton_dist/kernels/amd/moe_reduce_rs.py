@@ -91,11 +91,13 @@ class MoEReduceRSContext:
 
 
 def create_moe_rs_context(pg, local_rank, world_size, local_world_size, max_token_num, hidden_dim, num_experts, topk,
-                          input_dtype, output_dtype, device, moe_block_size, router_logits, peer_router_logits=None):
+                          input_dtype, output_dtype, device, moe_block_size, router_logits, peer_router_logits=None, split_k=True):
     """reference :280-361. ``pg`` may be None on one GPU (``local_rank`` is then the rank)."""
     if not torch.cuda.is_available():
         raise RuntimeError("create_moe_rs_context needs a GPU")
     _lib.check(_lib.load().tdist_init())
+    if split_k:
+        _lib.enable_split_k()   # (see create_ag_group_gemm_intra_node_context)
     if output_dtype != torch.bfloat16:
         raise NotImplementedError("the top-k reduction writes bf16 (reference: the input dtype, fp16 in its test)")
     rank = local_rank if pg is None else pg.rank()
