@@ -82,7 +82,7 @@ def test_null_pointers_are_rejected_without_touching_the_gpu():
     assert lib.tdist_producer_wait_until(None, 1000, None) == _lib.TDIST_ERR_INVALID
     assert lib.tdist_producer_wait_until(p, -1, None) == _lib.TDIST_ERR_INVALID
     assert lib.tdist_producer_wait_until(p, 100000001, None) == _lib.TDIST_ERR_INVALID and "100 ms" in _lib.last_error()
-    assert lib.tdist_moe_workspace_bytes(32768, 256) == (32 + 1) * 256 * 4
+    assert lib.tdist_moe_workspace_bytes(32768, 256) == (128 + 1) * 256 * 4 + 256
 
 
 def test_ops_fail_loudly_without_gpu():

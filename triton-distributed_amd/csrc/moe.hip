@@ -15,7 +15,7 @@
 namespace tdist {
 
 constexpr int kMoeThreads = 256;              // 4 waves
-constexpr int kMoeItemsPerBlock = 1024;       // ids ranked by one block (256 per wave)
+constexpr int kMoeItemsPerBlock = 256;        // ids ranked by one block (64 per wave: one pass)
 constexpr int kMoeMaxExperts = 4096;          // LDS: 4 waves * G * 4 B
 constexpr int kScanThreads = 1024;
 
@@ -27,8 +27,10 @@ __host__ __device__ static inline int id_bits(int g) {
 
 // hist[b][g] = #ids equal to g among block b's items.
 __global__ __launch_bounds__(kMoeThreads) void moe_hist_kernel(const int32_t* __restrict__ ids, int64_t n, int G,
-                                                              int32_t* __restrict__ hist) {
+                                                              int32_t* __restrict__ hist,
+                                                              int32_t* __restrict__ scan_counter) {
   extern __shared__ int32_t s_hist[];
+  if (blockIdx.x == 0 && threadIdx.x == 0) *scan_counter = 0;  // arrival counter of the scan that follows
   for (int g = threadIdx.x; g < G; g += kMoeThreads) s_hist[g] = 0;
   __syncthreads();
   const int64_t base = (int64_t)blockIdx.x * kMoeItemsPerBlock;
@@ -45,52 +47,77 @@ __global__ __launch_bounds__(kMoeThreads) void moe_hist_kernel(const int32_t* __
   for (int g = threadIdx.x; g < G; g += kMoeThreads) out[g] = s_hist[g];
 }
 
-// One block. Turns hist[b][g] into the exclusive prefix over b, writes splits[g] and cumsum[0..G].
+// Turns hist[b][g] into the exclusive prefix over b, writes splits[g] and cumsum[0..G]. One workgroup per 256
+// columns (a single workgroup would move the whole table through one compute unit: 19 us for 2048 groups x 32
+// blocks), four row ranges per column; the workgroup that finishes last adds up the column totals. `counter` is zero
+// on entry (the histogram kernel clears it) and zero again on exit.
 // splits is never NULL here: the host substitutes a row of the workspace when the caller has none.
+constexpr int kScanCols = 256, kScanParts = kScanThreads / kScanCols;
 __global__ __launch_bounds__(kScanThreads) void moe_scan_kernel(int32_t* __restrict__ hist, int num_blocks, int G,
                                                                int32_t* __restrict__ splits,
-                                                               int32_t* __restrict__ cumsum) {
+                                                               int32_t* __restrict__ cumsum,
+                                                               int32_t* __restrict__ counter) {
+  __shared__ int32_t s_tot[kScanParts][kScanCols];
   __shared__ int32_t s_part[kScanThreads];
-  const int per = (G + kScanThreads - 1) / kScanThreads;  // consecutive experts per thread
-  const int g0 = threadIdx.x * per;
-  int32_t local_total = 0;
-  // two experts and 32 blocks at a time: 64 independent loads in flight per thread, then their exclusive prefixes
-  // (the kernel is one workgroup and all latency, so the depth of each round of loads is what it costs)
-  constexpr int kCols = 2, kDepth = 32;
-  for (int j0 = 0; j0 < per; j0 += kCols) {
-    int32_t run[kCols];
+  __shared__ int s_last;
+  const int c = threadIdx.x % kScanCols, q = threadIdx.x / kScanCols;
+  const int g = blockIdx.x * kScanCols + c;
+  const int rows_per = (num_blocks + kScanParts - 1) / kScanParts;
+  const int b_begin = min(q * rows_per, num_blocks), b_end = min(b_begin + rows_per, num_blocks);
+  constexpr int kDepth = 32;  // loads in flight per thread and round
+  int32_t h[kDepth];
+  int32_t total = 0;
+  if (g < G) {
+    for (int b0 = b_begin; b0 < b_end; b0 += kDepth) {
 #pragma unroll
-    for (int c = 0; c < kCols; ++c) run[c] = 0;
-    for (int b0 = 0; b0 < num_blocks; b0 += kDepth) {
-      int32_t h[kCols][kDepth];
+      for (int u = 0; u < kDepth; ++u) h[u] = b0 + u < b_end ? hist[(int64_t)(b0 + u) * G + g] : 0;
 #pragma unroll
-      for (int c = 0; c < kCols; ++c) {
-        const int g = g0 + j0 + c;
-        const bool col_ok = j0 + c < per && g < G;
-#pragma unroll
-        for (int u = 0; u < kDepth; ++u)
-          h[c][u] = (col_ok && b0 + u < num_blocks) ? hist[(int64_t)(b0 + u) * G + g] : 0;
-      }
-#pragma unroll
-      for (int c = 0; c < kCols; ++c) {
-        const int g = g0 + j0 + c;
-        const bool col_ok = j0 + c < per && g < G;
-#pragma unroll
-        for (int u = 0; u < kDepth; ++u) {
-          if (col_ok && b0 + u < num_blocks) hist[(int64_t)(b0 + u) * G + g] = run[c];
-          run[c] += h[c][u];
-        }
-      }
+      for (int u = 0; u < kDepth; ++u) total += h[u];
     }
+  }
+  s_tot[q][c] = total;
+  __syncthreads();
+  int32_t run = 0, column = 0;
 #pragma unroll
-    for (int c = 0; c < kCols; ++c) {
-      const int g = g0 + j0 + c;
-      if (j0 + c < per && g < G) {
-        splits[g] = run[c];
-        local_total += run[c];
+  for (int p = 0; p < kScanParts; ++p) {
+    if (p < q) run += s_tot[p][c];
+    column += s_tot[p][c];
+  }
+  if (g < G) {
+    if (q == 0) splits[g] = column;
+    const bool kept = b_end - b_begin <= kDepth;  // the only round's values are still in registers
+    for (int b0 = b_begin; b0 < b_end; b0 += kDepth) {
+      if (!kept) {
+#pragma unroll
+        for (int u = 0; u < kDepth; ++u) h[u] = b0 + u < b_end ? hist[(int64_t)(b0 + u) * G + g] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < kDepth; ++u) {
+        if (b0 + u < b_end) hist[(int64_t)(b0 + u) * G + g] = run;
+        run += h[u];
       }
     }
   }
+  // ---- the last workgroup: cumsum over all columns -------------------------------------------
+  if (gridDim.x > 1) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      __threadfence();  // this workgroup's splits are visible before its arrival is
+      const int arrived = atomicAdd(counter, 1);
+      s_last = arrived == (int)gridDim.x - 1;
+      if (s_last) {
+        *counter = 0;
+        __threadfence();
+      }
+    }
+    __syncthreads();
+    if (!s_last) return;
+  }
+  const int per = (G + kScanThreads - 1) / kScanThreads;  // consecutive columns per thread
+  const int g0 = threadIdx.x * per;
+  int32_t local_total = 0;
+  for (int j = 0; j < per; ++j)
+    if (g0 + j < G) local_total += __hip_atomic_load(splits + g0 + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   s_part[threadIdx.x] = local_total;
   __syncthreads();
   // Hillis-Steele inclusive scan over the per-thread totals.
@@ -100,13 +127,13 @@ __global__ __launch_bounds__(kScanThreads) void moe_scan_kernel(int32_t* __restr
     s_part[threadIdx.x] += v;
     __syncthreads();
   }
-  int32_t run = s_part[threadIdx.x] - local_total;  // exclusive prefix of this thread's first expert
+  int32_t acc = s_part[threadIdx.x] - local_total;  // exclusive prefix of this thread's first column
   if (threadIdx.x == 0) cumsum[0] = 0;
   for (int j = 0; j < per; ++j) {
-    const int g = g0 + j;
-    if (g < G) {
-      run += splits[g];
-      cumsum[g + 1] = run;
+    const int gg = g0 + j;
+    if (gg < G) {
+      acc += __hip_atomic_load(splits + gg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      cumsum[gg + 1] = acc;
     }
   }
 }
@@ -713,8 +740,11 @@ static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, 
   const int num_blocks = (int)ceil_div(n_ids > 0 ? n_ids : 1, kMoeItemsPerBlock);
   int32_t* hist = (int32_t*)workspace;
   int32_t* splits_buf = splits ? splits : hist + (int64_t)num_blocks * G;
-  hipLaunchKernelGGL(moe_hist_kernel, dim3(num_blocks), dim3(kMoeThreads), (size_t)G * 4, stream, ids, n_ids, G, hist);
-  hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, hist, num_blocks, G, splits_buf, cumsum);
+  int32_t* scan_counter = hist + (int64_t)(num_blocks + 1) * G;
+  hipLaunchKernelGGL(moe_hist_kernel, dim3(num_blocks), dim3(kMoeThreads), (size_t)G * 4, stream, ids, n_ids, G, hist,
+                     scan_counter);
+  hipLaunchKernelGGL(moe_scan_kernel, dim3((G + kScanCols - 1) / kScanCols), dim3(kScanThreads), 0, stream, hist, num_blocks,
+                     G, splits_buf, cumsum, scan_counter);
   if (want_index && n_ids > 0) {
     hipLaunchKernelGGL(moe_rank_kernel, dim3(num_blocks), dim3(kMoeThreads), (size_t)G * 4 * (kMoeThreads / 64), stream,
                        ids, n_ids, topk, G, id_bits(G), hist, cumsum, scatter_idx, gather_idx, topk_idx);
@@ -731,7 +761,7 @@ extern "C" {
 int64_t tdist_moe_workspace_bytes(int64_t n_ids, int num_experts) {
   if (n_ids < 0 || num_experts <= 0) return 0;
   const int64_t num_blocks = ceil_div(n_ids > 0 ? n_ids : 1, kMoeItemsPerBlock);
-  return (num_blocks + 1) * (int64_t)num_experts * 4;  // block histograms + one splits row
+  return (num_blocks + 1) * (int64_t)num_experts * 4 + 256;  // block histograms + one splits row + the scan's counter
 }
 
 int tdist_moe_splits_cumsum(const int32_t* ids, int64_t n_ids, int num_experts, int32_t* splits, int32_t* cumsum,
