@@ -312,11 +312,21 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
     paced = ctx is not None and ctx.link_gbps > 0 and num_ranks > 1
     if paced:
         _lib.call("tdist_producer_mark", ctx.start_stamp.data_ptr(), current_stream.cuda_stream)
-    gemm_stream.wait_stream(current_stream)
-    for ag_stream in ag_streams:
-        ag_stream.wait_stream(current_stream)
-
     use_kernel = ctx is not None and ctx.producer_kernel
+    # Fork: one event on the caller's stream, waited for by the GEMM stream and by the producer streams that this
+    # call really uses (the kernel producer needs one; the copy producer stream r % n for every peer r). The host
+    # cost of a call is what bounds the small shapes, so nothing is forked, joined or entered that is not used.
+    if num_ranks <= 1:
+        used_ag_streams = []
+    elif use_kernel:
+        used_ag_streams = [ag_streams[0]]
+    else:
+        used = sorted(set(r % len(ag_streams) for r in range(num_ranks) if r != rank))
+        used_ag_streams = [ag_streams[i] for i in used]
+    fork = current_stream.record_event()
+    gemm_stream.wait_event(fork)
+    for ag_stream in used_ag_streams:
+        ag_stream.wait_event(fork)
 
     def call_ag():
         if num_ranks > 1 and use_kernel:
@@ -330,16 +340,16 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
                 link_gbps=ctx.link_gbps if paced else 0.0, start_stamp=ctx.start_stamp if paced else None)
 
     def call_gemm(max_wgs):
-        with torch.cuda.stream(gemm_stream):
-            gated_gemm(workspace[:M], a, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
-                       row_scale=row_scale, col_scale=col_scale, wait_value=1,
-                       spin_limit=ctx.spin_limit if ctx is not None else 0,
-                       status=ctx.status if ctx is not None else None, max_workgroups=max_wgs, stream=gemm_stream)
+        # (the launch names its stream; nothing here runs on torch's current stream)
+        gated_gemm(workspace[:M], a, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
+                   row_scale=row_scale, col_scale=col_scale, wait_value=1,
+                   spin_limit=ctx.spin_limit if ctx is not None else 0,
+                   status=ctx.status if ctx is not None else None, max_workgroups=max_wgs, stream=gemm_stream)
 
     if serial or (ctx is not None and ctx.preset_flags):
         # every chunk delivered before the GEMM starts
         call_ag()
-        for ag_stream in ag_streams:
+        for ag_stream in used_ag_streams:
             gemm_stream.wait_stream(ag_stream)
         if serial:
             torch.cuda.synchronize()
@@ -355,8 +365,9 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
             call_ag()  # the reference's order (:300-304)
             call_gemm(max_wgs)
     current_stream.wait_stream(gemm_stream)
-    for ag_stream in ag_streams:
+    for ag_stream in used_ag_streams:
         current_stream.wait_stream(ag_stream)
+    # (c and the operands are used on gemm_stream by kernels queued before this join; the caller's stream owns them)
     return None
 
 

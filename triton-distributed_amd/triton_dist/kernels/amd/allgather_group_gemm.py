@@ -240,8 +240,10 @@ def ag_group_gemm_intra_node(a, b, ctx=None, full_topk_ids=None, num_experts=Non
     workspace, barrier = ctx.workspace_tensors[rank], ctx.barrier_tensors[rank]
     current = torch.cuda.current_stream()
     gemm_stream = current if ctx.group_gemm_stream is None else ctx.group_gemm_stream
-    ctx.ag_stream.wait_stream(current)
-    gemm_stream.wait_stream(current)
+    fork = current.record_event()   # one event for both streams; a GEMM on the caller's own stream needs none
+    ctx.ag_stream.wait_event(fork)
+    if gemm_stream is not current:
+        gemm_stream.wait_event(fork)
     # producer: one copy and one flag per peer rank (reference :354-361)
     nbytes = M_per_rank * K * a.element_size()
     for idx in range(1, W):
@@ -251,12 +253,13 @@ def ag_group_gemm_intra_node(a, b, ctx=None, full_topk_ids=None, num_experts=Non
         _lib.call("tdist_producer_push_chunk", workspace.data_ptr() + r * nbytes, ctx.peer_shards[r].data_ptr(), nbytes,
                   barrier.data_ptr() + 4 * r, ctx.one.data_ptr(), 0, ctx.ag_stream.cuda_stream)
     max_wgs = max(1, _lib.load().tdist_num_cus() - ctx.producer_cus) if (W > 1 and ctx.producer_cus > 0) else 0
-    with torch.cuda.stream(gemm_stream):
-        group_gemm_gated(workspace[:M_per_rank * W], a, rank * M_per_rank, b_nk, C, ctx.sorted_topk_ids,
-                         ctx.aligned_expert_ids, ctx.aligned_barrier_ids, ctx.aligned_num_tokens, ctx.BLOCK_M,
-                         ctx.full_num_tokens, ctx.topk, M_per_rank, ctx.first_block, barrier, rank,
-                         spin_limit=ctx.spin_limit, status=ctx.status, max_workgroups=max_wgs, stream=gemm_stream)
+    # (the launch names its stream; nothing here runs on torch's current stream)
+    group_gemm_gated(workspace[:M_per_rank * W], a, rank * M_per_rank, b_nk, C, ctx.sorted_topk_ids,
+                     ctx.aligned_expert_ids, ctx.aligned_barrier_ids, ctx.aligned_num_tokens, ctx.BLOCK_M,
+                     ctx.full_num_tokens, ctx.topk, M_per_rank, ctx.first_block, barrier, rank,
+                     spin_limit=ctx.spin_limit, status=ctx.status, max_workgroups=max_wgs, stream=gemm_stream)
     current.wait_stream(ctx.ag_stream)
-    current.wait_stream(gemm_stream)
+    if gemm_stream is not current:
+        current.wait_stream(gemm_stream)
     fill_flags(barrier, 0)   # the reference's block_barriers[rank].zero_() (:399)
     return C
