@@ -143,6 +143,43 @@ def test_gemm_rs_scatter_and_grouped_forms(cuda, split_k):
         assert torch.equal(c.float().cpu(), ref.to(c.dtype).float()), (dtype, block)
 
 
+def test_graph_replay_with_new_inputs(cuda, split_k):
+    """A captured launch carries one epoch for all its replays: the flags must be back down after every replay, and a
+    replay on new operands must not see anything of the one before."""
+    from triton_dist.kernels.amd import gated_gemm
+    M, N, K, wgs = 1024, 768, 1024, 40
+    announce("split-k graph replay")
+    g = torch.Generator().manual_seed(11)
+    a_d = torch.empty((M, K), dtype=torch.bfloat16, device=cuda)
+    b_d = torch.empty((N, K), dtype=torch.bfloat16, device=cuda)
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=cuda)
+    status = torch.zeros(2, dtype=torch.int32, device=cuda)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        gated_gemm(a_d, None, 0, b_d, c, None, 0, 0, 1, status=status, max_workgroups=wgs)   # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gated_gemm(a_d, None, 0, b_d, c, None, 0, 0, 1, status=status, max_workgroups=wgs, stream=torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    for replay in range(4):
+        a, b = ints((M, K), g, torch.bfloat16), ints((N, K), g, torch.bfloat16)
+        a_d.copy_(a)
+        b_d.copy_(b)
+        c.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert status.tolist() == [0, 0]
+        assert torch.equal(c.cpu(), (a.float() @ b.float().T).to(torch.bfloat16)), "replay %d" % replay
+    # and an eager launch afterwards (a new epoch) on the same workspace
+    gated_gemm(a_d, None, 0, b_d, c, None, 0, 0, 1, status=status, max_workgroups=wgs)
+    torch.cuda.synchronize()
+    assert torch.equal(c.cpu(), (a.float() @ b.float().T).to(torch.bfloat16))
+
+
 def test_workspace_argument_errors(cuda):
     from triton_dist import _lib
     lib = _lib.load()

@@ -586,6 +586,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
             }
             __builtin_amdgcn_s_sleep(4);
           }
+          // this workgroup is the flag's only reader: lower it again, so that a launch replayed from a captured
+          // graph (same epoch every time) starts from lowered flags as well
+          if (ok) __hip_atomic_store(p.sk_flags + w, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           if (!ok && p.status != nullptr) {
             if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = -1 - w;
           }
