@@ -469,6 +469,21 @@ def bench_mfma_ceiling(dev, steps, warmup):
     return out
 
 
+def bench_library_gemm(dev, steps, warmup):
+    """Yardstick, not product: the vendor library's GEMM (torch.matmul = hipBLASLt) on the headline shape and the
+    same seeded operands, timed the same way. Says what fraction of the nominal peak AMD's own kernel sustains on
+    this data under the same power limit."""
+    import torch
+    M, N, K = 8192, 8192, 3584
+    g = torch.Generator().manual_seed(3 + 1)
+    a = torch.randn((M, K), generator=g).to(torch.bfloat16).to(dev)
+    b = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(dev)
+    bt = b.t()
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    s = time_launches(lambda: torch.matmul(a, bt, out=out), steps, warmup)
+    return roof("mfma", 2.0 * M * N * K, s, "bf16")
+
+
 def main():
     global LIVE_PRODUCER, SETTLE_SECONDS
     ap = argparse.ArgumentParser()
@@ -477,7 +492,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle-seconds", type=float, default=SETTLE_SECONDS,
                     help="untimed period of the same launches before each warm-up, to reach the sustained clock")
-    ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,moe_gemm,copy,mfma (c2 always runs)")
+    ap.add_argument("--only", default="", help="comma list of c1,c2,c3,c4,c5,moe_gemm,copy,mfma,library (c2 always runs)")
     ap.add_argument("--no-live-producer", action="store_true",
                     help="skip the AG-GEMM legs in which a copy stream releases the flags while the GEMM spins: a "
                     "counter-collecting profiler serialises dispatches, so the producer could never run beside it")
@@ -496,7 +511,7 @@ def main():
     _lib.check(_lib.load().tdist_init())
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    want = set(x for x in args.only.split(",") if x) or {"c1", "c2", "c3", "c4", "c5", "moe_gemm", "copy", "mfma"}
+    want = set(x for x in args.only.split(",") if x) or {"c1", "c2", "c3", "c4", "c5", "moe_gemm", "copy", "mfma", "library"}
 
     step_s, gemm_roof, red_roof, cpu, err = bench_c2(dev, args.steps, args.warmup)
     log("c2 step %.1f us, gemm %s, reduce %s" % (step_s * 1e6, gemm_roof, red_roof))
@@ -524,6 +539,9 @@ def main():
     if "mfma" in want:
         kernels["mfma_only_rate_yardstick"] = bench_mfma_ceiling(dev, args.steps, args.warmup)
         log("mfma", kernels["mfma_only_rate_yardstick"])
+    if "library" in want:
+        kernels["hipblaslt_matmul_c2_shape_yardstick"] = bench_library_gemm(dev, args.steps, args.warmup)
+        log("library", kernels["hipblaslt_matmul_c2_shape_yardstick"])
 
     flops = 2.0 * 8192 * 8192 * 3584
     line = {
