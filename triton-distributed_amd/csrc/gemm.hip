@@ -26,6 +26,7 @@
 #include <stdlib.h>
 
 #include <mutex>
+#include <utility>
 
 #include "common.h"
 
@@ -82,6 +83,8 @@ struct GemmParams {
 struct ElemBF16 {
   static constexpr int kBytes = 2;
   static constexpr int kLaneBytes = 16;  // K bytes one lane feeds to one MFMA
+  static constexpr int kRows = 32;       // rows (and columns) of one MFMA block
+  typedef float16v acc_t;                // its accumulators in one lane
   typedef int4v frag;
   __device__ static __forceinline__ frag load(const TDIST_AS3 unsigned char* c0, const TDIST_AS3 unsigned char*) {
     return *(const TDIST_AS3 int4v*)c0;
@@ -95,6 +98,8 @@ struct ElemBF16 {
 struct ElemF16 {
   static constexpr int kBytes = 2;
   static constexpr int kLaneBytes = 16;
+  static constexpr int kRows = 32;
+  typedef float16v acc_t;
   typedef int4v frag;
   __device__ static __forceinline__ frag load(const TDIST_AS3 unsigned char* c0, const TDIST_AS3 unsigned char*) {
     return *(const TDIST_AS3 int4v*)c0;
@@ -105,9 +110,34 @@ struct ElemF16 {
   }
   __device__ static __forceinline__ uint32_t pack(float a, float b) { return pack_f16x2(a, b); }
 };
+// The same element types on the 16x16x32 MFMA: four lane groups along K instead of two, sixteen rows per block.
+// Per flop it draws less power than the 32x32x16 form, which is what the clock of a long GEMM on real data
+// is limited by.
+// Its four-register result is not tied to its accumulator input in the compiler's instruction model; with all 256
+// accumulation registers in use the allocator then shuffles accumulators between registers inside the K loop. Written
+// as assembly with one read-write operand the instruction works in place. (The compiler then knows none of its
+// hazards: the K loop never reads an accumulator, and the code after it waits out the last MFMA before it does.)
+struct ElemBF16N : ElemBF16 {
+  static constexpr int kRows = 16;
+  typedef float4v acc_t;
+  __device__ static __forceinline__ float4v mma(frag a, frag b, float4v c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    return c;
+  }
+};
+struct ElemF16N : ElemF16 {
+  static constexpr int kRows = 16;
+  typedef float4v acc_t;
+  __device__ static __forceinline__ float4v mma(frag a, frag b, float4v c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    return c;
+  }
+};
 struct ElemFP8 {
   static constexpr int kBytes = 1;
   static constexpr int kLaneBytes = 32;
+  static constexpr int kRows = 32;
+  typedef float16v acc_t;
   typedef int8v frag;
   __device__ static __forceinline__ frag load(const TDIST_AS3 unsigned char* c0, const TDIST_AS3 unsigned char* c1) {
     const int4v lo = *(const TDIST_AS3 int4v*)c0;
@@ -143,10 +173,12 @@ struct GemmCfg {
   static constexpr int kBBytes = BN * KB;
   static constexpr int kStageBytes = kABytes + kBBytes;
   static constexpr int kP = NST - 1;
-  static constexpr int kKSteps = KB / (2 * E::kLaneBytes);
+  static constexpr int kLaneGroups = 64 / E::kRows;  // lane groups along K within one MFMA
+  static constexpr int kAccLen = E::kRows * E::kRows / 64;  // accumulators per lane and MFMA block
+  static constexpr int kKSteps = KB / (kLaneGroups * E::kLaneBytes);
   static constexpr int kFragVecs = E::kLaneBytes / 16;  // 16-byte pieces per operand fragment (1 or 2)
   static constexpr int kWaveM = BM / WM, kWaveN = BN / WN;
-  static constexpr int kTM = kWaveM / 32, kTN = kWaveN / 32;
+  static constexpr int kTM = kWaveM / E::kRows, kTN = kWaveN / E::kRows;
   // NST == 5 selects the split ring: three stages of A rows and two of B rows (five half stages, exactly the
   // 160 KB of LDS at 256x256x128). A freed B stage is refilled at once; the A refill then has a whole K tile of
   // time, so the DMA issue can be spread evenly over the K steps instead of bunching up behind the barrier.
@@ -186,6 +218,17 @@ struct GemmCfg {
   static_assert(kEpiBytes * kWaves <= kLdsBytes, "epilogue staging must fit in the stage ring");
   static_assert(kWaveM % 32 == 0 && kWaveN % 32 == 0, "wave tile");
 };
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a constant in every trip
+// without leaning on the unroller (which gives up on bodies as long as a K step's schedule)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 // Waits until at most `kOutstanding` of this wave's DMA loads are in flight and for its LDS reads, then joins
 // the workgroup barrier.
@@ -233,7 +276,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int wm = wave / WN, wn = wave % WN;
-  const int l32 = lane & 31, lh = lane >> 5;
+  const int lrow = lane % E::kRows, lgrp = lane / E::kRows;
 
   const int num_pid_m = (p.M + BM - 1) / BM;
   const int num_pid_n = (p.N + BN - 1) / BN;
@@ -391,15 +434,15 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     typename E::frag a_cur[C::kTM], b_cur[C::kTN], a_nxt[C::kTM], b_nxt[C::kTN];
     // f-th operand fragment (A fragments first) of K step ks of tile kt
     auto load_frag = [&](int kt, int ks, int f, typename E::frag* af, typename E::frag* bf) {
-      const int c0 = (ks * 2 + lh) * C::kFragVecs;  // first 16-byte chunk of this lane's K bytes
+      const int c0 = (ks * C::kLaneGroups + lgrp) * C::kFragVecs;  // first 16-byte chunk of this lane's K bytes
       const int c1 = c0 + C::kFragVecs - 1;         // last one (== c0 for 16-byte fragments)
       if (f < C::kTM) {
-        const int r = wm * C::kWaveM + f * 32 + l32;
+        const int r = wm * C::kWaveM + f * E::kRows + lrow;
         lds_u8 const row = a_stage(kt) + r * KB;
         af[f] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
       } else {
         const int j = f - C::kTM;
-        const int r = wn * C::kWaveN + j * 32 + l32;
+        const int r = wn * C::kWaveN + j * E::kRows + lrow;
         lds_u8 const row = b_stage(kt) + r * KB;
         bf[j] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
       }
@@ -409,16 +452,77 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       for (int f = 0; f < C::kTM + C::kTN; ++f) load_frag(kt, ks, f, af, bf);
     };
 
-    float16v acc[C::kTN][C::kTM];
+    typename E::acc_t acc[C::kTN][C::kTM];
 #pragma unroll
     for (int j = 0; j < C::kTN; ++j)
 #pragma unroll
       for (int i = 0; i < C::kTM; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[j][i][e] = 0.f;
+        for (int e = 0; e < C::kAccLen; ++e) acc[j][i][e] = 0.f;
 
     constexpr int kMfmaPerStep = C::kTM * C::kTN;
-    if constexpr (C::kSplit) {
+    if constexpr (C::kSplit && E::kRows == 16) {
+      // ---- split ring, 16-row MFMA blocks ------------------------------------------------------------
+      // The MFMAs of a K step run in B-fragment-major order: a B fragment serves kTM MFMAs in a row and is then dead,
+      // so the next step's B fragment is read into the same registers right behind them; only the A fragments, which
+      // the whole step uses, are double-buffered. No read sits in the first kLead slots: the last step of a tile holds
+      // its barrier there (the reads before it come from the stages the barrier releases, and the last of them,
+      // issued behind the previous step's final MFMA, has those slots to come back).
+      static_assert(C::kKSteps == 2 && C::kTM >= 4, "schedule written for two K steps per tile");
+      constexpr int kLead = C::kTM - 1 < 4 ? C::kTM - 1 : 4;
+      constexpr int kAStride = (kMfmaPerStep - kLead - 2) / C::kTM;  // slots between two A fragment reads
+      auto issue_list = [&](int cyc, int q) {
+        if (q < C::kBInstr) issue_b(cyc + 2, q);
+        else issue_a(cyc + 3, q - C::kBInstr);
+      };
+#pragma unroll
+      for (int t = 0; t < C::kAInstr; ++t) issue_a(0, t);
+#pragma unroll
+      for (int u = 0; u < C::kBInstr; ++u) issue_b(0, u);
+#pragma unroll
+      for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+#pragma unroll
+      for (int q = 0; q < C::kDmaPerStep; ++q) issue_list(-1, q);
+      wait_tiles_and_barrier<C::kAInstr + C::kDmaPerStep>();
+      load_frags(0, 0, a_cur, b_cur);
+      __builtin_amdgcn_sched_barrier(0);
+      for (int kt = 0; kt < KTp; ++kt) {
+        const int kt_next = min(kt + 1, KTp - 1);
+        auto step = [&](auto ks_c, typename E::frag* a_now, typename E::frag* a_new) {
+          constexpr int ks = decltype(ks_c)::value;
+          constexpr bool last = ks == C::kKSteps - 1;
+          constexpr int first = last ? kLead : 0;
+          constexpr int nslots = kMfmaPerStep - first;
+          constexpr int pos = (ks + 1) % C::kKSteps;
+          const int r_kt = last ? kt_next : kt;   // tile and K step the reads of this step fetch
+          constexpr int r_ks = last ? 0 : ks + 1;
+          static_for<kMfmaPerStep>([&](auto idx_c) {
+            constexpr int idx = decltype(idx_c)::value;
+            constexpr int j = idx / C::kTM, i = idx % C::kTM;
+            acc[j][i] = E::mma(b_cur[j], a_now[i], acc[j][i]);
+            if constexpr (last && idx == kLead - 1) {
+              __builtin_amdgcn_sched_barrier(0);
+              wait_tiles_and_barrier<C::kAInstr>();
+              __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (i == C::kTM - 1) load_frag(r_kt, r_ks, C::kTM + j, a_new, b_cur);  // B fragment j, in place
+            if constexpr (idx > kLead && (idx - kLead - 1) % kAStride == 0 && (idx - kLead - 1) / kAStride < C::kTM)
+              load_frag(r_kt, r_ks, (idx - kLead - 1) / kAStride, a_new, b_cur);
+            if constexpr (idx >= first) {
+              constexpr int slot = idx - first;
+#pragma unroll
+              for (int d = 0; d < C::kDmaPerStep; ++d)
+                if (slot == (d * nslots) / C::kDmaPerStep) issue_list(last ? kt : kt - 1, pos * C::kDmaPerStep + d);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          });
+        };
+        step(std::integral_constant<int, 0>{}, a_cur, a_nxt);
+        step(std::integral_constant<int, 1>{}, a_nxt, a_cur);
+      }
+      // the last MFMAs' results are readable 4 passes + 3 cycles after issue
+      asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+    } else if constexpr (C::kSplit) {
       // ---- split ring ------------------------------------------------------------------------------
       // The DMA list of one cycle is [B(kt+2) rows..., A(kt+3) rows...]; it starts right after the barrier in the
       // last K step of tile kt (B stage kt%2 and A stage kt%3 have just been released) and runs, kDmaPerStep
@@ -557,7 +661,17 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     }
 
     // ---- epilogue ---------------------------------------------------------------------------------
-    // acc[j][i][e]: output row m = wm*kWaveM + 32i + l32, column n = wn*kWaveN + 32j + 8*(e/4) + 4*lh + e%4
+    // A lane's accumulators, seen as kRowBlocks blocks of 32 rows of the wave tile times kGroups groups of four
+    // consecutive columns of one row. Group g of row block ib is
+    //   32-row MFMA blocks: acc[g/4][ib][4*(g%4) ...],   row 32*ib + lrow,              column 8*g + 4*lgrp
+    //   16-row MFMA blocks: acc[g/2][2*ib + g%2][0 ...], row 32*ib + 16*(g%2) + lrow,   column 16*(g/2) + 4*lgrp
+    constexpr int kRowBlocks = C::kWaveM / 32, kGroups = C::kWaveN / 8;
+    constexpr bool kWide = E::kRows == 32;
+    // 256 accumulators live in AGPRs; they are then read one by one where they are used, instead of letting the
+    // compiler copy all of them to VGPRs at the loop exit (which spills)
+    constexpr bool kAgpr = C::kTM * C::kTN * C::kAccLen >= 256;
+#define TDIST_ACC(ib, g, e) \
+  acc[kWide ? (g) / 4 : (g) / 2][kWide ? (ib) : 2 * (ib) + (g) % 2][kWide ? 4 * ((g) % 4) + (e) : (e)]
     wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
     if (p.sk_on && KTp < KT) {
       // ---- split last round: this piece is not the whole K range -------------------------------
@@ -566,8 +680,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       // tile then hands its sum on through its slot; the piece that does start there runs the epilogue. (The pieces
       // are equally long and start together, so the chain costs its length times one hand-over.)
       constexpr int kThreads = C::kWaves * 64;
-      constexpr int kQuads = C::kTM * C::kTN * 4;  // float4 groups of accumulators per lane
-      constexpr bool kAgpr = C::kTM * C::kTN * 16 >= 256;
+      constexpr int kQuads = kRowBlocks * kGroups;  // float4 groups of accumulators per lane
       // slot addresses: a uniform base per float4 group plus one 32-bit lane offset (from an opaque copy of the
       // thread id, so that nothing of this is computed ahead and held across the K loop)
       uint32_t sk_voff = threadIdx.x;
@@ -608,17 +721,17 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
           for (int r = 0; r < kLoadBatch; ++r) t[r] = *(const TDIST_AS1 float4v*)(src + (size_t)(r0 + r) * (kThreads * 16) + sk_voff);
 #pragma unroll
           for (int r = 0; r < kLoadBatch; ++r) {
-            const int j = (r0 + r) / (C::kTM * 4), i = ((r0 + r) / 4) % C::kTM, q = (r0 + r) % 4;
+            const int ib = (r0 + r) / kGroups, g = (r0 + r) % kGroups;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               if constexpr (kAgpr) {
                 // in place, so that the accumulators stay where they are on both sides of this branch
                 float tmp;
                 asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_add_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
-                             : "+a"(acc[j][i][4 * q + e]), "=&v"(tmp)
+                             : "+a"(TDIST_ACC(ib, g, e)), "=&v"(tmp)
                              : "v"(t[r][e]));
               } else {
-                acc[j][i][4 * q + e] += t[r][e];
+                TDIST_ACC(ib, g, e) += t[r][e];
               }
             }
           }
@@ -634,15 +747,15 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         unsigned char* slot = (unsigned char*)(p.sk_partials + (int64_t)wg_pos * (BM * BN)) + sk_voff;
 #pragma unroll
         for (int r = 0; r < kQuads; ++r) {
-          const int j = r / (C::kTM * 4), i = (r / 4) % C::kTM, q = r % 4;
+          const int ib = r / kGroups, g = r % kGroups;
           float4v t;
           if constexpr (kAgpr) {
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[0]) : "a"(acc[j][i][4 * q + 0]));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[1]) : "a"(acc[j][i][4 * q + 1]));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[2]) : "a"(acc[j][i][4 * q + 2]));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[3]) : "a"(acc[j][i][4 * q + 3]));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[0]) : "a"(TDIST_ACC(ib, g, 0)));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[1]) : "a"(TDIST_ACC(ib, g, 1)));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[2]) : "a"(TDIST_ACC(ib, g, 2)));
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[3]) : "a"(TDIST_ACC(ib, g, 3)));
           } else {
-            t = float4v{acc[j][i][4 * q + 0], acc[j][i][4 * q + 1], acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]};
+            t = float4v{TDIST_ACC(ib, g, 0), TDIST_ACC(ib, g, 1), TDIST_ACC(ib, g, 2), TDIST_ACC(ib, g, 3)};
           }
           asm volatile("s_nop 1\n\tglobal_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(slot), "v"(t) : "memory");
           slot += kThreads * 16;
@@ -660,7 +773,12 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // rebuilt per tile (a few dozen instructions) instead of being held in ~100 registers across the K loop.
     int e_lane = lane;
     asm volatile("" : "+v"(e_lane));
-    const int e_l32 = e_lane & 31, e_lh = e_lane >> 5;
+    const int e_lrow = e_lane % E::kRows, e_lgrp = e_lane / E::kRows;
+    // row (within its 32-row block) and first column of this lane's group g
+    auto group_row = [&](int g) { return kWide ? e_lrow : 16 * (g % 2) + e_lrow; };
+    auto group_col = [&](int g) { return kWide ? 8 * g + 4 * e_lgrp : 16 * (g / 2) + 4 * e_lgrp; };
+    // index of group g's row among the row scales held per MFMA row block
+    auto scale_slot = [&](int ib, int g) { return kWide ? ib : 2 * ib + g % 2; };
     // destination of this tile's rows
     unsigned char* Cbase;
     int64_t crow0;
@@ -677,39 +795,38 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     const int er = e_lane / kLanesPerRow, ec = e_lane % kLanesPerRow;
     const bool n_vec_ok = (p.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(Cbase) & 15) == 0);
 
-    // packs the 32 x 32 block (i, j) of the wave tile into its staging rows
-    // packs four columns x 32 rows (column group q of block (i, j)) into the staging rows
-    auto stage_group_at = [&](int i, int j, int q, float rsi, const float4v* cs, lds_u8 where) {
+    // packs group g of row block ib (four columns of one row per lane; `rs` holds the row scales by scale_slot,
+    // `csg` the group's four column scales) and writes it to `where` in the staging rows
+    auto stage_group_at = [&](int ib, int g, const float* rs, const float4v csg, lds_u8 where) {
       float v0, v1, v2, v3;
-      if constexpr (C::kTM * C::kTN * 16 >= 256) {
-        // 256 accumulators live in AGPRs; read each one here, where it is packed, instead of letting the
-        // compiler copy all of them to VGPRs at the loop exit (which spills)
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v0) : "a"(acc[j][i][4 * q + 0]));
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v1) : "a"(acc[j][i][4 * q + 1]));
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v2) : "a"(acc[j][i][4 * q + 2]));
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v3) : "a"(acc[j][i][4 * q + 3]));
+      if constexpr (kAgpr) {
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v0) : "a"(TDIST_ACC(ib, g, 0)));
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v1) : "a"(TDIST_ACC(ib, g, 1)));
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v2) : "a"(TDIST_ACC(ib, g, 2)));
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v3) : "a"(TDIST_ACC(ib, g, 3)));
       } else {
-        v0 = acc[j][i][4 * q + 0], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2], v3 = acc[j][i][4 * q + 3];
+        v0 = TDIST_ACC(ib, g, 0), v1 = TDIST_ACC(ib, g, 1), v2 = TDIST_ACC(ib, g, 2), v3 = TDIST_ACC(ib, g, 3);
       }
-      if (kScales) {
-        v0 *= rsi * cs[q][0];
-        v1 *= rsi * cs[q][1];
-        v2 *= rsi * cs[q][2];
-        v3 *= rsi * cs[q][3];
+      if constexpr (kScales) {
+        const float rsi = rs[scale_slot(ib, g)];
+        v0 *= rsi * csg[0];
+        v1 *= rsi * csg[1];
+        v2 *= rsi * csg[2];
+        v3 *= rsi * csg[3];
       }
       const int2v w = {(int)E::pack(v0, v1), (int)E::pack(v2, v3)};
       *(TDIST_AS3 int2v*)where = w;
     };
-    auto stage_group = [&](int i, int j, int q, float rsi, const float4v* cs) {
-      const int mrow = 32 * i + e_l32;
-      const int ncol = 32 * j + 8 * q + 4 * e_lh;
-      stage_group_at(i, j, q, rsi, cs,
+    auto stage_group = [&](int ib, int g, const float* rs, const float4v csg) {
+      const int mrow = 32 * ib + group_row(g);
+      const int ncol = group_col(g);
+      stage_group_at(ib, g, rs, csg,
                      epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2);
     };
-    // the same for the 32 x 32 block (i, j)
-    auto stage_block = [&](int i, int j, float rsi, const float4v* cs) {
+    // the same for the four groups of the 32 x 32 block (ib, jb); cs4[g % 4] are their column scales
+    auto stage_block = [&](int ib, int jb, const float* rs, const float4v* cs4) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) stage_group(i, j, q, rsi, cs);
+      for (int q = 0; q < 4; ++q) stage_group(ib, 4 * jb + q, rs, kScales ? cs4[q] : float4v{1.f, 1.f, 1.f, 1.f});
       __builtin_amdgcn_sched_barrier(0);  // keep the accumulator read-out block by block (register pressure)
     };
     // staged rows [row0, row0 + nrows) of the wave tile → global memory, 16 bytes per lane
@@ -758,43 +875,41 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       if (m0 + BM <= p.M && n0 + BN <= p.N && n_vec_ok) {
         stored = true;
         constexpr int kPasses = 32 / kRowsPerPass;
-        static_assert(2 * kPasses == 4 * C::kTN, "one read or store per column group of a row block");
+        static_assert(2 * kPasses == kGroups, "one read or store per column group of a row block");
         const int64_t row_bytes = p.ldc * 2;
         unsigned char* const tile_dst = Cbase + ((crow0 + wm * C::kWaveM) * p.ldc + n0 + wn * C::kWaveN) * 2;
         const uint32_t lane_off = (uint32_t)er * (uint32_t)row_bytes + (uint32_t)ec * 16u;
         const bool streaming = p.scatter_bufs == nullptr;
-        float rs[C::kTM];
-        float4v cs[kScales ? C::kTN : 1][4];
-#pragma unroll
-        for (int i = 0; i < C::kTM; ++i) {
-          rs[i] = 1.f;
-          if (kScales && p.row_scale) rs[i] = p.row_scale[m0 + wm * C::kWaveM + 32 * i + e_l32];
-        }
+        float rs[kScales ? C::kTM : 1] = {1.f};
+        float4v cs[kScales ? kGroups : 1] = {float4v{1.f, 1.f, 1.f, 1.f}};
         if constexpr (kScales) {
 #pragma unroll
-          for (int j = 0; j < C::kTN; ++j) {
+          for (int i = 0; i < C::kTM; ++i) {
+            rs[i] = 1.f;
+            if (p.row_scale) rs[i] = p.row_scale[m0 + wm * C::kWaveM + E::kRows * i + e_lrow];
+          }
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {  // the four column scales of each of this lane's four column groups in block j
-              cs[j][q] = float4v{1.f, 1.f, 1.f, 1.f};
-              if (p.col_scale) cs[j][q] = *(const float4v*)(p.col_scale + n0 + wn * C::kWaveN + 32 * j + 8 * q + 4 * e_lh);
-            }
+          for (int g = 0; g < kGroups; ++g) {  // the four column scales of each of this lane's column groups
+            cs[g] = float4v{1.f, 1.f, 1.f, 1.f};
+            if (p.col_scale) cs[g] = *(const float4v*)(p.col_scale + n0 + wn * C::kWaveN + group_col(g));
           }
         }
         // Staging addresses: a row block adds a constant to them (32 rows leave the swizzle term alone), so one
         // address per column group and one per swizzle phase of the read-back serve the whole tile, with the row
         // block in the instruction's offset field.
-        constexpr int kGroups = 4 * C::kTN;
         constexpr int kReadPhases = (C::kEpiSwz + 1) / kRowsPerPass > 1 ? (C::kEpiSwz + 1) / kRowsPerPass : 1;
         static_assert(kPasses % kReadPhases == 0 && (C::kEpiSwz + 1) <= 32, "swizzle period within a row block");
         lds_u8 wbase[kGroups], rbase[kReadPhases];
 #pragma unroll
-        for (int c = 0; c < kGroups; ++c)
-          wbase[c] = epi + e_l32 * C::kEpiPitch + ((c ^ (e_l32 & C::kEpiSwz)) << 4) + 8 * e_lh;
+        for (int g = 0; g < kGroups; ++g) {
+          const int mrow = group_row(g), ncol = group_col(g);
+          wbase[g] = epi + mrow * C::kEpiPitch + (((ncol >> 3) ^ (mrow & C::kEpiSwz)) << 4) + (ncol & 7) * 2;
+        }
 #pragma unroll
         for (int ph = 0; ph < kReadPhases; ++ph)
           rbase[ph] = epi + er * C::kEpiPitch + ((ec ^ ((ph * kRowsPerPass + er) & C::kEpiSwz)) << 4);
         auto stage_fast = [&](int i, int g) {
-          stage_group_at(i, g / 4, g % 4, rs[i], cs[kScales ? g / 4 : 0], wbase[g] + i * 32 * C::kEpiPitch);
+          stage_group_at(i, g, rs, cs[kScales ? g : 0], wbase[g] + i * 32 * C::kEpiPitch);
         };
 #pragma unroll
         for (int g = 0; g < kGroups; ++g) stage_fast(0, g);
@@ -816,11 +931,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         constexpr int kLag = 2;
         static_assert(kPasses >= 2 * kLag, "the store of a piece follows its read by kLag reads");
 #pragma unroll
-        for (int i = 0; i + 1 < C::kTM; ++i) {
+        for (int i = 0; i + 1 < kRowBlocks; ++i) {
           __builtin_amdgcn_wave_barrier();
 #pragma unroll
-          for (int g = 0; g < 4 * C::kTN; ++g) {
-            stage_fast(i + 1 < C::kTM ? i + 1 : 0, g);
+          for (int g = 0; g < kGroups; ++g) {
+            stage_fast(i + 1, g);
             if (g % 2 == 0) {
               read_piece(i, g / 2);
             } else {
@@ -832,7 +947,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
           }
         }
         {
-          constexpr int i = C::kTM - 1;  // nothing left to pack behind the last block
+          constexpr int i = kRowBlocks - 1;  // nothing left to pack behind the last block
           __builtin_amdgcn_wave_barrier();
 #pragma unroll
           for (int u = 0; u < kPasses - kLag; ++u) read_piece(i, u);
@@ -848,12 +963,12 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       }
     }
     if (stored) {
-    } else if constexpr (!kScales && C::kTM * C::kTN * 16 >= 256) {
+    } else if constexpr (!kScales && kAgpr) {
       // row block by row block: the stores of block i drain while block i+1 is being packed
 #pragma unroll
-      for (int i = 0; i < C::kTM; ++i) {
+      for (int i = 0; i < kRowBlocks; ++i) {
 #pragma unroll
-        for (int j = 0; j < C::kTN; ++j) stage_block(i, j, 1.f, nullptr);
+        for (int j = 0; j < kGroups / 4; ++j) stage_block(i, j, nullptr, nullptr);
         __builtin_amdgcn_wave_barrier();
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         store_rows(32 * i, 32);
@@ -863,24 +978,24 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 #pragma unroll
       for (int i = 0; i < C::kTM; ++i) {
         rs[i] = 1.f;
-        if (kScales && p.row_scale) rs[i] = p.row_scale[min(m0 + wm * C::kWaveM + 32 * i + e_l32, p.M - 1)];
+        if (kScales && p.row_scale) rs[i] = p.row_scale[min(m0 + wm * C::kWaveM + E::kRows * i + e_lrow, p.M - 1)];
       }
 #pragma unroll
-      for (int j = 0; j < C::kTN; ++j) {
+      for (int j = 0; j < kGroups / 4; ++j) {
         // the four column scales of each of this lane's four column groups in this 32-column block
         float4v cs[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           cs[q] = float4v{1.f, 1.f, 1.f, 1.f};
           if (kScales && p.col_scale) {
-            const int gn = n0 + wn * C::kWaveN + 32 * j + 8 * q + 4 * e_lh;
+            const int gn = n0 + wn * C::kWaveN + group_col(4 * j + q);
             if (gn + 3 < p.N) cs[q] = *(const float4v*)(p.col_scale + gn);
             else
               for (int e = 0; e < 4; ++e) cs[q][e] = p.col_scale[min(gn + e, p.N - 1)];
           }
         }
 #pragma unroll
-        for (int i = 0; i < C::kTM; ++i) stage_block(i, j, rs[i], cs);
+        for (int i = 0; i < kRowBlocks; ++i) stage_block(i, j, rs, cs);
       }
       __builtin_amdgcn_wave_barrier();
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -889,6 +1004,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // the next tile's prologue overwrites the ring: every wave must be done reading its staging area
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   }
+#undef TDIST_ACC
 }
 
 // ---- host side ------------------------------------------------------------------------------------
@@ -944,6 +1060,13 @@ struct SkWorkspace {
 };
 static SkWorkspace g_sk[kSkMaxDevices];
 static std::mutex g_sk_mutex;
+
+// The 16-bit 256-row tiles run on the 16x16x32 MFMA; TDIST_GEMM_MFMA16=0 puts them back on 32x32x16 (measurement
+// aid: the two give the same bits, at different power)
+static bool narrow_mfma_env() {
+  if (const char* v = getenv("TDIST_GEMM_MFMA16")) return atoi(v) != 0;
+  return true;
+}
 
 // 0 = off, 1 = on wherever the workspace allows, -1 = by the cost estimate
 static int sk_env() {
@@ -1046,6 +1169,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   const int BM = kChoices[pick].bm;
   const int BN = kChoices[pick].bn;
   const bool big = pick == 0;
+  const bool narrow_mfma = narrow_mfma_env();
 
   GemmParams p;
   p.A = (const unsigned char*)c.A;
@@ -1135,11 +1259,19 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       return scales ? launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, true>(p, grid, c.stream, who)          \
                     : launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);        \
   }
+    if (narrow_mfma && variant == 6 && elem != kElemFP8) {
+      if (elem == kElemBF16) return launch_gemm_cfg<ElemBF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      return launch_gemm_cfg<ElemF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+    }
     switch (variant) {
       case 2: TDIST_BIG(256, 128, 2, 4, 2)
       case 5: TDIST_BIG(256, 128, 2, 4, 5)
       default: TDIST_BIG(256, 128, 2, 2, 5)
     }
+  }
+  if (pick == 1 && narrow_mfma && elem != kElemFP8) {
+    if (elem == kElemBF16) return launch_gemm_cfg<ElemBF16N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+    return launch_gemm_cfg<ElemF16N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
   }
   if (pick == 1) { TDIST_BIG(128, 128, 2, 2, 5) }
 #undef TDIST_BIG
@@ -1258,6 +1390,12 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
       sk_attach(p);
     }
   }
+  const bool narrow_mfma = narrow_mfma_env();
+#define TDIST_GROUPED_NARROW(BM_, BN_, KB_, NST_)                                                                         \
+  if (narrow_mfma && elem == kElemBF16)                                                                                   \
+    return launch_gemm_cfg<ElemBF16N, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);                    \
+  if (narrow_mfma && elem == kElemF16)                                                                                    \
+    return launch_gemm_cfg<ElemF16N, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);
 #define TDIST_GROUPED(BM_, BN_, KB_, NST_)                                                                            \
   switch (elem) {                                                                                                    \
     case kElemBF16: return launch_gemm_cfg<ElemBF16, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who); \
@@ -1266,11 +1404,16 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   }
   if (c.block_size == 256) {
     if (!k128) return fail(TDIST_ERR_UNSUPPORTED, "%s: 256-row blocks need K*elem_size to be a multiple of 128 bytes", who);
+    TDIST_GROUPED_NARROW(256, 256, 128, 5)
     TDIST_GROUPED(256, 256, 128, 5)
   }
-  if (k128) { TDIST_GROUPED(128, 256, 128, 5) }   // 64 x 128 per wave on the split ring
+  if (k128) {  // 64 x 128 per wave on the split ring
+    TDIST_GROUPED_NARROW(128, 256, 128, 5)
+    TDIST_GROUPED(128, 256, 128, 5)
+  }
   TDIST_GROUPED(128, 128, 64, 4)
 #undef TDIST_GROUPED
+#undef TDIST_GROUPED_NARROW
 }
 
 }  // namespace tdist
