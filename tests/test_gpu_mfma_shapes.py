@@ -1,0 +1,94 @@
+"""The 256-row GEMM tiles run on the 16-row MFMA blocks (16x16x32 for bf16/f16, 16x16x128 for e4m3) by default and on
+the 32-row blocks (32x32x16 / 32x32x64) with TDIST_GEMM_MFMA16=0. Both forms add the same products in the same order
+per accumulator, so they must agree bit for bit; each is also held against the exact result on integer-valued inputs
+(every partial sum is an integer that fp32 holds) and, on random inputs, to max relative error <= 1e-2 of fp32."""
+import os
+
+import pytest
+import torch
+
+from tests.conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def mfma_env():
+    keys = ("TDIST_GEMM_MFMA16", "TDIST_GEMM_TILE")
+    old = {k: os.environ.get(k) for k in keys}
+    yield
+    torch.cuda.synchronize()
+    for k in keys:
+        if old[k] is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = old[k]
+
+
+def run_both(cuda, a, b, out_dtype, tile, **kw):
+    from triton_dist.kernels.amd import gated_gemm
+    out = {}
+    for mode in ("0", "1"):
+        os.environ["TDIST_GEMM_MFMA16"] = mode
+        os.environ["TDIST_GEMM_TILE"] = str(tile)
+        c = torch.full((a.shape[0], b.shape[0]), float("nan"), dtype=out_dtype, device=cuda)
+        status = torch.zeros(2, dtype=torch.int32, device=cuda)
+        gated_gemm(a, None, 0, b, c, None, 0, 0, 1, status=status, **kw)
+        torch.cuda.synchronize()
+        assert status.tolist() == [0, 0]
+        out[mode] = c
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
+@pytest.mark.parametrize("tile", [0, 1])
+@pytest.mark.parametrize("M,N,K", [(512, 512, 128), (768, 512, 384), (300, 200, 640), (1024, 1280, 1152)])
+def test_exact_and_bit_equal_on_integer_inputs(cuda, mfma_env, dtype, tile, M, N, K):
+    """One K tile (e4m3) or two; an odd number of K tiles (the e4m3 loop works in pairs of tiles); a ragged shape (the
+    bounds-checked epilogue); several tiles per workgroup row. tile 0 = 256x256, 1 = 256x128."""
+    announce("mfma shapes exact %s tile %d %dx%dx%d" % (dtype, tile, M, N, K))
+    g = torch.Generator().manual_seed(M + N + K + tile)
+    a = torch.randint(-2, 3, (M, K), generator=g).float().to(dtype).to(cuda)
+    b = torch.randint(-2, 3, (N, K), generator=g).float().to(dtype).to(cuda)
+    out_dtype = torch.bfloat16 if dtype == torch.float8_e4m3fn else dtype
+    out = run_both(cuda, a, b, out_dtype, tile)
+    ref = (a.float() @ b.float().T).to(out_dtype)
+    assert torch.equal(out["0"], ref)
+    assert torch.equal(out["1"], ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
+def test_random_inputs_bit_equal_and_close(cuda, mfma_env, dtype):
+    M, N, K = 1536, 1024, 4224
+    announce("mfma shapes random %s %dx%dx%d" % (dtype, M, N, K))
+    g = torch.Generator().manual_seed(11)
+    a = torch.randn((M, K), generator=g).to(dtype).to(cuda)
+    b = (torch.randn((N, K), generator=g) * 0.05).to(dtype).to(cuda)
+    kw = {}
+    ref = a.float() @ b.float().T
+    if dtype == torch.float8_e4m3fn:
+        kw["row_scale"] = (torch.rand(M, generator=g) * 0.09 + 0.01).to(cuda)
+        kw["col_scale"] = (torch.rand(N, generator=g) * 0.9 + 0.1).to(cuda)
+        ref = ref * kw["row_scale"][:, None] * kw["col_scale"][None, :]
+    out_dtype = torch.bfloat16
+    out = run_both(cuda, a, b, out_dtype, 0, **kw)
+    assert torch.equal(out["0"], out["1"])
+    rel = (out["1"].float() - ref).abs().max() / ref.abs().max()
+    assert rel.item() <= 1e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
+@pytest.mark.parametrize("block", [128, 256])
+def test_grouped_blocks_exact_in_both_forms(cuda, mfma_env, dtype, block):
+    """The grouped form (gathered A rows, per-block expert weights, scattered C rows) on both block sizes."""
+    from oracle import golden
+    from tests.test_gpu_group_gemm import make_case, run
+    world, mpr, K, N, E, topk = 4, 96, 640, 328, 6, 2
+    announce("mfma shapes grouped %s block %d" % (dtype, block))
+    shards, w, ids = make_case(world, mpr, K, N, E, topk, dtype, seed=block, integer=True)
+    ref = golden.ag_group_gemm_fp32(shards, w, ids)
+    for mode in ("0", "1"):
+        os.environ["TDIST_GEMM_MFMA16"] = mode
+        ctx, c = run(cuda, shards, w, ids, 1, E, block)
+        ctx.check_status()
+        assert torch.equal(c.float().cpu(), ref.to(c.dtype).float()), "TDIST_GEMM_MFMA16=%s" % mode

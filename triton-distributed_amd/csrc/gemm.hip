@@ -8,9 +8,10 @@
 // (kernels/amd/gemm_reduce_scatter.py:125-229) and kernel_consumer_m_parallel_scatter_group_gemm
 // (kernels/nvidia/allgather_group_gemm.py:238-314) as one hand-scheduled kernel:
 //
-//  * workgroup = WM x WN waves, macro tile BM x BN, each wave owns (BM/WM) x (BN/WN) of it as 32x32
-//    MFMA tiles: v_mfma_f32_32x32x16_{bf16,f16} (16 B of K per lane) or v_mfma_f32_32x32x64_f8f6f4
-//    (32 B of K per lane) with fp32 accumulators;
+//  * workgroup = WM x WN waves, macro tile BM x BN, each wave owns (BM/WM) x (BN/WN) of it as MFMA blocks with
+//    fp32 accumulators: on the 256-row tiles 16 x 16 blocks (v_mfma_f32_16x16x32_{bf16,f16}, 16 B of K per lane,
+//    and v_mfma_f32_16x16x128_f8f6f4, 32 B per lane), which spend the least power per flop and so hold the highest
+//    clock on real data; elsewhere 32 x 32 blocks (v_mfma_f32_32x32x16_{bf16,f16}, v_mfma_f32_32x32x64_f8f6f4);
 //  * A and B tiles go HBM/L2 → LDS with asynchronous 16-byte-per-lane LDS-DMA loads into a ring of NST
 //    stages, P = NST-1 tiles in flight (NST == 5: a split ring of three A and two B half stages whose refill is
 //    spread over the K steps); rows are stored with an XOR swizzle of the 16-byte chunk index
@@ -155,6 +156,16 @@ struct ElemFP8 {
 // A ds_read_b128 is served 16 lanes at a time (16 x 16 B = 256 B = one pass over the 64 banks), and the 16
 // lanes of a pass read the same logical chunk of 16 consecutive rows. Those rows cover 256 B / KB positions
 // "for free" through their row offset; the XOR term has to spread the rest, i.e. change every (256 / KB) rows.
+// e4m3 on the 16x16x128 MFMA: a lane feeds the same 32 bytes of K, four lane groups cover a whole 128-byte tile row
+struct ElemFP8N : ElemFP8 {
+  static constexpr int kRows = 16;
+  typedef float4v acc_t;
+  __device__ static __forceinline__ float4v mma(frag a, frag b, float4v c) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    return c;
+  }
+};
+
 template <int KB>
 __host__ __device__ constexpr int swz(int r) {
   return KB >= 128 ? ((r >> 1) & 7) : ((r >> 2) & 3);
@@ -461,7 +472,74 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         for (int e = 0; e < C::kAccLen; ++e) acc[j][i][e] = 0.f;
 
     constexpr int kMfmaPerStep = C::kTM * C::kTN;
-    if constexpr (C::kSplit && E::kRows == 16) {
+    if constexpr (C::kSplit && E::kRows == 16 && C::kKSteps == 1) {
+      // ---- split ring, 16-row MFMA blocks, the whole K tile in one MFMA depth (e4m3) --------------------
+      // The 64 MFMAs of a tile run as four quarters of 4 x 4 blocks: A fragments 0-3 against one half of the B
+      // fragments, then against the other half, then A fragments 4-7 against that other half and against the first
+      // one again. Every quarter reads the four fragments whose registers have just fallen idle:
+      //   quarter 0: the B half that quarter 1 needs;     quarter 1: A fragments 4-7 of this tile;
+      //   quarter 2: A fragments 0-3 of the next tile;     quarter 3: the B half quarter 2 has finished with, for the
+      //                                                    next tile, which therefore starts with that half.
+      // So the B halves swap roles from one tile to the next, the fragment registers are never doubled, and the LDS
+      // sees the same eight reads per wave in every quarter. The barrier (tile kt+1 has landed everywhere, nobody
+      // reads tile kt's stages any more) stands in front of quarter 2; the refill DMA ([B(kt+2) rows, A(kt+3) rows],
+      // as in the other split-ring loops) goes out one instruction every fourth slot from there to the next barrier.
+      static_assert(C::kTM == 8 && C::kTN == 8 && C::kLoadsPerTile == 16, "schedule written for a 128x128 wave tile");
+      constexpr int kBar = 33;                         // the barrier sits in front of this slot's MFMA
+      constexpr int kProDma = (64 - kBar + 3) / 4;     // list entries that fall between a barrier and the tile's end
+      auto issue_list = [&](int cyc, int q) {
+        if (q < C::kBInstr) issue_b(cyc + 2, q);
+        else issue_a(cyc + 3, q - C::kBInstr);
+      };
+#pragma unroll
+      for (int t = 0; t < C::kAInstr; ++t) issue_a(0, t);
+#pragma unroll
+      for (int u = 0; u < C::kBInstr; ++u) issue_b(0, u);
+#pragma unroll
+      for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+#pragma unroll
+      for (int q = 0; q < kProDma; ++q) issue_list(-1, q);
+      wait_tiles_and_barrier<C::kAInstr + kProDma>();
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        load_frag(0, 0, f, a_cur, b_cur);            // A fragments 0-3
+        load_frag(0, 0, C::kTM + f, a_cur, b_cur);   // B fragments 0-3
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // one tile; kOdd: the B halves in the order (4-7, 0-3)
+      auto tile = [&](auto odd_c, int kt) {
+        constexpr int kOdd = decltype(odd_c)::value;
+        const int kt_next = min(kt + 1, KTp - 1);
+        static_for<kMfmaPerStep>([&](auto u_c) {
+          constexpr int u = decltype(u_c)::value;
+          constexpr int quarter = u / 16, w = u % 16;
+          constexpr int a_half = quarter / 2;
+          constexpr int b_half = ((quarter == 1 || quarter == 2) ? 1 : 0) ^ kOdd;
+          constexpr int j = 4 * b_half + w / 4, i = 4 * a_half + w % 4;
+          if constexpr (u == kBar) {
+            __builtin_amdgcn_sched_barrier(0);
+            wait_tiles_and_barrier<C::kAInstr>();
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+          if constexpr (w % 3 == 2 && w / 3 < 4) {  // slots 2, 5, 8, 11 of the quarter
+            constexpr int f = w / 3;
+            if constexpr (quarter == 0) load_frag(kt, 0, C::kTM + 4 * (1 ^ kOdd) + f, a_cur, b_cur);
+            if constexpr (quarter == 1) load_frag(kt, 0, 4 + f, a_cur, b_cur);
+            if constexpr (quarter == 2) load_frag(kt_next, 0, f, a_cur, b_cur);
+            if constexpr (quarter == 3) load_frag(kt_next, 0, C::kTM + 4 * (1 ^ kOdd) + f, a_cur, b_cur);
+          }
+          constexpr int since = (u - kBar + 64) % 64;  // slots since the last barrier
+          if constexpr (since % 4 == 0) issue_list(u >= kBar ? kt : kt - 1, since / 4);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      };
+      for (int kt = 0; kt < KTp; kt += 2) {
+        tile(std::integral_constant<int, 0>{}, kt);
+        if (kt + 1 < KTp) tile(std::integral_constant<int, 1>{}, kt + 1);
+      }
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the last MFMAs' results: 8 passes + 3 cycles after issue
+    } else if constexpr (C::kSplit && E::kRows == 16) {
       // ---- split ring, 16-row MFMA blocks ------------------------------------------------------------
       // The MFMAs of a K step run in B-fragment-major order: a B fragment serves kTM MFMAs in a row and is then dead,
       // so the next step's B fragment is read into the same registers right behind them; only the A fragments, which
@@ -881,7 +959,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         const uint32_t lane_off = (uint32_t)er * (uint32_t)row_bytes + (uint32_t)ec * 16u;
         const bool streaming = p.scatter_bufs == nullptr;
         float rs[kScales ? C::kTM : 1] = {1.f};
-        float4v cs[kScales ? kGroups : 1] = {float4v{1.f, 1.f, 1.f, 1.f}};
+        // (the two groups of a 16-column block share their column scales)
+        constexpr int kColSlots = kWide ? kGroups : kGroups / 2;
+        float4v cs[kScales ? kColSlots : 1] = {float4v{1.f, 1.f, 1.f, 1.f}};
         if constexpr (kScales) {
 #pragma unroll
           for (int i = 0; i < C::kTM; ++i) {
@@ -889,9 +969,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
             if (p.row_scale) rs[i] = p.row_scale[m0 + wm * C::kWaveM + E::kRows * i + e_lrow];
           }
 #pragma unroll
-          for (int g = 0; g < kGroups; ++g) {  // the four column scales of each of this lane's column groups
-            cs[g] = float4v{1.f, 1.f, 1.f, 1.f};
-            if (p.col_scale) cs[g] = *(const float4v*)(p.col_scale + n0 + wn * C::kWaveN + group_col(g));
+          for (int c = 0; c < kColSlots; ++c) {  // the four column scales of each of this lane's column groups
+            cs[c] = float4v{1.f, 1.f, 1.f, 1.f};
+            if (p.col_scale) cs[c] = *(const float4v*)(p.col_scale + n0 + wn * C::kWaveN + group_col(kWide ? c : 2 * c));
           }
         }
         // Staging addresses: a row block adds a constant to them (32 rows leave the swizzle term alone), so one
@@ -909,7 +989,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         for (int ph = 0; ph < kReadPhases; ++ph)
           rbase[ph] = epi + er * C::kEpiPitch + ((ec ^ ((ph * kRowsPerPass + er) & C::kEpiSwz)) << 4);
         auto stage_fast = [&](int i, int g) {
-          stage_group_at(i, g, rs, cs[kScales ? g : 0], wbase[g] + i * 32 * C::kEpiPitch);
+          stage_group_at(i, g, rs, cs[kScales ? (kWide ? g : g / 2) : 0], wbase[g] + i * 32 * C::kEpiPitch);
         };
 #pragma unroll
         for (int g = 0; g < kGroups; ++g) stage_fast(0, g);
@@ -1259,6 +1339,10 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       return scales ? launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, true>(p, grid, c.stream, who)          \
                     : launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);        \
   }
+    if (narrow_mfma && variant == 6 && elem == kElemFP8) {
+      return scales ? launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, true>(p, grid, c.stream, who)
+                    : launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+    }
     if (narrow_mfma && variant == 6 && elem != kElemFP8) {
       if (elem == kElemBF16) return launch_gemm_cfg<ElemBF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
       return launch_gemm_cfg<ElemF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
@@ -1405,6 +1489,8 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   if (c.block_size == 256) {
     if (!k128) return fail(TDIST_ERR_UNSUPPORTED, "%s: 256-row blocks need K*elem_size to be a multiple of 128 bytes", who);
     TDIST_GROUPED_NARROW(256, 256, 128, 5)
+    if (narrow_mfma && elem == kElemFP8)
+      return launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, false, true>(p, grid, c.stream, who);
     TDIST_GROUPED(256, 256, 128, 5)
   }
   if (k128) {  // 64 x 128 per wave on the split ring
