@@ -1,7 +1,8 @@
 """The 256-row GEMM tiles run on the 16-row MFMA blocks (16x16x32 for bf16/f16, 16x16x128 for e4m3) by default and on
-the 32-row blocks (32x32x16 / 32x32x64) with TDIST_GEMM_MFMA16=0. Both forms add the same products in the same order
-per accumulator, so they must agree bit for bit; each is also held against the exact result on integer-valued inputs
-(every partial sum is an integer that fp32 holds) and, on random inputs, to max relative error <= 1e-2 of fp32."""
+the 32-row blocks (32x32x16 / 32x32x64) with TDIST_GEMM_MFMA16=0. Both forms walk K in the same tile order with one
+fp32 accumulator per output element, and they agree bit for bit on every case here; each is also held against the
+exact result on integer-valued inputs (every partial sum is an integer that fp32 holds) and, on random inputs, to max
+relative error <= 1e-2 of fp32."""
 import os
 
 import pytest

@@ -445,8 +445,13 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     typename E::frag a_cur[C::kTM], b_cur[C::kTN], a_nxt[C::kTM], b_nxt[C::kTN];
     // f-th operand fragment (A fragments first) of K step ks of tile kt
     auto load_frag = [&](int kt, int ks, int f, typename E::frag* af, typename E::frag* bf) {
-      const int c0 = (ks * C::kLaneGroups + lgrp) * C::kFragVecs;  // first 16-byte chunk of this lane's K bytes
-      const int c1 = c0 + C::kFragVecs - 1;         // last one (== c0 for 16-byte fragments)
+      // 16-byte chunks of this lane's K bytes (c1 == c0 for 16-byte fragments). With four lane groups and two chunks
+      // per lane, group g takes chunks g and g + 4 rather than 2g and 2g + 1: any assignment of K bytes to lanes gives
+      // the same product as long as A and B share it, and only with the four groups of one read on consecutive chunks
+      // is the swizzle free of bank conflicts (every other chunk per read: half of the LDS cycles were conflicts).
+      constexpr bool kStridedPieces = C::kLaneGroups == 4 && C::kFragVecs == 2;
+      const int c0 = kStridedPieces ? lgrp : (ks * C::kLaneGroups + lgrp) * C::kFragVecs;
+      const int c1 = kStridedPieces ? lgrp + 4 : c0 + C::kFragVecs - 1;
       if (f < C::kTM) {
         const int r = wm * C::kWaveM + f * E::kRows + lrow;
         lds_u8 const row = a_stage(kt) + r * KB;
