@@ -458,14 +458,17 @@ def bench_mfma_ceiling(dev, steps, warmup):
     from triton_dist import _lib
     cus = _lib.load().tdist_num_cus()
     sink = torch.empty(cus * 256, dtype=torch.float32, device=dev)
-    iters = 2000
+    iters = 1000
     out = {}
-    for name, code, per in (("bf16", _lib.TDIST_BF16, 32768.0), ("fp8", _lib.TDIST_F8E4M3, 131072.0)):
-        for rnd in (0, 1):
-            s = time_launches(lambda: _lib.call("tdist_mfma_rate_probe", code, rnd, iters, sink.data_ptr(), _lib.stream_ptr()),
-                              max(steps // 4, 5), warmup)
-            tf = cus * 4 * iters * 8 * per / s / 1e12
-            out["%s_%s_operands_TFLOPs" % (name, "random" if rnd else "constant")] = round(tf, 1)
+    for name, code, kstep in (("bf16", _lib.TDIST_BF16, 16), ("fp8", _lib.TDIST_F8E4M3, 64)):
+        for entry, rows, ks in (("tdist_mfma_rate_probe", "", kstep), ("tdist_mfma_rate_probe_16row", "_16row_mfma", 2 * kstep)):
+            for rnd in (0, 1):
+                if rows and not rnd:
+                    continue
+                s = time_launches(lambda: _lib.call(entry, code, rnd, iters, sink.data_ptr(), _lib.stream_ptr()),
+                                  max(steps // 4, 5), warmup)
+                tf = cus * 4 * iters * 2.0 * 128 * 128 * ks / s / 1e12
+                out["%s_%s_operands%s_TFLOPs" % (name, "random" if rnd else "constant", rows)] = round(tf, 1)
     return out
 
 

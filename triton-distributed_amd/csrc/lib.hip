@@ -171,9 +171,11 @@ __global__ __launch_bounds__(256) void copy_bytes_kernel(int4v* __restrict__ dst
   }
 }
 
-// MFMA-only loop for the rate yardstick: no memory traffic at all, eight independent accumulators, and operand
-// fragments that change from one MFMA to the next (eight A and eight B fragments in registers, paired differently
-// every time). kRandom fills them with hashed bit patterns (random sign, mantissa and low exponent bits), else with 1.0.
+// MFMA-only loop for the rate yardstick: the K loop of a 128 x 128 wave tile with no memory traffic at all. 256
+// accumulators, eight A and eight B operand fragments in registers, and the GEMM kernel's order of use: a B fragment
+// serves a row of MFMAs against every A fragment in turn. kRandom fills the fragments with hashed bit patterns (random
+// sign, mantissa and low exponent bits), else with 1.0. kRows = 32: 4 x 4 blocks of 32x32x16 (bf16) / 32x32x64 (e4m3);
+// kRows = 16: 8 x 8 blocks of 16x16x32 / 16x16x128, i.e. twice the K per round.
 __device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
   x ^= x >> 16;
   x *= 0x7feb352dU;
@@ -183,10 +185,13 @@ __device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
   return x;
 }
 
-template <bool kFp8, bool kRandom>
+template <bool kFp8, bool kRandom, int kRows>
 __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(float* __restrict__ sink, int iters) {
   typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
   typedef int int8v_ __attribute__((ext_vector_type(8)));
+  constexpr int kT = 128 / kRows;            // blocks per side of the wave tile
+  constexpr int kAcc = kRows * kRows / 64;   // accumulators per lane and block
+  typedef float acc_t __attribute__((ext_vector_type(kAcc)));
   int8v_ a[8], b[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -201,29 +206,38 @@ __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(float* __restrict__ s
         b[i][e] = kRandom ? (int)((h2 & 0x81ff81ffu) | 0x3e003e00u) : 0x3f803f80;
       }
     }
-  float16v acc[8];
+  acc_t acc[kT][kT];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int j = 0; j < kT; ++j)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
-  for (int it = 0; it < iters; it += 4) {
+    for (int i = 0; i < kT; ++i)
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+      for (int e = 0; e < kAcc; ++e) acc[j][i][e] = 0.f;
+  for (int it = 0; it < iters; it += 2) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int8v_ av = a[(i + u) & 7], bv = b[(i * 3 + u) & 7];
-        if (kFp8) {
-          acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i], 0, 0, 0, 0, 0, 0);
-        } else {
-          const int4v a4 = __builtin_shufflevector(av, av, 0, 1, 2, 3), b4 = __builtin_shufflevector(bv, bv, 0, 1, 2, 3);
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8v, a4), __builtin_bit_cast(bf16x8v, b4),
-                                                           acc[i], 0, 0, 0);
+    for (int u = 0; u < 2; ++u)  // (two rounds with the fragments paired differently, as two K steps would be)
+#pragma unroll
+      for (int j = 0; j < kT; ++j)
+#pragma unroll
+        for (int i = 0; i < kT; ++i) {
+          const int8v_ av = a[(i + 4 * u) & 7], bv = b[(j + 4 * u) & 7];
+          if constexpr (kFp8) {
+            if constexpr (kRows == 32) acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc[j][i], 0, 0, 0, 0, 0, 0);
+            else acc[j][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[j][i], 0, 0, 0, 0, 0, 0);
+          } else {
+            const int4v a4 = __builtin_shufflevector(av, av, 0, 1, 2, 3), b4 = __builtin_shufflevector(bv, bv, 0, 1, 2, 3);
+            if constexpr (kRows == 32)
+              acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8v, b4), __builtin_bit_cast(bf16x8v, a4), acc[j][i], 0, 0, 0);
+            else
+              acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8v, b4), __builtin_bit_cast(bf16x8v, a4), acc[j][i], 0, 0, 0);
+          }
         }
-      }
   }
   float s = 0.f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) s += acc[i][0];
+  for (int j = 0; j < kT; ++j)
+#pragma unroll
+    for (int i = 0; i < kT; ++i) s += acc[j][i][0];
   sink[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
@@ -350,21 +364,33 @@ int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
   return launch_status("tdist_copy_bytes");
 }
 
-int tdist_mfma_rate_probe(int dtype, int random_operands, int iters, float* sink, void* stream) {
-  if (!sink || iters <= 0 || iters % 4 != 0) return fail(TDIST_ERR_INVALID, "tdist_mfma_rate_probe: sink, iters (multiple of 4)");
-  if (dtype != TDIST_BF16 && dtype != TDIST_F8E4M3) return fail(TDIST_ERR_UNSUPPORTED, "tdist_mfma_rate_probe: bf16 or e4m3");
+static int mfma_rate_probe(const char* who, bool narrow, int dtype, int random_operands, int iters, float* sink, void* stream) {
+  if (!sink || iters <= 0 || iters % 2 != 0) return fail(TDIST_ERR_INVALID, "%s: sink, iters (even)", who);
+  if (dtype != TDIST_BF16 && dtype != TDIST_F8E4M3) return fail(TDIST_ERR_UNSUPPORTED, "%s: bf16 or e4m3", who);
   const DeviceInfo& di = device_info();
-  if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "tdist_mfma_rate_probe: current device is not gfx950");
+  if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "%s: current device is not gfx950", who);
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(di.num_cus), block(256);
-  if (dtype == TDIST_BF16) {
-    if (random_operands) hipLaunchKernelGGL((mfma_rate_kernel<false, true>), grid, block, 0, st, sink, iters);
-    else hipLaunchKernelGGL((mfma_rate_kernel<false, false>), grid, block, 0, st, sink, iters);
-  } else {
-    if (random_operands) hipLaunchKernelGGL((mfma_rate_kernel<true, true>), grid, block, 0, st, sink, iters);
-    else hipLaunchKernelGGL((mfma_rate_kernel<true, false>), grid, block, 0, st, sink, iters);
+  const int which = (narrow ? 4 : 0) + (dtype == TDIST_F8E4M3 ? 2 : 0) + (random_operands ? 1 : 0);
+  switch (which) {
+    case 0: hipLaunchKernelGGL((mfma_rate_kernel<false, false, 32>), grid, block, 0, st, sink, iters); break;
+    case 1: hipLaunchKernelGGL((mfma_rate_kernel<false, true, 32>), grid, block, 0, st, sink, iters); break;
+    case 2: hipLaunchKernelGGL((mfma_rate_kernel<true, false, 32>), grid, block, 0, st, sink, iters); break;
+    case 3: hipLaunchKernelGGL((mfma_rate_kernel<true, true, 32>), grid, block, 0, st, sink, iters); break;
+    case 4: hipLaunchKernelGGL((mfma_rate_kernel<false, false, 16>), grid, block, 0, st, sink, iters); break;
+    case 5: hipLaunchKernelGGL((mfma_rate_kernel<false, true, 16>), grid, block, 0, st, sink, iters); break;
+    case 6: hipLaunchKernelGGL((mfma_rate_kernel<true, false, 16>), grid, block, 0, st, sink, iters); break;
+    default: hipLaunchKernelGGL((mfma_rate_kernel<true, true, 16>), grid, block, 0, st, sink, iters); break;
   }
-  return launch_status("tdist_mfma_rate_probe");
+  return launch_status(who);
+}
+
+int tdist_mfma_rate_probe(int dtype, int random_operands, int iters, float* sink, void* stream) {
+  return mfma_rate_probe("tdist_mfma_rate_probe", false, dtype, random_operands, iters, sink, stream);
+}
+
+int tdist_mfma_rate_probe_16row(int dtype, int random_operands, int iters, float* sink, void* stream) {
+  return mfma_rate_probe("tdist_mfma_rate_probe_16row", true, dtype, random_operands, iters, sink, stream);
 }
 
 }  // extern "C"

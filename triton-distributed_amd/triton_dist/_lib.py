@@ -66,6 +66,7 @@ PROTOTYPES = {
     "tdist_decode_combine": (_I, [_P, _I, _P, _I, _I, _P, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P, _I, _L, _L, _P, _P]),
     "tdist_copy_bytes": (_I, [_P, _P, _L, _P]),
     "tdist_mfma_rate_probe": (_I, [_I, _I, _I, _P, _P]),
+    "tdist_mfma_rate_probe_16row": (_I, [_I, _I, _I, _P, _P]),
 }
 
 
