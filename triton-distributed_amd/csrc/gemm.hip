@@ -479,19 +479,32 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     constexpr int kMfmaPerStep = C::kTM * C::kTN;
     if constexpr (C::kSplit && E::kRows == 16 && C::kKSteps == 1) {
       // ---- split ring, 16-row MFMA blocks, the whole K tile in one MFMA depth (e4m3) --------------------
-      // The 64 MFMAs of a tile run as four quarters of 4 x 4 blocks: A fragments 0-3 against one half of the B
-      // fragments, then against the other half, then A fragments 4-7 against that other half and against the first
-      // one again. Every quarter reads the four fragments whose registers have just fallen idle:
-      //   quarter 0: the B half that quarter 1 needs;     quarter 1: A fragments 4-7 of this tile;
-      //   quarter 2: A fragments 0-3 of the next tile;     quarter 3: the B half quarter 2 has finished with, for the
+      // The MFMAs of a tile run as four quarters: the lower half of the A fragments against one half of the B
+      // fragments, then against the other half, then the upper A half against that other half and against the first
+      // one again (128 x 128 wave tile: 4 x 4 blocks per quarter). Every quarter reads the fragments whose registers
+      // have just fallen idle:
+      //   quarter 0: the B half that quarter 1 needs;     quarter 1: the upper A half of this tile;
+      //   quarter 2: the lower A half of the next tile;   quarter 3: the B half quarter 2 has finished with, for the
       //                                                    next tile, which therefore starts with that half.
       // So the B halves swap roles from one tile to the next, the fragment registers are never doubled, and the LDS
-      // sees the same eight reads per wave in every quarter. The barrier (tile kt+1 has landed everywhere, nobody
-      // reads tile kt's stages any more) stands in front of quarter 2; the refill DMA ([B(kt+2) rows, A(kt+3) rows],
-      // as in the other split-ring loops) goes out one instruction every fourth slot from there to the next barrier.
-      static_assert(C::kTM == 8 && C::kTN == 8 && C::kLoadsPerTile == 16, "schedule written for a 128x128 wave tile");
-      constexpr int kBar = 33;                         // the barrier sits in front of this slot's MFMA
-      constexpr int kProDma = (64 - kBar + 3) / 4;     // list entries that fall between a barrier and the tile's end
+      // reads are spread evenly over the tile. The barrier (tile kt+1 has landed everywhere, nobody reads tile kt's
+      // stages any more) stands in front of quarter 2; the refill DMA ([B(kt+2) rows, A(kt+3) rows], as in the other
+      // split-ring loops) goes out evenly spaced from there to the next barrier.
+      constexpr int kHA = C::kTM / 2, kHB = C::kTN / 2, kQuarter = kHA * kHB;
+      static_assert(C::kTM % 2 == 0 && C::kTN % 2 == 0 && kQuarter - 2 >= kHA && kQuarter - 2 >= kHB,
+                    "a quarter has a slot for each of its fragment reads");
+      constexpr int kBar = 2 * kQuarter + 1;           // the barrier sits in front of this slot's MFMA
+      // list entry q goes out ceil(q * slots / entries) slots after the barrier
+      auto dma_due = [](int since) constexpr {
+        for (int q = 0; q < C::kLoadsPerTile; ++q)
+          if ((q * kMfmaPerStep + C::kLoadsPerTile - 1) / C::kLoadsPerTile == since) return q;
+        return -1;
+      };
+      constexpr int kProDma = [&]() constexpr {        // entries that fall between a barrier and the tile's end
+        int n = 0;
+        for (int since = 0; since < kMfmaPerStep - kBar; ++since) n += dma_due(since) >= 0 ? 1 : 0;
+        return n;
+      }();
       auto issue_list = [&](int cyc, int q) {
         if (q < C::kBInstr) issue_b(cyc + 2, q);
         else issue_a(cyc + 3, q - C::kBInstr);
@@ -506,36 +519,39 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       for (int q = 0; q < kProDma; ++q) issue_list(-1, q);
       wait_tiles_and_barrier<C::kAInstr + kProDma>();
 #pragma unroll
-      for (int f = 0; f < 4; ++f) {
-        load_frag(0, 0, f, a_cur, b_cur);            // A fragments 0-3
-        load_frag(0, 0, C::kTM + f, a_cur, b_cur);   // B fragments 0-3
-      }
+      for (int f = 0; f < kHA; ++f) load_frag(0, 0, f, a_cur, b_cur);            // lower A half
+#pragma unroll
+      for (int f = 0; f < kHB; ++f) load_frag(0, 0, C::kTM + f, a_cur, b_cur);   // lower B half
       __builtin_amdgcn_sched_barrier(0);
-      // one tile; kOdd: the B halves in the order (4-7, 0-3)
+      // one tile; kOdd: the B halves in the order (upper, lower)
       auto tile = [&](auto odd_c, int kt) {
         constexpr int kOdd = decltype(odd_c)::value;
         const int kt_next = min(kt + 1, KTp - 1);
         static_for<kMfmaPerStep>([&](auto u_c) {
           constexpr int u = decltype(u_c)::value;
-          constexpr int quarter = u / 16, w = u % 16;
+          constexpr int quarter = u / kQuarter, w = u % kQuarter;
           constexpr int a_half = quarter / 2;
           constexpr int b_half = ((quarter == 1 || quarter == 2) ? 1 : 0) ^ kOdd;
-          constexpr int j = 4 * b_half + w / 4, i = 4 * a_half + w % 4;
+          constexpr int j = kHB * b_half + w / kHA, i = kHA * a_half + w % kHA;
           if constexpr (u == kBar) {
             __builtin_amdgcn_sched_barrier(0);
             wait_tiles_and_barrier<C::kAInstr>();
             __builtin_amdgcn_sched_barrier(0);
           }
           acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
-          if constexpr (w % 3 == 2 && w / 3 < 4) {  // slots 2, 5, 8, 11 of the quarter
-            constexpr int f = w / 3;
-            if constexpr (quarter == 0) load_frag(kt, 0, C::kTM + 4 * (1 ^ kOdd) + f, a_cur, b_cur);
-            if constexpr (quarter == 1) load_frag(kt, 0, 4 + f, a_cur, b_cur);
+          // the quarter's fragment reads, from its slot 2 on (128 x 128 wave tile: slots 2, 5, 8, 11)
+          constexpr int n_reads = (quarter == 0 || quarter == 3) ? kHB : kHA;
+          constexpr int stride = (kQuarter - 2) / n_reads;
+          if constexpr (w >= 2 && (w - 2) % stride == 0 && (w - 2) / stride < n_reads) {
+            constexpr int f = (w - 2) / stride;
+            if constexpr (quarter == 0) load_frag(kt, 0, C::kTM + kHB * (1 ^ kOdd) + f, a_cur, b_cur);
+            if constexpr (quarter == 1) load_frag(kt, 0, kHA + f, a_cur, b_cur);
             if constexpr (quarter == 2) load_frag(kt_next, 0, f, a_cur, b_cur);
-            if constexpr (quarter == 3) load_frag(kt_next, 0, C::kTM + 4 * (1 ^ kOdd) + f, a_cur, b_cur);
+            if constexpr (quarter == 3) load_frag(kt_next, 0, C::kTM + kHB * (1 ^ kOdd) + f, a_cur, b_cur);
           }
-          constexpr int since = (u - kBar + 64) % 64;  // slots since the last barrier
-          if constexpr (since % 4 == 0) issue_list(u >= kBar ? kt : kt - 1, since / 4);
+          constexpr int since = (u - kBar + kMfmaPerStep) % kMfmaPerStep;  // slots since the last barrier
+          constexpr int due = dma_due(since);
+          if constexpr (due >= 0) issue_list(u >= kBar ? kt : kt - 1, due);
           __builtin_amdgcn_sched_barrier(0);
         });
       };
@@ -1358,6 +1374,10 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       default: TDIST_BIG(256, 128, 2, 2, 5)
     }
   }
+  if (pick == 1 && narrow_mfma && elem == kElemFP8) {
+    return scales ? launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, true>(p, grid, c.stream, who)
+                  : launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+  }
   if (pick == 1 && narrow_mfma && elem != kElemFP8) {
     if (elem == kElemBF16) return launch_gemm_cfg<ElemBF16N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
     return launch_gemm_cfg<ElemF16N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
@@ -1500,6 +1520,8 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   }
   if (k128) {  // 64 x 128 per wave on the split ring
     TDIST_GROUPED_NARROW(128, 256, 128, 5)
+    if (narrow_mfma && elem == kElemFP8)
+      return launch_gemm_cfg<ElemFP8N, 128, 256, 128, 2, 2, 5, false, true>(p, grid, c.stream, who);
     TDIST_GROUPED(128, 256, 128, 5)
   }
   TDIST_GROUPED(128, 128, 64, 4)
