@@ -560,6 +560,15 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         if (kt + 1 < KTp) tile(std::integral_constant<int, 1>{}, kt + 1);
       }
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the last MFMAs' results: 8 passes + 3 cycles after issue
+
+      // (every later use of an accumulator depends on these empty statements, which stay behind the wait above: the
+      // compiler, which does not know that the assembly before it was an MFMA, cannot move a read in front of it)
+      if constexpr (C::kTM * C::kTN * C::kAccLen < 256) {  // (with 256 of them they are only ever read in assembly)
+#pragma unroll
+        for (int j = 0; j < C::kTN; ++j)
+#pragma unroll
+          for (int i = 0; i < C::kTM; ++i) asm volatile("" : "+a"(acc[j][i]));
+      }
     } else if constexpr (C::kSplit && E::kRows == 16) {
       // ---- split ring, 16-row MFMA blocks ------------------------------------------------------------
       // The MFMAs of a K step run in B-fragment-major order: a B fragment serves kTM MFMAs in a row and is then dead,
@@ -621,6 +630,15 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       }
       // the last MFMAs' results are readable 4 passes + 3 cycles after issue
       asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+
+      // (every later use of an accumulator depends on these empty statements, which stay behind the wait above: the
+      // compiler, which does not know that the assembly before it was an MFMA, cannot move a read in front of it)
+      if constexpr (C::kTM * C::kTN * C::kAccLen < 256) {  // (with 256 of them they are only ever read in assembly)
+#pragma unroll
+        for (int j = 0; j < C::kTN; ++j)
+#pragma unroll
+          for (int i = 0; i < C::kTM; ++i) asm volatile("" : "+a"(acc[j][i]));
+      }
     } else if constexpr (C::kSplit) {
       // ---- split ring ------------------------------------------------------------------------------
       // The DMA list of one cycle is [B(kt+2) rows..., A(kt+3) rows...]; it starts right after the barrier in the
