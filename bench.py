@@ -77,22 +77,13 @@ def time_launches(fn, steps, warmup):
 
 
 def time_live_ag_gemm(call, ctx, steps, warmup):
-    """Times the AG-GEMM with its producer running: first with the GEMM queued before the chunk copies
-    (ctx.gemm_first), and if the copy streams turn out to share a hardware queue with the GEMM stream in this
-    process (the bounded flag wait reports a timeout), in the reference's order. Returns (seconds, order)."""
-    from triton_dist import _lib
-    ctx.gemm_first = True
+    """Times the AG-GEMM with its producer running, in the reference's order (producer queued first, then the gated
+    GEMM); a bounded flag wait that expired is an error. Returns (seconds, order)."""
     call()
-    try:
-        ctx.check_status()
-        s = time_launches(call, steps, warmup)
-        ctx.check_status()
-        return s, "gemm_first"
-    except _lib.TdistError:
-        ctx.gemm_first = False
-        s = time_launches(call, steps, warmup)
-        ctx.check_status()
-        return s, "copies_first"
+    ctx.check_status()
+    s = time_launches(call, steps, warmup)
+    ctx.check_status()
+    return s, "copies_first"
 
 
 XGMI_LINK_GBPS = 153.0   # one xGMI link of MI355X: the rate at which one peer's rows arrive
@@ -177,17 +168,6 @@ def bench_c2(dev, steps, warmup):
     stream = torch.cuda.current_stream()
     gemm_s = time_launches(lambda: matmul_fuse_scatter(a_d, b_d, ctx.scatter_bufs_ptr, rank, W, False, stream=stream),
                            steps, warmup)
-    # the same kernel on the 32-row MFMA blocks (same bits out, more power per flop), for reference
-    saved = os.environ.get("TDIST_GEMM_MFMA16")
-    os.environ["TDIST_GEMM_MFMA16"] = "0"
-    try:
-        gemm32_s = time_launches(lambda: matmul_fuse_scatter(a_d, b_d, ctx.scatter_bufs_ptr, rank, W, False, stream=stream),
-                                 max(steps // 2, 5), warmup)
-    finally:
-        if saved is None:
-            del os.environ["TDIST_GEMM_MFMA16"]
-        else:
-            os.environ["TDIST_GEMM_MFMA16"] = saved
     scatter_out = ctx.scatter_bufs[rank][:M]
     red_s = time_launches(lambda: ring_reduce_after_scatter(rank, W, scatter_out, stream), steps, warmup)
     red_bytes = (W + 1) * (M // W) * N * 2
@@ -215,7 +195,6 @@ def bench_c2(dev, steps, warmup):
         cpu = {"value": round(flops / 8 / probe / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                "sample": "1/8 of the rows (1024 of 8192) of the fp32 up-cast golden GEMM, %.2f s" % probe}
     gemm_roof = roof("mfma", flops, gemm_s, "bf16", MEASURED_TRAFFIC_BYTES["c2_gemm"])
-    gemm_roof["on_32row_mfma_blocks_us"] = round(gemm32_s * 1e6, 2)
     return (step_s, gemm_roof, roof("hbm", red_bytes, red_s, "hbm", MEASURED_TRAFFIC_BYTES["c2_reduce"]), cpu, err)
 
 
@@ -460,7 +439,7 @@ def bench_copy(dev, steps, warmup):
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device=dev)
     dst = torch.empty(n, dtype=torch.uint8, device=dev)
-    s = time_launches(lambda: _lib.call("tdist_copy_bytes", dst.data_ptr(), src.data_ptr(), n, _lib.stream_ptr()), steps, warmup)
+    s = time_launches(lambda: _lib.bench_call("tdist_copy_bytes", dst.data_ptr(), src.data_ptr(), n, _lib.stream_ptr()), steps, warmup)
     return roof("hbm", 2 * n, s, "hbm")
 
 
@@ -477,7 +456,7 @@ def bench_mfma_ceiling(dev, steps, warmup):
             for rnd in (0, 1):
                 if rows and not rnd:
                     continue
-                s = time_launches(lambda: _lib.call(entry, code, rnd, iters, sink.data_ptr(), _lib.stream_ptr()),
+                s = time_launches(lambda: _lib.bench_call(entry, code, rnd, iters, sink.data_ptr(), _lib.stream_ptr()),
                                   max(steps // 4, 5), warmup)
                 tf = cus * 4 * iters * 2.0 * 128 * 128 * ks / s / 1e12
                 out["%s_%s_operands%s_TFLOPs" % (name, "random" if rnd else "constant", rows)] = round(tf, 1)
@@ -531,7 +510,6 @@ def main():
     step_s, gemm_roof, red_roof, cpu, err = bench_c2(dev, args.steps, args.warmup)
     log("c2 step %.1f us, gemm %s, reduce %s" % (step_s * 1e6, gemm_roof, red_roof))
     kernels = {"c2_gemm_rs_scatter_gemm_bf16": dict(gemm_roof), "c2_reduce_slices_bf16": red_roof}
-    gemm_roof.pop("on_32row_mfma_blocks_us", None)   # (the headline roofline object keeps to its fields)
     if "c1" in want:
         kernels["c1_ag_gemm_bf16_gated"] = bench_c1(dev, args.steps, args.warmup)
         log("c1", kernels["c1_ag_gemm_bf16_gated"])

@@ -80,13 +80,15 @@ int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local,
                                 int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
                                 int64_t ldc, int M, int N, int K, const int32_t* flags, int m_per_chunk,
                                 int wait_value, const int32_t* chunk_order, int rank, int world_size,
-                                int spin_limit, int32_t* status, int max_workgroups, void* stream);
+                                int spin_limit, int32_t* status, int max_workgroups,
+    void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 
 int tdist_gemm_chunk_gated_f16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
                                int64_t ldc, int M, int N, int K, const int32_t* flags, int m_per_chunk,
                                int wait_value, const int32_t* chunk_order, int rank, int world_size,
-                               int spin_limit, int32_t* status, int max_workgroups, void* stream);
+                               int spin_limit, int32_t* status, int max_workgroups,
+    void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 
 /* fp8-e4m3 inputs, bf16 output, C = (sum_k A8*B8) * row_scale[m] * col_scale[n].
  * The scale epilogue has no counterpart in the reference (fp8 is a dtype passthrough there,
@@ -96,7 +98,8 @@ int tdist_gemm_chunk_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
                                    void* C, int64_t ldc, int M, int N, int K, const float* row_scale,
                                    const float* col_scale, const int32_t* flags, int m_per_chunk,
                                    int wait_value, const int32_t* chunk_order, int rank, int world_size,
-                                   int spin_limit, int32_t* status, int max_workgroups, void* stream);
+                                   int spin_limit, int32_t* status, int max_workgroups,
+    void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 
 /* Producer side of the gate on the same GPU: copy one chunk, then release its flag, both ordered on
  * `stream`.   replaces cp_engine_producer_all_gather_full_mesh_push_multi_stream
@@ -153,10 +156,12 @@ int tdist_flag_fill(int32_t* flags, int n, int value, void* stream);
  * Requirements: M % (256*world_size) == 0, K % 64 == 0. */
 int tdist_gemm_rs_scatter_bf16(const void* A, int64_t lda, const void* B, int64_t ldb,
                                void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank,
-                               int world_size, void* stream);
+                               int world_size,
+    void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t ldb,
                               void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank,
-                              int world_size, void* stream);
+                              int world_size,
+    void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 
 /* out[e] = round( sum_{i=0..n_slices-1} float(c[((i + first_slice) % n_slices) * slice_stride + e]) )
  * for e in [0, n_elems): fp32 accumulation in exactly that order (the reference's order is
@@ -293,14 +298,16 @@ int tdist_group_gemm_gated_bf16(const void* A, int64_t lda, const void* A_local,
                                 const int32_t* block_barrier_ids, const int32_t* num_tokens_post_padded, int num_blocks,
                                 int block_size, int num_valid_tokens, int topk, int tokens_per_rank, int first_block,
                                 const int32_t* flags, int wait_value, int rank, int spin_limit, int32_t* status,
-                                int max_workgroups, void* stream);
+                                int max_workgroups,
+    void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 int tdist_group_gemm_gated_f16(const void* A, int64_t lda, const void* A_local, int64_t lda_local, int local_row_begin,
                                int local_rows, const void* B, int64_t ldb, int64_t expert_stride, void* C, int64_t ldc,
                                int a_rows, int N, int K, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                                const int32_t* block_barrier_ids, const int32_t* num_tokens_post_padded, int num_blocks,
                                int block_size, int num_valid_tokens, int topk, int tokens_per_rank, int first_block,
                                const int32_t* flags, int wait_value, int rank, int spin_limit, int32_t* status,
-                               int max_workgroups, void* stream);
+                               int max_workgroups,
+    void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 int tdist_group_gemm_gated_fp8e4m3(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                    int local_row_begin, int local_rows, const void* B, int64_t ldb,
                                    int64_t expert_stride, void* C, int64_t ldc, int a_rows, int N, int K,
@@ -308,28 +315,36 @@ int tdist_group_gemm_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
                                    const int32_t* block_barrier_ids, const int32_t* num_tokens_post_padded,
                                    int num_blocks, int block_size, int num_valid_tokens, int topk, int tokens_per_rank,
                                    int first_block, const int32_t* flags, int wait_value, int rank, int spin_limit,
-                                   int32_t* status, int max_workgroups, void* stream);
+                                   int32_t* status, int max_workgroups,
+    void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
- * Split-K workspace for the GEMM entry points above (tdist_gemm_chunk_gated_*, tdist_gemm_rs_scatter_*,
- * tdist_group_gemm_gated_*). Optional. The reference's kernels run whole tiles per program and leave a last round
- * that does not fill the grid to its autotuner's tile choice (kernels/amd/all_gather_gemm.py:151-246 persistent
- * loop; kernels/nvidia/allgather_group_gemm.py:238-314). Here, with a workspace registered for the current device,
- * a last round that fills at most half of the grid is cut along K: each of its tiles goes to s = grid / tiles
- * workgroups (at most 8, pieces of at least 4 K tiles), which add their fp32 accumulators through the workspace
- * before the usual epilogue (same products, other order of the sums: results stay within the stated tolerance
- * and are exact on integer-valued inputs). Whole rounds run as before. Bounded waits as for the chunk flags: a
- * piece that never arrives sets status to {TDIST_ERR_TIMEOUT, -1 - workgroup}.
- *   tdist_gemm_split_k_workspace_bytes(): size that serves every call on the current device (one fp32 256 x 256
- *     tile per compute unit + 4096 bytes of flags: 64 MiB + 4 KiB on MI355X); 0 if the device is not gfx950.
- *   tdist_gemm_split_k_set_workspace(workspace, bytes, stream): registers (workspace != NULL; 256-byte aligned
- *     device memory; the call clears the flag words on `stream`) or unregisters (NULL) the current device's
- *     workspace. The caller keeps the memory alive until it unregisters. One GEMM launch at a time may use it:
- *     launches of these entry points that can overlap on the device (different streams without an ordering) must
- *     not both find a workspace registered.
- * TDIST_GEMM_SPLIT_K=0 in the environment turns the path off, =1 takes it wherever a round can be split. */
+ * Workspace of the GEMM entry points above (tdist_gemm_chunk_gated_*, tdist_gemm_rs_scatter_*,
+ * tdist_group_gemm_gated_*): their sk_workspace / sk_workspace_bytes arguments. Optional (NULL, 0). The reference's
+ * kernels run whole tiles per program in a fixed order and leave a last round that does not fill the grid to the
+ * autotuner's tile choice (kernels/amd/all_gather_gemm.py:151-246 persistent loop;
+ * kernels/nvidia/allgather_group_gemm.py:238-314). With a workspace:
+ *   - a last round of tiles that fills at most half of the grid is cut along K: each of its tiles goes to s = 2, 4 or
+ *     8 workgroups (pieces of at least 4 K tiles); every piece's fp32 accumulators go through the workspace, and each
+ *     of the s workgroups adds up and stores 1/s of the tile, the pieces in their K order (same products, another
+ *     order of the sums than a whole tile's: results stay within the stated tolerance, are exact on integer-valued
+ *     inputs and do not depend on timing);
+ *   - the chunk-gated GEMM (flags != NULL, at most 64 chunks) schedules by arrival: a round of tiles is made up, when
+ *     the workgroups get to it, of the chunks whose flags are set by then, in the order given by chunk_order / rank;
+ *     when fewer tiles are ready than half of the workgroups, they are cut along K as above instead of leaving
+ *     workgroups idle until the next chunk lands. Without a workspace the tiles are taken in the fixed order and each
+ *     workgroup waits for its own tile's flag, as in the reference.
+ * Bounded waits as for the chunk flags: an exchange that does not complete sets status to
+ * {TDIST_ERR_TIMEOUT, -1 - workgroup} and the tile is not stored.
+ * The workspace is plain device memory, 256-byte aligned, of at least tdist_gemm_split_k_workspace_bytes() bytes (one
+ * fp32 256 x 256 tile per compute unit + a 20 KiB header: 64 MiB + 20 KiB on MI355X; 0 if the device is not gfx950),
+ * ZERO when it is first used; the kernels keep it consistent from then on (also across a launch that timed out). It
+ * carries no state that the library holds: any number of workspaces may be in use, one per launch in flight —
+ * launches that share one must be ordered (same stream, or events). A workspace that is misaligned or smaller than
+ * the header plus one 128 x 128 tile is rejected (TDIST_ERR_WORKSPACE); one too small for the call's tiles and grid
+ * is left unused.
+ * TDIST_GEMM_SPLIT_K=0 in the environment turns both uses off, =1 splits a last round wherever it can be split. */
 int64_t tdist_gemm_split_k_workspace_bytes(void);
-int tdist_gemm_split_k_set_workspace(void* workspace, int64_t bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * (d) split-KV GQA flash decode + LSE combine.
@@ -393,26 +408,6 @@ int tdist_decode_combine(const void* part, int part_dtype, const float* lse, int
                          int64_t part_stride_b, int64_t part_stride_h, int64_t lse_stride_p,
                          int64_t lse_stride_b, int64_t lse_stride_h, void* out, int out_dtype,
                          int64_t out_stride_b, int64_t out_stride_h, float* lse_out, void* stream);
-
-/* ---------------------------------------------------------------------------------------------
- * Measurement helper: plain 16-byte-vector device copy of nbytes (multiple of 16). Used to calibrate
- * rocprof FETCH_SIZE / WRITE_SIZE readings and as the HBM streaming yardstick; not on the hot path.
- * ------------------------------------------------------------------------------------------- */
-int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
-
-/* Measurement helper: the MFMA rate this chip sustains with no memory traffic at all. One workgroup of four waves per
- * compute unit runs iters (even) K steps of a 128 x 128 wave tile on register operands, in the GEMM kernel's order (a B
- * fragment against every A fragment in turn, 256 accumulators per lane): 4 x 4 MFMAs of 32x32x16 (bf16, K step 16) or
- * 32x32x64 (e4m3, K step 64) per K step. random_operands != 0 fills the fragments with random bit patterns, else with
- * 1.0. FLOP per launch = tdist_num_cus() * 4 * iters * 2 * 128 * 128 * K step. sink: tdist_num_cus() * 256 floats.
- * With random operands the chip is power-limited well below its nominal rate: this is the ceiling any GEMM on random
- * data sits under. Not on the hot path. */
-int tdist_mfma_rate_probe(int dtype, int random_operands, int iters, float* sink, void* stream);
-
-/* The same on the 16-row MFMA blocks the 256-row GEMM tiles use: 8 x 8 MFMAs of 16x16x32 (bf16, K step 32) or
- * 16x16x128 (e4m3, K step 128) per K step. They move a quarter of the accumulator registers per FLOP and sustain a
- * higher rate under the power limit. */
-int tdist_mfma_rate_probe_16row(int dtype, int random_operands, int iters, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -10,10 +10,11 @@ from triton_dist import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "tdist.h")
+BENCH_HEADER = os.path.join(ROOT, "include", "tdist_bench.h")
 
 
-def header_functions():
-    text = open(HEADER).read()
+def header_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tdist_[a-z0-9_]+)\s*\(", text)))
 
@@ -32,6 +33,18 @@ def test_library_exports_every_declared_symbol():
 
 def test_python_prototypes_cover_header():
     assert sorted(_lib.PROTOTYPES) == header_functions()
+
+
+def test_bench_library_is_separate_and_complete():
+    """The measurement helpers live in libtdist_bench.so: declared in tdist_bench.h, exported there, and absent from
+    the product library."""
+    names = header_functions(BENCH_HEADER)
+    assert sorted(_lib.BENCH_PROTOTYPES) == names
+    bench, product = _lib.load_bench(), _lib.load()
+    for name in names:
+        assert hasattr(bench, name), "libtdist_bench.so does not export %s" % name
+        assert not hasattr(product, name), "libtdist_hip.so still exports %s" % name
+    assert bench.tdist_copy_bytes(None, None, 16, None) == _lib.TDIST_ERR_INVALID
 
 
 def test_prototype_arity_matches_header():
@@ -57,7 +70,6 @@ def test_null_pointers_are_rejected_without_touching_the_gpu():
     assert "null" in _lib.last_error()
     assert lib.tdist_flag_set(None, 1, None) == _lib.TDIST_ERR_INVALID
     assert lib.tdist_moe_dispatch(None, 16, None, None, None, 0, 1, 1, 1, None, None, None, None) == _lib.TDIST_ERR_INVALID
-    assert lib.tdist_copy_bytes(None, None, 16, None) == _lib.TDIST_ERR_INVALID
     buf = ctypes.create_string_buffer(64)
     p = ctypes.addressof(buf)
     # bad sizes are caught before any launch

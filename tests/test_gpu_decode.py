@@ -248,6 +248,52 @@ def test_full_size_shard_sampled(cuda):
         assert (merged_lse[b].cpu().double() - exact_lse[0]).abs().max() <= ATOL
 
 
+def test_config5_end_to_end_with_seven_peers(cuda):
+    """BASELINE config 5 end to end at full size through the layer: split-KV over the shard (32 x 32768 keys, page 16),
+    merge of its splits, then the LSE merge with 7 seeded peer shards (out ~N(0,1) bf16, LSE ~N(log 32768, 2) fp32)
+    into [32, 64, 128]. Checked on 8 sequences against the exact closed form (decode_exact for the own shard, lse_merge
+    over the 8 shards): the fp32 form of the final output at 2e-3 absolute with no allowance, and the bf16 output
+    as exactly that fp32 result rounded to bf16 (its values are O(1), so bf16 rounding alone is up to 2^-8 |x|)."""
+    from triton_dist.kernels.amd import gqa_fwd_batch_decode_inter_rank_combine
+    from triton_dist.layers.nvidia import SpGQAFlashDecodeAttention
+    announce("decode C5 end to end, 8 shards")
+    R, rank, B, Hq, Hkv, D, L, page = 8, 0, 32, 64, 8, 128, 32768, 16
+    g = torch.Generator(device="cuda").manual_seed(3 + 4)
+    pages_per_seq = L // page
+    num_pages = B * pages_per_seq
+    k_dev = torch.randn((num_pages, page, Hkv, D), generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    v_dev = torch.randn((num_pages, page, Hkv, D), generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    q_dev = torch.randn((B, Hq, D), generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    table = torch.randperm(num_pages, generator=torch.Generator().manual_seed(6)).view(B, pages_per_seq).int()
+    gp = torch.Generator().manual_seed(3 + 4 + 100)
+    peer_out = torch.randn((R, B, Hq, D), generator=gp).to(torch.bfloat16)
+    peer_lse = torch.randn((R, B, Hq), generator=gp) * 2 + math.log(L)
+    global_lens = torch.full((R, B), L, dtype=torch.int32)
+    scale = D**-0.5
+    layer = SpGQAFlashDecodeAttention(rank, 0, R, 1, Hq, Hkv, D, D, page_size=page, scale=scale, max_allowed_batch=B)
+    layer.kv_split = 16                                   # the config's 16 splits
+    all_out = peer_out.float().to(cuda)                    # gather buffer in fp32: the own fp32 partial loses nothing
+    all_lse = peer_lse.to(cuda)
+    out = layer(q_dev, k_dev, v_dev, global_lens.to(cuda), table.to(cuda), peer_partials=(all_out, all_lse))
+    # the same merge with an fp32 result (all_out / all_lse now hold the own shard in row `rank`)
+    out32 = gqa_fwd_batch_decode_inter_rank_combine(all_out, all_lse, global_lens.to(cuda), out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16 and out.shape == (B, Hq, D)
+    assert torch.equal(out, out32.to(torch.bfloat16)), "the bf16 output is the fp32 result rounded to nearest even"
+    seqs = [0, 3, 7, 12, 16, 21, 26, 31]
+    for b in seqs:
+        pages = table[b].long().to(cuda)
+        k_b, v_b = k_dev[pages].cpu(), v_dev[pages].cpu()
+        t_b = torch.arange(pages_per_seq, dtype=torch.int32).view(1, -1)
+        own, own_lse = golden.decode_exact(q_dev[b:b + 1].cpu(), k_b, v_b, [L], t_b, scale)
+        shard_out = peer_out[:, b:b + 1].double().clone()
+        shard_lse = peer_lse[:, b:b + 1].double().clone()
+        shard_out[rank], shard_lse[rank] = own, own_lse
+        want, _ = golden.lse_merge(shard_out, shard_lse)
+        err = float((out32[b].cpu().double() - want[0]).abs().max())
+        assert err <= ATOL, "sequence %d: %g" % (b, err)
+
+
 @pytest.mark.parametrize("variant", [1, 2, 3, 4])
 def test_alternative_block_shapes(cuda, monkeypatch, variant):
     """The other compiled block shapes for D = 128 (keys per block, waves, stages), selectable for measurements:

@@ -99,32 +99,18 @@ def test_ag_gemm_config1(cuda):
             assert int(ctx.barrier_tensors[rank].abs().sum()) == 0
 
 
-def test_ag_gemm_gemm_first_and_sdma_options(cuda):
-    """The two producer options: the GEMM queued before the chunk copies, and copies on the copy engines. Queuing
-    the GEMM first needs the copy streams on hardware queues of their own; where this process has too many streams
-    for that, the bounded wait reports a timeout (never a hang) and the default order is checked instead."""
-    from triton_dist import _lib
+def test_ag_gemm_copy_engine_option(cuda):
+    """The chunk copies on the copy engines (hipMemcpyDeviceToDeviceNoCU), flags still published after the data."""
     from triton_dist.kernels.amd import ag_gemm_intra_node
-    announce("ag_gemm gemm_first / use_sdma")
+    announce("ag_gemm use_sdma")
     shards, b = make_ag_case(4, 512, 1024, 768, torch.bfloat16, seed=17)
     ref = golden.ag_gemm_fp32(shards, b)
     rank = 1
     ctx = run_ag_gemm(cuda, shards, b, rank, 256, use_sdma=True)
-    c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx)
-    ctx.check_status()
-    assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
-    ctx = run_ag_gemm(cuda, shards, b, rank, 256, gemm_first=True, spin_limit=1 << 18)
-    c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx)
-    try:
-        ctx.check_status()
-    except _lib.TdistError as e:
-        assert e.code == _lib.TDIST_ERR_TIMEOUT
-        ctx.gemm_first = False
+    for _ in range(2):
         c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx)
         ctx.check_status()
         assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
-        pytest.skip("a copy stream shares a hardware queue with the GEMM stream in this process")
-    assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
@@ -182,7 +168,8 @@ def test_gate_holds_and_times_out(cuda):
 
 
 def test_gate_released_by_a_stream_while_the_gemm_waits(cuda):
-    """Flags are set by a second stream after the GEMM has been launched (explicit chunk order, last chunk first)."""
+    """Flags are set by a second stream while the GEMM waits for them (explicit chunk order, last chunk first)."""
+    from triton_dist import _lib
     from triton_dist.kernels.amd import gated_gemm
     from triton_dist.kernels.amd.common_ops import set_signal
     announce("gate released late")
@@ -196,10 +183,15 @@ def test_gate_released_by_a_stream_while_the_gemm_waits(cuda):
     c = torch.empty((M, N), dtype=torch.bfloat16, device=cuda)
     a_dev, b_dev = a.to(cuda), b.to(cuda)
     side = torch.cuda.Stream()
+    stamp = torch.zeros(1, dtype=torch.int64, device=cuda)
     torch.cuda.synchronize()
-    gated_gemm(a_dev, None, 0, b_dev, c, flags, mpc, 0, 1, chunk_order=order, status=status)
+    # The releases are queued BEFORE the GEMM (work queued behind a spinning GEMM may share its hardware queue and never
+    # run) and held back on the device: a one-wave kernel sleeps 300 us past the stamp before the flags are set.
+    _lib.call("tdist_producer_mark", stamp.data_ptr(), side.cuda_stream)
+    _lib.call("tdist_producer_wait_until", stamp.data_ptr(), 300000, side.cuda_stream)
     for chunk in (3, 1, 0, 2):
         set_signal(flags.data_ptr() + 4 * chunk, 1, side)
+    gated_gemm(a_dev, None, 0, b_dev, c, flags, mpc, 0, 1, chunk_order=order, status=status)
     torch.cuda.synchronize()
     assert status.tolist() == [0, 0]
     assert golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32([a], b)) <= 1e-2
@@ -267,12 +259,16 @@ def test_fp8_ag_gemm_config3_full_size(cuda):
     c = ag_gemm_intra_node(shards[rank].to(cuda), b.to(cuda), False, ctx, row_scale=sa.to(cuda), col_scale=sb.to(cuda))
     ctx.check_status()
     assert c.shape == (16384, 7168) and c.dtype == torch.bfloat16
-    got = c.float().cpu()
-    # closed form on a band of rows from every chunk (the full fp32 product is 1.9 TFLOP on the CPU)
+    # closed form on every row of every chunk: the fp32 golden of one 2048-row chunk is a fraction of a second of CPU
+    # work, so all 16384 x 7168 outputs are compared (the stated bar against the chunk's own largest value, and
+    # element by element to the bf16 rounding of C, which a tile stored in the wrong place cannot meet)
     for r in range(world):
-        rows = slice(r * m_per_rank + 37, r * m_per_rank + 37 + 64)
-        ref = golden.fp8_scaled_gemm_fp32(shards[r][37:37 + 64], sa[rows], b, sb)
-        assert golden.max_rel_err(got[rows], ref) <= 1e-2, "chunk %d" % r
+        rows = slice(r * m_per_rank, (r + 1) * m_per_rank)
+        ref = golden.fp8_scaled_gemm_fp32(shards[r], sa[rows], b, sb)
+        got = c[rows].float().cpu()
+        assert golden.max_rel_err(got, ref) <= 1e-2, "chunk %d" % r
+        assert torch.allclose(got, ref, rtol=2.0**-7, atol=2e-3 * float(ref.abs().max())), "chunk %d" % r
+        del ref, got
     # linearity in the scales: doubling a row scale doubles that row (size-independent property)
     sa2 = sa.clone()
     sa2[::2] *= 2
@@ -469,33 +465,6 @@ def test_ag_gemm_kernel_producer_and_graph_replay(cuda, producer_kernel, link_gb
     ctx.check_status()
     if producer_kernel:
         assert int(ctx.producer_counters.abs().sum()) == 0
-
-
-@pytest.mark.parametrize("variant", [2, 5])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
-def test_alternative_schedules_of_the_large_tile(cuda, monkeypatch, variant, dtype):
-    """The two other compiled schedules of the 256 x 256 tile (eight waves on a two-stage ring and on the split
-    ring), selectable for measurements, give the same exact result on integer-valued inputs."""
-    from triton_dist.kernels.amd import gated_gemm
-    monkeypatch.setenv("TDIST_GEMM_VARIANT", str(variant))
-    monkeypatch.setenv("TDIST_GEMM_TILE", "0")
-    esz = 1 if dtype == torch.float8_e4m3fn else 2
-    M, N, K = 1100, 780, 640 // esz
-    announce("gemm schedule variant %d %s" % (variant, dtype))
-    g = torch.Generator().manual_seed(variant)
-    a = torch.randint(-2, 3, (M, K), generator=g).float()
-    b = torch.randint(-2, 3, (N, K), generator=g).float()
-    c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
-    sa = sb = None
-    if dtype == torch.float8_e4m3fn:
-        sa = (2.0 ** torch.randint(-3, 3, (M,), generator=g).float()).to(cuda)
-        sb = (2.0 ** torch.randint(-3, 3, (N,), generator=g).float()).to(cuda)
-    gated_gemm(a.to(dtype).to(cuda), None, 0, b.to(dtype).to(cuda), c, None, 0, 0, 1, row_scale=sa, col_scale=sb)
-    torch.cuda.synchronize()
-    ref = a.to(cuda) @ b.to(cuda).T
-    if sa is not None:
-        ref = ref * sa[:, None] * sb[None, :]
-    assert torch.equal(c, ref.to(torch.bfloat16))
 
 
 @pytest.mark.parametrize("m_per,K", [(256, 256), (200, 320), (72, 96)])

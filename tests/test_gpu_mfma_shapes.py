@@ -1,8 +1,8 @@
-"""The 256-row GEMM tiles run on the 16-row MFMA blocks (16x16x32 for bf16/f16, 16x16x128 for e4m3) by default and on
-the 32-row blocks (32x32x16 / 32x32x64) with TDIST_GEMM_MFMA16=0. Both forms walk K in the same tile order with one
-fp32 accumulator per output element, and they agree bit for bit on every case here; each is also held against the
-exact result on integer-valued inputs (every partial sum is an integer that fp32 holds) and, on random inputs, to max
-relative error <= 1e-2 of fp32."""
+"""The 256-row GEMM tiles run on the 16-row MFMA blocks (16x16x32 for bf16/f16, 16x16x128 for e4m3) with their
+accumulators in fixed registers; the 128 x 128 tile runs on the 32-row blocks (32x32x16 / 32x32x64) with accumulators
+the compiler places. Each form is held against the exact result on integer-valued inputs (every partial sum is an
+integer that fp32 holds) over the K-loop's corner cases, and on random inputs to max relative error <= 1e-2 of fp32 and
+to each other within the rounding of the output."""
 import os
 
 import pytest
@@ -14,52 +14,44 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture
-def mfma_env():
-    keys = ("TDIST_GEMM_MFMA16", "TDIST_GEMM_TILE")
-    old = {k: os.environ.get(k) for k in keys}
+def tile_env():
+    old = os.environ.get("TDIST_GEMM_TILE")
     yield
     torch.cuda.synchronize()
-    for k in keys:
-        if old[k] is None:
-            os.environ.pop(k, None)
-        else:
-            os.environ[k] = old[k]
+    if old is None:
+        os.environ.pop("TDIST_GEMM_TILE", None)
+    else:
+        os.environ["TDIST_GEMM_TILE"] = old
 
 
-def run_both(cuda, a, b, out_dtype, tile, **kw):
+def run_tile(cuda, a, b, out_dtype, tile, **kw):
     from triton_dist.kernels.amd import gated_gemm
-    out = {}
-    for mode in ("0", "1"):
-        os.environ["TDIST_GEMM_MFMA16"] = mode
-        os.environ["TDIST_GEMM_TILE"] = str(tile)
-        c = torch.full((a.shape[0], b.shape[0]), float("nan"), dtype=out_dtype, device=cuda)
-        status = torch.zeros(2, dtype=torch.int32, device=cuda)
-        gated_gemm(a, None, 0, b, c, None, 0, 0, 1, status=status, **kw)
-        torch.cuda.synchronize()
-        assert status.tolist() == [0, 0]
-        out[mode] = c
-    return out
+    os.environ["TDIST_GEMM_TILE"] = str(tile)
+    c = torch.full((a.shape[0], b.shape[0]), float("nan"), dtype=out_dtype, device=cuda)
+    status = torch.zeros(2, dtype=torch.int32, device=cuda)
+    gated_gemm(a, None, 0, b, c, None, 0, 0, 1, status=status, **kw)
+    torch.cuda.synchronize()
+    assert status.tolist() == [0, 0]
+    return c
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
-@pytest.mark.parametrize("tile", [0, 1])
+@pytest.mark.parametrize("tile", [0, 1, 2])
 @pytest.mark.parametrize("M,N,K", [(512, 512, 128), (768, 512, 384), (300, 200, 640), (1024, 1280, 1152)])
-def test_exact_and_bit_equal_on_integer_inputs(cuda, mfma_env, dtype, tile, M, N, K):
+def test_exact_on_integer_inputs(cuda, tile_env, dtype, tile, M, N, K):
     """One K tile (e4m3) or two; an odd number of K tiles (the e4m3 loop works in pairs of tiles); a ragged shape (the
-    bounds-checked epilogue); several tiles per workgroup row. tile 0 = 256x256, 1 = 256x128."""
+    bounds-checked epilogue); several tiles per workgroup row. tile 0 = 256x256, 1 = 256x128, 2 = 128x128."""
     announce("mfma shapes exact %s tile %d %dx%dx%d" % (dtype, tile, M, N, K))
     g = torch.Generator().manual_seed(M + N + K + tile)
     a = torch.randint(-2, 3, (M, K), generator=g).float().to(dtype).to(cuda)
     b = torch.randint(-2, 3, (N, K), generator=g).float().to(dtype).to(cuda)
     out_dtype = torch.bfloat16 if dtype == torch.float8_e4m3fn else dtype
-    out = run_both(cuda, a, b, out_dtype, tile)
     ref = (a.float() @ b.float().T).to(out_dtype)
-    assert torch.equal(out["0"], ref)
-    assert torch.equal(out["1"], ref)
+    assert torch.equal(run_tile(cuda, a, b, out_dtype, tile), ref)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
-def test_random_inputs_bit_equal_and_close(cuda, mfma_env, dtype):
+def test_random_inputs_close_in_every_form(cuda, tile_env, dtype):
     M, N, K = 1536, 1024, 4224
     announce("mfma shapes random %s %dx%dx%d" % (dtype, M, N, K))
     g = torch.Generator().manual_seed(11)
@@ -71,16 +63,17 @@ def test_random_inputs_bit_equal_and_close(cuda, mfma_env, dtype):
         kw["row_scale"] = (torch.rand(M, generator=g) * 0.09 + 0.01).to(cuda)
         kw["col_scale"] = (torch.rand(N, generator=g) * 0.9 + 0.1).to(cuda)
         ref = ref * kw["row_scale"][:, None] * kw["col_scale"][None, :]
-    out_dtype = torch.bfloat16
-    out = run_both(cuda, a, b, out_dtype, 0, **kw)
-    assert torch.equal(out["0"], out["1"])
-    rel = (out["1"].float() - ref).abs().max() / ref.abs().max()
-    assert rel.item() <= 1e-2
+    out = [run_tile(cuda, a, b, torch.bfloat16, tile, **kw) for tile in (0, 1, 2)]
+    for c in out:
+        rel = (c.float() - ref).abs().max() / ref.abs().max()
+        assert rel.item() <= 1e-2
+        # (the forms differ in the order of the fp32 sums only: one rounding step of the bf16 output at most)
+        assert torch.allclose(c.float(), out[0].float(), rtol=2.0**-7, atol=1e-3 * float(ref.abs().max()))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
 @pytest.mark.parametrize("block", [128, 256])
-def test_grouped_blocks_exact_in_both_forms(cuda, mfma_env, dtype, block):
+def test_grouped_blocks_exact(cuda, dtype, block):
     """The grouped form (gathered A rows, per-block expert weights, scattered C rows) on both block sizes."""
     from oracle import golden
     from tests.test_gpu_group_gemm import make_case, run
@@ -88,8 +81,6 @@ def test_grouped_blocks_exact_in_both_forms(cuda, mfma_env, dtype, block):
     announce("mfma shapes grouped %s block %d" % (dtype, block))
     shards, w, ids = make_case(world, mpr, K, N, E, topk, dtype, seed=block, integer=True)
     ref = golden.ag_group_gemm_fp32(shards, w, ids)
-    for mode in ("0", "1"):
-        os.environ["TDIST_GEMM_MFMA16"] = mode
-        ctx, c = run(cuda, shards, w, ids, 1, E, block)
-        ctx.check_status()
-        assert torch.equal(c.float().cpu(), ref.to(c.dtype).float()), "TDIST_GEMM_MFMA16=%s" % mode
+    ctx, c = run(cuda, shards, w, ids, 1, E, block)
+    ctx.check_status()
+    assert torch.equal(c.float().cpu(), ref.to(c.dtype).float())

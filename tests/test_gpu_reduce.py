@@ -72,7 +72,7 @@ def test_copy_bytes_helper(cuda):
     announce("copy_bytes")
     src = torch.randint(0, 255, (1 << 20, ), dtype=torch.uint8, device=cuda)
     dst = torch.zeros_like(src)
-    _lib.call("tdist_copy_bytes", dst.data_ptr(), src.data_ptr(), src.numel(), _lib.stream_ptr())
+    _lib.bench_call("tdist_copy_bytes", dst.data_ptr(), src.data_ptr(), src.numel(), _lib.stream_ptr())
     torch.cuda.synchronize()
     assert torch.equal(src, dst)
 
@@ -84,23 +84,23 @@ def test_mfma_rate_probe_runs(cuda):
     sink = torch.full((cus * 256, ), float("nan"), dtype=torch.float32, device=cuda)
     for code in (_lib.TDIST_BF16, _lib.TDIST_F8E4M3):
         for rnd in (0, 1):
-            _lib.call("tdist_mfma_rate_probe", code, rnd, 8, sink.data_ptr(), _lib.stream_ptr())
+            _lib.bench_call("tdist_mfma_rate_probe", code, rnd, 8, sink.data_ptr(), _lib.stream_ptr())
             torch.cuda.synchronize()
             assert torch.isfinite(sink).all()
     # constant operands: 1.0 x 1.0 summed over K (16 per bf16 MFMA), 8 K steps, the first accumulator of 16 blocks
-    _lib.call("tdist_mfma_rate_probe", _lib.TDIST_BF16, 0, 8, sink.data_ptr(), _lib.stream_ptr())
+    _lib.bench_call("tdist_mfma_rate_probe", _lib.TDIST_BF16, 0, 8, sink.data_ptr(), _lib.stream_ptr())
     torch.cuda.synchronize()
     assert torch.all(sink == 16 * 8 * 16.0)
     with pytest.raises(_lib.TdistError):
-        _lib.call("tdist_mfma_rate_probe", _lib.TDIST_BF16, 0, 7, sink.data_ptr(), _lib.stream_ptr())
+        _lib.bench_call("tdist_mfma_rate_probe", _lib.TDIST_BF16, 0, 7, sink.data_ptr(), _lib.stream_ptr())
     # the 16-row blocks: 64 blocks, K = 32 per bf16 MFMA
     for code in (_lib.TDIST_BF16, _lib.TDIST_F8E4M3):
         for rnd in (0, 1):
-            _lib.call("tdist_mfma_rate_probe_16row", code, rnd, 8, sink.data_ptr(), _lib.stream_ptr())
+            _lib.bench_call("tdist_mfma_rate_probe_16row", code, rnd, 8, sink.data_ptr(), _lib.stream_ptr())
             torch.cuda.synchronize()
             assert torch.isfinite(sink).all()
-    _lib.call("tdist_mfma_rate_probe_16row", _lib.TDIST_BF16, 0, 8, sink.data_ptr(), _lib.stream_ptr())
+    _lib.bench_call("tdist_mfma_rate_probe_16row", _lib.TDIST_BF16, 0, 8, sink.data_ptr(), _lib.stream_ptr())
     torch.cuda.synchronize()
     assert torch.all(sink == 64 * 8 * 32.0)
     with pytest.raises(_lib.TdistError):
-        _lib.call("tdist_mfma_rate_probe_16row", _lib.TDIST_BF16, 0, 7, sink.data_ptr(), _lib.stream_ptr())
+        _lib.bench_call("tdist_mfma_rate_probe_16row", _lib.TDIST_BF16, 0, 7, sink.data_ptr(), _lib.stream_ptr())

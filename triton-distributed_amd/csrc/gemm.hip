@@ -66,18 +66,36 @@ struct GemmParams {
   const int32_t* post_pad;       // device scalar: rows of the sorted space in use (a multiple of BM)
   int64_t b_expert_stride_b;     // bytes between the experts' weight matrices
   int num_valid, topk, first_block, a_rows;
-  // Split last round (sk_on != 0): whole rounds of the grid run tile by tile as always; the tiles of a last round
-  // that fills at most half of the grid are cut along K into s = grid / tiles equal pieces (at most kSkMaxSplit, at
-  // least kSkMinPiece K tiles each), one per workgroup, so that the round takes 1/s of a tile's time. Workgroups
-  // s*t .. s*t+s-1 share tile t: each but the last adds the next one's accumulators (fp32, in register order,
-  // through slot [workgroup] of sk_partials, announced by sk_flags[workgroup] == sk_epoch) to its own, and the
-  // first runs the epilogue. (Cutting every tile of the schedule into equal shares of K tiles, "stream-K",
-  // was measured slower than whole tiles: workgroups that share an operand panel are then at different K
-  // positions, and the panel is fetched once per workgroup instead of once per XCD.)
+  // Split rounds (sk_ctrl != NULL: the caller handed in a workspace). A tile may be cut along K into s = 2, 4 or 8
+  // equal pieces (at least kSkMinPiece K tiles each), one per workgroup: workgroups s*t .. s*t+s-1 of the round share
+  // tile t. Every piece writes its fp32 accumulators (register order) to slot [workgroup] of sk_partials and raises
+  // flag [workgroup] to the round's tag; then each of the s workgroups adds up 1/s of the tile from the s slots, in
+  // slot order (so the sum does not depend on timing), and stores that part of C. A slot is written again only after
+  // its s readers have acknowledged (ack [workgroup] counts them). Tags are unique per launch and round: the header
+  // word kSkCtrlEpoch is read at the start and advanced by the last workgroup to leave, so nothing has to be cleared
+  // between launches, a launch that ran into a timeout included. Launches that share a workspace must not overlap.
+  //   sk_mode 1: static schedule, only a last round that fills at most half of the grid is split;
+  //   sk_mode 2: dynamic rounds (chunk-gated calls): see the scheduler in the kernel.
+  // (Cutting every tile of the schedule into equal shares of K tiles, "stream-K", was measured slower than whole
+  // tiles: workgroups that share an operand panel are then at different K positions, and the panel is fetched once
+  // per workgroup instead of once per XCD.)
+  int32_t* sk_ctrl;
   float* sk_partials;
-  int32_t* sk_flags;
-  int sk_on, sk_epoch;
+  int sk_mode;
 };
+
+// Workspace header, in int32 words
+constexpr int kSkCtrlEpoch = 0;          // tag base of the next launch
+constexpr int kSkCtrlDone = 1;           // workgroups of the running launch that have left
+constexpr int kSkMaxWorkgroups = 1024;
+constexpr int kSkFlagsOff = 1024;        // [kSkMaxWorkgroups] tag of the partial in the slot
+constexpr int kSkAcksOff = 2048;         // [kSkMaxWorkgroups] readers that are done with the slot, ever
+constexpr int kSkDecOff = 3072;          // [kSkMaxDecisions][kSkDecWords] scheduler decisions of the running launch
+constexpr int kSkMaxDecisions = 256, kSkDecWords = 8;
+constexpr int kSkHeaderWords = kSkDecOff + kSkMaxDecisions * kSkDecWords;
+constexpr int64_t kSkHeaderBytes = (int64_t)kSkHeaderWords * 4;
+constexpr int kSkTagStride = 1024;       // tags per launch (rounds that may be split or decided)
+static_assert(kSkHeaderBytes % 256 == 0, "the partial slots start 256-byte aligned");
 
 // Operand fragment of one lane: K bytes [0, kLaneBytes) of one row; chunk0 / chunk1 are LDS addresses of its
 // 16-byte pieces.
@@ -114,24 +132,28 @@ struct ElemF16 {
 // The same element types on the 16x16x32 MFMA: four lane groups along K instead of two, sixteen rows per block.
 // Per flop it draws less power than the 32x32x16 form, which is what the clock of a long GEMM on real data
 // is limited by.
-// Its four-register result is not tied to its accumulator input in the compiler's instruction model; with all 256
-// accumulation registers in use the allocator then shuffles accumulators between registers inside the K loop. Written
-// as assembly with one read-write operand the instruction works in place. (The compiler then knows none of its
-// hazards: the K loop never reads an accumulator, and the code after it waits out the last MFMA before it does.)
+// Its four-register result is not tied to its accumulator input in the compiler's instruction model, and with all 256
+// accumulation registers in use the register allocator, left to place the accumulators itself, has shuffled them
+// between registers and spilled them inside the K loop, after edits far from the loop. The kernels on these blocks
+// therefore keep their accumulators in FIXED accumulation registers: block (j, i) of the wave tile lives in
+// a[4*(j*kTM+i) .. +3], the instruction is written as assembly that names those registers, and the compiler never
+// allocates an accumulation register in these kernels (see acc_reserve). (The compiler then knows none of the
+// instruction's hazards: the K loop never reads an accumulator, and the code after it waits out the last MFMA
+// before it does.)
 struct ElemBF16N : ElemBF16 {
   static constexpr int kRows = 16;
   typedef float4v acc_t;
-  __device__ static __forceinline__ float4v mma(frag a, frag b, float4v c) {
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-    return c;
+  template <int kBase>
+  __device__ static __forceinline__ void mma_at(frag a, frag b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(kBase), "n"(kBase + 3));
   }
 };
 struct ElemF16N : ElemF16 {
   static constexpr int kRows = 16;
   typedef float4v acc_t;
-  __device__ static __forceinline__ float4v mma(frag a, frag b, float4v c) {
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-    return c;
+  template <int kBase>
+  __device__ static __forceinline__ void mma_at(frag a, frag b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(kBase), "n"(kBase + 3));
   }
 };
 struct ElemFP8 {
@@ -160,9 +182,9 @@ struct ElemFP8 {
 struct ElemFP8N : ElemFP8 {
   static constexpr int kRows = 16;
   typedef float4v acc_t;
-  __device__ static __forceinline__ float4v mma(frag a, frag b, float4v c) {
-    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-    return c;
+  template <int kBase>
+  __device__ static __forceinline__ void mma_at(frag a, frag b) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(kBase), "n"(kBase + 3));
   }
 };
 
@@ -249,11 +271,38 @@ __device__ __forceinline__ void wait_tiles_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kOutstanding) : "memory");
 }
 
-// Split last round: most pieces per tile, fewest K tiles per piece
+// Split rounds: most pieces per tile, fewest K tiles per piece
 constexpr int kSkMaxSplit = 8, kSkMinPiece = 4;
+// pieces per tile when `tiles` tiles are all that `workgroups` workgroups have to do: the largest power of two that
+// the workgroups and the K tiles allow (1 = whole tiles)
+__host__ __device__ inline int sk_split_for(int workgroups, int tiles, int k_tiles) {
+  int s = 1;
+  while (2 * s <= kSkMaxSplit && (int64_t)2 * s * tiles <= workgroups && k_tiles / (2 * s) >= kSkMinPiece) s *= 2;
+  return s;
+}
 
 // Instruction classes for __builtin_amdgcn_sched_group_barrier
 constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
+
+// Kernels with fixed accumulators: declares a[0 .. kN) in use, so that the kernel is given them and the compiler
+// neither parks spilled vector registers in them nor counts them as free; nothing else in such a kernel is ever of
+// the accumulation register class. Then clears them.
+#define TDIST_A10(n) "a" #n "0", "a" #n "1", "a" #n "2", "a" #n "3", "a" #n "4", "a" #n "5", "a" #n "6", "a" #n "7", "a" #n "8", "a" #n "9"
+#define TDIST_A_0_99 "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", TDIST_A10(1), TDIST_A10(2), TDIST_A10(3), TDIST_A10(4), \
+    TDIST_A10(5), TDIST_A10(6), TDIST_A10(7), TDIST_A10(8), TDIST_A10(9)
+#define TDIST_A_100_127 TDIST_A10(10), TDIST_A10(11), "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127"
+#define TDIST_A_128_255 "a128", "a129", TDIST_A10(13), TDIST_A10(14), TDIST_A10(15), TDIST_A10(16), TDIST_A10(17), TDIST_A10(18), \
+    TDIST_A10(19), TDIST_A10(20), TDIST_A10(21), TDIST_A10(22), TDIST_A10(23), TDIST_A10(24), "a250", "a251", "a252", "a253", "a254", "a255"
+template <int kN>
+__device__ __forceinline__ void acc_reserve() {
+  static_assert(kN == 128 || kN == 256, "accumulators of a 128 x 64 or a 128 x 128 wave tile");
+  if constexpr (kN == 256) asm volatile("" ::: TDIST_A_0_99, TDIST_A_100_127, TDIST_A_128_255);
+  else asm volatile("" ::: TDIST_A_0_99, TDIST_A_100_127);
+}
+template <int kN>
+__device__ __forceinline__ void acc_clear() {
+  static_for<kN>([&](auto r_c) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(decltype(r_c)::value)); });
+}
 
 // schedule position → chunk id
 __device__ __forceinline__ int chunk_of(const GemmParams& p, int oc) {
@@ -278,6 +327,9 @@ template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kSca
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams p) {
   typedef GemmCfg<E, BM, BN, KB, WM, WN, NST> C;
   typedef TDIST_AS3 unsigned char* lds_u8;
+  constexpr bool kFixedAcc = E::kRows == 16;
+  constexpr int kAccRegs = C::kTM * C::kTN * C::kAccLen;
+  if constexpr (kFixedAcc) acc_reserve<kAccRegs>();
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem_generic[];
   lds_u8 const smem = (lds_u8)smem_generic;
   // gate result (1 = tile may proceed, 0 = wait expired) lives in the first word of the ring, which is idle
@@ -307,25 +359,48 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   // XCD-aware position within a round: workgroups of XCD x take a contiguous range
   int wg_pos = blockIdx.x;
   if (p.num_xcds > 1 && G % p.num_xcds == 0) wg_pos = (wg_pos % p.num_xcds) * (G / p.num_xcds) + wg_pos / p.num_xcds;
-  // split last round: s pieces per tile (1 = not split)
+  // ---- workspace state of this launch ---------------------------------------------------------------------
+  int32_t* const sk_flags = p.sk_ctrl + kSkFlagsOff;
+  int32_t* const sk_acks = p.sk_ctrl + kSkAcksOff;
+  int tag_base = 0;   // tags of this launch are tag_base + 1 + round
+  int sk_need = 0;    // value of this workgroup's ack word once every reader of its last partial is done
+  if (p.sk_mode != 0) {
+    if (threadIdx.x == 0) {
+      s_gate[0] = __hip_atomic_load(p.sk_ctrl + kSkCtrlEpoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_gate[1] = __hip_atomic_load(sk_acks + wg_pos, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    tag_base = __builtin_amdgcn_readfirstlane(s_gate[0]);
+    sk_need = __builtin_amdgcn_readfirstlane(s_gate[1]);
+    __syncthreads();
+  }
+  // static schedule: the last round is cut into s pieces per tile (1 = not split)
   const int sk_tail_tiles = total_sched % G;
   int sk_split = 1;
-  if (p.sk_on && sk_tail_tiles > 0) sk_split = min(min(G / sk_tail_tiles, kSkMaxSplit), KT / kSkMinPiece);
-  if (sk_split < 2) sk_split = 1;
+  if (p.sk_mode == 1 && sk_tail_tiles > 0) sk_split = sk_split_for(G, sk_tail_tiles, KT);
 
-  for (int sbase = 0;; sbase += G) {
-    int sidx, ka = 0, kb = KT;  // the piece: K tiles [ka, kb) of scheduled tile sidx
-    if (sbase >= total_sched) break;
-    if (sk_split > 1 && sbase + G > total_sched) {
-      // the last round, split: workgroup s*t + j takes piece j of the round's tile t
-      const int t = wg_pos / sk_split, j = wg_pos - t * sk_split;
-      if (t >= sk_tail_tiles) break;
-      sidx = __builtin_amdgcn_readfirstlane(sbase + t);
-      ka = __builtin_amdgcn_readfirstlane(KT * j / sk_split);  // (KT < 2^20 and j < 8: 32-bit scalar arithmetic)
-      kb = __builtin_amdgcn_readfirstlane(KT * (j + 1) / sk_split);
-    } else {
-      sidx = sbase + wg_pos;
-      if (sidx >= total_sched) continue;
+  int sbase = 0;
+  for (;;) {
+    // ---- next piece of work: K tiles [ka, kb) of scheduled tile sidx, as piece sk_j of sk_s --------------
+    int sidx, ka = 0, kb = KT, sk_s = 1, sk_j = 0, sk_tag = 0;
+    {
+      if (sbase >= total_sched) break;
+      const int round_base = sbase;
+      sbase += G;
+      if (sk_split > 1 && round_base + G > total_sched) {
+        // the last round, split: workgroup s*t + j takes piece j of the round's tile t
+        const int t = wg_pos / sk_split, j = wg_pos - t * sk_split;
+        if (t >= sk_tail_tiles) break;
+        sidx = __builtin_amdgcn_readfirstlane(round_base + t);
+        sk_s = sk_split;
+        sk_j = __builtin_amdgcn_readfirstlane(j);
+        sk_tag = tag_base + 1;
+        ka = __builtin_amdgcn_readfirstlane(KT * j / sk_split);  // (KT < 2^20 and j < 8: 32-bit scalar arithmetic)
+        kb = __builtin_amdgcn_readfirstlane(KT * (j + 1) / sk_split);
+      } else {
+        sidx = round_base + wg_pos;
+        if (sidx >= total_sched) continue;
+      }
     }
     const int KTp = kb - ka;
     const int oc = sidx / tiles_per_chunk;
@@ -468,15 +543,21 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       for (int f = 0; f < C::kTM + C::kTN; ++f) load_frag(kt, ks, f, af, bf);
     };
 
-    typename E::acc_t acc[C::kTN][C::kTM];
+    // accumulators: fixed registers a[0 .. kAccRegs) for the 16-row MFMA blocks, else the compiler's
+    typename E::acc_t acc[kFixedAcc ? 1 : C::kTN][kFixedAcc ? 1 : C::kTM];
+    if constexpr (kFixedAcc) {
+      acc_clear<kAccRegs>();
+    } else {
 #pragma unroll
-    for (int j = 0; j < C::kTN; ++j)
+      for (int j = 0; j < C::kTN; ++j)
 #pragma unroll
-      for (int i = 0; i < C::kTM; ++i)
+        for (int i = 0; i < C::kTM; ++i)
 #pragma unroll
-        for (int e = 0; e < C::kAccLen; ++e) acc[j][i][e] = 0.f;
+          for (int e = 0; e < C::kAccLen; ++e) acc[j][i][e] = 0.f;
+    }
 
     constexpr int kMfmaPerStep = C::kTM * C::kTN;
+    static_assert(!C::kSplit || E::kRows == 16, "the split ring's K loops are written for the 16-row MFMA blocks");
     if constexpr (C::kSplit && E::kRows == 16 && C::kKSteps == 1) {
       // ---- split ring, 16-row MFMA blocks, the whole K tile in one MFMA depth (e4m3) --------------------
       // The MFMAs of a tile run as four quarters: the lower half of the A fragments against one half of the B
@@ -538,7 +619,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
             wait_tiles_and_barrier<C::kAInstr>();
             __builtin_amdgcn_sched_barrier(0);
           }
-          acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
+          E::template mma_at<(j * C::kTM + i) * C::kAccLen>(b_cur[j], a_cur[i]);
           // the quarter's fragment reads, from its slot 2 on (128 x 128 wave tile: slots 2, 5, 8, 11)
           constexpr int n_reads = (quarter == 0 || quarter == 3) ? kHB : kHA;
           constexpr int stride = (kQuarter - 2) / n_reads;
@@ -560,15 +641,6 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         if (kt + 1 < KTp) tile(std::integral_constant<int, 1>{}, kt + 1);
       }
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the last MFMAs' results: 8 passes + 3 cycles after issue
-
-      // (every later use of an accumulator depends on these empty statements, which stay behind the wait above: the
-      // compiler, which does not know that the assembly before it was an MFMA, cannot move a read in front of it)
-      if constexpr (C::kTM * C::kTN * C::kAccLen < 256) {  // (with 256 of them they are only ever read in assembly)
-#pragma unroll
-        for (int j = 0; j < C::kTN; ++j)
-#pragma unroll
-          for (int i = 0; i < C::kTM; ++i) asm volatile("" : "+a"(acc[j][i]));
-      }
     } else if constexpr (C::kSplit && E::kRows == 16) {
       // ---- split ring, 16-row MFMA blocks ------------------------------------------------------------
       // The MFMAs of a K step run in B-fragment-major order: a B fragment serves kTM MFMAs in a row and is then dead,
@@ -607,7 +679,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
           static_for<kMfmaPerStep>([&](auto idx_c) {
             constexpr int idx = decltype(idx_c)::value;
             constexpr int j = idx / C::kTM, i = idx % C::kTM;
-            acc[j][i] = E::mma(b_cur[j], a_now[i], acc[j][i]);
+            E::template mma_at<(j * C::kTM + i) * C::kAccLen>(b_cur[j], a_now[i]);
             if constexpr (last && idx == kLead - 1) {
               __builtin_amdgcn_sched_barrier(0);
               wait_tiles_and_barrier<C::kAInstr>();
@@ -630,81 +702,6 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       }
       // the last MFMAs' results are readable 4 passes + 3 cycles after issue
       asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
-
-      // (every later use of an accumulator depends on these empty statements, which stay behind the wait above: the
-      // compiler, which does not know that the assembly before it was an MFMA, cannot move a read in front of it)
-      if constexpr (C::kTM * C::kTN * C::kAccLen < 256) {  // (with 256 of them they are only ever read in assembly)
-#pragma unroll
-        for (int j = 0; j < C::kTN; ++j)
-#pragma unroll
-          for (int i = 0; i < C::kTM; ++i) asm volatile("" : "+a"(acc[j][i]));
-      }
-    } else if constexpr (C::kSplit) {
-      // ---- split ring ------------------------------------------------------------------------------
-      // The DMA list of one cycle is [B(kt+2) rows..., A(kt+3) rows...]; it starts right after the barrier in the
-      // last K step of tile kt (B stage kt%2 and A stage kt%3 have just been released) and runs, kDmaPerStep
-      // instructions per K step, through the K steps of tile kt+1. At the barrier of tile kt+1 only the A rows
-      // of that list may still be in flight.
-      constexpr int kFrags = C::kTM + C::kTN;
-      // q-th instruction of the list whose cycle started in tile `cyc`
-      auto issue_list = [&](int cyc, int q) {
-        if (q < C::kBInstr) issue_b(cyc + 2, q);
-        else issue_a(cyc + 3, q - C::kBInstr);
-      };
-#pragma unroll
-      for (int t = 0; t < C::kAInstr; ++t) issue_a(0, t);
-#pragma unroll
-      for (int u = 0; u < C::kBInstr; ++u) issue_b(0, u);
-#pragma unroll
-      for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
-#pragma unroll
-      for (int q = 0; q < C::kDmaPerStep; ++q) issue_list(-1, q);
-      wait_tiles_and_barrier<C::kAInstr + C::kDmaPerStep>();
-      load_frags(0, 0, a_cur, b_cur);
-      __builtin_amdgcn_sched_barrier(0);
-      for (int kt = 0; kt < KTp; ++kt) {
-        const int kt_next = min(kt + 1, KTp - 1);
-#pragma unroll
-        for (int ks = 0; ks < C::kKSteps; ++ks) {
-          constexpr int kLast = C::kKSteps - 1;
-          const bool last = ks == kLast;
-          const int first = last ? C::kLeadMfma : 0;
-          const int nslots = kMfmaPerStep - first;
-          const int pos = (ks + 1) % C::kKSteps;  // K steps since the list's cycle began
-          if (last) {
-#pragma unroll
-            for (int idx = 0; idx < C::kLeadMfma; ++idx) {
-              const int j = idx / C::kTM, i = idx % C::kTM;
-              acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            wait_tiles_and_barrier<C::kAInstr>();
-            __builtin_amdgcn_sched_barrier(0);
-          }
-#pragma unroll
-          for (int idx = first; idx < kMfmaPerStep; ++idx) {
-            const int j = idx / C::kTM, i = idx % C::kTM;
-            acc[j][i] = E::mma(b_cur[j], a_cur[i], acc[j][i]);
-            const int slot = idx - first;
-            // next K step's fragments in the order of their first use; the shorter last step reads two at once
-            if (last) {
-              if (slot == 0) load_frag(kt_next, 0, C::frag_order(0), a_nxt, b_nxt);
-              if (slot + 1 < kFrags) load_frag(kt_next, 0, C::frag_order(slot + 1), a_nxt, b_nxt);
-            } else if (slot < kFrags) {
-              load_frag(kt, ks + 1, C::frag_order(slot), a_nxt, b_nxt);
-            }
-#pragma unroll
-            for (int d = 0; d < C::kDmaPerStep; ++d)
-              if (slot == (d * nslots) / C::kDmaPerStep)
-                issue_list(last ? kt : kt - 1, pos * C::kDmaPerStep + d);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-#pragma unroll
-          for (int i = 0; i < C::kTM; ++i) a_cur[i] = a_nxt[i];
-#pragma unroll
-          for (int j = 0; j < C::kTN; ++j) b_cur[j] = b_nxt[j];
-        }
-      }
     } else {
     // ---- prologue: P tiles in flight, wait for tile 0 ------------------------------------------
 #pragma unroll
@@ -784,107 +781,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     //   16-row MFMA blocks: acc[g/2][2*ib + g%2][0 ...], row 32*ib + 16*(g%2) + lrow,   column 16*(g/2) + 4*lgrp
     constexpr int kRowBlocks = C::kWaveM / 32, kGroups = C::kWaveN / 8;
     constexpr bool kWide = E::kRows == 32;
-    // 256 accumulators live in AGPRs; they are then read one by one where they are used, instead of letting the
-    // compiler copy all of them to VGPRs at the loop exit (which spills)
-    constexpr bool kAgpr = C::kTM * C::kTN * C::kAccLen >= 256;
-#define TDIST_ACC(ib, g, e) \
-  acc[kWide ? (g) / 4 : (g) / 2][kWide ? (ib) : 2 * (ib) + (g) % 2][kWide ? 4 * ((g) % 4) + (e) : (e)]
     wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
-    if (p.sk_on && KTp < KT) {
-      // ---- split last round: this piece is not the whole K range -------------------------------
-      // The pieces of a tile form a chain along the workgroup order: a piece that does not reach the tile's last K
-      // tile waits for the next workgroup's piece and adds it; a piece that does not start at the tile's first K
-      // tile then hands its sum on through its slot; the piece that does start there runs the epilogue. (The pieces
-      // are equally long and start together, so the chain costs its length times one hand-over.)
-      constexpr int kThreads = C::kWaves * 64;
-      constexpr int kQuads = kRowBlocks * kGroups;  // float4 groups of accumulators per lane
-      // slot addresses: a uniform base per float4 group plus one 32-bit lane offset (from an opaque copy of the
-      // thread id, so that nothing of this is computed ahead and held across the K loop)
-      uint32_t sk_voff = threadIdx.x;
-      asm volatile("" : "+v"(sk_voff));
-      sk_voff *= 16u;
-      if (kb < KT) {
-        const int w = wg_pos + 1;  // the workgroup with the next piece of this tile
-        if (threadIdx.x == 0) {
-          int ok = 0;
-          // (the full limit even after an error elsewhere: this piece is being computed, not awaited from outside;
-          // if its workgroup gave it up at a chunk flag, the wait runs out and the tile is not stored)
-          for (int it = 0; it < p.spin_limit; ++it) {
-            if (__hip_atomic_load(p.sk_flags + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.sk_epoch) {
-              ok = 1;
-              break;
-            }
-            __builtin_amdgcn_s_sleep(4);
-          }
-          // this workgroup is the flag's only reader: lower it again, so that a launch replayed from a captured
-          // graph (same epoch every time) starts from lowered flags as well
-          if (ok) __hip_atomic_store(p.sk_flags + w, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if (!ok && p.status != nullptr) {
-            if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = -1 - w;
-          }
-          *s_gate = ok;
-        }
-        __syncthreads();
-        const int ok = *s_gate;
-        __syncthreads();
-        if (!ok) continue;  // (a piece further up the chain then runs out of its wait as well: the tile is not stored)
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        const TDIST_AS1 unsigned char* src = (const TDIST_AS1 unsigned char*)(p.sk_partials + (int64_t)w * (BM * BN));
-        constexpr int kLoadBatch = 16;
-#pragma unroll
-        for (int r0 = 0; r0 < kQuads; r0 += kLoadBatch) {
-          float4v t[kLoadBatch];
-#pragma unroll
-          for (int r = 0; r < kLoadBatch; ++r) t[r] = *(const TDIST_AS1 float4v*)(src + (size_t)(r0 + r) * (kThreads * 16) + sk_voff);
-#pragma unroll
-          for (int r = 0; r < kLoadBatch; ++r) {
-            const int ib = (r0 + r) / kGroups, g = (r0 + r) % kGroups;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              if constexpr (kAgpr) {
-                // in place, so that the accumulators stay where they are on both sides of this branch
-                float tmp;
-                asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_add_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
-                             : "+a"(TDIST_ACC(ib, g, e)), "=&v"(tmp)
-                             : "v"(t[r][e]));
-              } else {
-                TDIST_ACC(ib, g, e) += t[r][e];
-              }
-            }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      if (ka != 0) {
-        // hand the sum on: coherent at device scope, every store instruction a contiguous KiB
-        // The store sits in inline assembly (the cache-policy bit has no builtin), where the compiler sees neither
-        // a memory instruction nor its hazards. Hence: a vector address (a scalar base that the compiler happened
-        // to reload from a spill lane with v_readlane would need five wait states before the store), and a wait
-        // state after the store before anything may overwrite its data registers.
-        unsigned char* slot = (unsigned char*)(p.sk_partials + (int64_t)wg_pos * (BM * BN)) + sk_voff;
-#pragma unroll
-        for (int r = 0; r < kQuads; ++r) {
-          const int ib = r / kGroups, g = r % kGroups;
-          float4v t;
-          if constexpr (kAgpr) {
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[0]) : "a"(TDIST_ACC(ib, g, 0)));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[1]) : "a"(TDIST_ACC(ib, g, 1)));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[2]) : "a"(TDIST_ACC(ib, g, 2)));
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[3]) : "a"(TDIST_ACC(ib, g, 3)));
-          } else {
-            t = float4v{TDIST_ACC(ib, g, 0), TDIST_ACC(ib, g, 1), TDIST_ACC(ib, g, 2), TDIST_ACC(ib, g, 3)};
-          }
-          asm volatile("s_nop 1\n\tglobal_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(slot), "v"(t) : "memory");
-          slot += kThreads * 16;
-          asm volatile("" : "+v"(slot));  // one running address, not sixty-four precomputed ones
-          if (r % 4 == 3) __builtin_amdgcn_sched_barrier(0);
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (threadIdx.x == 0) __hip_atomic_store(p.sk_flags + wg_pos, p.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        continue;
-      }
-    }
     lds_u8 const epi = smem + wave * C::kEpiBytes;
     // The epilogue's lane-dependent addresses are the same for every tile; computed from these opaque copies they are
     // rebuilt per tile (a few dozen instructions) instead of being held in ~100 registers across the K loop.
@@ -896,6 +793,23 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     auto group_col = [&](int g) { return kWide ? 8 * g + 4 * e_lgrp : 16 * (g / 2) + 4 * e_lgrp; };
     // index of group g's row among the row scales held per MFMA row block
     auto scale_slot = [&](int ib, int g) { return kWide ? ib : 2 * ib + g % 2; };
+    // the four accumulators of group g of row block ib (fixed accumulators: read out of their registers here, one
+    // by one where they are used, so that no copy of the whole set is ever held in vector registers)
+    auto acc4 = [&](auto ib_c, auto g_c) -> float4v {
+      constexpr int ib = decltype(ib_c)::value, g = decltype(g_c)::value;
+      constexpr int j = kWide ? g / 4 : g / 2, i = kWide ? ib : 2 * ib + g % 2, e0 = kWide ? 4 * (g % 4) : 0;
+      if constexpr (kFixedAcc) {
+        constexpr int r = (j * C::kTM + i) * C::kAccLen + e0;
+        float v0, v1, v2, v3;
+        asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v0) : "n"(r));
+        asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v1) : "n"(r + 1));
+        asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v2) : "n"(r + 2));
+        asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v3) : "n"(r + 3));
+        return float4v{v0, v1, v2, v3};
+      } else {
+        return float4v{acc[j][i][e0], acc[j][i][e0 + 1], acc[j][i][e0 + 2], acc[j][i][e0 + 3]};
+      }
+    };
     // destination of this tile's rows
     unsigned char* Cbase;
     int64_t crow0;
@@ -912,45 +826,41 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     const int er = e_lane / kLanesPerRow, ec = e_lane % kLanesPerRow;
     const bool n_vec_ok = (p.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(Cbase) & 15) == 0);
 
-    // packs group g of row block ib (four columns of one row per lane; `rs` holds the row scales by scale_slot,
-    // `csg` the group's four column scales) and writes it to `where` in the staging rows
-    auto stage_group_at = [&](int ib, int g, const float* rs, const float4v csg, lds_u8 where) {
-      float v0, v1, v2, v3;
-      if constexpr (kAgpr) {
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v0) : "a"(TDIST_ACC(ib, g, 0)));
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v1) : "a"(TDIST_ACC(ib, g, 1)));
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v2) : "a"(TDIST_ACC(ib, g, 2)));
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v3) : "a"(TDIST_ACC(ib, g, 3)));
-      } else {
-        v0 = TDIST_ACC(ib, g, 0), v1 = TDIST_ACC(ib, g, 1), v2 = TDIST_ACC(ib, g, 2), v3 = TDIST_ACC(ib, g, 3);
-      }
+    // scales and packs four columns of one row (row scale rsi, column scales csg) and writes them to `where` in the
+    // staging rows
+    auto stage_vals = [&](float4v v, float rsi, const float4v csg, lds_u8 where) {
       if constexpr (kScales) {
-        const float rsi = rs[scale_slot(ib, g)];
-        v0 *= rsi * csg[0];
-        v1 *= rsi * csg[1];
-        v2 *= rsi * csg[2];
-        v3 *= rsi * csg[3];
+        v[0] *= rsi * csg[0];
+        v[1] *= rsi * csg[1];
+        v[2] *= rsi * csg[2];
+        v[3] *= rsi * csg[3];
       }
-      const int2v w = {(int)E::pack(v0, v1), (int)E::pack(v2, v3)};
+      const int2v w = {(int)E::pack(v[0], v[1]), (int)E::pack(v[2], v[3])};
       *(TDIST_AS3 int2v*)where = w;
     };
-    auto stage_group = [&](int ib, int g, const float* rs, const float4v csg) {
-      const int mrow = 32 * ib + group_row(g);
-      const int ncol = group_col(g);
-      stage_group_at(ib, g, rs, csg,
-                     epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2);
+    // staging address of this lane's group g in row block ib
+    auto stage_addr = [&](int ib, int g) -> lds_u8 {
+      const int mrow = 32 * ib + group_row(g), ncol = group_col(g);
+      return epi + mrow * C::kEpiPitch + ((((ncol >> 3) ^ (mrow & C::kEpiSwz))) << 4) + (ncol & 7) * 2;
+    };
+    // group g of row block ib (`rs` holds the row scales by scale_slot, `csg` the group's four column scales)
+    auto stage_group = [&](auto ib_c, auto g_c, const float* rs, const float4v csg) {
+      constexpr int ib = decltype(ib_c)::value, g = decltype(g_c)::value;
+      stage_vals(acc4(ib_c, g_c), kScales ? rs[scale_slot(ib, g)] : 1.f, csg, stage_addr(ib, g));
     };
     // the same for the four groups of the 32 x 32 block (ib, jb); cs4[g % 4] are their column scales
-    auto stage_block = [&](int ib, int jb, const float* rs, const float4v* cs4) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) stage_group(ib, 4 * jb + q, rs, kScales ? cs4[q] : float4v{1.f, 1.f, 1.f, 1.f});
+    auto stage_block = [&](auto ib_c, auto jb_c, const float* rs, const float4v* cs4) {
+      constexpr int jb = decltype(jb_c)::value;
+      static_for<4>([&](auto q_c) {
+        constexpr int q = decltype(q_c)::value;
+        stage_group(ib_c, std::integral_constant<int, 4 * jb + q>{}, rs, kScales ? cs4[q] : float4v{1.f, 1.f, 1.f, 1.f});
+      });
       __builtin_amdgcn_sched_barrier(0);  // keep the accumulator read-out block by block (register pressure)
     };
-    // staged rows [row0, row0 + nrows) of the wave tile → global memory, 16 bytes per lane
     // one staged 16-byte piece → global memory
-    auto store_piece = [&](int mrow, const int4v v) {
+    auto store_piece_at = [&](int mrow, int piece, const int4v v) {
       const int gm = m0 + wm * C::kWaveM + mrow;
-      const int gn = n0 + wn * C::kWaveN + ec * 8;
+      const int gn = n0 + wn * C::kWaveN + piece * 8;
       int64_t crow = crow0 + wm * C::kWaveM + mrow;
       bool row_ok = gm < p.M;
       if constexpr (kGrouped) {
@@ -969,18 +879,153 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         }
       }
     };
-    auto staged_piece = [&](int mrow) -> int4v {
-      return *(const TDIST_AS3 int4v*)(epi + mrow * C::kEpiPitch + ((ec ^ (mrow & C::kEpiSwz)) << 4));
+    auto staged_piece_at = [&](int mrow, int piece) -> int4v {
+      return *(const TDIST_AS3 int4v*)(epi + mrow * C::kEpiPitch + ((piece ^ (mrow & C::kEpiSwz)) << 4));
     };
     // staged rows [row0, row0 + nrows) of the wave tile → global memory, 16 bytes per lane
     auto store_rows = [&](int row0, int nrows) {
 #pragma unroll 4
       for (int pass = 0; pass < nrows / kRowsPerPass; ++pass) {
         const int mrow = row0 + pass * kRowsPerPass + er;
-        store_piece(mrow, staged_piece(mrow));
+        store_piece_at(mrow, ec, staged_piece_at(mrow, ec));
       }
     };
     static_assert(32 % kRowsPerPass == 0, "a 32-row block is a whole number of store passes");
+
+    if (sk_s > 1) {
+      // ---- this piece is 1/sk_s of the tile's K range: exchange through the workspace --------------------------
+      constexpr int kThreads = C::kWaves * 64;
+      constexpr int kQuads = kRowBlocks * kGroups;  // float4 groups of accumulators per lane
+      const int w0 = wg_pos - sk_j;                 // first workgroup of this tile's pieces
+      // slot addresses: a uniform base per float4 group plus one 32-bit lane offset (from an opaque copy of the
+      // thread id, so that nothing of this is computed ahead and held across the K loop)
+      uint32_t sk_voff = threadIdx.x;
+      asm volatile("" : "+v"(sk_voff));
+      sk_voff *= 16u;
+      // (1) the slot is free once the readers of this workgroup's previous partial are done with it
+      if (threadIdx.x == 0) {
+        int ok = 0;
+        for (int it = 0; it < p.spin_limit; ++it) {
+          if (__hip_atomic_load(sk_acks + wg_pos, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == sk_need) {
+            ok = 1;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
+        }
+        *s_gate = ok;
+      }
+      __syncthreads();
+      const int slot_ok = *s_gate;
+      __syncthreads();
+      sk_need += sk_s;
+      if (slot_ok) {
+        // (2) the partial, coherent at device scope, every store instruction a contiguous KiB.
+        // The store sits in inline assembly (the cache-policy bit has no builtin), where the compiler sees neither
+        // a memory instruction nor its hazards. Hence: a vector address (a scalar base that the compiler happened
+        // to reload from a spill lane with v_readlane would need five wait states before the store), and a wait
+        // state after the store before anything may overwrite its data registers.
+        unsigned char* slot = (unsigned char*)(p.sk_partials + (int64_t)wg_pos * (BM * BN)) + sk_voff;
+        static_for<kQuads>([&](auto r_c) {
+          constexpr int r = decltype(r_c)::value;
+          const float4v t = acc4(std::integral_constant<int, r / kGroups>{}, std::integral_constant<int, r % kGroups>{});
+          asm volatile("s_nop 1\n\tglobal_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(slot), "v"(t) : "memory");
+          slot += kThreads * 16;
+          asm volatile("" : "+v"(slot));  // one running address, not sixty-four precomputed ones
+          if constexpr (r % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        });
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0) __hip_atomic_store(sk_flags + wg_pos, sk_tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      // (3) all pieces of the tile: thread i waits for the flag of piece i. (The full limit even after an error
+      // elsewhere: these pieces are being computed, not awaited from outside; if a workgroup gave its piece up at a
+      // chunk flag, the wait runs out and the tile is not stored.)
+      if (threadIdx.x < 64) {
+        int ok = 1;
+        if ((int)threadIdx.x < sk_s) {
+          ok = 0;
+          for (int it = 0; it < p.spin_limit; ++it) {
+            if (__hip_atomic_load(sk_flags + w0 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == sk_tag) {
+              ok = 1;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+          }
+        }
+        const int all_ok = __ballot(ok != 0) == ~0ull;
+        if (threadIdx.x == 0) {
+          if (!(all_ok && slot_ok) && p.status != nullptr) {
+            if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = -1 - wg_pos;
+          }
+          *s_gate = all_ok && slot_ok;
+        }
+      }
+      __syncthreads();
+      const int pieces_ok = *s_gate;
+      __syncthreads();
+      if (!pieces_ok) continue;
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      // (4) this workgroup's share of the sum: float4 groups [q0, q0 + nq) of every lane, over the sk_s slots in slot
+      // order, packed into the staging rows as the plain epilogue packs them
+      const int nq = kQuads / sk_s, q0 = sk_j * nq;
+      const TDIST_AS1 unsigned char* const part0 =
+          (const TDIST_AS1 unsigned char*)(p.sk_partials + (int64_t)w0 * (BM * BN)) + sk_voff;
+      auto reduce_share = [&](auto s_c) {
+        constexpr int kS = decltype(s_c)::value;
+        constexpr int kBatch = 16 / kS < kQuads / kS ? 16 / kS : kQuads / kS;  // float4 groups per round of loads
+        for (int qb = 0; qb < nq; qb += kBatch) {
+          float4v t[kBatch][kS];
+#pragma unroll
+          for (int u = 0; u < kBatch; ++u)
+#pragma unroll
+            for (int i = 0; i < kS; ++i)
+              t[u][i] = *(const TDIST_AS1 float4v*)(part0 + (size_t)i * (BM * BN * 4) + (size_t)(q0 + qb + u) * (kThreads * 16));
+#pragma unroll
+          for (int u = 0; u < kBatch; ++u) {
+            float4v v = t[u][0];
+#pragma unroll
+            for (int i = 1; i < kS; ++i) v += t[u][i];
+            const int r = q0 + qb + u;
+            const int ib = r / kGroups, g = r % kGroups;
+            float rsi = 1.f;
+            float4v csg = {1.f, 1.f, 1.f, 1.f};
+            if constexpr (kScales) {
+              if (p.row_scale) rsi = p.row_scale[min(m0 + wm * C::kWaveM + 32 * ib + group_row(g), p.M - 1)];
+              if (p.col_scale) {
+                const int gn = n0 + wn * C::kWaveN + group_col(g);
+                for (int e = 0; e < 4; ++e) csg[e] = p.col_scale[min(gn + e, p.N - 1)];
+              }
+            }
+            stage_vals(v, rsi, csg, stage_addr(ib, g));
+          }
+        }
+      };
+      if (sk_s == 2) reduce_share(std::integral_constant<int, 2>{});
+      else if (sk_s == 4) reduce_share(std::integral_constant<int, 4>{});
+      else reduce_share(std::integral_constant<int, 8>{});
+      // the slots have been read: acknowledge to their writers
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if ((int)threadIdx.x < sk_s) __hip_atomic_fetch_add(sk_acks + w0 + threadIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // (5) the staged share → C. It is whole 32-row blocks of the wave tile, or a column range of one block:
+      // float4 groups [g0, g0 + n) of a row block are its 16-byte pieces [g0, g0 + n).
+      {
+        const int ib0 = q0 / kGroups;
+        const int n_rows = nq >= kGroups ? 32 * (nq / kGroups) : 32;
+        const int p0 = nq >= kGroups ? 0 : q0 % kGroups;
+        const int np = nq >= kGroups ? kGroups : nq;          // pieces per row: a power of two, 2 .. 16
+        const int rows_per_pass = 64 / np;
+        const int s_er = e_lane / np, s_ec = p0 + e_lane % np;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        for (int row = 0; row < n_rows; row += rows_per_pass) {
+          const int mrow = 32 * ib0 + row + s_er;
+          store_piece_at(mrow, s_ec, staged_piece_at(mrow, s_ec));
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      continue;
+    }
 
     // A tile that lies inside C with 16-byte-aligned rows. Row block by row block, software-pipelined: the staged rows
     // of block i are read back (LDS serves one wave's instructions in order, so the reads see the writes before them
@@ -1020,18 +1065,16 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         static_assert(kPasses % kReadPhases == 0 && (C::kEpiSwz + 1) <= 32, "swizzle period within a row block");
         lds_u8 wbase[kGroups], rbase[kReadPhases];
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) {
-          const int mrow = group_row(g), ncol = group_col(g);
-          wbase[g] = epi + mrow * C::kEpiPitch + (((ncol >> 3) ^ (mrow & C::kEpiSwz)) << 4) + (ncol & 7) * 2;
-        }
+        for (int g = 0; g < kGroups; ++g) wbase[g] = stage_addr(0, g);
 #pragma unroll
         for (int ph = 0; ph < kReadPhases; ++ph)
           rbase[ph] = epi + er * C::kEpiPitch + ((ec ^ ((ph * kRowsPerPass + er) & C::kEpiSwz)) << 4);
-        auto stage_fast = [&](int i, int g) {
-          stage_group_at(i, g, rs, cs[kScales ? (kWide ? g : g / 2) : 0], wbase[g] + i * 32 * C::kEpiPitch);
+        auto stage_fast = [&](auto i_c, auto g_c) {
+          constexpr int i = decltype(i_c)::value, g = decltype(g_c)::value;
+          stage_vals(acc4(i_c, g_c), kScales ? rs[scale_slot(i, g)] : 1.f, cs[kScales ? (kWide ? g : g / 2) : 0],
+                     wbase[g] + i * 32 * C::kEpiPitch);
         };
-#pragma unroll
-        for (int g = 0; g < kGroups; ++g) stage_fast(0, g);
+        static_for<kGroups>([&](auto g_c) { stage_fast(std::integral_constant<int, 0>{}, g_c); });
         __builtin_amdgcn_sched_barrier(0);
         int4v v[kPasses];
         auto read_piece = [&](int i, int u) {
@@ -1049,22 +1092,22 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         // kLag stores of a block go behind the first groups of the next one.
         constexpr int kLag = 2;
         static_assert(kPasses >= 2 * kLag, "the store of a piece follows its read by kLag reads");
-#pragma unroll
-        for (int i = 0; i + 1 < kRowBlocks; ++i) {
+        static_for<kRowBlocks - 1>([&](auto i_c) {
+          constexpr int i = decltype(i_c)::value;
           __builtin_amdgcn_wave_barrier();
-#pragma unroll
-          for (int g = 0; g < kGroups; ++g) {
-            stage_fast(i + 1, g);
-            if (g % 2 == 0) {
+          static_for<kGroups>([&](auto g_c) {
+            constexpr int g = decltype(g_c)::value;
+            stage_fast(std::integral_constant<int, i + 1>{}, g_c);
+            if constexpr (g % 2 == 0) {
               read_piece(i, g / 2);
             } else {
-              const int u = (g - 1) / 2 - kLag;
-              if (u >= 0) store_fast(i, u);
-              else if (i > 0) store_fast(i - 1, u + kPasses);
+              constexpr int u = (g - 1) / 2 - kLag;
+              if constexpr (u >= 0) store_fast(i, u);
+              else if constexpr (i > 0) store_fast(i - 1, u + kPasses);
             }
             __builtin_amdgcn_sched_barrier(0);
-          }
-        }
+          });
+        });
         {
           constexpr int i = kRowBlocks - 1;  // nothing left to pack behind the last block
           __builtin_amdgcn_wave_barrier();
@@ -1082,16 +1125,15 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       }
     }
     if (stored) {
-    } else if constexpr (!kScales && kAgpr) {
+    } else if constexpr (!kScales && kFixedAcc) {
       // row block by row block: the stores of block i drain while block i+1 is being packed
-#pragma unroll
-      for (int i = 0; i < kRowBlocks; ++i) {
-#pragma unroll
-        for (int j = 0; j < kGroups / 4; ++j) stage_block(i, j, nullptr, nullptr);
+      static_for<kRowBlocks>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        static_for<kGroups / 4>([&](auto j_c) { stage_block(i_c, j_c, nullptr, nullptr); });
         __builtin_amdgcn_wave_barrier();
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         store_rows(32 * i, 32);
-      }
+      });
     } else {
       float rs[C::kTM];
 #pragma unroll
@@ -1099,8 +1141,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         rs[i] = 1.f;
         if (kScales && p.row_scale) rs[i] = p.row_scale[min(m0 + wm * C::kWaveM + E::kRows * i + e_lrow, p.M - 1)];
       }
-#pragma unroll
-      for (int j = 0; j < kGroups / 4; ++j) {
+      static_for<kGroups / 4>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
         // the four column scales of each of this lane's four column groups in this 32-column block
         float4v cs[4];
 #pragma unroll
@@ -1113,9 +1155,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
               for (int e = 0; e < 4; ++e) cs[q][e] = p.col_scale[min(gn + e, p.N - 1)];
           }
         }
-#pragma unroll
-        for (int i = 0; i < kRowBlocks; ++i) stage_block(i, j, rs, cs);
-      }
+        static_for<kRowBlocks>([&](auto i_c) { stage_block(i_c, j_c, rs, cs); });
+      });
       __builtin_amdgcn_wave_barrier();
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       store_rows(0, C::kWaveM);
@@ -1123,7 +1164,22 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // the next tile's prologue overwrites the ring: every wave must be done reading its staging area
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   }
-#undef TDIST_ACC
+  // ---- leave: the last workgroup out advances the workspace's tag base for the next launch -------------------
+  if (p.sk_mode != 0 && threadIdx.x == 0) {
+    int32_t* const done = p.sk_ctrl + kSkCtrlDone;
+    if (__hip_atomic_fetch_add(done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == G - 1) {
+      __hip_atomic_store(done, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      int next = tag_base + kSkTagStride;
+      if (next > 0x3fff0000) {
+        // tags start over: no word may still hold a value that a tag will take again
+        next = 0;
+        for (int i = 0; i < kSkMaxWorkgroups; ++i) __hip_atomic_store(sk_flags + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int i = 0; i < kSkMaxDecisions; ++i)
+          __hip_atomic_store(p.sk_ctrl + kSkDecOff + i * kSkDecWords, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __hip_atomic_store(p.sk_ctrl + kSkCtrlEpoch, next, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
 }
 
 // ---- host side ------------------------------------------------------------------------------------
@@ -1149,6 +1205,8 @@ struct GemmCall {
   int rank, world_size, spin_limit;
   int32_t* status;
   int max_workgroups;
+  void* sk_workspace;
+  int64_t sk_workspace_bytes;
   hipStream_t stream;
   const char* who;
 };
@@ -1167,25 +1225,10 @@ static int launch_gemm_cfg(const GemmParams& prm, int grid, hipStream_t stream, 
   return launch_status(who);
 }
 
-// ---- split-K workspace (one per device, handed in by the caller) -------------------------------------------
-// [0, kSkFlagBytes): one flag word per workgroup; then one fp32 tile per workgroup. A launch that uses it gets a
-// fresh epoch: its flags count as raised when they hold that value, so nothing is cleared between launches.
-constexpr int64_t kSkFlagBytes = 4096;
-constexpr int kSkMaxDevices = 64;
-struct SkWorkspace {
-  unsigned char* base = nullptr;
-  int64_t bytes = 0;
-  int epoch = 0;
-};
-static SkWorkspace g_sk[kSkMaxDevices];
-static std::mutex g_sk_mutex;
-
-// The 16-bit 256-row tiles run on the 16x16x32 MFMA; TDIST_GEMM_MFMA16=0 puts them back on 32x32x16 (measurement
-// aid: the two give the same bits, at different power)
-static bool narrow_mfma_env() {
-  if (const char* v = getenv("TDIST_GEMM_MFMA16")) return atoi(v) != 0;
-  return true;
-}
+// ---- split-K workspace (the caller's, per call) ------------------------------------------------------------
+// [0, kSkHeaderBytes): control words, one flag and one acknowledgement word per workgroup, the scheduler's decision
+// records; then one fp32 tile per workgroup. The memory must be zero when it is first used; the kernels keep it
+// consistent from then on (tags, never cleared flags).
 
 // 0 = off, 1 = on wherever the workspace allows, -1 = by the cost estimate
 static int sk_env() {
@@ -1193,25 +1236,28 @@ static int sk_env() {
   return -1;
 }
 
-static bool sk_workspace_fits(int workgroups, int bm, int bn) {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSkMaxDevices) return false;
-  std::lock_guard<std::mutex> lock(g_sk_mutex);
-  const SkWorkspace& w = g_sk[dev];
-  return w.base != nullptr && workgroups * 4 <= kSkFlagBytes && w.bytes >= kSkFlagBytes + (int64_t)workgroups * bm * bn * 4;
+static bool sk_workspace_fits(const void* ws, int64_t bytes, int workgroups, int bm, int bn) {
+  return ws != nullptr && workgroups <= kSkMaxWorkgroups && bytes >= kSkHeaderBytes + (int64_t)workgroups * bm * bn * 4;
 }
 
-static void sk_attach(GemmParams& p) {
-  int dev = 0;
-  (void)hipGetDevice(&dev);
-  std::lock_guard<std::mutex> lock(g_sk_mutex);
-  SkWorkspace& w = g_sk[dev];
-  w.epoch = w.epoch == 0x7fffffff ? 1 : w.epoch + 1;
-  p.sk_on = 1;
-  p.sk_epoch = w.epoch;
-  p.sk_flags = (int32_t*)w.base;
-  p.sk_partials = (float*)(w.base + kSkFlagBytes);
+// a workspace that is handed in must be usable at least for the smallest tile
+static int sk_workspace_check(const void* ws, int64_t bytes, const char* who) {
+  if (ws == nullptr) return TDIST_OK;
+  if ((reinterpret_cast<uintptr_t>(ws) & 255u) != 0 || bytes < kSkHeaderBytes + 128 * 128 * 4)
+    return fail(TDIST_ERR_WORKSPACE, "%s: sk_workspace of %lld bytes at %p (256-byte aligned, at least %lld bytes; see "
+                "tdist_gemm_split_k_workspace_bytes)", who, (long long)bytes, ws, (long long)(kSkHeaderBytes + 128 * 128 * 4));
+  return TDIST_OK;
 }
+
+static void sk_attach(GemmParams& p, void* ws, int mode) {
+  p.sk_ctrl = (int32_t*)ws;
+  p.sk_partials = (float*)((unsigned char*)ws + kSkHeaderBytes);
+  p.sk_mode = mode;
+}
+
+// cost of handing a tile's pieces through the workspace, in K tiles of that tile's work (one compute unit writes the
+// tile's fp32 accumulators and reads as much back)
+static double sk_handover_k_tiles(int bm, int bn) { return 2.0 + 6.0 * bm * bn / 65536.0; }
 
 static int run_gemm(const GemmCall& c, GemmElem elem) {
   const char* who = c.who;
@@ -1226,6 +1272,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (c.lda < c.K || c.ldb < c.K || c.ldc < c.N) return fail(TDIST_ERR_INVALID, "%s: leading dimension smaller than row", who);
   if (c.lda * esz > (1 << 22) || c.ldb * esz > (1 << 22) || (c.A_local && c.lda_local * esz > (1 << 22)))
     return fail(TDIST_ERR_UNSUPPORTED, "%s: row strides above 4 MiB are not supported", who);
+  if (int rc = sk_workspace_check(c.sk_workspace, c.sk_workspace_bytes, who)) return rc;
   const DeviceInfo& di = device_info();
   if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "%s: current device is not gfx950", who);
 
@@ -1242,9 +1289,9 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (c.max_workgroups > 0 && c.max_workgroups < cap_wgs) cap_wgs = c.max_workgroups;
   struct TileChoice { int bm, bn; double eff; };
   static const TileChoice kChoices[3] = {{256, 256, 1.0}, {256, 128, 0.9}, {128, 128, 0.6}};
-  // With a workspace registered, a last round that fills at most half of the grid is split along K (see GemmParams):
-  // it then costs 1/s of a round plus s-1 hand-overs of a tile's accumulators (priced at 2 + 2 * tile/64Ki K tiles
-  // of work each), and that form is taken where it beats whole tiles by a margin.
+  // With a workspace, a last round that fills at most half of the grid is split along K (see GemmParams): it then
+  // costs 1/s of a round plus one exchange of the tile's accumulators, and that form is taken where it beats whole
+  // tiles by a margin.
   const int sk_mode = sk_env();
   int pick = 2;
   bool use_sk = false;
@@ -1258,16 +1305,14 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
     const double cost = (double)ceil_div(tiles, cap_wgs) * kt * per_k_tile;
     if (best == 0 || cost < best) best = cost, pick = t, use_sk = false;
     const int64_t tail = tiles % cap_wgs;
-    int64_t split = tail > 0 ? cap_wgs / tail : 1;
-    if (split > kSkMaxSplit) split = kSkMaxSplit;
-    if (split > kt / kSkMinPiece) split = kt / kSkMinPiece;
-    if (sk_mode != 0 && split >= 2 && sk_workspace_fits(cap_wgs, bm, bn)) {
-      const double cost_sk = ((double)(tiles / cap_wgs) * kt + (double)kt / split + (split - 1) * (2.0 + 2.0 * bm * bn / 65536.0)) * per_k_tile;
+    const int split = tail > 0 ? sk_split_for(cap_wgs, (int)tail, (int)(kt < 0x7fffffff ? kt : 0x7fffffff)) : 1;
+    if (sk_mode != 0 && split >= 2 && sk_workspace_fits(c.sk_workspace, c.sk_workspace_bytes, cap_wgs, bm, bn)) {
+      const double cost_sk = ((double)(tiles / cap_wgs) * kt + (double)kt / split + sk_handover_k_tiles(bm, bn)) * per_k_tile;
       if (cost_sk < 0.95 * best || (sk_mode == 1 && (!use_sk || cost_sk < best))) best = cost_sk, pick = t, use_sk = true;
     }
   }
-  // TDIST_GEMM_TILE forces a tile (measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128; a 256-row tile that the
-  // call's row blocks do not admit is not taken.
+  // TDIST_GEMM_TILE forces a tile (test and measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128; a 256-row tile
+  // that the call's row blocks do not admit is not taken.
   if (const char* v = getenv("TDIST_GEMM_TILE")) {
     const int t = atoi(v);
     if (t >= 0 && t < 3 && (kChoices[t].bm != 256 || rows256)) {
@@ -1276,19 +1321,12 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       const int64_t tiles = ceil_div(c.M, kChoices[t].bm) * ceil_div(c.N, kChoices[t].bn);
       const int64_t kt = (int64_t)c.K * esz / (kChoices[t].bm == 256 ? 128 : 64);
       const int64_t tail = tiles % cap_wgs;
-      use_sk = sk_mode != 0 && use_sk && tail > 0 && cap_wgs / tail >= 2 && kt / kSkMinPiece >= 2 &&
-               sk_workspace_fits(cap_wgs, kChoices[t].bm, kChoices[t].bn);
+      use_sk = sk_mode != 0 && use_sk && tail > 0 && sk_split_for(cap_wgs, (int)tail, (int)kt) >= 2 &&
+               sk_workspace_fits(c.sk_workspace, c.sk_workspace_bytes, cap_wgs, kChoices[t].bm, kChoices[t].bn);
     }
   }
-  // TDIST_GEMM_VARIANT picks another compiled schedule of the 256x256 tile (measurement aid): 2 = 2x4 waves on a
-  // two-stage ring, 5 = 2x4 waves on the split ring. The default is 2x2 waves of 128x128 on the split ring
-  // (3 A stages + 2 B stages).
-  int variant = 6;
-  if (const char* v = getenv("TDIST_GEMM_VARIANT")) variant = atoi(v);
   const int BM = kChoices[pick].bm;
   const int BN = kChoices[pick].bn;
-  const bool big = pick == 0;
-  const bool narrow_mfma = narrow_mfma_env();
 
   GemmParams p;
   p.A = (const unsigned char*)c.A;
@@ -1320,9 +1358,9 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   p.sorted_ids = p.block_expert = p.block_segment = p.post_pad = nullptr;
   p.b_expert_stride_b = 0;
   p.num_valid = p.topk = p.first_block = p.a_rows = 0;
+  p.sk_ctrl = nullptr;
   p.sk_partials = nullptr;
-  p.sk_flags = nullptr;
-  p.sk_on = p.sk_epoch = 0;
+  p.sk_mode = 0;
 
   if (c.scatter_bufs) {
     if (c.world_size <= 0 || c.rank < 0 || c.rank >= c.world_size)
@@ -1365,43 +1403,30 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   int grid = (int)(sched < cap_wgs ? sched : cap_wgs);
   if (use_sk) {
     grid = cap_wgs;
-    sk_attach(p);
+    sk_attach(p, c.sk_workspace, 1);
   }
   const bool scales = elem == kElemFP8 && (c.row_scale || c.col_scale);
 
-  if (big) {
-#define TDIST_BIG(BN_, KB_, WM_, WN_, NST_)                                                                          \
-  switch (elem) {                                                                                                    \
-    case kElemBF16: return launch_gemm_cfg<ElemBF16, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);  \
-    case kElemF16: return launch_gemm_cfg<ElemF16, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);    \
-    default:                                                                                                         \
-      return scales ? launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, true>(p, grid, c.stream, who)          \
-                    : launch_gemm_cfg<ElemFP8, 256, BN_, KB_, WM_, WN_, NST_, false>(p, grid, c.stream, who);        \
-  }
-    if (narrow_mfma && variant == 6 && elem == kElemFP8) {
-      return scales ? launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, true>(p, grid, c.stream, who)
-                    : launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
-    }
-    if (narrow_mfma && variant == 6 && elem != kElemFP8) {
-      if (elem == kElemBF16) return launch_gemm_cfg<ElemBF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
-      return launch_gemm_cfg<ElemF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
-    }
-    switch (variant) {
-      case 2: TDIST_BIG(256, 128, 2, 4, 2)
-      case 5: TDIST_BIG(256, 128, 2, 4, 5)
-      default: TDIST_BIG(256, 128, 2, 2, 5)
+  // 256-row tiles: 2 x 2 waves on the split ring (3 A stages + 2 B stages), 16-row MFMA blocks
+  if (BM == 256 && BN == 256) {
+    switch (elem) {
+      case kElemBF16: return launch_gemm_cfg<ElemBF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      case kElemF16: return launch_gemm_cfg<ElemF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      default:
+        return scales ? launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, true>(p, grid, c.stream, who)
+                      : launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
     }
   }
-  if (pick == 1 && narrow_mfma && elem == kElemFP8) {
-    return scales ? launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, true>(p, grid, c.stream, who)
-                  : launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+  if (BM == 256) {
+    switch (elem) {
+      case kElemBF16: return launch_gemm_cfg<ElemBF16N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      case kElemF16: return launch_gemm_cfg<ElemF16N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      default:
+        return scales ? launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, true>(p, grid, c.stream, who)
+                      : launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+    }
   }
-  if (pick == 1 && narrow_mfma && elem != kElemFP8) {
-    if (elem == kElemBF16) return launch_gemm_cfg<ElemBF16N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
-    return launch_gemm_cfg<ElemF16N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
-  }
-  if (pick == 1) { TDIST_BIG(128, 128, 2, 2, 5) }
-#undef TDIST_BIG
+  // the 128 x 128 tile on a four-stage ring of 64-byte K tiles, 32-row MFMA blocks: every shape
   switch (elem) {
     case kElemBF16: return launch_gemm_cfg<ElemBF16, 128, 128, 64, 2, 2, 4, false>(p, grid, c.stream, who);
     case kElemF16: return launch_gemm_cfg<ElemF16, 128, 128, 64, 2, 2, 4, false>(p, grid, c.stream, who);
@@ -1428,6 +1453,8 @@ struct GroupGemmCall {
   int wait_value, rank, spin_limit;
   int32_t* status;
   int max_workgroups;
+  void* sk_workspace;
+  int64_t sk_workspace_bytes;
   hipStream_t stream;
   const char* who;
 };
@@ -1455,6 +1482,7 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   if ((int64_t)c.num_blocks * c.block_size > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many rows", who);
   if (c.first_block < 0 || c.first_block >= c.num_blocks) return fail(TDIST_ERR_INVALID, "%s: first_block %d", who, c.first_block);
   if (c.A_local && (c.rank < 0 || c.local_rows <= 0)) return fail(TDIST_ERR_INVALID, "%s: local shard without rank / rows", who);
+  if (int rc = sk_workspace_check(c.sk_workspace, c.sk_workspace_bytes, who)) return rc;
   const DeviceInfo& di = device_info();
   if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "%s: current device is not gfx950", who);
 
@@ -1496,9 +1524,9 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   p.topk = c.topk;
   p.first_block = c.first_block;
   p.a_rows = c.a_rows;
+  p.sk_ctrl = nullptr;
   p.sk_partials = nullptr;
-  p.sk_flags = nullptr;
-  p.sk_on = p.sk_epoch = 0;
+  p.sk_mode = 0;
 
   const bool k128 = ((int64_t)c.K * esz) % 128 == 0;
   const int BN = (c.block_size == 256 || k128) ? 256 : 128;
@@ -1512,39 +1540,26 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   {
     const int bm = c.block_size == 256 ? 256 : 128;
     const int64_t kt = (int64_t)c.K * esz / (c.block_size == 256 || k128 ? 128 : 64);
-    if (sk_env() != 0 && kt >= 2 * kSkMinPiece && sk_workspace_fits(cap_wgs, bm, BN)) {
+    if (sk_env() != 0 && kt >= 2 * kSkMinPiece && sk_workspace_fits(c.sk_workspace, c.sk_workspace_bytes, cap_wgs, bm, BN)) {
       grid = cap_wgs;
-      sk_attach(p);
+      sk_attach(p, c.sk_workspace, 1);
     }
   }
-  const bool narrow_mfma = narrow_mfma_env();
-#define TDIST_GROUPED_NARROW(BM_, BN_, KB_, NST_)                                                                         \
-  if (narrow_mfma && elem == kElemBF16)                                                                                   \
-    return launch_gemm_cfg<ElemBF16N, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);                    \
-  if (narrow_mfma && elem == kElemF16)                                                                                    \
-    return launch_gemm_cfg<ElemF16N, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);
-#define TDIST_GROUPED(BM_, BN_, KB_, NST_)                                                                            \
-  switch (elem) {                                                                                                    \
-    case kElemBF16: return launch_gemm_cfg<ElemBF16, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who); \
-    case kElemF16: return launch_gemm_cfg<ElemF16, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);   \
-    default: return launch_gemm_cfg<ElemFP8, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);         \
+#define TDIST_GROUPED(EB, EH, E8, BM_, BN_, KB_, NST_)                                                          \
+  switch (elem) {                                                                                               \
+    case kElemBF16: return launch_gemm_cfg<EB, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who); \
+    case kElemF16: return launch_gemm_cfg<EH, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);  \
+    default: return launch_gemm_cfg<E8, BM_, BN_, KB_, 2, 2, NST_, false, true>(p, grid, c.stream, who);        \
   }
   if (c.block_size == 256) {
     if (!k128) return fail(TDIST_ERR_UNSUPPORTED, "%s: 256-row blocks need K*elem_size to be a multiple of 128 bytes", who);
-    TDIST_GROUPED_NARROW(256, 256, 128, 5)
-    if (narrow_mfma && elem == kElemFP8)
-      return launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, false, true>(p, grid, c.stream, who);
-    TDIST_GROUPED(256, 256, 128, 5)
+    TDIST_GROUPED(ElemBF16N, ElemF16N, ElemFP8N, 256, 256, 128, 5)
   }
   if (k128) {  // 64 x 128 per wave on the split ring
-    TDIST_GROUPED_NARROW(128, 256, 128, 5)
-    if (narrow_mfma && elem == kElemFP8)
-      return launch_gemm_cfg<ElemFP8N, 128, 256, 128, 2, 2, 5, false, true>(p, grid, c.stream, who);
-    TDIST_GROUPED(128, 256, 128, 5)
+    TDIST_GROUPED(ElemBF16N, ElemF16N, ElemFP8N, 128, 256, 128, 5)
   }
-  TDIST_GROUPED(128, 128, 64, 4)
+  TDIST_GROUPED(ElemBF16, ElemF16, ElemFP8, 128, 128, 64, 4)
 #undef TDIST_GROUPED
-#undef TDIST_GROUPED_NARROW
 }
 
 }  // namespace tdist
@@ -1558,7 +1573,8 @@ using namespace tdist;
   c.B = B; c.ldb = ldb; c.C = C; c.scatter_bufs = nullptr; c.ldc = ldc; c.M = M; c.N = N; c.K = K;                  \
   c.row_scale = RS; c.col_scale = CS; c.flags = flags; c.m_per_chunk = m_per_chunk; c.wait_value = wait_value;      \
   c.chunk_order = chunk_order; c.rank = rank; c.world_size = world_size; c.spin_limit = spin_limit;                 \
-  c.status = status; c.max_workgroups = max_workgroups; c.stream = (hipStream_t)stream; c.who = WHO;                                                   \
+  c.status = status; c.max_workgroups = max_workgroups; c.sk_workspace = sk_workspace;                              \
+  c.sk_workspace_bytes = sk_workspace_bytes; c.stream = (hipStream_t)stream; c.who = WHO;                           \
   return run_gemm(c, ELEM);
 
 extern "C" {
@@ -1566,41 +1582,22 @@ extern "C" {
 int64_t tdist_gemm_split_k_workspace_bytes(void) {
   const tdist::DeviceInfo& di = tdist::device_info();
   if (di.ok != 1) return 0;
-  return tdist::kSkFlagBytes + (int64_t)di.num_cus * 256 * 256 * 4;
-}
-
-int tdist_gemm_split_k_set_workspace(void* workspace, int64_t bytes, void* stream) {
-  using namespace tdist;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSkMaxDevices)
-    return fail(TDIST_ERR_DEVICE, "tdist_gemm_split_k_set_workspace: no current device");
-  if (workspace != nullptr) {
-    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || bytes < kSkFlagBytes + 128 * 128 * 4)
-      return fail(TDIST_ERR_WORKSPACE, "tdist_gemm_split_k_set_workspace: %lld bytes at %p (256-byte aligned, see "
-                  "tdist_gemm_split_k_workspace_bytes)", (long long)bytes, workspace);
-    // flags start below every epoch
-    if (hipMemsetAsync(workspace, 0, kSkFlagBytes, (hipStream_t)stream) != hipSuccess)
-      return fail(TDIST_ERR_LAUNCH, "tdist_gemm_split_k_set_workspace: clearing the flags failed");
-  }
-  std::lock_guard<std::mutex> lock(g_sk_mutex);
-  g_sk[dev].base = (unsigned char*)workspace;
-  g_sk[dev].bytes = workspace ? bytes : 0;
-  g_sk[dev].epoch = 0;
-  return TDIST_OK;
+  return tdist::kSkHeaderBytes + (int64_t)di.num_cus * 256 * 256 * 4;
 }
 
 int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                 int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C, int64_t ldc,
                                 int M, int N, int K, const int32_t* flags, int m_per_chunk, int wait_value,
                                 const int32_t* chunk_order, int rank, int world_size, int spin_limit, int32_t* status,
-                                int max_workgroups, void* stream) {
+                                int max_workgroups, void* sk_workspace, int64_t sk_workspace_bytes, void* stream) {
   TDIST_GATED_BODY(kElemBF16, nullptr, nullptr, "tdist_gemm_chunk_gated_bf16")
 }
 
 int tdist_gemm_chunk_gated_f16(const void* A, int64_t lda, const void* A_local, int64_t lda_local, int local_row_begin,
                                int local_rows, const void* B, int64_t ldb, void* C, int64_t ldc, int M, int N, int K,
                                const int32_t* flags, int m_per_chunk, int wait_value, const int32_t* chunk_order,
-                               int rank, int world_size, int spin_limit, int32_t* status, int max_workgroups, void* stream) {
+                               int rank, int world_size, int spin_limit, int32_t* status, int max_workgroups,
+                               void* sk_workspace, int64_t sk_workspace_bytes, void* stream) {
   TDIST_GATED_BODY(kElemF16, nullptr, nullptr, "tdist_gemm_chunk_gated_f16")
 }
 
@@ -1609,34 +1606,36 @@ int tdist_gemm_chunk_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
                                    int64_t ldc, int M, int N, int K, const float* row_scale, const float* col_scale,
                                    const int32_t* flags, int m_per_chunk, int wait_value, const int32_t* chunk_order,
                                    int rank, int world_size, int spin_limit, int32_t* status, int max_workgroups,
-                                   void* stream) {
+                                   void* sk_workspace, int64_t sk_workspace_bytes, void* stream) {
   TDIST_GATED_BODY(kElemFP8, row_scale, col_scale, "tdist_gemm_chunk_gated_fp8e4m3")
 }
 
 static int gemm_rs_scatter(GemmElem elem, const void* A, int64_t lda, const void* B, int64_t ldb,
                            void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank, int world_size,
-                           void* stream, const char* who) {
+                           void* sk_workspace, int64_t sk_workspace_bytes, void* stream, const char* who) {
   if (!scatter_bufs) return fail(TDIST_ERR_INVALID, "%s: null scatter_bufs", who);
   GemmCall c;
   c.A = A; c.lda = lda; c.A_local = nullptr; c.lda_local = 0; c.local_row_begin = 0; c.local_rows = 0;
   c.B = B; c.ldb = ldb; c.C = nullptr; c.scatter_bufs = scatter_bufs; c.ldc = ldc; c.M = M; c.N = N; c.K = K;
   c.row_scale = nullptr; c.col_scale = nullptr; c.flags = nullptr; c.m_per_chunk = 0; c.wait_value = 0;
   c.chunk_order = nullptr; c.rank = rank; c.world_size = world_size; c.spin_limit = 0; c.status = nullptr;
-  c.max_workgroups = 0;
+  c.max_workgroups = 0; c.sk_workspace = sk_workspace; c.sk_workspace_bytes = sk_workspace_bytes;
   c.stream = (hipStream_t)stream; c.who = who;
   return run_gemm(c, elem);
 }
 
 int tdist_gemm_rs_scatter_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, void* const* scatter_bufs,
-                               int64_t ldc, int M, int N, int K, int rank, int world_size, void* stream) {
-  return gemm_rs_scatter(kElemBF16, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, stream,
-                         "tdist_gemm_rs_scatter_bf16");
+                               int64_t ldc, int M, int N, int K, int rank, int world_size, void* sk_workspace,
+                               int64_t sk_workspace_bytes, void* stream) {
+  return gemm_rs_scatter(kElemBF16, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, sk_workspace,
+                         sk_workspace_bytes, stream, "tdist_gemm_rs_scatter_bf16");
 }
 
 int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t ldb, void* const* scatter_bufs,
-                              int64_t ldc, int M, int N, int K, int rank, int world_size, void* stream) {
-  return gemm_rs_scatter(kElemF16, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, stream,
-                         "tdist_gemm_rs_scatter_f16");
+                              int64_t ldc, int M, int N, int K, int rank, int world_size, void* sk_workspace,
+                              int64_t sk_workspace_bytes, void* stream) {
+  return gemm_rs_scatter(kElemF16, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, sk_workspace,
+                         sk_workspace_bytes, stream, "tdist_gemm_rs_scatter_f16");
 }
 
 #define TDIST_GROUP_GEMM_BODY(ELEM, WHO)                                                                              \
@@ -1647,7 +1646,8 @@ int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t
   c.block_segment = block_barrier_ids; c.post_pad = num_tokens_post_padded; c.num_blocks = num_blocks;                \
   c.block_size = block_size; c.num_valid = num_valid_tokens; c.topk = topk; c.tokens_per_rank = tokens_per_rank;      \
   c.first_block = first_block; c.flags = flags; c.wait_value = wait_value; c.rank = rank; c.spin_limit = spin_limit;  \
-  c.status = status; c.max_workgroups = max_workgroups; c.stream = (hipStream_t)stream; c.who = WHO;                  \
+  c.status = status; c.max_workgroups = max_workgroups; c.sk_workspace = sk_workspace;                                \
+  c.sk_workspace_bytes = sk_workspace_bytes; c.stream = (hipStream_t)stream; c.who = WHO;                             \
   return run_group_gemm(c, ELEM);
 
 #define TDIST_GROUP_GEMM_ARGS                                                                                         \
@@ -1656,7 +1656,7 @@ int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t
       const int32_t *sorted_token_ids, const int32_t *expert_ids, const int32_t *block_barrier_ids,                   \
       const int32_t *num_tokens_post_padded, int num_blocks, int block_size, int num_valid_tokens, int topk,          \
       int tokens_per_rank, int first_block, const int32_t *flags, int wait_value, int rank, int spin_limit,           \
-      int32_t *status, int max_workgroups, void *stream
+      int32_t *status, int max_workgroups, void *sk_workspace, int64_t sk_workspace_bytes, void *stream
 
 int tdist_group_gemm_gated_bf16(TDIST_GROUP_GEMM_ARGS) { TDIST_GROUP_GEMM_BODY(kElemBF16, "tdist_group_gemm_gated_bf16") }
 int tdist_group_gemm_gated_f16(TDIST_GROUP_GEMM_ARGS) { TDIST_GROUP_GEMM_BODY(kElemF16, "tdist_group_gemm_gated_f16") }

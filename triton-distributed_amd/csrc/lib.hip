@@ -101,7 +101,7 @@ struct PushParams {
   int world, rank, chunks_per_rank, flag_value;
 };
 
-__global__ __launch_bounds__(256) void producer_push_kernel(const PushParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(24))) void producer_push_kernel(const PushParams p) {
   const int r = (p.rank + 1 + (int)blockIdx.y) % p.world;
   const unsigned char* src = p.peer_src[r];
   unsigned char* dst = p.workspace + (long long)r * p.rank_bytes;
@@ -124,7 +124,8 @@ __global__ __launch_bounds__(256) void producer_push_kernel(const PushParams p) 
       }
       __syncthreads();
     }
-    // Four loads in flight per lane: more would cost the registers that let these waves sit beside a GEMM wave.
+    // Two loads in flight per lane: more would cost the registers that let these waves sit beside a GEMM wave
+    // (the kernel is held to 24 registers per lane; the GEMM's wave takes up to 488 of the SIMD's 512).
     // Addresses are a wave-uniform chunk base plus a 32-bit byte offset (chunks are below 4 GiB): one register
     // per lane instead of a 64-bit pointer per load.
     const unsigned char* const sbase = (const unsigned char*)src + (long long)c * p.chunk_bytes;
@@ -134,15 +135,11 @@ __global__ __launch_bounds__(256) void producer_push_kernel(const PushParams p) 
     auto put = [&](uint32_t off, const int4v v) { __builtin_nontemporal_store(v, (int4v*)(dbase + off)); };
     uint32_t off = (blockIdx.x * 256u + threadIdx.x) * 16u;
     // (the host keeps chunk_bytes + 4 * stride below 2^32, so the offsets cannot wrap)
-    for (; off + 3 * stride < nbytes; off += 4 * stride) {
+    for (; off + stride < nbytes; off += 2 * stride) {
       const int4v v0 = __builtin_nontemporal_load((const int4v*)(sbase + off));
       const int4v v1 = __builtin_nontemporal_load((const int4v*)(sbase + off + stride));
-      const int4v v2 = __builtin_nontemporal_load((const int4v*)(sbase + off + 2 * stride));
-      const int4v v3 = __builtin_nontemporal_load((const int4v*)(sbase + off + 3 * stride));
       put(off, v0);
       put(off + stride, v1);
-      put(off + 2 * stride, v2);
-      put(off + 3 * stride, v3);
     }
     for (; off < nbytes; off += stride) put(off, __builtin_nontemporal_load((const int4v*)(sbase + off)));
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -159,86 +156,6 @@ __global__ __launch_bounds__(256) void producer_push_kernel(const PushParams p) 
       }
     }
   }
-}
-
-__global__ __launch_bounds__(256) void copy_bytes_kernel(int4v* __restrict__ dst, const int4v* __restrict__ src,
-                                                         int64_t n16) {
-  int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    int64_t j = i + u * 256;
-    if (j < n16) __builtin_nontemporal_store(__builtin_nontemporal_load(src + j), dst + j);
-  }
-}
-
-// MFMA-only loop for the rate yardstick: the K loop of a 128 x 128 wave tile with no memory traffic at all. 256
-// accumulators, eight A and eight B operand fragments in registers, and the GEMM kernel's order of use: a B fragment
-// serves a row of MFMAs against every A fragment in turn. kRandom fills the fragments with hashed bit patterns (random
-// sign, mantissa and low exponent bits), else with 1.0. kRows = 32: 4 x 4 blocks of 32x32x16 (bf16) / 32x32x64 (e4m3);
-// kRows = 16: 8 x 8 blocks of 16x16x32 / 16x16x128, i.e. twice the K per round.
-__device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
-  x ^= x >> 16;
-  x *= 0x7feb352dU;
-  x ^= x >> 15;
-  x *= 0x846ca68bU;
-  x ^= x >> 16;
-  return x;
-}
-
-template <bool kFp8, bool kRandom, int kRows>
-__global__ __launch_bounds__(256, 1) void mfma_rate_kernel(float* __restrict__ sink, int iters) {
-  typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
-  typedef int int8v_ __attribute__((ext_vector_type(8)));
-  constexpr int kT = 128 / kRows;            // blocks per side of the wave tile
-  constexpr int kAcc = kRows * kRows / 64;   // accumulators per lane and block
-  typedef float acc_t __attribute__((ext_vector_type(kAcc)));
-  int8v_ a[8], b[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const uint32_t h1 = probe_hash(threadIdx.x * 131u + i * 17u + e), h2 = probe_hash(threadIdx.x * 71u + i * 29u + e + 1000u);
-      if (kFp8) {  // e4m3 bytes: random sign, exponent 4..7, random mantissa
-        a[i][e] = kRandom ? (int)((h1 & 0x9f9f9f9fu) | 0x20202020u) : 0x38383838;
-        b[i][e] = kRandom ? (int)((h2 & 0x9f9f9f9fu) | 0x20202020u) : 0x38383838;
-      } else {     // bf16 pairs: random sign, exponent 124..127, random mantissa
-        a[i][e] = kRandom ? (int)((h1 & 0x81ff81ffu) | 0x3e003e00u) : 0x3f803f80;
-        b[i][e] = kRandom ? (int)((h2 & 0x81ff81ffu) | 0x3e003e00u) : 0x3f803f80;
-      }
-    }
-  acc_t acc[kT][kT];
-#pragma unroll
-  for (int j = 0; j < kT; ++j)
-#pragma unroll
-    for (int i = 0; i < kT; ++i)
-#pragma unroll
-      for (int e = 0; e < kAcc; ++e) acc[j][i][e] = 0.f;
-  for (int it = 0; it < iters; it += 2) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u)  // (two rounds with the fragments paired differently, as two K steps would be)
-#pragma unroll
-      for (int j = 0; j < kT; ++j)
-#pragma unroll
-        for (int i = 0; i < kT; ++i) {
-          const int8v_ av = a[(i + 4 * u) & 7], bv = b[(j + 4 * u) & 7];
-          if constexpr (kFp8) {
-            if constexpr (kRows == 32) acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc[j][i], 0, 0, 0, 0, 0, 0);
-            else acc[j][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[j][i], 0, 0, 0, 0, 0, 0);
-          } else {
-            const int4v a4 = __builtin_shufflevector(av, av, 0, 1, 2, 3), b4 = __builtin_shufflevector(bv, bv, 0, 1, 2, 3);
-            if constexpr (kRows == 32)
-              acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8v, b4), __builtin_bit_cast(bf16x8v, a4), acc[j][i], 0, 0, 0);
-            else
-              acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8v, b4), __builtin_bit_cast(bf16x8v, a4), acc[j][i], 0, 0, 0);
-          }
-        }
-  }
-  float s = 0.f;
-#pragma unroll
-  for (int j = 0; j < kT; ++j)
-#pragma unroll
-    for (int i = 0; i < kT; ++i) s += acc[j][i][0];
-  sink[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
 }  // namespace tdist
@@ -350,47 +267,6 @@ int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int 
   p.flag_value = flag_value;
   hipLaunchKernelGGL(producer_push_kernel, dim3(workgroups_per_peer, world_size - 1), dim3(256), 0, (hipStream_t)stream, p);
   return launch_status(who);
-}
-
-int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
-  if (!dst || !src || nbytes < 0 || (nbytes & 15) || !aligned16(dst) || !aligned16(src))
-    return fail(TDIST_ERR_INVALID, "tdist_copy_bytes: pointers and size must be 16-byte aligned");
-  if (nbytes == 0) return TDIST_OK;
-  int64_t n16 = nbytes / 16;
-  int64_t blocks = ceil_div(n16, 1024);
-  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_copy_bytes: too large");
-  hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (int4v*)dst,
-                     (const int4v*)src, n16);
-  return launch_status("tdist_copy_bytes");
-}
-
-static int mfma_rate_probe(const char* who, bool narrow, int dtype, int random_operands, int iters, float* sink, void* stream) {
-  if (!sink || iters <= 0 || iters % 2 != 0) return fail(TDIST_ERR_INVALID, "%s: sink, iters (even)", who);
-  if (dtype != TDIST_BF16 && dtype != TDIST_F8E4M3) return fail(TDIST_ERR_UNSUPPORTED, "%s: bf16 or e4m3", who);
-  const DeviceInfo& di = device_info();
-  if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "%s: current device is not gfx950", who);
-  hipStream_t st = (hipStream_t)stream;
-  const dim3 grid(di.num_cus), block(256);
-  const int which = (narrow ? 4 : 0) + (dtype == TDIST_F8E4M3 ? 2 : 0) + (random_operands ? 1 : 0);
-  switch (which) {
-    case 0: hipLaunchKernelGGL((mfma_rate_kernel<false, false, 32>), grid, block, 0, st, sink, iters); break;
-    case 1: hipLaunchKernelGGL((mfma_rate_kernel<false, true, 32>), grid, block, 0, st, sink, iters); break;
-    case 2: hipLaunchKernelGGL((mfma_rate_kernel<true, false, 32>), grid, block, 0, st, sink, iters); break;
-    case 3: hipLaunchKernelGGL((mfma_rate_kernel<true, true, 32>), grid, block, 0, st, sink, iters); break;
-    case 4: hipLaunchKernelGGL((mfma_rate_kernel<false, false, 16>), grid, block, 0, st, sink, iters); break;
-    case 5: hipLaunchKernelGGL((mfma_rate_kernel<false, true, 16>), grid, block, 0, st, sink, iters); break;
-    case 6: hipLaunchKernelGGL((mfma_rate_kernel<true, false, 16>), grid, block, 0, st, sink, iters); break;
-    default: hipLaunchKernelGGL((mfma_rate_kernel<true, true, 16>), grid, block, 0, st, sink, iters); break;
-  }
-  return launch_status(who);
-}
-
-int tdist_mfma_rate_probe(int dtype, int random_operands, int iters, float* sink, void* stream) {
-  return mfma_rate_probe("tdist_mfma_rate_probe", false, dtype, random_operands, iters, sink, stream);
-}
-
-int tdist_mfma_rate_probe_16row(int dtype, int random_operands, int iters, float* sink, void* stream) {
-  return mfma_rate_probe("tdist_mfma_rate_probe_16row", true, dtype, random_operands, iters, sink, stream);
 }
 
 }  // extern "C"

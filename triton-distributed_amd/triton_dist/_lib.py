@@ -30,17 +30,17 @@ PROTOTYPES = {
     "tdist_last_error_string": (c_char_p, []),
     "tdist_init": (_I, []),
     "tdist_num_cus": (_I, []),
-    "tdist_gemm_chunk_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
-    "tdist_gemm_chunk_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
-    "tdist_gemm_chunk_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
+    "tdist_gemm_chunk_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
+    "tdist_gemm_chunk_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
+    "tdist_gemm_chunk_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
     "tdist_producer_push_chunk": (_I, [_P, _P, _L, _P, _P, _I, _P]),
     "tdist_producer_push_peers": (_I, [_P, _P, _I, _I, _L, _L, _P, _I, _P, _P, _P, _L, _I, _P]),
     "tdist_producer_mark": (_I, [_P, _P]),
     "tdist_producer_wait_until": (_I, [_P, _L, _P]),
     "tdist_flag_set": (_I, [_P, _I, _P]),
     "tdist_flag_fill": (_I, [_P, _I, _I, _P]),
-    "tdist_gemm_rs_scatter_bf16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P]),
-    "tdist_gemm_rs_scatter_f16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P]),
+    "tdist_gemm_rs_scatter_bf16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P]),
+    "tdist_gemm_rs_scatter_f16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P]),
     "tdist_reduce_slices": (_I, [_P, _L, _I, _I, _L, _P, _I, _P]),
     "tdist_moe_workspace_bytes": (_L, [_L, _I]),
     "tdist_moe_splits_cumsum": (_I, [_P, _L, _I, _P, _P, _P, _L, _P]),
@@ -53,17 +53,22 @@ PROTOTYPES = {
     "tdist_moe_dispatch_tokens_quant": (_I, [_P, _I, _I, _P, _I, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_align_workspace_bytes": (_L, [_L, _I, _I]),
     "tdist_moe_align_block_size": (_I, [_P, _I, _L, _I, _I, _L, _I, _P, _P, _P, _P, _P, _P, _L, _P]),
-    "tdist_group_gemm_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
-    "tdist_group_gemm_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
-    "tdist_group_gemm_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P]),
+    "tdist_group_gemm_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
+    "tdist_group_gemm_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
+    "tdist_group_gemm_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
     "tdist_gemm_split_k_workspace_bytes": (_L, []),
-    "tdist_gemm_split_k_set_workspace": (_I, [_P, _L, _P]),
     "tdist_decode_split_kv": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                    _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
     "tdist_decode_fused_counters": (_L, [_I, _I, _I]),
     "tdist_decode_fused": (_I, [_P, _P, _P, _P, _P, _F, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                 _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P, _L, _P, _I, _L, _L, _P, _P]),
     "tdist_decode_combine": (_I, [_P, _I, _P, _I, _I, _P, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P, _I, _L, _L, _P, _P]),
+}
+
+# libtdist_bench.so (include/tdist_bench.h): measurement helpers for bench.py, kept out of the product library
+BENCH_LIB_PATH = os.path.join(_HERE, "_lib", "libtdist_bench.so")
+BENCH_PROTOTYPES = {
+    "tdist_bench_last_error_string": (c_char_p, []),
     "tdist_copy_bytes": (_I, [_P, _P, _L, _P]),
     "tdist_mfma_rate_probe": (_I, [_I, _I, _I, _P, _P]),
     "tdist_mfma_rate_probe_16row": (_I, [_I, _I, _I, _P, _P]),
@@ -136,35 +141,49 @@ def dtype_code(dtype):
     raise TypeError("unsupported dtype %s" % dtype)
 
 
-_split_k_workspaces = {}   # device index -> uint8 tensor registered with the library (kept alive here)
+_bench_lib = None
 
 
-def enable_split_k(device=None):
-    """Allocates and registers the current (or given) device's split-K workspace once; the GEMM entry points then
-    cut the tiles of a last round that fills at most half of the grid along K. Returns the workspace tensor."""
+def load_bench():
+    """Loads libtdist_bench.so (once): the copy and MFMA-rate yardsticks of bench.py."""
+    global _bench_lib
+    if _bench_lib is None:
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise RuntimeError("libtdist_bench.so is missing at %s: build it with `python triton-distributed_amd/build.py`"
+                               % BENCH_LIB_PATH)
+        lib = ctypes.CDLL(BENCH_LIB_PATH)
+        for name, (restype, argtypes) in BENCH_PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _bench_lib = lib
+    return _bench_lib
+
+
+def bench_call(name, *args):
+    lib = load_bench()
+    code = getattr(lib, name)(*args)
+    if code != TDIST_OK:
+        msg = lib.tdist_bench_last_error_string()
+        raise TdistError(code, msg.decode("utf-8", "replace") if msg else "")
+
+
+def new_split_k_workspace(device=None):
+    """A zero-filled workspace for the GEMM entry points' sk_workspace argument (tdist_gemm_split_k_workspace_bytes()
+    bytes: 64 MiB + 20 KiB on MI355X). Every context owns one: launches that share a workspace must be ordered, and
+    contexts may run on streams of their own. Returns a uint8 tensor."""
     import torch
     dev = torch.cuda.current_device() if device is None else torch.device(device).index
-    if dev in _split_k_workspaces:
-        return _split_k_workspaces[dev]
     with torch.cuda.device(dev):
         nbytes = load().tdist_gemm_split_k_workspace_bytes()
         if nbytes <= 0:
             raise TdistError(TDIST_ERR_DEVICE, "split-K workspace: device %d is not gfx950" % dev)
-        ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda:%d" % dev)
-        call("tdist_gemm_split_k_set_workspace", ws.data_ptr(), nbytes, stream_ptr())
-        torch.cuda.current_stream().synchronize()
-    _split_k_workspaces[dev] = ws
-    return ws
+        return torch.zeros(nbytes, dtype=torch.uint8, device="cuda:%d" % dev)
 
 
-def disable_split_k(device=None):
-    import torch
-    dev = torch.cuda.current_device() if device is None else torch.device(device).index
-    if dev in _split_k_workspaces:
-        with torch.cuda.device(dev):
-            torch.cuda.synchronize()
-            call("tdist_gemm_split_k_set_workspace", None, 0, stream_ptr())
-        del _split_k_workspaces[dev]
+def workspace_args(ws):
+    """(pointer, bytes) of an optional workspace tensor for the sk_workspace / sk_workspace_bytes arguments."""
+    return (None, 0) if ws is None else (ws.data_ptr(), ws.numel() * ws.element_size())
 
 
 def require_cuda(*tensors):

@@ -127,11 +127,6 @@ class AllGatherGEMMTensorParallelContext:
     # producer does across GPUs. On one GPU the engines move ~55 GB/s each, far below a kernel copy inside HBM, so
     # the default is the blit path.
     use_sdma: bool = False
-    # True: queue the gated GEMM before the chunk copies, so that it works on the caller's own rows while the host
-    # is still queueing copies. Only safe when the GEMM stream and the copy streams sit on different hardware
-    # queues (a process has 4 by default and streams beyond that share them): a copy queued behind the spinning
-    # GEMM on the same queue can never run, and the bounded wait then reports a timeout.
-    gemm_first: bool = False
     preset_flags: bool = False   # debug: release every flag before the GEMM starts (no overlap)
     # > 0: pace the arrivals like one xGMI link per peer (GB/s; a link of MI355X moves ~153): a peer's n-th chunk is
     # copied no earlier than n * chunk_bytes / rate after the op started. 0: chunks are copied as fast as this GPU can.
@@ -149,6 +144,10 @@ class AllGatherGEMMTensorParallelContext:
     # units of this GPU; measured on MI355X they make no progress next to a full-chip persistent grid
     # unless 32 units stay free. A peer's copy engine pushing over xGMI would need none.
     producer_cus: int = 32
+    # The context's workspace for the GEMM (tdist_gemm_split_k_workspace_bytes() bytes, zero-filled once): with it the
+    # gated GEMM schedules its tiles by arrival and cuts tiles along K where workgroups would otherwise idle. It
+    # belongs to this context, so contexts on different streams never share scheduling state. None: fixed order.
+    sk_workspace: Optional[torch.Tensor] = None
 
     def update(self, rank, num_ranks, BLOCK_M=128, BLOCK_N=256, BLOCK_K=64, stages=3, ag_streams=None, gemm_stream=None,
                serial=False, autotune=False):
@@ -193,9 +192,9 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
     """create context for allgather gemm intra-node (reference :360-429).
 
     ``tp_group`` may be None: one GPU holds the only real rank. BLOCK_*/stages/autotune are accepted for
-    signature compatibility; the HIP kernel picks its own tiling. ``split_k``: register the device's split-K
-    workspace (64 MiB, once per device), with which a last round of tiles that fills at most half of the grid is cut
-    along K (one GEMM launch at a time per device may use it).
+    signature compatibility; the HIP kernel picks its own tiling. ``split_k``: give the context a workspace
+    (64 MiB) with which the gated GEMM schedules its tiles by arrival and cuts tiles along K where workgroups would
+    otherwise stand idle; False keeps the reference's fixed tile order.
     """
     assert M_PER_CHUNK % BLOCK_M == 0
     assert max_M % num_ranks == 0
@@ -204,9 +203,8 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
     if not torch.cuda.is_available():
         raise RuntimeError("create_ag_gemm_intra_node_context needs a GPU")
     _lib.check(_lib.load().tdist_init())
-    if split_k:
-        _lib.enable_split_k()
     device = torch.device("cuda", torch.cuda.current_device())
+    sk_workspace = _lib.new_split_k_workspace(device) if split_k else None
     workspace = torch.empty([max_M, K], dtype=input_dtype, device=device)
     m_chunk_num = (max_M + M_PER_CHUNK - 1) // M_PER_CHUNK
     barrier = torch.zeros([m_chunk_num], dtype=torch.int32, device=device)
@@ -246,6 +244,7 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
         output_dtype=output_dtype,
         status=status,
         start_stamp=start_stamp,
+        sk_workspace=sk_workspace,
     )
 
 
@@ -258,10 +257,12 @@ _GEMM_ENTRY = {
 
 def gated_gemm(a_ws, a_local, local_row_begin, b, c, flags, m_per_chunk, rank, num_ranks, *, row_scale=None,
                col_scale=None, chunk_order=None, wait_value=1, spin_limit=0, status=None, max_workgroups=0,
-               stream=None):
+               sk_workspace=None, stream=None):
     """Thin wrapper over tdist_gemm_chunk_gated_*: C[M,N] = A[M,K] @ B[N,K]^T with per-chunk gating.
     ``a_ws`` [M,K] gathered rows, ``a_local`` own shard or None, ``b`` [N,K]. ``max_workgroups`` > 0 caps the
-    persistent grid (leave compute units to a producer that copies on this same GPU)."""
+    persistent grid (leave compute units to a producer that copies on this same GPU). ``sk_workspace``: an optional
+    zero-initialised uint8 tensor of tdist_gemm_split_k_workspace_bytes() bytes (_lib.new_split_k_workspace); launches
+    that share one must be ordered."""
     _lib.require_cuda(a_ws, b, c)
     M, K = a_ws.shape
     N = b.shape[0]
@@ -281,7 +282,8 @@ def gated_gemm(a_ws, a_local, local_row_begin, b, c, flags, m_per_chunk, rank, n
         raise ValueError("scales are only defined for fp8 inputs")
     args += [
         _lib.ptr(flags), int(m_per_chunk), int(wait_value), _lib.ptr(chunk_order), int(rank), int(num_ranks),
-        int(spin_limit), _lib.ptr(status), int(max_workgroups), _lib.stream_ptr(stream),
+        int(spin_limit), _lib.ptr(status), int(max_workgroups), *_lib.workspace_args(sk_workspace),
+        _lib.stream_ptr(stream),
     ]
     _lib.call(_GEMM_ENTRY[a_ws.dtype], *args)
     return c
@@ -344,7 +346,8 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
         gated_gemm(workspace[:M], a, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
                    row_scale=row_scale, col_scale=col_scale, wait_value=1,
                    spin_limit=ctx.spin_limit if ctx is not None else 0,
-                   status=ctx.status if ctx is not None else None, max_workgroups=max_wgs, stream=gemm_stream)
+                   status=ctx.status if ctx is not None else None, max_workgroups=max_wgs,
+                   sk_workspace=ctx.sk_workspace if ctx is not None else None, stream=gemm_stream)
 
     if serial or (ctx is not None and ctx.preset_flags):
         # every chunk delivered before the GEMM starts
@@ -358,12 +361,11 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
         max_wgs = 0
         if ctx is not None and num_ranks > 1 and ctx.producer_cus > 0 and not use_kernel:
             max_wgs = max(1, _lib.load().tdist_num_cus() - ctx.producer_cus)
-        if ctx is not None and ctx.gemm_first:
-            call_gemm(max_wgs)
-            call_ag()
-        else:
-            call_ag()  # the reference's order (:300-304)
-            call_gemm(max_wgs)
+        # The reference's order (:300-304): producer first. (Queuing the GEMM first would let it start on the own
+        # rows while the host still queues copies, but a copy that lands behind the spinning GEMM on a shared
+        # hardware queue can never run, and which streams share a queue is not under the caller's control.)
+        call_ag()
+        call_gemm(max_wgs)
     current_stream.wait_stream(gemm_stream)
     for ag_stream in used_ag_streams:
         current_stream.wait_stream(ag_stream)

@@ -89,7 +89,7 @@ _GROUP_GEMM_ENTRY = {
 
 def group_gemm_gated(a_ws, a_local, local_row_begin, b_nk, c, sorted_token_ids, expert_ids, block_barrier_ids,
                      num_tokens_post_padded, block_size, num_valid_tokens, topk, tokens_per_rank, first_block, flags, rank,
-                     *, wait_value=1, spin_limit=0, status=None, max_workgroups=0, stream=None):
+                     *, wait_value=1, spin_limit=0, status=None, max_workgroups=0, sk_workspace=None, stream=None):
     """Thin wrapper over tdist_group_gemm_gated_*. ``a_ws`` [tokens, K] gathered rows, ``a_local`` the own shard or
     None, ``b_nk`` [E, N, K] (K contiguous), ``c`` [num_valid_tokens, N]."""
     _lib.require_cuda(a_ws, b_nk, c, sorted_token_ids, expert_ids, block_barrier_ids, num_tokens_post_padded)
@@ -106,7 +106,8 @@ def group_gemm_gated(a_ws, a_local, local_row_begin, b_nk, c, sorted_token_ids, 
               c.stride(0), a_ws.shape[0], N, K, sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
               block_barrier_ids.data_ptr(), num_tokens_post_padded.data_ptr(), num_blocks, int(block_size),
               int(num_valid_tokens), int(topk), int(tokens_per_rank), int(first_block), _lib.ptr(flags), int(wait_value),
-              int(rank), int(spin_limit), _lib.ptr(status), int(max_workgroups), _lib.stream_ptr(stream))
+              int(rank), int(spin_limit), _lib.ptr(status), int(max_workgroups), *_lib.workspace_args(sk_workspace),
+              _lib.stream_ptr(stream))
     return c
 
 
@@ -144,6 +145,7 @@ class MoE_AllGatherGroupGEMMTensorParallelContext:
     producer_cus: int = 32               # compute units left to the copies (see the AG-GEMM context)
     weight_nk: Optional[torch.Tensor] = None   # [E, N, K] copy of a [E, K, N] weight, made once per weight tensor
     weight_key: Optional[tuple] = None
+    sk_workspace: Optional[torch.Tensor] = None   # the context's GEMM workspace (split of a last round along K); None = off
 
     def set_peer_shards(self, shards):
         """``shards``: dict rank -> [M_per_rank, K] tensor (or a list; the own entry is ignored): the token rows that
@@ -173,14 +175,12 @@ def create_ag_group_gemm_intra_node_context(tp_pg, tensor_A, tensor_B, full_topk
     tensor_A [M_per_rank, K] local tokens, tensor_B [E, K, N_per_rank] local expert weights, full_topk_ids
     [M_per_rank * num_ranks, topk]. ``tp_pg`` may be None on one GPU: pass ``rank`` / ``num_ranks``. BLOCK_M is the
     row block of the align / sort and of the GEMM tile (128 or 256); the other tiling arguments are accepted for
-    signature compatibility. ``split_k``: register the device's split-K workspace (64 MiB, once per device): the
-    number of row blocks in use is seldom a multiple of the grid, and with the workspace the grouped GEMM cuts the tiles
-    of a last round that fills at most half of the grid along K (one GEMM launch at a time per device may use it)."""
+    signature compatibility. ``split_k``: give the context a GEMM workspace (64 MiB): the number of row blocks
+    in use is seldom a multiple of the grid, and with the workspace the grouped GEMM cuts the tiles of a last round that
+    fills at most half of the grid along K."""
     if not torch.cuda.is_available():
         raise RuntimeError("create_ag_group_gemm_intra_node_context needs a GPU")
     _lib.check(_lib.load().tdist_init())
-    if split_k:
-        _lib.enable_split_k()
     M_per_rank, K = tensor_A.shape
     _, topk = full_topk_ids.shape
     assert tensor_B.shape[1] == K, "tensor_B should have shape [E, %d, N_per_rank], got %s" % (K, tuple(tensor_B.shape))
@@ -205,7 +205,8 @@ def create_ag_group_gemm_intra_node_context(tp_pg, tensor_A, tensor_B, full_topk
         ag_stream=torch.cuda.Stream() if ag_stream is None else ag_stream,
         group_gemm_stream=group_gemm_stream, BLOCK_M=BLOCK_M, BLOCK_N=BLOCK_N, BLOCK_K=BLOCK_K,
         GROUP_SIZE_M=GROUP_SIZE_M, stages=stages, warps=warps, rank_block_num=rank_block_num, first_block=first_block,
-        one=torch.ones((16, ), dtype=torch.int32, device=device), status=torch.zeros((2, ), dtype=torch.int32, device=device))
+        one=torch.ones((16, ), dtype=torch.int32, device=device), status=torch.zeros((2, ), dtype=torch.int32, device=device),
+        sk_workspace=_lib.new_split_k_workspace(device) if split_k else None)
 
 
 def _weight_nk(ctx, b):
@@ -257,7 +258,8 @@ def ag_group_gemm_intra_node(a, b, ctx=None, full_topk_ids=None, num_experts=Non
     group_gemm_gated(workspace[:M_per_rank * W], a, rank * M_per_rank, b_nk, C, ctx.sorted_topk_ids,
                      ctx.aligned_expert_ids, ctx.aligned_barrier_ids, ctx.aligned_num_tokens, ctx.BLOCK_M,
                      ctx.full_num_tokens, ctx.topk, M_per_rank, ctx.first_block, barrier, rank,
-                     spin_limit=ctx.spin_limit, status=ctx.status, max_workgroups=max_wgs, stream=gemm_stream)
+                     spin_limit=ctx.spin_limit, status=ctx.status, max_workgroups=max_wgs, sk_workspace=ctx.sk_workspace,
+                     stream=gemm_stream)
     current.wait_stream(ctx.ag_stream)
     if gemm_stream is not current:
         current.wait_stream(gemm_stream)

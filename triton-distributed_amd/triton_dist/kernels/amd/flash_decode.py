@@ -67,21 +67,24 @@ def _split_kv(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_sp
     return out_split, lse_split, kv_lens
 
 
-_fused_counters = {}   # device index -> zero-initialised int32 counters (the kernel leaves them zero)
+_fused_counters = {}   # (device index, stream handle) -> zero-initialised int32 counters (the kernel leaves them zero)
 
 
 def _counters_for(q, kv_heads, workspace):
     """Arrival counters of the fused launch: a caller's ``workspace`` when it is a contiguous int32 tensor on the
-    device that is large enough (it must be ALL ZERO; the kernel leaves it zero), else a cached per-device buffer."""
+    device that is large enough (it must be ALL ZERO; the kernel leaves it zero), else a buffer cached per
+    (device, current stream): launches on one stream are ordered, so they may share it, and launches on different
+    streams never do."""
     batch, q_heads, _ = q.shape
     need = _lib.load().tdist_decode_fused_counters(batch, q_heads, kv_heads)
     if (isinstance(workspace, torch.Tensor) and workspace.is_cuda and workspace.dtype == torch.int32
             and workspace.is_contiguous() and workspace.numel() >= need):
         return workspace, workspace.numel()
-    buf = _fused_counters.get(q.device.index)
+    key = (q.device.index, torch.cuda.current_stream(q.device).cuda_stream)
+    buf = _fused_counters.get(key)
     if buf is None or buf.numel() < need:
         buf = torch.zeros(max(int(need), 4096), dtype=torch.int32, device=q.device)
-        _fused_counters[q.device.index] = buf
+        _fused_counters[key] = buf
     return buf, buf.numel()
 
 
@@ -134,15 +137,17 @@ def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_
 def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
                                     output_split=None, output_combine=None, kv_split=-1):
     """Same result as gqa_fwd_batch_decode in one launch (reference :931-1004: split-KV, a grid barrier on
-    ``workspace``, then the combine). Here the last workgroup to finish a (sequence, head block) merges its splits;
-    the arrival counters are a cached per-device buffer that the kernel leaves at zero (``workspace`` is accepted
-    and unused: nothing here depends on what a caller left in it). ``output_split`` is ignored (partials are fp32
-    internally). Calls on different streams of one device share the counters and must not overlap."""
+    ``workspace``, then the combine). Here the last workgroup to finish a (sequence, head block) merges its splits.
+    The arrival counters live in ``workspace`` when it is a zero-filled contiguous int32 device tensor of at least
+    tdist_decode_fused_counters(batch, q_heads, kv_heads) entries (the reference's barrier workspace is such a
+    tensor; the kernel leaves it zero), else in a zeroed buffer cached per (device, stream). ``output_split`` is
+    ignored (partials are fp32 internally)."""
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
     batch, q_heads, _ = q.shape
     if output_combine is None:
         output_combine = torch.empty((batch, q_heads, v_cache.shape[-1]), dtype=q.dtype, device=q.device)
-    decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, output_combine)
+    decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, output_combine,
+                 workspace=workspace)
     return output_combine
 
 
@@ -160,7 +165,8 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
     out32 = torch.empty((batch, q_heads, dv), dtype=torch.float32, device=q.device)
     lse32 = torch.empty((batch, q_heads), dtype=torch.float32, device=q.device)
     # split-KV and the merge of the splits (keeping the LSE) in one launch
-    decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, out32, lse32)
+    decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, out32, lse32,
+                 workspace=workspace)
     output_combine[..., :dv].copy_(out32)
     output_combine[..., dv].copy_(lse32)
     if return_lse:

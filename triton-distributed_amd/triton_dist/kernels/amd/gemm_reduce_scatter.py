@@ -29,6 +29,8 @@ class GEMMReduceScatterTensorParallelContext:
     # rows every rank's slice is padded to in the scatter buffer (the NVIDIA-side entry point pads M_per_rank to its
     # BLOCK_M, kernels/nvidia/gemm_reduce_scatter.py:468-479); None = no padding
     block_m: Optional[int] = None
+    # workspace of the context's GEMM launches (a last round that does not fill the grid is cut along K); None = off
+    sk_workspace: Optional[torch.Tensor] = None
 
     def set_peer_partials(self, partials):
         """``partials``: dict rank -> [M_per_rank, N] tensor, or a list of num_ranks entries (the entry of
@@ -48,7 +50,7 @@ class GEMMReduceScatterTensorParallelContext:
 def create_gemm_rs_intra_node_context(max_M, N, output_dtype, rank, num_ranks, tp_group, fuse_scatter=True,
                                       transpose_weight=False, split_k=True):
     """create context for gemm reduce-scatter intra-node (reference :381-426). ``tp_group`` may be None.
-    ``split_k``: register the device's split-K workspace (see create_ag_gemm_intra_node_context)."""
+    ``split_k``: give the context a GEMM workspace (see create_ag_gemm_intra_node_context)."""
     if not fuse_scatter:
         raise NotImplementedError()
     if transpose_weight:
@@ -56,9 +58,8 @@ def create_gemm_rs_intra_node_context(max_M, N, output_dtype, rank, num_ranks, t
     if not torch.cuda.is_available():
         raise RuntimeError("create_gemm_rs_intra_node_context needs a GPU")
     _lib.check(_lib.load().tdist_init())
-    if split_k:
-        _lib.enable_split_k()
     device = torch.device("cuda", torch.cuda.current_device())
+    sk_workspace = _lib.new_split_k_workspace(device) if split_k else None
     scatter_bufs = [torch.zeros([max_M, N], dtype=output_dtype, device=device) for _ in range(num_ranks)]
     scatter_bufs_ptr = torch.tensor([t.data_ptr() for t in scatter_bufs], dtype=torch.int64, device=device)
     torch.cuda.synchronize()
@@ -72,6 +73,7 @@ def create_gemm_rs_intra_node_context(max_M, N, output_dtype, rank, num_ranks, t
         output_dtype=output_dtype,
         fuse_scatter=fuse_scatter,
         transpose_weight=transpose_weight,
+        sk_workspace=sk_workspace,
     )
 
 
@@ -79,7 +81,7 @@ _SCATTER_ENTRY = {torch.bfloat16: "tdist_gemm_rs_scatter_bf16", torch.float16: "
 
 
 def matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weight, ldc=None, stream=None,
-                        strict_alignment=True):
+                        strict_alignment=True, sk_workspace=None):
     """GEMM with the scatter epilogue (reference :289-314). ``b`` is [N, K]. ``strict_alignment`` keeps the
     reference's assertion (M, N, K multiples of 256); without it the library's own limits apply (M / num_ranks a
     multiple of 128, K rows a multiple of 64 bytes)."""
@@ -95,7 +97,7 @@ def matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weigh
         raise TypeError("unsupported GEMM-RS dtype %s" % a.dtype)
     _lib.call(_SCATTER_ENTRY[a.dtype], a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
               scatter_bufs_ptr.data_ptr(), N if ldc is None else ldc, M, N, K, rank, num_ranks,
-              _lib.stream_ptr(stream))
+              *_lib.workspace_args(sk_workspace), _lib.stream_ptr(stream))
 
 
 def ring_reduce_after_scatter(rank, num_ranks, scatter_out, stream):
@@ -111,7 +113,7 @@ def ring_reduce_after_scatter(rank, num_ranks, scatter_out, stream):
 
 
 def gemm_rs_intra_node_op(a, b, output_dtype, rank, num_ranks, scatter_bufs, scatter_bufs_ptr, sync_bufs_ptr,
-                          fuse_scatter=True, transpose_weight=False):
+                          fuse_scatter=True, transpose_weight=False, sk_workspace=None):
     """gemm reduce scatter for intra-node (reference :317-365)."""
     if not fuse_scatter:
         raise NotImplementedError()
@@ -127,7 +129,7 @@ def gemm_rs_intra_node_op(a, b, output_dtype, rank, num_ranks, scatter_bufs, sca
                         "for %s, inputs are %s" % (scatter_bufs[rank].dtype, a.dtype))
     current_stream = torch.cuda.current_stream()
     matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weight=transpose_weight,
-                        ldc=scatter_bufs[rank].stride(0), stream=current_stream)
+                        ldc=scatter_bufs[rank].stride(0), stream=current_stream, sk_workspace=sk_workspace)
     scatter_out = scatter_bufs[rank][:M]
     output = ring_reduce_after_scatter(rank, num_ranks, scatter_out, current_stream)
     return output
@@ -145,4 +147,5 @@ def gemm_rs_intra_node(a, b, ctx):
         c (torch.Tensor<bfloat16/float16>): shape [M // world_size, N]
     """
     return gemm_rs_intra_node_op(a, b, ctx.output_dtype, ctx.rank, ctx.num_ranks, ctx.scatter_bufs,
-                                 ctx.scatter_bufs_ptr, ctx.sync_bufs_ptr, ctx.fuse_scatter, ctx.transpose_weight)
+                                 ctx.scatter_bufs_ptr, ctx.sync_bufs_ptr, ctx.fuse_scatter, ctx.transpose_weight,
+                                 sk_workspace=ctx.sk_workspace)

@@ -78,6 +78,7 @@ class MoEReduceRSContext:
     output_dtype: torch.dtype = torch.bfloat16
     weight_nk: Optional[torch.Tensor] = None
     weight_key: Optional[tuple] = None
+    sk_workspace: Optional[torch.Tensor] = None   # the context's GEMM workspace; None = off
 
     def set_peer_partials(self, partials):
         """``partials``: dict rank -> [tokens_per_rank, hidden]: what rank r computed (over its share of the intermediate
@@ -96,8 +97,6 @@ def create_moe_rs_context(pg, local_rank, world_size, local_world_size, max_toke
     if not torch.cuda.is_available():
         raise RuntimeError("create_moe_rs_context needs a GPU")
     _lib.check(_lib.load().tdist_init())
-    if split_k:
-        _lib.enable_split_k()   # (see create_ag_group_gemm_intra_node_context)
     if output_dtype != torch.bfloat16:
         raise NotImplementedError("the top-k reduction writes bf16 (reference: the input dtype, fp16 in its test)")
     rank = local_rank if pg is None else pg.rank()
@@ -112,7 +111,8 @@ def create_moe_rs_context(pg, local_rank, world_size, local_world_size, max_toke
         precompute_ctx=pre, rank=rank, world_size=world_size, rs_buffers=rs_buffers,
         final_output_buffer=torch.zeros((max_token_num * topk, hidden_dim), dtype=output_dtype, device=device),
         topk_weight_f32=pre.full_topk_weight.float().contiguous(),
-        identity_index=torch.arange(M * topk, dtype=torch.int32, device=device).view(M, topk), output_dtype=output_dtype)
+        identity_index=torch.arange(M * topk, dtype=torch.int32, device=device).view(M, topk), output_dtype=output_dtype,
+        sk_workspace=_lib.new_split_k_workspace(device) if split_k else None)
 
 
 def _weight_nk(ctx, b):
@@ -141,7 +141,7 @@ def moe_reduce_rs(rank, world_size, local_world_size, a, b, ctx, dump_ir=False, 
     # every sorted id names its own row of ``a`` (topk = 1 for the gather), no flag to wait for: the rows are local
     group_gemm_gated(a, None, 0, _weight_nk(ctx, b), out, pre.full_sorted_token_ids, pre.full_token_expert_ids,
                      pre.block_wait_barriers, pre.full_num_tokens_post_padded_list, pre.BLOCK_M, pre.full_numel, 1,
-                     pre.num_tokens_per_rank * topk, 0, flags, rank)
+                     pre.num_tokens_per_rank * topk, 0, flags, rank, sk_workspace=ctx.sk_workspace)
     y = moe_weighted_combine(None, out, None, ctx.identity_index, ctx.topk_weight_f32, from_slots=False)   # [M, hidden]
     m_per = M // world_size
     buf = ctx.rs_buffers[ctx.rank]

@@ -8,6 +8,7 @@ the gather has nobody to talk to: the partial results of the other ranks are pas
 """
 import torch
 
+from triton_dist import _lib
 from triton_dist.kernels.amd.flash_decode import (gqa_fwd_batch_decode_intra_rank,
                                                    gqa_fwd_batch_decode_inter_rank_combine)
 
@@ -16,22 +17,23 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
 
     def __init__(self, rank, node, num_ranks, num_nodes, num_q_heads, num_kv_heads, q_head_dim, v_head_dim, page_size=1,
                  scale=1, soft_cap=0, max_allowed_batch=1, thrink_buffer_threshold=500, stages=20):
+        """Same arguments as the reference's constructor (:45-47, including its spelling of
+        ``thrink_buffer_threshold``). ``node``, ``num_nodes``, ``stages`` and the threshold describe the all-gather
+        buffers of the multi-GPU layer; here they are recorded and otherwise unused, because the gather is the
+        caller handing in ``peer_partials``."""
         super().__init__()
-        self.rank = rank
-        self.num_ranks = num_ranks
-        self.node = node
-        self.num_nodes = num_nodes
-
-        self.workspace = None  # gqa_fwd doesn't need workspace
-        self.num_q_heads = num_q_heads
-        self.num_kv_heads = num_kv_heads
-        self.q_head_dim = q_head_dim
-        self.v_head_dim = v_head_dim
+        # where this shard sits among the sequence-parallel ranks
+        self.rank, self.num_ranks = rank, num_ranks
+        self.node, self.num_nodes = node, num_nodes
+        # attention geometry
+        self.num_q_heads, self.num_kv_heads = num_q_heads, num_kv_heads
+        self.q_head_dim, self.v_head_dim = q_head_dim, v_head_dim
         self.page_size = page_size
-        self.soft_cap = soft_cap
-        self.scale = scale
-        self.kv_split = 32
+        self.scale, self.soft_cap = scale, soft_cap
+        self.kv_split = 32                    # splits of the local shard (the reference fixes 32, :59)
         self.max_allowed_batch = max_allowed_batch
+        # the fused decode keeps its arrival counters per layer, so that two layers may run on two streams
+        self.workspace = None
         self.stages = stages
         self.shrink_buffer_threshold = thrink_buffer_threshold
 
@@ -48,6 +50,9 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         assert global_kv_lens.shape[0] == self.num_ranks
         assert global_kv_lens.shape[1] == batch
         assert batch <= self.max_allowed_batch, f"Only support {self.max_allowed_batch} queries decode now"
+        if self.workspace is None or self.workspace.device != q.device:
+            n = _lib.load().tdist_decode_fused_counters(self.max_allowed_batch, self.num_q_heads, self.num_kv_heads)
+            self.workspace = torch.zeros(max(int(n), 1), dtype=torch.int32, device=q.device)
         _, out32, lse32 = gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, self.workspace, [1] * batch,
                                                           global_kv_lens[self.rank], block_table, self.scale,
                                                           soft_cap=self.soft_cap, kv_split=self.kv_split,
