@@ -178,7 +178,10 @@ int tdist_reduce_slices(const void* c, int64_t slice_stride, int n_slices, int f
  *            combine + index_add_         test/nvidia/test_all_to_all.py:360-370
  *            weighted top-k reduce        test/nvidia/test_moe_reduce_rs.py:103-129
  * ------------------------------------------------------------------------------------------- */
-/* Scratch bytes needed by tdist_moe_scatter_index / tdist_moe_splits_cumsum for n_ids ids. */
+/* Scratch bytes needed by tdist_moe_scatter_index / tdist_moe_splits_cumsum for n_ids ids. The first 256 bytes of the
+ * workspace are control words: they must be ZERO when the workspace is first used and are left zero by every call
+ * (so one zero-initialised buffer serves all later calls; calls that share it must not overlap). The rest is plain
+ * scratch. */
 int64_t tdist_moe_workspace_bytes(int64_t n_ids, int num_experts);
 
 /* splits[g] = #{i : ids[i] == g} (torch.bincount(..., minlength=G), test_all_to_all.py:314);
@@ -269,7 +272,8 @@ int tdist_moe_dispatch_tokens_quant(const void* tokens_bf16, int hidden, int gro
  *                           n_total / block_size + num_experts * num_iterations blocks are written (the reference
  *                           allocates n_total + num_experts * num_iterations entries)
  *   rank_block_num[r]     = blocks of segment r;  *total_tokens_post_pad = padded total.
- * Needs num_experts * num_iterations <= 4096. Workspace: tdist_moe_align_workspace_bytes (0 = unsupported sizes). */
+ * Needs num_experts * num_iterations <= 4096. Workspace: tdist_moe_align_workspace_bytes (0 = unsupported sizes); its
+ * first 256 bytes are control words, ZERO on first use and left zero by every call (see tdist_moe_workspace_bytes). */
 int64_t tdist_moe_align_workspace_bytes(int64_t n_total, int num_experts, int num_iterations);
 int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_total, int num_experts,
                                int num_iterations, int64_t n_per_iteration, int block_size, int32_t* sorted_token_ids,

@@ -51,6 +51,54 @@ def test_preprocess_repeated_ids_and_skewed_load(cuda):
         assert torch.equal(a.cpu(), b)
 
 
+@pytest.mark.parametrize("launches", ["one", "three"])
+def test_preprocess_paths_sizes_in_turn_and_context_buffers(cuda, monkeypatch, launches):
+    """The one-launch index build and the three-launch form it falls back to (forced here through the library's
+    switch; taken by itself beyond one block per compute unit, as the 560 000 ids below do): calls of different sizes
+    in turn on the same cached scratch, ids outside [0, G) (dropped: scatter index -1), and the context-owned result
+    tensors, two sets used in turn."""
+    from triton_dist.kernels.amd import create_all_to_all_context, moe_dispatch_preprocess
+    if launches == "three":
+        monkeypatch.setenv("TDIST_MOE_INDEX_LAUNCHES", "3")
+    announce("moe preprocess paths (%s launch)" % launches)
+    g = torch.Generator().manual_seed(9)
+    for T, topk, G in [(4096, 8, 256), (300, 4, 2048), (70000, 8, 64), (1000, 8, 256), (5, 3, 4096)]:
+        ids = torch.randint(0, G, (T, topk), generator=g).to(torch.int32)
+        out = moe_dispatch_preprocess(ids.to(cuda), G, want_topk_index=True)
+        torch.cuda.synchronize()
+        for a, b in zip(out, golden.moe_preprocess(ids, G)):
+            assert torch.equal(a.cpu(), b), (T, topk, G)
+    # ids outside the range take no place in the order
+    T, topk, G = 777, 4, 32
+    ids = torch.randint(0, G, (T, topk), generator=g).to(torch.int32)
+    bad = torch.rand((T, topk), generator=g) < 0.1
+    ids_bad = torch.where(bad, torch.where(torch.rand((T, topk), generator=g) < 0.5, torch.tensor(-1), torch.tensor(G + 5)), ids).int()
+    splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids_bad.to(cuda), G)
+    torch.cuda.synchronize()
+    flat, keep = ids_bad.view(-1), ~bad.view(-1)
+    want_splits = torch.bincount(flat[keep].long(), minlength=G).int()
+    assert torch.equal(splits.cpu(), want_splits) and torch.equal(cumsum.cpu(), golden.splits_to_cumsum(want_splits))
+    order = torch.argsort(flat[keep], stable=True)
+    want_scatter = torch.full((T * topk, ), -1, dtype=torch.int32)
+    kept_pos = torch.nonzero(keep).view(-1)
+    want_scatter[kept_pos[order]] = torch.arange(order.numel(), dtype=torch.int32)
+    assert torch.equal(scatter.cpu().view(-1), want_scatter)
+    assert torch.equal(gather.cpu()[:order.numel()], (kept_pos[order] // topk).int())
+    # context-owned tensors: the result of a call stays valid through the next call
+    ctx = create_all_to_all_context(64, 128, 0, 16, 4, 4, dtype=torch.float8_e4m3fn)
+    ids_a = torch.randint(0, 16, (200, 4), generator=g).to(torch.int32)
+    ids_b = torch.randint(0, 16, (200, 4), generator=g).to(torch.int32)
+    out_a = moe_dispatch_preprocess(ids_a.to(cuda), 16, ctx=ctx)
+    out_b = moe_dispatch_preprocess(ids_b.to(cuda), 16, ctx=ctx)
+    torch.cuda.synchronize()
+    for a, b in zip(out_a, golden.moe_preprocess(ids_a, 16)[:4]):
+        assert torch.equal(a.cpu(), b)
+    for a, b in zip(out_b, golden.moe_preprocess(ids_b, 16)[:4]):
+        assert torch.equal(a.cpu(), b)
+    out_c = moe_dispatch_preprocess(ids_a.to(cuda), 16, ctx=ctx)
+    assert out_c[2].data_ptr() == out_a[2].data_ptr() and out_c[2].data_ptr() != out_b[2].data_ptr()
+
+
 def test_splits_cumsum_entry_point(cuda):
     from triton_dist import _lib
     announce("moe splits_cumsum")
@@ -58,7 +106,7 @@ def test_splits_cumsum_entry_point(cuda):
     dev_ids = ids.to(cuda)
     splits = torch.empty(100, dtype=torch.int32, device=cuda)
     cumsum = torch.empty(101, dtype=torch.int32, device=cuda)
-    ws = torch.empty(_lib.load().tdist_moe_workspace_bytes(ids.numel(), 100), dtype=torch.uint8, device=cuda)
+    ws = torch.zeros(_lib.load().tdist_moe_workspace_bytes(ids.numel(), 100), dtype=torch.uint8, device=cuda)
     _lib.call("tdist_moe_splits_cumsum", dev_ids.data_ptr(), ids.numel(), 100, splits.data_ptr(), cumsum.data_ptr(),
               ws.data_ptr(), ws.numel(), _lib.stream_ptr())
     torch.cuda.synchronize()

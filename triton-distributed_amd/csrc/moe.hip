@@ -4,12 +4,17 @@
 // of the flat [T*topk] expert ids, restating in parallel form what the reference does with
 //   torch.bincount / cumsum / argsort(stable).argsort()      test/nvidia/test_all_to_all.py:42-46,95-96,314
 //   calc_gather_index                                         test/nvidia/test_all_to_all.py:49-92
-// Three launches: per-block histograms, one scan block, per-block ranking. Inside a wave the rank of
-// an entry among equal ids is found with ballots (one per id bit), so no sort is involved and the
-// order of equal ids is their flat order (stability).
+// One launch when the ids fit one co-resident grid (moe_index_fused_kernel: per-block histograms, a grid-wide
+// rendezvous, then every block derives its own prefixes and ranks its ids), else three launches (per-block
+// histograms, scan, per-block ranking). Inside a wave the rank of an entry among equal ids is found with ballots
+// (one per id bit), so no sort is involved and the order of equal ids is their flat order (stability).
 //
 // Row movement restates all_to_all_kernel (kernels/nvidia/low_latency_all_to_all.py:56-103): the rows
 // of destination d are contiguous in the sorted order, and land in that destination's receive slot.
+#include <stdlib.h>
+
+#include <mutex>
+
 #include "common.h"
 
 namespace tdist {
@@ -198,6 +203,183 @@ __global__ __launch_bounds__(kMoeThreads) void moe_rank_kernel(const int32_t* __
       const int32_t start = pos[e];
       const int rank_in = __popcll(peers & lt_mask);
       const int32_t p = start + rank_in;
+      scatter_idx[i] = p;
+      gather_idx[p] = (int32_t)(i / topk);
+      if (topk_idx) topk_idx[p] = (int32_t)(i % topk);
+    } else if (i < n) {
+      scatter_idx[i] = -1;
+    }
+    // every lane of the wave has read pos[] before the leaders advance it
+    __builtin_amdgcn_wave_barrier();
+    if (valid && (peers & lt_mask) == 0) pos[e] = pos[e] + __popcll(peers);
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// ---- the same in one launch ---------------------------------------------------------------------
+// Block b owns ids [b * kItems, (b+1) * kItems), kPerWave consecutive ones per wave, in flat order.
+//   1. every wave counts its ids per expert in its own row of LDS counters; the block's sum goes to hist[b][.];
+//   2. rendezvous: every block needs every other block's histogram (cumsum is a prefix over ALL ids), so the blocks
+//      wait for each other. That is safe because the host only takes this path when the grid is at most one block per
+//      compute unit, i.e. co-resident (ctrl[0] counts arrivals and is put back to zero by the last one, ctrl[1] is a
+//      generation number that the last arrival bumps; the wait is bounded all the same: if it ran out, the block leaves
+//      without writing and cumsum[0] is set to -1 instead of 0);
+//   3. every block adds up the histogram columns (all rows: the split of the expert; rows before its own: its offset
+//      within the expert), scans the splits into cumsum, and turns its waves' counters into start positions;
+//   4. ranking as in moe_rank_kernel.
+// ctrl[0] must be zero on entry and is zero again on exit.
+// A block is 8 waves x 256 ids. (One block of 16 waves x 2048 ids for all of a decode step's 32768 ids, with no
+// rendezvous at all, was measured 4 x slower: a wave ranks its ids 64 at a time, each pass behind the previous one's
+// counter update, and 32 such passes in a row cost more than the trips through memory they save.) A single block
+// (up to 2048 ids) skips the rendezvous.
+constexpr int kFusedSpinLimit = 1 << 22;
+constexpr int kFusedThreads = 512, kFusedPerWave = 256, kFusedItems = kFusedThreads / 64 * kFusedPerWave;
+
+template <int kThreads, int kPerWave>
+__global__ __launch_bounds__(kThreads) void moe_index_fused_kernel(const int32_t* __restrict__ ids, int64_t n, int topk,
+                                                                  int G, int nbits, int32_t* hist, int32_t* ctrl,
+                                                                  int32_t* __restrict__ splits,
+                                                                  int32_t* __restrict__ cumsum,
+                                                                  int32_t* __restrict__ scatter_idx,
+                                                                  int32_t* __restrict__ gather_idx,
+                                                                  int32_t* __restrict__ topk_idx) {
+  constexpr int kWaves = kThreads / 64, kItems = kWaves * kPerWave, kPasses = kPerWave / 64;
+  extern __shared__ int32_t s_mem[];  // [kWaves][G] wave counters, [G] column sums
+  int32_t* const s_cnt = s_mem;
+  int32_t* const s_col = s_mem + kWaves * G;
+  __shared__ int32_t s_part[kWaves];
+  __shared__ int s_flag;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int B = gridDim.x, b = blockIdx.x;
+  int gen0 = 0;
+  if (B > 1 && threadIdx.x == 0) gen0 = __hip_atomic_load(ctrl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // the wave's ids first: the loads are in flight while the counters are cleared
+  const int64_t wbase = (int64_t)b * kItems + (int64_t)wave * kPerWave;
+  int e_of[kPasses];
+#pragma unroll
+  for (int u = 0; u < kPasses; ++u) {
+    const int64_t i = wbase + u * 64 + lane;
+    e_of[u] = i < n ? ids[i] : -1;
+  }
+  for (int g = threadIdx.x; g < kWaves * G; g += kThreads) s_cnt[g] = 0;
+  __syncthreads();
+  // 1. per-wave counts
+  int32_t* const my_cnt = s_cnt + wave * G;
+#pragma unroll
+  for (int u = 0; u < kPasses; ++u) {
+    if (e_of[u] < 0 || e_of[u] >= G) e_of[u] = -1;
+    if (e_of[u] >= 0) atomicAdd(&my_cnt[e_of[u]], 1);
+  }
+  __syncthreads();
+  if (B > 1) {
+    for (int g = threadIdx.x; g < G; g += kThreads) {
+      int32_t t = 0;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) t += s_cnt[w * G + g];
+      // (device-coherent store: it goes through to memory, so no cache has to be written back before the arrival)
+      __hip_atomic_store(hist + (int64_t)b * G + g, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // 2. rendezvous. No fence on either side (a release or acquire fence at device scope writes back or invalidates
+    // the whole L2 of this XCD, microseconds after a kernel that left it full of dirty lines): every wave waits for
+    // its own coherent stores, then the arrival is counted; the histograms are read back with coherent loads.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int ok = 1;
+      if (__hip_atomic_fetch_add(ctrl, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == B - 1) {
+        __hip_atomic_store(ctrl, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(ctrl + 1, gen0 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        ok = 0;
+        for (int it = 0; it < kFusedSpinLimit; ++it) {
+          if (__hip_atomic_load(ctrl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != gen0) {
+            ok = 1;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+      }
+      s_flag = ok;
+    }
+    __syncthreads();
+    if (!s_flag) {
+      if (threadIdx.x == 0) cumsum[0] = -1;
+      return;
+    }
+  }
+  // 3. column sums: s_col[g] = ids of expert g in all blocks; the blocks before this one go into wave 0's start
+  for (int g = threadIdx.x; g < G; g += kThreads) {
+    int32_t total = 0, before = 0;
+    if (B > 1) {
+      for (int r = 0; r < B; ++r) {
+        const int32_t h = __hip_atomic_load(hist + (int64_t)r * G + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        total += h;
+        before += r < b ? h : 0;
+      }
+    }
+    // wave starts within the expert: blocks before, then the earlier waves of this block
+    int32_t run = before;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const int32_t c = s_cnt[w * G + g];
+      s_cnt[w * G + g] = run;
+      run += c;
+    }
+    s_col[g] = B > 1 ? total : run;
+  }
+  __syncthreads();
+  // exclusive scan of s_col over the experts: consecutive experts per thread, an inclusive scan of the threads' totals
+  // within the wave by shuffles, then the waves' totals through LDS
+  const int per = (G + kThreads - 1) / kThreads;
+  const int g0 = threadIdx.x * per;
+  int32_t local_total = 0;
+  for (int j = 0; j < per; ++j)
+    if (g0 + j < G) local_total += s_col[g0 + j];
+  int32_t incl = local_total;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int32_t t = __shfl_up(incl, off);
+    if (lane >= off) incl += t;
+  }
+  if (lane == 63) s_part[wave] = incl;
+  __syncthreads();
+  int32_t acc = incl - local_total;  // ids of the experts before this thread's first one
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) acc += w < wave ? s_part[w] : 0;
+  if (b == 0 && threadIdx.x == 0) cumsum[0] = 0;
+  for (int j = 0; j < per; ++j) {
+    const int g = g0 + j;
+    if (g < G) {
+      const int32_t c = s_col[g];
+      if (b == 0) {
+        if (splits) splits[g] = c;
+        cumsum[g + 1] = acc + c;
+      }
+      // the expert's first position goes into every wave's start
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) s_cnt[w * G + g] += acc;
+      acc += c;
+    }
+  }
+  __syncthreads();
+  if (scatter_idx == nullptr) return;  // splits and cumsum only
+  // 4. walk the wave's ids in flat order, 64 at a time
+  volatile int32_t* pos = my_cnt;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+  for (int u = 0; u < kPasses; ++u) {
+    if (wbase + u * 64 >= n) break;  // (the whole wave is past the end)
+    const int64_t i = wbase + u * 64 + lane;
+    const int e = e_of[u];
+    const bool valid = e >= 0;
+    uint64_t peers = __ballot(valid);
+    for (int bit = 0; bit < nbits; ++bit) {
+      const bool one = (e >> bit) & 1;
+      const uint64_t m = __ballot(valid && one);
+      peers &= one ? m : ~m;
+    }
+    if (valid) {
+      const int32_t p = pos[e] + __popcll(peers & lt_mask);
       scatter_idx[i] = p;
       gather_idx[p] = (int32_t)(i / topk);
       if (topk_idx) topk_idx[p] = (int32_t)(i % topk);
@@ -738,9 +920,29 @@ static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, 
   if (!workspace || workspace_bytes < need)
     return fail(TDIST_ERR_WORKSPACE, "%s: workspace %lld B < %lld B", who, (long long)workspace_bytes, (long long)need);
   const int num_blocks = (int)ceil_div(n_ids > 0 ? n_ids : 1, kMoeItemsPerBlock);
-  int32_t* hist = (int32_t*)workspace;
+  // workspace: 256 bytes of control words (always at the start, whatever the sizes of the call), the block
+  // histograms, one row for the splits
+  int32_t* scan_counter = (int32_t*)workspace;
+  int32_t* hist = scan_counter + 64;
   int32_t* splits_buf = splits ? splits : hist + (int64_t)num_blocks * G;
-  int32_t* scan_counter = hist + (int64_t)(num_blocks + 1) * G;
+  // One launch when every block of it is resident at once (one per compute unit at most): the blocks wait for each
+  // other's histograms. Its histogram rows (one per 2048 ids) fit the rows the workspace holds (one per 256 ids).
+  const DeviceInfo& di = device_info();
+  const int64_t fused_blocks = ceil_div(n_ids > 0 ? n_ids : 1, kFusedItems);
+  if (di.ok == 1 && fused_blocks <= di.num_cus && getenv("TDIST_MOE_INDEX_LAUNCHES") == nullptr) {
+    auto kern = moe_index_fused_kernel<kFusedThreads, kFusedPerWave>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (kFusedThreads / 64 + 1) * kMoeMaxExperts * 4) != hipSuccess)
+        return fail(TDIST_ERR_LAUNCH, "%s: cannot reserve LDS for the index kernel", who);
+      attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)fused_blocks), dim3(kFusedThreads), (size_t)(kFusedThreads / 64 + 1) * G * 4, stream,
+                       ids, n_ids, want_index ? topk : 1, G, id_bits(G), hist, scan_counter, splits, cumsum,
+                       want_index ? scatter_idx : nullptr, gather_idx, topk_idx);
+    return launch_status(who);
+  }
   hipLaunchKernelGGL(moe_hist_kernel, dim3(num_blocks), dim3(kMoeThreads), (size_t)G * 4, stream, ids, n_ids, G, hist,
                      scan_counter);
   hipLaunchKernelGGL(moe_scan_kernel, dim3((G + kScanCols - 1) / kScanCols), dim3(kScanThreads), 0, stream, hist, num_blocks,
@@ -761,7 +963,7 @@ extern "C" {
 int64_t tdist_moe_workspace_bytes(int64_t n_ids, int num_experts) {
   if (n_ids < 0 || num_experts <= 0) return 0;
   const int64_t num_blocks = ceil_div(n_ids > 0 ? n_ids : 1, kMoeItemsPerBlock);
-  return (num_blocks + 1) * (int64_t)num_experts * 4 + 256;  // block histograms + one splits row + the scan's counter
+  return 256 + (num_blocks + 1) * (int64_t)num_experts * 4;  // control words + block histograms + one splits row
 }
 
 int tdist_moe_splits_cumsum(const int32_t* ids, int64_t n_ids, int num_experts, int32_t* splits, int32_t* cumsum,
@@ -935,13 +1137,15 @@ int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_to
   if (!workspace || workspace_bytes < need)
     return fail(TDIST_ERR_WORKSPACE, "%s: workspace %lld B < %lld B", who, (long long)workspace_bytes, (long long)need);
   hipStream_t st = (hipStream_t)stream;
-  int32_t* keys = (int32_t*)workspace;
+  // the index build's own scratch first, so that its control words are the workspace's first 256 bytes whatever the
+  // sizes; then keys, scatter index, gather index, group sizes and two prefix rows
+  void* index_ws = workspace;
+  int32_t* keys = (int32_t*)((unsigned char*)workspace + tdist_moe_workspace_bytes(n_total, (int)G));
   int32_t* scatter = keys + n_total;
   int32_t* gather = scatter + n_total;
   int32_t* splits = gather + n_total;
   int32_t* cumsum = splits + (G + 1);
   int32_t* pad_cum = cumsum + (G + 1);
-  void* index_ws = pad_cum + (G + 1);
   const int64_t blocks = ceil_div(n_total > 0 ? n_total : 1, 256);
   if (n_total > 0)
     hipLaunchKernelGGL(moe_align_keys_kernel, dim3((unsigned)blocks), dim3(256), 0, st, topk_ids, ids_int64, n_total,

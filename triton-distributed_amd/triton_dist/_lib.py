@@ -181,6 +181,24 @@ def new_split_k_workspace(device=None):
         return torch.zeros(nbytes, dtype=torch.uint8, device="cuda:%d" % dev)
 
 
+_zero_scratch = {}   # (device index, stream handle) -> uint8 tensor whose control words the kernels keep at zero
+
+
+def zeroed_scratch(nbytes, device):
+    """A scratch tensor of at least ``nbytes`` for entry points whose workspace starts with control words that must be
+    zero on first use and are left zero by every call (the MoE index build, the align / sort): allocated zero-filled
+    once per (device, current stream) and handed out again on later calls, so a call allocates nothing. Launches on
+    one stream are ordered and may share it; launches on different streams never do."""
+    import torch
+    device = torch.device(device)
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _zero_scratch.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.zeros(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _zero_scratch[key] = buf
+    return buf
+
+
 def workspace_args(ws):
     """(pointer, bytes) of an optional workspace tensor for the sk_workspace / sk_workspace_bytes arguments."""
     return (None, 0) if ws is None else (ws.data_ptr(), ws.numel() * ws.element_size())

@@ -55,9 +55,8 @@ def sort_topk_ids_align_block_size(
     if ws_bytes == 0:
         raise _lib.TdistError(_lib.TDIST_ERR_UNSUPPORTED,
                               "num_experts * num_ranks = %d is above what the align kernel handles" % (num_experts * num_ranks))
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-
     def launch(stream):
+        workspace = _lib.zeroed_scratch(ws_bytes, dev)   # (cached per stream: current is `stream` here)
         sorted_ids.fill_(n_total)
         _lib.call("tdist_moe_align_block_size", topk_ids.data_ptr(), 1 if topk_ids.dtype == torch.int64 else 0, n_total,
                   num_experts, num_ranks, n_per, block_size, sorted_ids.data_ptr(), expert_ids.data_ptr(),
@@ -70,7 +69,6 @@ def sort_topk_ids_align_block_size(
         with torch.cuda.stream(moe_stream):
             launch(moe_stream)
         torch.cuda.current_stream().wait_stream(moe_stream)
-        workspace.record_stream(moe_stream)
     return (
         sorted_ids,
         expert_ids,

@@ -78,6 +78,8 @@ class AllToAllContext:
         # start from 1, as the reference does (:161-163)
         self.call_count = 1
         self.MOD_VALUE = 1000000
+        # index tensors of moe_dispatch_preprocess(..., ctx=self): two sets, allocated on first use for a shape
+        self.index_sets, self.index_key, self.index_calls = None, None, 0
 
 
 def create_all_to_all_context(
@@ -119,7 +121,8 @@ def splits_to_cumsum(splits: torch.Tensor):
     return out
 
 
-def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_topk_index: bool = False):
+def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_topk_index: bool = False,
+                            ctx: Optional[AllToAllContext] = None):
     """GPU version of the reference test's index preparation (test/nvidia/test_all_to_all.py:314-320):
 
         splits       int32[G]        torch.bincount(exp_indices.view(-1), minlength=G)
@@ -127,7 +130,9 @@ def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_to
         scatter_idx  int32[T, topk]  exp_indices.flatten().argsort(stable=True).argsort()
         gather_idx   int32[T*topk]   token of each expert-sorted row (calc_gather_index)
 
-    Returns (splits, split_cumsum, scatter_idx, gather_idx[, topk_idx])."""
+    One kernel launch. With ``ctx`` the five tensors are the context's own (allocated on the first call for a shape,
+    two sets used in turn like the receive buffers, so a result stays valid until the call after next) and the call
+    allocates nothing. Returns (splits, split_cumsum, scatter_idx, gather_idx[, topk_idx])."""
     _lib.require_cuda(exp_indices)
     if exp_indices.dtype != torch.int32:
         exp_indices = exp_indices.to(torch.int32)
@@ -135,13 +140,26 @@ def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_to
     T, topk = exp_indices.shape
     n = T * topk
     dev = exp_indices.device
-    splits = torch.empty(num_experts, dtype=torch.int32, device=dev)
-    cumsum = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
-    scatter_idx = torch.empty((T, topk), dtype=torch.int32, device=dev)
-    gather_idx = torch.empty(n, dtype=torch.int32, device=dev)
-    topk_idx = torch.empty(n, dtype=torch.int32, device=dev) if want_topk_index else None
+
+    def alloc():
+        return (torch.empty(num_experts, dtype=torch.int32, device=dev),
+                torch.empty(num_experts + 1, dtype=torch.int32, device=dev),
+                torch.empty((T, topk), dtype=torch.int32, device=dev),
+                torch.empty(n, dtype=torch.int32, device=dev),
+                torch.empty(n, dtype=torch.int32, device=dev))
+
+    if ctx is not None:
+        key = (T, topk, num_experts, dev)
+        if ctx.index_key != key:
+            ctx.index_sets, ctx.index_key, ctx.index_calls = [alloc(), alloc()], key, 0
+        splits, cumsum, scatter_idx, gather_idx, topk_idx = ctx.index_sets[ctx.index_calls % 2]
+        ctx.index_calls += 1
+    else:
+        splits, cumsum, scatter_idx, gather_idx, topk_idx = alloc()
+    if not want_topk_index:
+        topk_idx = None
     ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
-    workspace = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+    workspace = _lib.zeroed_scratch(ws_bytes, dev)
     _lib.call("tdist_moe_scatter_index", exp_indices.data_ptr(), n, topk, num_experts, splits.data_ptr(),
               cumsum.data_ptr(), scatter_idx.data_ptr(), gather_idx.data_ptr(), _lib.ptr(topk_idx),
               workspace.data_ptr(), workspace.numel(), _lib.stream_ptr())
