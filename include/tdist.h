@@ -45,8 +45,9 @@ typedef enum tdist_dtype {
  * ------------------------------------------------------------------------------------------- */
 int tdist_version(void);
 const char* tdist_last_error_string(void);
-/* Caches properties of the current device (CU count, XCD count). Optional: every entry point calls
- * it lazily. Returns TDIST_ERR_DEVICE when the current device is not gfx950. */
+/* Caches properties of the current device (CU count, XCD count) and the device address of the library's built-in
+ * scratch (tdist_moe_scatter_index_static). Optional: every entry point does its part lazily. Returns
+ * TDIST_ERR_DEVICE when the current device is not gfx950. */
 int tdist_init(void);
 int tdist_num_cus(void);
 
@@ -199,6 +200,16 @@ int tdist_moe_splits_cumsum(const int32_t* ids, int64_t n_ids, int num_experts, 
 int tdist_moe_scatter_index(const int32_t* ids, int64_t n_ids, int topk, int num_experts, int32_t* splits,
                             int32_t* cumsum, int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx,
                             void* workspace, int64_t workspace_bytes, void* stream);
+
+/* tdist_moe_scatter_index for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses
+ * that forbid hipMalloc). It has no counterpart in the reference. Same arguments and same results, without the
+ * workspace: the scratch is a 1 MiB array inside the library (one copy per GPU, held until the process ends), so the
+ * call allocates nothing. Sizes whose scratch (tdist_moe_workspace_bytes) exceeds 1 MiB are rejected with
+ * TDIST_ERR_UNSUPPORTED: e.g. 256 experts take up to 261 632 ids. All calls on one GPU share that GPU's array: calls
+ * that overlap on one GPU (different streams without an ordering) race. */
+int tdist_moe_scatter_index_static(const int32_t* ids, int64_t n_ids, int topk, int num_experts, int32_t* splits,
+                                   int32_t* cumsum, int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx,
+                                   void* stream);
 
 /* Dispatch: sorted row p (0 <= p < cumsum[G]) of expert e goes to destination d = e / experts_per_rank,
  * slot row d*max_m + (p - cumsum[d*experts_per_rank]) of slot_rows / slot_scales

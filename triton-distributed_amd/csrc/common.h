@@ -22,6 +22,9 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 // hipGetLastError() → TDIST_OK or TDIST_ERR_LAUNCH (message recorded).
 int launch_status(const char* what);
 const DeviceInfo& device_info();
+// Looks up, once per device and with that device current, the device address of the built-in scratch of
+// tdist_moe_scatter_index_static (moe.hip). Called by tdist_init and, lazily, by that entry point.
+int moe_static_scratch_init();
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

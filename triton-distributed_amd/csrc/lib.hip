@@ -171,7 +171,9 @@ const char* tdist_last_error_string(void) { return g_err; }
 int tdist_init(void) {
   const DeviceInfo& di = device_info();
   if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "tdist_init: current device is not a gfx950 GPU");
-  return TDIST_OK;
+  // the address of the current device's copy of the library's built-in scratch (tdist_moe_scatter_index_static), so
+  // that a caller that may not run set-up work later (under graph capture) finds it ready
+  return moe_static_scratch_init();
 }
 
 int tdist_num_cus(void) {

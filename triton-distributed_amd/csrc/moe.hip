@@ -954,11 +954,63 @@ static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, 
   return launch_status(who);
 }
 
+// ---- the index build without a caller's workspace ---------------------------------------------------------
+// Scratch for tdist_moe_scatter_index_static: every GPU the library runs on holds its own copy of this array until the
+// process ends. Host code never uses the array's name as an address: the per-device address comes from
+// hipGetSymbolAddress, once per device, and is what the kernels are given.
+constexpr int64_t kMoeStaticScratchBytes = 1 << 20;
+static __device__ __align__(256) unsigned char scratch[kMoeStaticScratchBytes];
+
+constexpr int kMoeMaxDevices = 64;
+static void* g_scratch_ptr[kMoeMaxDevices];   // device address of `scratch` per device, NULL until looked up
+static std::mutex g_scratch_mutex;
+
+// Device address of the current device's copy of `scratch` (looked up on first use, with that device current).
+static int moe_static_scratch(void** out, const char* who) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMoeMaxDevices)
+    return fail(TDIST_ERR_DEVICE, "%s: no current device (or more than %d devices)", who, kMoeMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(TDIST_ERR_DEVICE, "%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return TDIST_OK;
+}
+
+int moe_static_scratch_init() {
+  void* ptr = nullptr;
+  return moe_static_scratch(&ptr, "tdist_init");
+}
+
 }  // namespace tdist
 
 using namespace tdist;
 
 extern "C" {
+
+int tdist_moe_scatter_index_static(const int32_t* ids, int64_t n_ids, int topk, int num_experts, int32_t* splits,
+                                   int32_t* cumsum, int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx,
+                                   void* stream) {
+  const char* who = "tdist_moe_scatter_index_static";
+  const int64_t need = tdist_moe_workspace_bytes(n_ids, num_experts);
+  if (need <= 0) return fail(TDIST_ERR_INVALID, "%s: bad sizes", who);
+  if (need > kMoeStaticScratchBytes)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: %lld ids over %d experts need %lld bytes of scratch, the built-in buffer holds "
+                "%lld (use tdist_moe_scatter_index with a workspace)", who, (long long)n_ids, num_experts, (long long)need,
+                (long long)kMoeStaticScratchBytes);
+  void* ws = nullptr;
+  if (int rc = moe_static_scratch(&ws, who)) return rc;
+  // (the control words are the array's first 256 bytes whatever the call's sizes; they are zero between calls: the
+  // kernels leave them so, and the array starts out zero. The rest needs no clearing, every word is written before it
+  // is read, so a call after a larger one is not disturbed by what that one left behind.)
+  return moe_index_common(ids, n_ids, topk, num_experts, splits, cumsum, scatter_idx, gather_idx, topk_idx, ws, need,
+                          (hipStream_t)stream, true, who);
+}
 
 int64_t tdist_moe_workspace_bytes(int64_t n_ids, int num_experts) {
   if (n_ids < 0 || num_experts <= 0) return 0;

@@ -45,6 +45,7 @@ PROTOTYPES = {
     "tdist_moe_workspace_bytes": (_L, [_L, _I]),
     "tdist_moe_splits_cumsum": (_I, [_P, _L, _I, _P, _P, _P, _L, _P]),
     "tdist_moe_scatter_index": (_I, [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _L, _P]),
+    "tdist_moe_scatter_index_static": (_I, [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P]),
     "tdist_moe_dispatch": (_I, [_P, _L, _P, _P, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_dispatch_tokens": (_I, [_P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_post_process": (_I, [_P, _L, _P, _P, _L, _I, _I, _I, _P, _P, _P]),
