@@ -119,9 +119,10 @@ int tdist_producer_push_chunk(void* dst, const void* src, int64_t nbytes, int32_
  * system scope) — the data-then-flag protocol of kernels/amd/all_gather_gemm.py:80-100.
  * peer_src: device array of world_size device pointers (entry `rank` unused). counters: int32
  * [world_size*chunks_per_rank], zero on entry, left zero. held: optional int32 mask of chunks never to deliver
- * (test hook for the consumer's bounded wait). stamp + ns_per_chunk > 0: chunk c of every peer is held back
- * until (c+1)*ns_per_chunk after the stamp (tdist_producer_mark), the pace of one link per peer; the total must
- * stay within 100 ms. The kernel needs 32 registers per lane and no LDS, so its waves fit on a SIMD beside a
+ * (test hook for the consumer's bounded wait). stamp + ns_per_chunk > 0: the pace of one link per peer: chunk c of
+ * every peer is copied from c*ns_per_chunk after the stamp (tdist_producer_mark) on and its flag is released no
+ * earlier than (c+1)*ns_per_chunk after it, when a link of that rate would have delivered the chunk's last byte; the
+ * total must stay within 100 ms. The kernel needs 32 registers per lane and no LDS, so its waves fit on a SIMD beside a
  * resident wave of the consumer GEMM; nothing in it waits for another workgroup. */
 int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int world_size, int rank,
                               int64_t rank_bytes, int64_t chunk_bytes, int32_t* flags, int flag_value,
@@ -338,27 +339,22 @@ int tdist_group_gemm_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
  * tdist_group_gemm_gated_*): their sk_workspace / sk_workspace_bytes arguments. Optional (NULL, 0). The reference's
  * kernels run whole tiles per program in a fixed order and leave a last round that does not fill the grid to the
  * autotuner's tile choice (kernels/amd/all_gather_gemm.py:151-246 persistent loop;
- * kernels/nvidia/allgather_group_gemm.py:238-314). With a workspace:
- *   - a last round of tiles that fills at most half of the grid is cut along K: each of its tiles goes to s = 2, 4 or
- *     8 workgroups (pieces of at least 4 K tiles); every piece's fp32 accumulators go through the workspace, and each
- *     of the s workgroups adds up and stores 1/s of the tile, the pieces in their K order (same products, another
- *     order of the sums than a whole tile's: results stay within the stated tolerance, are exact on integer-valued
- *     inputs and do not depend on timing);
- *   - the chunk-gated GEMM (flags != NULL, at most 64 chunks) schedules by arrival: a round of tiles is made up, when
- *     the workgroups get to it, of the chunks whose flags are set by then, in the order given by chunk_order / rank;
- *     when fewer tiles are ready than half of the workgroups, they are cut along K as above instead of leaving
- *     workgroups idle until the next chunk lands. Without a workspace the tiles are taken in the fixed order and each
- *     workgroup waits for its own tile's flag, as in the reference.
+ * kernels/nvidia/allgather_group_gemm.py:238-314). With a workspace,
+ * a last round of tiles that fills at most half of the grid is cut along K: each of its tiles goes to s = 2, 4 or 8
+ * workgroups (pieces of at least 4 K tiles); every piece's fp32 accumulators go through the workspace, and each of the
+ * s workgroups adds up and stores 1/s of the tile, the pieces in their K order (same products, another order of the
+ * sums than a whole tile's: results stay within the stated tolerance, are exact on integer-valued inputs and do not
+ * depend on timing). Whole rounds run as before.
  * Bounded waits as for the chunk flags: an exchange that does not complete sets status to
  * {TDIST_ERR_TIMEOUT, -1 - workgroup} and the tile is not stored.
  * The workspace is plain device memory, 256-byte aligned, of at least tdist_gemm_split_k_workspace_bytes() bytes (one
- * fp32 256 x 256 tile per compute unit + a 20 KiB header: 64 MiB + 20 KiB on MI355X; 0 if the device is not gfx950),
+ * fp32 256 x 256 tile per compute unit + a 12 KiB header: 64 MiB + 12 KiB on MI355X; 0 if the device is not gfx950),
  * ZERO when it is first used; the kernels keep it consistent from then on (also across a launch that timed out). It
  * carries no state that the library holds: any number of workspaces may be in use, one per launch in flight —
  * launches that share one must be ordered (same stream, or events). A workspace that is misaligned or smaller than
  * the header plus one 128 x 128 tile is rejected (TDIST_ERR_WORKSPACE); one too small for the call's tiles and grid
  * is left unused.
- * TDIST_GEMM_SPLIT_K=0 in the environment turns both uses off, =1 splits a last round wherever it can be split. */
+ * TDIST_GEMM_SPLIT_K=0 in the environment turns the split off, =1 takes it wherever a last round can be split. */
 int64_t tdist_gemm_split_k_workspace_bytes(void);
 
 /* ---------------------------------------------------------------------------------------------

@@ -217,7 +217,7 @@ def test_workspace_argument_errors(cuda):
     from triton_dist.kernels.amd import gated_gemm
     lib = _lib.load()
     need = lib.tdist_gemm_split_k_workspace_bytes()
-    assert need == 20480 + lib.tdist_num_cus() * 256 * 256 * 4
+    assert need == 12288 + lib.tdist_num_cus() * 256 * 256 * 4
     a = torch.zeros((128, 64), dtype=torch.bfloat16, device=cuda)
     c = torch.zeros((128, 128), dtype=torch.bfloat16, device=cuda)
     buf = torch.zeros(1 << 20, dtype=torch.uint8, device=cuda)

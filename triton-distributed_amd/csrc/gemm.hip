@@ -74,8 +74,7 @@ struct GemmParams {
   // its s readers have acknowledged (ack [workgroup] counts them). Tags are unique per launch and round: the header
   // word kSkCtrlEpoch is read at the start and advanced by the last workgroup to leave, so nothing has to be cleared
   // between launches, a launch that ran into a timeout included. Launches that share a workspace must not overlap.
-  //   sk_mode 1: static schedule, only a last round that fills at most half of the grid is split;
-  //   sk_mode 2: dynamic rounds (chunk-gated calls): see the scheduler in the kernel.
+  // Only a last round that fills at most half of the grid is split (sk_mode 1; 0 = no workspace in use).
   // (Cutting every tile of the schedule into equal shares of K tiles, "stream-K", was measured slower than whole
   // tiles: workgroups that share an operand panel are then at different K positions, and the panel is fetched once
   // per workgroup instead of once per XCD.)
@@ -90,11 +89,9 @@ constexpr int kSkCtrlDone = 1;           // workgroups of the running launch tha
 constexpr int kSkMaxWorkgroups = 1024;
 constexpr int kSkFlagsOff = 1024;        // [kSkMaxWorkgroups] tag of the partial in the slot
 constexpr int kSkAcksOff = 2048;         // [kSkMaxWorkgroups] readers that are done with the slot, ever
-constexpr int kSkDecOff = 3072;          // [kSkMaxDecisions][kSkDecWords] scheduler decisions of the running launch
-constexpr int kSkMaxDecisions = 256, kSkDecWords = 8;
-constexpr int kSkHeaderWords = kSkDecOff + kSkMaxDecisions * kSkDecWords;
+constexpr int kSkHeaderWords = 3072;
 constexpr int64_t kSkHeaderBytes = (int64_t)kSkHeaderWords * 4;
-constexpr int kSkTagStride = 1024;       // tags per launch (rounds that may be split or decided)
+constexpr int kSkTagStride = 16;         // tags per launch (rounds that may be split)
 static_assert(kSkHeaderBytes % 256 == 0, "the partial slots start 256-byte aligned");
 
 // Operand fragment of one lane: K bytes [0, kLaneBytes) of one row; chunk0 / chunk1 are LDS addresses of its
@@ -362,6 +359,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   // ---- workspace state of this launch ---------------------------------------------------------------------
   int32_t* const sk_flags = p.sk_ctrl + kSkFlagsOff;
   int32_t* const sk_acks = p.sk_ctrl + kSkAcksOff;
+  // the workgroups of one XCD hold a contiguous range of positions (see wg_pos): pieces of a tile share an XCD when
+  // the pieces per tile (2, 4 or 8) divide the workgroups per XCD
+  const bool sk_xcd_local = p.num_xcds > 1 && G % p.num_xcds == 0 && (G / p.num_xcds) % kSkMaxSplit == 0;
   int tag_base = 0;   // tags of this launch are tag_base + 1 + round
   int sk_need = 0;    // value of this workgroup's ack word once every reader of its last partial is done
   if (p.sk_mode != 0) {
@@ -381,9 +381,10 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 
   int sbase = 0;
   for (;;) {
-    // ---- next piece of work: K tiles [ka, kb) of scheduled tile sidx, as piece sk_j of sk_s --------------
-    int sidx, ka = 0, kb = KT, sk_s = 1, sk_j = 0, sk_tag = 0;
+    // ---- next piece of work: K tiles [ka, kb) of tile `within` of chunk position oc, as piece sk_j of sk_s -----
+    int oc, within, ka = 0, kb = KT, sk_s = 1, sk_j = 0, sk_tag = 0;
     {
+      int sidx;
       if (sbase >= total_sched) break;
       const int round_base = sbase;
       sbase += G;
@@ -401,10 +402,10 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         sidx = round_base + wg_pos;
         if (sidx >= total_sched) continue;
       }
+      oc = sidx / tiles_per_chunk;
+      within = sidx - oc * tiles_per_chunk;
     }
     const int KTp = kb - ka;
-    const int oc = sidx / tiles_per_chunk;
-    const int within = sidx - oc * tiles_per_chunk;
     const int chunk = kGrouped ? (oc + p.first_block) % n_chunks : chunk_of(p, oc);
     const int pid_m = chunk * cm + within % cm;
     const int pid_n = within / cm;
@@ -918,8 +919,13 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       const int slot_ok = *s_gate;
       __syncthreads();
       sk_need += sk_s;
+
       if (slot_ok) {
-        // (2) the partial, coherent at device scope, every store instruction a contiguous KiB.
+        // (2) the partial, every store instruction a contiguous KiB. The pieces of a tile sit on workgroups s*t ..
+        // s*t+s-1 of the round, which the XCD-aware order puts on ONE XCD whenever s divides the workgroups per XCD:
+        // the partials then need to go no further than that XCD's L2 (plain stores; the readers invalidate their
+        // own first-level cache and find the lines in the L2 they share with the writers). Otherwise the stores are
+        // coherent at device scope (written through to memory).
         // The store sits in inline assembly (the cache-policy bit has no builtin), where the compiler sees neither
         // a memory instruction nor its hazards. Hence: a vector address (a scalar base that the compiler happened
         // to reload from a spill lane with v_readlane would need five wait states before the store), and a wait
@@ -928,7 +934,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         static_for<kQuads>([&](auto r_c) {
           constexpr int r = decltype(r_c)::value;
           const float4v t = acc4(std::integral_constant<int, r / kGroups>{}, std::integral_constant<int, r % kGroups>{});
-          asm volatile("s_nop 1\n\tglobal_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(slot), "v"(t) : "memory");
+          if (sk_xcd_local) asm volatile("s_nop 1\n\tglobal_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(slot), "v"(t) : "memory");
+          else asm volatile("s_nop 1\n\tglobal_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(slot), "v"(t) : "memory");
           slot += kThreads * 16;
           asm volatile("" : "+v"(slot));  // one running address, not sixty-four precomputed ones
           if constexpr (r % 4 == 3) __builtin_amdgcn_sched_barrier(0);
@@ -937,6 +944,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         __syncthreads();
         if (threadIdx.x == 0) __hip_atomic_store(sk_flags + wg_pos, sk_tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
+
       // (3) all pieces of the tile: thread i waits for the flag of piece i. (The full limit even after an error
       // elsewhere: these pieces are being computed, not awaited from outside; if a workgroup gave its piece up at a
       // chunk flag, the wait runs out and the tile is not stored.)
@@ -964,7 +972,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       const int pieces_ok = *s_gate;
       __syncthreads();
       if (!pieces_ok) continue;
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      // acquire: pieces from this XCD are in its L2 once their flags are up, so dropping this compute unit's own
+      // first-level lines is all it takes (a device-scope acquire would also sweep the whole L2, once per wave)
+      if (sk_xcd_local) asm volatile("buffer_inv sc0" ::: "memory");
+      else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+
       // (4) this workgroup's share of the sum: float4 groups [q0, q0 + nq) of every lane, over the sk_s slots in slot
       // order, packed into the staging rows as the plain epilogue packs them
       const int nq = kQuads / sk_s, q0 = sk_j * nq;
@@ -1006,6 +1018,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       // the slots have been read: acknowledge to their writers
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
+
       if ((int)threadIdx.x < sk_s) __hip_atomic_fetch_add(sk_acks + w0 + threadIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       // (5) the staged share → C. It is whole 32-row blocks of the wave tile, or a column range of one block:
       // float4 groups [g0, g0 + n) of a row block are its 16-byte pieces [g0, g0 + n).
@@ -1023,6 +1036,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
           store_piece_at(mrow, s_ec, staged_piece_at(mrow, s_ec));
         }
       }
+
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       continue;
     }
@@ -1174,8 +1188,6 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         // tags start over: no word may still hold a value that a tag will take again
         next = 0;
         for (int i = 0; i < kSkMaxWorkgroups; ++i) __hip_atomic_store(sk_flags + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (int i = 0; i < kSkMaxDecisions; ++i)
-          __hip_atomic_store(p.sk_ctrl + kSkDecOff + i * kSkDecWords, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       __hip_atomic_store(p.sk_ctrl + kSkCtrlEpoch, next, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }

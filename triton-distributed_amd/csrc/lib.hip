@@ -113,9 +113,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(24))) void prod
   for (int c = 0; c < p.chunks_per_rank; ++c) {
     const int chunk_pos = r * p.chunks_per_rank + c;
     if (p.held != nullptr && p.held[chunk_pos] != 0) continue;
-    if (p.stamp != nullptr) {
+    // Pacing: over a link the last byte of the peer's chunk c lands (c+1) chunk times after the start. The rows
+    // are therefore copied when their turn comes (they are "on the wire" once chunk c-1 is through) and the flag is
+    // held back until the chunk's arrival time: what the consumer sees is a chunk that is complete at that time.
+    if (p.stamp != nullptr && c > 0) {
       if (threadIdx.x == 0) {
-        const unsigned long long due = (unsigned long long)(c + 1) * p.ticks_per_chunk;
+        const unsigned long long due = (unsigned long long)c * p.ticks_per_chunk;
         while (true) {
           const unsigned long long now = wall_clock64();
           if (now - t0 >= due || now - begin >= due) break;
@@ -145,6 +148,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(24))) void prod
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
+      if (p.stamp != nullptr) {
+        const unsigned long long due = (unsigned long long)(c + 1) * p.ticks_per_chunk;
+        while (true) {
+          const unsigned long long now = wall_clock64();
+          if (now - t0 >= due || now - begin >= due) break;
+          __builtin_amdgcn_s_sleep(8);
+        }
+      }
       // one release per workgroup and chunk: writes this XCD's dirty lines (the workgroup's rows among them) back
       // to memory before the counter says that this part is in place
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");

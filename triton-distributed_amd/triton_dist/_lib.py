@@ -171,7 +171,7 @@ def bench_call(name, *args):
 
 def new_split_k_workspace(device=None):
     """A zero-filled workspace for the GEMM entry points' sk_workspace argument (tdist_gemm_split_k_workspace_bytes()
-    bytes: 64 MiB + 20 KiB on MI355X). Every context owns one: launches that share a workspace must be ordered, and
+    bytes: 64 MiB + 12 KiB on MI355X). Every context owns one: launches that share a workspace must be ordered, and
     contexts may run on streams of their own. Returns a uint8 tensor."""
     import torch
     dev = torch.cuda.current_device() if device is None else torch.device(device).index

@@ -144,9 +144,9 @@ class AllGatherGEMMTensorParallelContext:
     # units of this GPU; measured on MI355X they make no progress next to a full-chip persistent grid
     # unless 32 units stay free. A peer's copy engine pushing over xGMI would need none.
     producer_cus: int = 32
-    # The context's workspace for the GEMM (tdist_gemm_split_k_workspace_bytes() bytes, zero-filled once): with it the
-    # gated GEMM schedules its tiles by arrival and cuts tiles along K where workgroups would otherwise idle. It
-    # belongs to this context, so contexts on different streams never share scheduling state. None: fixed order.
+    # The context's workspace for the GEMM (tdist_gemm_split_k_workspace_bytes() bytes, zero-filled once): with it a
+    # last round of tiles that fills at most half of the grid is cut along K. It belongs to this context, so contexts
+    # on different streams share no state. None: whole tiles only.
     sk_workspace: Optional[torch.Tensor] = None
 
     def update(self, rank, num_ranks, BLOCK_M=128, BLOCK_N=256, BLOCK_K=64, stages=3, ag_streams=None, gemm_stream=None,
@@ -193,8 +193,7 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
 
     ``tp_group`` may be None: one GPU holds the only real rank. BLOCK_*/stages/autotune are accepted for
     signature compatibility; the HIP kernel picks its own tiling. ``split_k``: give the context a workspace
-    (64 MiB) with which the gated GEMM schedules its tiles by arrival and cuts tiles along K where workgroups would
-    otherwise stand idle; False keeps the reference's fixed tile order.
+    (64 MiB) with which a last round of tiles that fills at most half of the grid is cut along K.
     """
     assert M_PER_CHUNK % BLOCK_M == 0
     assert max_M % num_ranks == 0
