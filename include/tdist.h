@@ -74,8 +74,13 @@ int tdist_num_cus(void);
  *   max_workgroups  upper bound on the persistent grid; <= 0: one workgroup per compute unit. A producer
  *         whose copies run on this same GPU needs compute units of its own while the GEMM spins on a flag:
  *         leave it 32 (pass tdist_num_cus() - 32). Not needed when the rows arrive from a peer's copy engine.
- * Requirements: K * element size a multiple of 64 bytes, lda/ldb multiples of 8 (16 for fp8) elements,
- * 16-byte aligned bases, m_per_chunk % 128 == 0 when flags != NULL (% 256 selects the large tile).
+ * Requirements: K, lda and ldb multiples of 8 (16 for fp8) elements and 16-byte aligned bases. The large tiles are
+ * taken when K * element size is a multiple of 128 bytes and the row blocks (m_per_chunk, the local shard) are
+ * multiples of 256 rows; a K that ends inside a 64-byte K tile is filled up with zeros on its way in.
+ * m_per_chunk may be any positive number of rows: when it is not a multiple of 128, a tile waits for every chunk its
+ * rows touch (the reference's per-segment wait, kernels/nvidia/allgather_gemm.py:222-224), tiles are visited in row
+ * order starting inside the own rank's rows, chunk_order must be NULL and the local shard must either start and end
+ * on a multiple of 128 rows or be copied into A with its flags set (A_local = NULL).
  * ------------------------------------------------------------------------------------------- */
 int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                 int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,

@@ -315,7 +315,7 @@ def test_large_tiles_with_ragged_edges_and_padded_rows(cuda, M, N, K, pad):
 
 
 def test_randomised_shapes_gating_and_layouts(cuda):
-    """Forty seeded random cases over both tile paths: ragged M / N, K in 64-byte steps, padded row strides, the three
+    """Forty seeded random cases over both tile paths: ragged M / N, K in 64- or 16-byte steps, padded row strides, the three
     dtypes, gating with a local shard and pre-released flags in either chunk order, plain calls. Integer-valued inputs,
     so the only rounding is the final one."""
     import random
@@ -326,11 +326,11 @@ def test_randomised_shapes_gating_and_layouts(cuda):
         esz = 1 if dtype == torch.float8_e4m3fn else 2
         big = rnd.random() < 0.4
         gated = rnd.random() < 0.5
-        K = rnd.randrange(1, 9) * 64 // esz
+        K = rnd.randrange(1, 9) * 64 // esz if rnd.random() < 0.6 else rnd.randrange(1, 40) * 16 // esz
         pad_a, pad_b = rnd.choice([0, 16, 64]), rnd.choice([0, 16, 128])
         if gated:
             world = rnd.choice([2, 4, 8])
-            mpc = rnd.choice([256, 512]) if big else rnd.choice([128, 256, 384])
+            mpc = rnd.choice([256, 512]) if big else rnd.choice([128, 256, 384, 40, 200])
             cpr = rnd.choice([1, 2])
             M = world * cpr * mpc
             N = rnd.randrange(20, 30) * 256 - rnd.choice([0, 8, 100]) if big else rnd.randrange(1, 700)
@@ -353,7 +353,10 @@ def test_randomised_shapes_gating_and_layouts(cuda):
             mpr = M // world
             local = a_d[rank * mpr:(rank + 1) * mpr].contiguous()
             ws = a_d.clone()
-            ws[rank * mpr:(rank + 1) * mpr] = 0      # the own rows must come from the local shard
+            if mpc % 128 == 0:
+                ws[rank * mpr:(rank + 1) * mpr] = 0      # the own rows must come from the local shard
+            else:
+                local = None                              # (chunks that are no whole tiles: everything through the flags)
             flags = torch.ones(world * cpr, dtype=torch.int32, device=cuda)
             gated_gemm(ws, local, rank * mpr, b_d, c, flags, mpc, rank, world)
         else:
@@ -488,15 +491,83 @@ def test_nvidia_side_signatures(cuda, m_per, K):
     assert out.shape == (m_per, N)
     assert golden.max_rel_err(out.float().cpu(), golden.gemm_rs_fp32(a, b, peers, rank, W)) <= 1e-2
     # AG-GEMM gated per rank segment
-    if m_per % 128 == 0:
-        shards, bb = make_ag_case(W, m_per, K, N, torch.bfloat16, seed=K)
-        actx = create_ag_gemm_intra_node_context(shards[rank].to(cuda), bb.to(cuda), rank, W)
-        assert actx.barrier_tensors[rank].numel() == W and actx.M_PER_CHUNK == m_per
-        actx.set_peer_shards({r: s.to(cuda) for r, s in enumerate(shards) if r != rank})
+    # (rank segments of 200 and 72 rows are no whole tiles: a tile then waits for every segment it touches)
+    shards, bb = make_ag_case(W, m_per, K, N, torch.bfloat16, seed=K)
+    actx = create_ag_gemm_intra_node_context(shards[rank].to(cuda), bb.to(cuda), rank, W)
+    assert actx.barrier_tensors[rank].numel() == W and actx.M_PER_CHUNK == m_per
+    actx.set_peer_shards({r: s.to(cuda) for r, s in enumerate(shards) if r != rank})
+    for _ in range(2):   # (the second call finds the flags reset by the first)
+        actx.workspace_tensors[rank].view(torch.uint8).fill_(0x7B)
         c = ag_gemm_intra_node(shards[rank].to(cuda), bb.to(cuda), actx)
         actx.check_status()
         assert golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32(shards, bb)) <= 1e-2
-    else:
-        with pytest.raises(NotImplementedError):
-            create_ag_gemm_intra_node_context(torch.zeros((m_per, K), dtype=torch.bfloat16, device=cuda),
-                                              torch.zeros((N, K), dtype=torch.bfloat16, device=cuda), rank, W)
+
+
+@pytest.mark.parametrize("dtype,K", [(torch.bfloat16, 8), (torch.bfloat16, 40), (torch.float16, 72), (torch.bfloat16, 200),
+                                     (torch.bfloat16, 1000), (torch.float8_e4m3fn, 16), (torch.float8_e4m3fn, 80),
+                                     (torch.float8_e4m3fn, 1008), (torch.float16, 4104)])
+def test_k_ending_inside_a_k_tile(cuda, dtype, K):
+    """K rows of any whole number of 16-byte pieces: the last K tile is filled up with zeros on its way into the LDS.
+    The bytes behind a row's end are poisoned with NaN, so a lane that read them would show. Integer-valued inputs:
+    exact up to the final rounding. With and without a split last round."""
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import gated_gemm
+    announce("gemm K tail K=%d %s" % (K, dtype))
+    esz = 1 if dtype == torch.float8_e4m3fn else 2
+    pad = 48 // esz
+    out_dtype = torch.float16 if dtype == torch.float16 else torch.bfloat16
+    # (2176 x 2048 is 272 tiles: with the workspace and a long K the last 16 are cut along K)
+    for M, N, ws in [(300, 200, None), (1100, 1290, None), (2176, 2048, _lib.new_split_k_workspace(cuda))]:
+        g = torch.Generator().manual_seed(K + M)
+        a = torch.randint(-2, 3, (M, K + pad), generator=g).float()
+        b = torch.randint(-2, 3, (N, K + pad), generator=g).float()
+        a_d, b_d = a.to(dtype).to(cuda), b.to(dtype).to(cuda)
+        for t in (a_d, b_d):
+            if esz == 1:
+                t.view(torch.uint8)[:, K:] = 0x7F
+            else:
+                t.view(torch.int16)[:, K:] = 0x7FC0
+            assert torch.isnan(t[:, K:].float()).all()
+        c = torch.full((M, N), float("nan"), dtype=out_dtype, device=cuda)
+        gated_gemm(a_d[:, :K], None, 0, b_d[:, :K], c, None, 0, 0, 1, sk_workspace=ws)
+        torch.cuda.synchronize()
+        ref = a[:, :K].to(cuda) @ b[:, :K].to(cuda).T
+        assert torch.equal(c, ref.to(out_dtype)), "M=%d N=%d differs" % (M, N)
+    with pytest.raises(_lib.TdistError, match="16 bytes"):
+        gated_gemm(a_d[:, :K - 4 // esz], None, 0, b_d[:, :K - 4 // esz], c, None, 0, 0, 1)
+
+
+@pytest.mark.parametrize("world,mpc,rank", [(4, 200, 1), (8, 72, 7), (2, 1000, 0), (3, 130, 2)])
+def test_chunks_that_are_no_whole_tiles(cuda, world, mpc, rank):
+    """m_per_chunk of any size: a 128-row tile waits for every flag its rows touch. With every flag but one released,
+    exactly the tiles that hold rows of the withheld chunk give up (bounded wait, status names that chunk) and every
+    other row of C is right; with all flags released the whole result is."""
+    from triton_dist.kernels.amd import gated_gemm
+    announce("gemm ragged chunks world=%d mpc=%d rank=%d" % (world, mpc, rank))
+    M, N, K = world * mpc, 328, 160
+    g = torch.Generator().manual_seed(mpc)
+    a = torch.randint(-2, 3, (M, K), generator=g).float()
+    b = torch.randint(-2, 3, (N, K), generator=g).float()
+    a_d, b_d = a.to(torch.bfloat16).to(cuda), b.to(torch.bfloat16).to(cuda)
+    ref = (a.to(cuda) @ b.to(cuda).T).to(torch.bfloat16)
+    status = torch.zeros(2, dtype=torch.int32, device=cuda)
+    flags = torch.ones(world, dtype=torch.int32, device=cuda)
+    c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+    gated_gemm(a_d, None, 0, b_d, c, flags, mpc, rank, world, status=status)
+    torch.cuda.synchronize()
+    assert status.tolist() == [0, 0] and torch.equal(c, ref)
+    held = (rank + 1) % world
+    flags[held] = 0
+    c.fill_(float("nan"))
+    gated_gemm(a_d, None, 0, b_d, c, flags, mpc, rank, world, status=status, spin_limit=200)
+    torch.cuda.synchronize()
+    from triton_dist import _lib
+    assert status.tolist() == [_lib.TDIST_ERR_TIMEOUT, held]
+    rows = torch.arange(M, device=cuda)
+    tile_lo, tile_hi = rows // 128 * 128, torch.clamp(rows // 128 * 128 + 127, max=M - 1)
+    touches = (tile_lo // mpc <= held) & (tile_hi // mpc >= held)
+    assert torch.equal(c[~touches], ref[~touches])
+    assert torch.isnan(c[touches].float()).all()
+    # a local shard that is no whole number of tiles cannot be handed in beside such chunks
+    with pytest.raises(_lib.TdistError, match="local shard"):
+        gated_gemm(a_d, a_d[rank * mpc:(rank + 1) * mpc], rank * mpc, b_d, c, flags, mpc, rank, world)

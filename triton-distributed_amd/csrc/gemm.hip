@@ -50,6 +50,9 @@ struct GemmParams {
   int local_row_begin, local_rows;
   int m_per_chunk;   // rows per schedule chunk (multiple of BM)
   int n_chunks;      // ceil(M / m_per_chunk)
+  int gate_rows;     // rows per flag word: m_per_chunk, or (ragged chunks, walked in row order) any positive number:
+                     // a tile then waits for every flag its rows touch
+  int k_tail_bytes;  // bytes of K in the last K tile when K is not a whole number of them (128 x 128 tile only), else 0
   int chunks_per_rank;
   int wait_value;
   int rank, world_size;
@@ -301,6 +304,9 @@ __device__ __forceinline__ void acc_clear() {
   static_for<kN>([&](auto r_c) { asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(decltype(r_c)::value)); });
 }
 
+// what the DMA lanes of a ragged last K tile read for the bytes of K that do not exist
+static __device__ __align__(16) const unsigned char kZeroChunk[16] = {0};
+
 // schedule position → chunk id
 __device__ __forceinline__ int chunk_of(const GemmParams& p, int oc) {
   switch (p.order_mode) {
@@ -347,7 +353,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   if constexpr (kGrouped) n_chunks = min(n_chunks, __builtin_nontemporal_load(p.post_pad) / BM);
   const int total_sched = n_chunks * tiles_per_chunk;
   const int G = gridDim.x;
-  const int KT = p.K * E::kBytes / KB;
+  const int KT = (p.K * E::kBytes + KB - 1) / KB;   // (a ragged last K tile only on the plain ring: see k_tail_bytes)
 
   // DMA lane roles: row within an instruction's row group, and the LDS chunk position it fills
   const int dma_row = lane / C::kChunksPerRow;
@@ -422,23 +428,33 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
                                    : (p.A_local != nullptr && m0 >= p.local_row_begin && m0 < p.local_row_begin + p.local_rows);
     if (p.flags != nullptr && !is_local) {
       if (threadIdx.x == 0) {
-        const int32_t* f = p.flags + (kGrouped ? segment : chunk);
-        int ok = 0;
+        // the flags of the tile's rows: one (the tile lies inside a chunk), or, with ragged chunks, every flag from
+        // the first row's to the last row's (the reference's NVIDIA-side kernel waits for a range of rank segments
+        // in the same way, kernels/nvidia/allgather_gemm.py:222-224)
+        int f_lo = kGrouped ? segment : chunk, f_hi = f_lo;
+        if (!kGrouped && p.gate_rows != p.m_per_chunk) {
+          f_lo = m0 / p.gate_rows;
+          f_hi = min(m0 + BM - 1, p.M - 1) / p.gate_rows;
+        }
+        int ok = 1;
         int limit = p.spin_limit;
         if (p.status != nullptr && __hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) limit = 1;
-        // poll with plain coherent loads and acquire once, after the flag has been seen: an acquiring load
+        // poll with plain coherent loads and acquire once, after the flags have been seen: an acquiring load
         // invalidates this CU's and this XCD's caches every time it is executed
-        for (int it = 0; it < limit; ++it) {
-          if (__hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == p.wait_value) {
-            ok = 1;
-            break;
+        for (int f = f_lo; f <= f_hi && ok; ++f) {
+          ok = 0;
+          for (int it = 0; it < limit; ++it) {
+            if (__hip_atomic_load(p.flags + f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == p.wait_value) {
+              ok = 1;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(4);
           }
-          __builtin_amdgcn_s_sleep(4);
+          if (!ok && p.status != nullptr) {
+            if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = f;
+          }
         }
         if (ok) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-        if (!ok && p.status != nullptr) {
-          if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = kGrouped ? segment : chunk;
-        }
         *s_gate = ok;
       }
       __syncthreads();
@@ -502,11 +518,33 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
                    : "memory");
     };
+    // A ragged last K tile (plain ring only): the lanes whose 16 bytes of K lie beyond the row's end fetch zeros from
+    // kZeroChunk instead, through the load's 64-bit address form (the zero page is not within reach of a 32-bit
+    // offset from the operand). Only the tile that holds the end of K takes this path.
+    auto dma16_tail = [&](const unsigned char* sbase, uint32_t voff, int r, lds_u8 dst) {
+      const int chunk = dma_pos ^ swz<KB>(r);   // which 16 bytes of the K tile this lane fetches
+      const unsigned char* src = chunk * 16 < p.k_tail_bytes ? sbase + voff : kZeroChunk;
+      __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)src, (TDIST_AS3 void*)dst, 16, 0, 0);
+    };
     auto issue_a = [&](int kt, int t) {
-      dma16(a_base + (int64_t)min(kt, KTp - 1) * KB, a_off[t], a_stage(kt) + (wave * C::kAInstr + t) * 1024);
+      lds_u8 const dst = a_stage(kt) + (wave * C::kAInstr + t) * 1024;
+      if constexpr (!C::kSplit) {
+        if (p.k_tail_bytes != 0 && kb == KT && kt >= KTp - 1) {
+          dma16_tail(a_base + (int64_t)(KTp - 1) * KB, a_off[t], (wave * C::kAInstr + t) * C::kRowsPerInstr + dma_row, dst);
+          return;
+        }
+      }
+      dma16(a_base + (int64_t)min(kt, KTp - 1) * KB, a_off[t], dst);
     };
     auto issue_b = [&](int kt, int u) {
-      dma16(b_base + (int64_t)min(kt, KTp - 1) * KB, b_off[u], b_stage(kt) + (wave * C::kBInstr + u) * 1024);
+      lds_u8 const dst = b_stage(kt) + (wave * C::kBInstr + u) * 1024;
+      if constexpr (!C::kSplit) {
+        if (p.k_tail_bytes != 0 && kb == KT && kt >= KTp - 1) {
+          dma16_tail(b_base + (int64_t)(KTp - 1) * KB, b_off[u], (wave * C::kBInstr + u) * C::kRowsPerInstr + dma_row, dst);
+          return;
+        }
+      }
+      dma16(b_base + (int64_t)min(kt, KTp - 1) * KB, b_off[u], dst);
     };
     auto issue_dma = [&](int kt, int t) {
       if (t < C::kAInstr) issue_a(kt, t);
@@ -1276,11 +1314,18 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   const int esz = elem == kElemFP8 ? 1 : 2;
   if (!c.A || !c.B || (!c.C && !c.scatter_bufs)) return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
   if (c.M <= 0 || c.N <= 0 || c.K <= 0) return fail(TDIST_ERR_INVALID, "%s: M, N, K must be positive", who);
-  if (((int64_t)c.K * esz) % 64 != 0)
-    return fail(TDIST_ERR_UNSUPPORTED, "%s: K*elem_size = %lld must be a multiple of 64 bytes", who, (long long)c.K * esz);
+  if (((int64_t)c.K * esz) % 16 != 0)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: K*elem_size = %lld must be a multiple of 16 bytes", who, (long long)c.K * esz);
   if (!aligned16(c.A) || !aligned16(c.B) || (c.A_local && !aligned16(c.A_local)) || (c.lda * esz) % 16 ||
       (c.ldb * esz) % 16 || (c.A_local && (c.lda_local * esz) % 16))
     return fail(TDIST_ERR_UNSUPPORTED, "%s: A/B bases and row strides must be 16-byte aligned", who);
+  // a K that ends inside a 64-byte K tile: the 128 x 128 tile fetches zeros for the rest of its last K tile
+  const int k_tail_bytes = (int)(((int64_t)c.K * esz) % 64);
+  // chunks that are not whole 128-row tiles: tiles are walked in row order from the own rank's rows on, and each
+  // waits for every flag its rows touch
+  const bool ragged = !c.scatter_bufs && c.flags && c.m_per_chunk > 0 && c.m_per_chunk % 128 != 0;
+  if (ragged && c.chunk_order)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: chunk_order needs m_per_chunk (%d) to be a multiple of 128 rows", who, c.m_per_chunk);
   if (c.lda < c.K || c.ldb < c.K || c.ldc < c.N) return fail(TDIST_ERR_INVALID, "%s: leading dimension smaller than row", who);
   if (c.lda * esz > (1 << 22) || c.ldb * esz > (1 << 22) || (c.A_local && c.lda_local * esz > (1 << 22)))
     return fail(TDIST_ERR_UNSUPPORTED, "%s: row strides above 4 MiB are not supported", who);
@@ -1295,6 +1340,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   bool rows256 = true;
   if (c.scatter_bufs && c.world_size > 0 && (c.M % c.world_size != 0 || (c.M / c.world_size) % 256 != 0)) rows256 = false;
   if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) rows256 = false;
+  if (k_tail_bytes != 0) rows256 = false;
   if (c.A_local && (c.local_row_begin % 256 != 0 || c.local_rows % 256 != 0)) rows256 = false;
   if (((int64_t)c.K * esz) % 128 != 0) rows256 = false;  // the split ring steps through K 128 bytes at a time
   int cap_wgs = di.num_cus;
@@ -1312,7 +1358,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
     if (kChoices[t].bm == 256 && !rows256) continue;
     const int bm = kChoices[t].bm, bn = kChoices[t].bn;
     const int64_t tiles = ceil_div(c.M, bm) * ceil_div(c.N, bn);
-    const int64_t kt = (int64_t)c.K * esz / (bm == 256 ? 128 : 64);
+    const int64_t kt = ceil_div((int64_t)c.K * esz, bm == 256 ? 128 : 64);
     const double per_k_tile = (double)bm * bn / kChoices[t].eff;
     const double cost = (double)ceil_div(tiles, cap_wgs) * kt * per_k_tile;
     if (best == 0 || cost < best) best = cost, pick = t, use_sk = false;
@@ -1331,7 +1377,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       pick = t;
       // (the split is re-derived for the forced tile)
       const int64_t tiles = ceil_div(c.M, kChoices[t].bm) * ceil_div(c.N, kChoices[t].bn);
-      const int64_t kt = (int64_t)c.K * esz / (kChoices[t].bm == 256 ? 128 : 64);
+      const int64_t kt = ceil_div((int64_t)c.K * esz, kChoices[t].bm == 256 ? 128 : 64);
       const int64_t tail = tiles % cap_wgs;
       use_sk = sk_mode != 0 && use_sk && tail > 0 && sk_split_for(cap_wgs, (int)tail, (int)kt) >= 2 &&
                sk_workspace_fits(c.sk_workspace, c.sk_workspace_bytes, cap_wgs, kChoices[t].bm, kChoices[t].bn);
@@ -1373,6 +1419,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   p.sk_ctrl = nullptr;
   p.sk_partials = nullptr;
   p.sk_mode = 0;
+  p.k_tail_bytes = k_tail_bytes;
 
   if (c.scatter_bufs) {
     if (c.world_size <= 0 || c.rank < 0 || c.rank >= c.world_size)
@@ -1385,6 +1432,18 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
     p.n_chunks = c.world_size;
     p.order_mode = 2;
     p.flags = nullptr;
+  } else if (ragged) {
+    if (c.A_local && (c.local_row_begin % BM != 0 || c.local_rows % BM != 0))
+      return fail(TDIST_ERR_UNSUPPORTED, "%s: with m_per_chunk %d (not a multiple of %d rows) the local shard must start and end "
+                  "on a %d-row tile, or be copied into A with its flag set", who, c.m_per_chunk, BM, BM);
+    p.m_per_chunk = BM;
+    p.n_chunks = (int)ceil_div(c.M, BM);
+    p.order_mode = 0;
+    if (c.world_size > 1 && c.rank >= 0 && c.rank < c.world_size) {
+      // start with the first tile that lies inside the own rank's rows
+      p.order_mode = 4;
+      p.first_block = (int)(ceil_div((int64_t)c.rank * c.M / c.world_size, BM) % p.n_chunks);
+    }
   } else if (c.flags) {
     if (c.m_per_chunk <= 0 || c.m_per_chunk % BM != 0)
       return fail(TDIST_ERR_UNSUPPORTED, "%s: m_per_chunk %d must be a positive multiple of the %d-row tile", who,
@@ -1410,6 +1469,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
     if (c.A_local && (c.local_row_begin % BM != 0 || c.local_rows % BM != 0))
       return fail(TDIST_ERR_UNSUPPORTED, "%s: the local shard must start and end on a %d-row tile", who, BM);
   }
+  p.gate_rows = ragged ? c.m_per_chunk : p.m_per_chunk;
   const int64_t sched = (int64_t)p.n_chunks * (p.m_per_chunk / BM) * ceil_div(c.N, BN);
   if (sched > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many tiles", who);
   int grid = (int)(sched < cap_wgs ? sched : cap_wgs);
@@ -1539,6 +1599,8 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   p.sk_ctrl = nullptr;
   p.sk_partials = nullptr;
   p.sk_mode = 0;
+  p.gate_rows = p.m_per_chunk;
+  p.k_tail_bytes = 0;
 
   const bool k128 = ((int64_t)c.K * esz) % 128 == 0;
   const int BN = (c.block_size == 256 || k128) ? 256 : 128;

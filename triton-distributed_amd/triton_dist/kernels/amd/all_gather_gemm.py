@@ -188,14 +188,17 @@ class AllGatherGEMMTensorParallelContext:
 
 def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, rank, num_ranks, tp_group,
                                       ag_streams=None, gemm_stream=None, M_PER_CHUNK=1024, BLOCK_M=128, BLOCK_N=256,
-                                      BLOCK_K=64, stages=3, serial=False, autotune=False, split_k=True):
+                                      BLOCK_K=64, stages=3, serial=False, autotune=False, split_k=True,
+                                      ragged_chunks=False):
     """create context for allgather gemm intra-node (reference :360-429).
 
     ``tp_group`` may be None: one GPU holds the only real rank. BLOCK_*/stages/autotune are accepted for
     signature compatibility; the HIP kernel picks its own tiling. ``split_k``: give the context a workspace
     (64 MiB) with which a last round of tiles that fills at most half of the grid is cut along K.
+    ``ragged_chunks``: M_PER_CHUNK need not be a multiple of BLOCK_M (the reference asserts that it is, :375); a
+    tile of the GEMM then waits for every chunk its rows touch, and the own shard goes through the workspace.
     """
-    assert M_PER_CHUNK % BLOCK_M == 0
+    assert ragged_chunks or M_PER_CHUNK % BLOCK_M == 0
     assert max_M % num_ranks == 0
     M_per_rank = max_M // num_ranks
     assert M_per_rank % M_PER_CHUNK == 0
@@ -340,9 +343,25 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
                 use_sdma=ctx.use_sdma if ctx is not None else True,
                 link_gbps=ctx.link_gbps if paced else 0.0, start_stamp=ctx.start_stamp if paced else None)
 
+    # Chunks that are not whole 128-row tiles: a tile may hold rows of the own shard and of a neighbour's, so the
+    # own rows are copied into the workspace and released through their flags like everyone else's (what the
+    # reference's producer does with every local shard, :268-272).
+    local = a
+    if M_PER_CHUNK % 128 != 0 or (rank * M_per_rank) % 128 != 0 or M_per_rank % 128 != 0:
+        local = None
+
     def call_gemm(max_wgs):
+        if local is None:
+            if not a.is_contiguous():
+                raise ValueError("the local shard must be contiguous")
+            first, per_rank = rank * M_per_rank, M_per_rank // M_PER_CHUNK
+            own_flags = barrier.data_ptr() + rank * per_rank * 4
+            _lib.call("tdist_producer_push_chunk", workspace.data_ptr() + first * K * a.element_size(), a.data_ptr(),
+                      a.numel() * a.element_size(), own_flags, one.data_ptr(), 0, gemm_stream.cuda_stream)
+            if per_rank > 1:
+                _lib.call("tdist_flag_fill", own_flags, per_rank, 1, gemm_stream.cuda_stream)
         # (the launch names its stream; nothing here runs on torch's current stream)
-        gated_gemm(workspace[:M], a, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
+        gated_gemm(workspace[:M], local, rank * M_per_rank, b, c, barrier, M_PER_CHUNK, rank, num_ranks,
                    row_scale=row_scale, col_scale=col_scale, wait_value=1,
                    spin_limit=ctx.spin_limit if ctx is not None else 0,
                    status=ctx.status if ctx is not None else None, max_workgroups=max_wgs,
