@@ -160,7 +160,8 @@ int tdist_flag_fill(int32_t* flags, int n, int value, void* stream);
  * [rank*M/world, (rank+1)*M/world) (gemm_reduce_scatter.py:222-229), every buffer [M, ldc].
  * scatter_bufs is a DEVICE array of world_size device pointers (the reference's scatter_bufs_ptr).
  * Tiles are visited starting with the rows of rank+1 (:171-180).
- * Requirements: M % (256*world_size) == 0, K % 64 == 0. */
+ * Requirements: M / world_size a multiple of 128 rows (of 256 for the large tiles), K and the row strides
+ * multiples of 8 elements (16 for fp8). */
 int tdist_gemm_rs_scatter_bf16(const void* A, int64_t lda, const void* B, int64_t ldb,
                                void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank,
                                int world_size,
@@ -169,6 +170,15 @@ int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t
                               void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank,
                               int world_size,
     void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
+
+/* fp8-e4m3 inputs, bf16 partial results: P = (sum_k A8*B8) * row_scale[m] * col_scale[n], scattered as above
+ * (row_scale fp32 [M], col_scale fp32 [N], either may be NULL = 1). The reference's kernel takes its output type from
+ * its input (gemm_reduce_scatter.py:217-218), which for e4m3 inputs would round the partial sums to e4m3 before they
+ * are added up; here they stay bf16, as in the fp8 AG-GEMM above, and go through tdist_reduce_slices like the others. */
+int tdist_gemm_rs_scatter_fp8e4m3(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                  void* const* scatter_bufs, int64_t ldc, int M, int N, int K,
+                                  const float* row_scale, const float* col_scale, int rank, int world_size,
+                                  void* sk_workspace, int64_t sk_workspace_bytes, void* stream);
 
 /* out[e] = round( sum_{i=0..n_slices-1} float(c[((i + first_slice) % n_slices) * slice_stride + e]) )
  * for e in [0, n_elems): fp32 accumulation in exactly that order (the reference's order is
@@ -378,9 +388,11 @@ int64_t tdist_gemm_split_k_workspace_bytes(void);
  * block_table int32 [B, table_stride]; kv_lens int32 [B].
  * out_split fp32 [B,Hq,S,Dv] contiguous; lse_split fp32 [B,Hq,S] contiguous.
  * The reference keeps LSE in-band in the q dtype (column Dv of its [.., Dv+1] buffer, :235-239);
- * here it is a separate fp32 tensor. Supported (head_dim, head_dim_v): (64,64), (128,128), (256,256) and the
- * heads with extra key dimensions (BLOCK_DPE = D - 2^floor(log2 D), flash_decode.py:771-772): (192,128), (576,512);
- * dtype bf16 / f16. */
+ * here it is a separate fp32 tensor. Supported (head_dim, head_dim_v): every equal pair that is a multiple of 8 up
+ * to 256 ((64,64), (128,128) and (256,256) on shapes of their own, the others, e.g. 80, 96 and 160, on the shape of
+ * the next power of two with the missing dimensions read as zeros: the reference's BLOCK_DMODEL + BLOCK_DPE split
+ * with masks, flash_decode.py:771-772), and the heads whose keys carry 64 dimensions more than their values:
+ * (192,128), (576,512); dtype bf16 / f16. */
 int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cache, float* out_split,
                           float* lse_split, float sm_scale, float soft_cap, const int32_t* block_table,
                           const int32_t* kv_lens, int batch, int q_heads, int kv_heads, int head_dim,

@@ -78,10 +78,12 @@ def test_null_pointers_are_rejected_without_touching_the_gpu():
     assert lib.tdist_reduce_slices(p, 0, 4, 0, 16, p, _lib.TDIST_F8E4M3, None) == _lib.TDIST_ERR_UNSUPPORTED
     assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 6, 4, 128, 128, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
                                      _lib.TDIST_BF16, None) == _lib.TDIST_ERR_INVALID  # 6 % 4 != 0
-    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 96, 96, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
-                                     _lib.TDIST_BF16, None) == _lib.TDIST_ERR_UNSUPPORTED  # head_dim 96
-    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 192, 192, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
-                                     _lib.TDIST_BF16, None) == _lib.TDIST_ERR_UNSUPPORTED  # 192 goes with Dv = 128
+    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 100, 100, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                     _lib.TDIST_BF16, None) == _lib.TDIST_ERR_UNSUPPORTED  # head_dim 100: no multiple of 8
+    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 96, 64, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                     _lib.TDIST_BF16, None) == _lib.TDIST_ERR_UNSUPPORTED  # 96 goes with Dv = 96
+    assert lib.tdist_decode_split_kv(p, p, p, p, p, 1.0, 0.0, p, p, 1, 8, 4, 192, 64, 1, 4, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                     _lib.TDIST_BF16, None) == _lib.TDIST_ERR_UNSUPPORTED  # 192 goes with Dv = 128 or 192
     # the fused launch: 40 query heads over 2 kv heads = 2 blocks of 16 heads per kv head and sequence
     assert lib.tdist_decode_fused_counters(3, 40, 2) == 3 * 2 * 2
     assert lib.tdist_decode_fused_counters(3, 40, 3) == -1

@@ -294,21 +294,44 @@ def test_config5_end_to_end_with_seven_peers(cuda):
         assert err <= ATOL, "sequence %d: %g" % (b, err)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4])
-def test_alternative_block_shapes(cuda, monkeypatch, variant):
-    """The other compiled block shapes for D = 128 (keys per block, waves, stages), selectable for measurements:
-    same partials and LSE within the bar."""
-    from triton_dist.kernels.amd.flash_decode import _split_kv
-    monkeypatch.setenv("TDIST_DECODE_VARIANT", str(variant))
-    kv_lens, S, heads, D, page = [1320, 18, 463, 5], 8, (32, 8), 128, 16
-    announce("decode block shape variant %d" % variant)
-    q, k_cache, v_cache, table = build_case(kv_lens, heads, D, page, torch.bfloat16, seed=40 + variant)
+@pytest.mark.parametrize("D", [80, 96, 160, 8, 40, 248])
+@pytest.mark.parametrize("num_heads,kv_lens,S,block_size", [((16, 16), [1320, 18, 463], 4, 16), ((32, 8), [1, 54, 293, 70], 8, 1),
+                                                            ((6, 1), [777, 0, 5], 3, 16)])
+@pytest.mark.parametrize("dtype,soft_cap", [(torch.bfloat16, 0), (torch.float16, 30)])
+def test_head_dimensions_that_are_no_power_of_two(cuda, D, num_heads, kv_lens, S, block_size, dtype, soft_cap):
+    """Head dimensions like 80, 96 and 160 (the reference takes them as BLOCK_DMODEL + BLOCK_DPE with masks,
+    flash_decode.py:771-772): per-split partials and LSE, the merged 16-bit output, and the one-launch form bit for
+    bit against split + combine. The cache rows are D wide and packed, so a lane that read beyond its row would
+    read the next head's or token's values."""
+    from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine, decode_fused
+    announce("decode D=%d heads=%s kv_lens=%s S=%d page=%d %s cap=%s" % (D, num_heads, kv_lens, S, block_size, dtype, soft_cap))
+    q, k_cache, v_cache, table = build_case(kv_lens, num_heads, D, block_size, dtype, seed=D + S)
+    scale = D**-0.5
+    B, Hq = len(kv_lens), num_heads[0]
     lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
-    out_split, lse_split, _ = _split_kv(q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), lens_dev, table.to(cuda), D**-0.5, 0.0, S)
+    qd, kd, vd, td = q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), table.to(cuda)
+    out_split, lse_split, _ = _split_kv(qd, kd, vd, lens_dev, td, scale, soft_cap, S)
     torch.cuda.synchronize()
-    w_out, w_lse = golden.decode_split_exact(q, k_cache, v_cache, kv_lens, table, D**-0.5, S)
-    empty = torch.isinf(w_lse)
+    assert out_split.shape == (B, Hq, S, D)
+    w_out, w_lse = golden.decode_split_exact(q, k_cache, v_cache, kv_lens, table, scale, S, soft_cap)
     got_lse = lse_split.cpu().double()
+    empty = torch.isinf(w_lse)
     assert torch.equal(torch.isinf(got_lse), empty)
     assert (got_lse[~empty] - w_lse[~empty]).abs().max() <= ATOL
     assert (out_split.cpu().double() - w_out).abs().max() <= ATOL
+    want = torch.empty((B, Hq, D), dtype=dtype, device=cuda)
+    want_lse = torch.empty((B, Hq), dtype=torch.float32, device=cuda)
+    decode_combine(out_split, lse_split, S, 1, lens_dev, B, Hq, D,
+                   (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
+                   (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), want, want_lse)
+    got = torch.full((B, Hq, D), float("nan"), dtype=dtype, device=cuda)
+    got_lse = torch.full((B, Hq), float("nan"), dtype=torch.float32, device=cuda)
+    counters = torch.zeros(1024, dtype=torch.int32, device=cuda)
+    decode_fused(qd, kd, vd, lens_dev, td, scale, soft_cap, S, got, got_lse, workspace=counters)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(got_lse.view(torch.int32), want_lse.view(torch.int32))
+    assert int(counters.abs().sum()) == 0
+    exact, _ = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, scale, soft_cap)
+    eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    assert ((got.cpu().double() - exact).abs() <= ATOL + eps * exact.abs()).all()

@@ -225,6 +225,49 @@ def test_gemm_rs_small_and_owner_mapping(cuda):
     assert torch.equal(out.cpu().view(torch.int16), golden.reduce_slices_ordered(stored, (rank + 1) % W).view(torch.int16))
 
 
+@pytest.mark.parametrize("scaled", [False, True])
+def test_gemm_rs_with_e4m3_inputs(cuda, scaled):
+    """e4m3 inputs (optionally with per-row and per-column scales), bf16 partial results scattered to their owners'
+    buffers, fp32 sum of the slices: the scattered partials against the up-cast fp32 golden on random inputs, bit for
+    bit on integer-valued ones (power-of-two scales), and the reduction bit for bit given what the GEMM stored."""
+    from triton_dist.kernels.amd import create_gemm_rs_intra_node_context, gemm_rs_intra_node
+    announce("gemm_rs e4m3 scaled=%s" % scaled)
+    W, rank, M, N, K = 4, 1, 1024, 768, 512
+    m_per = M // W
+    g = torch.Generator().manual_seed(5)
+    ctx = create_gemm_rs_intra_node_context(M, N, torch.bfloat16, rank, W, None)
+    peers = [None if r == rank else torch.randn((m_per, N), generator=g).to(torch.bfloat16) for r in range(W)]
+    ctx.set_peer_partials(peers)
+    for integer in (True, False):
+        if integer:
+            a = torch.randint(-2, 3, (M, K), generator=g).float().to(torch.float8_e4m3fn)
+            b = torch.randint(-2, 3, (N, K), generator=g).float().to(torch.float8_e4m3fn)
+            sa = 2.0 ** torch.randint(-3, 3, (M,), generator=g).float() if scaled else None
+            sb = 2.0 ** torch.randint(-3, 3, (N,), generator=g).float() if scaled else None
+        else:
+            a = torch.randn((M, K), generator=g).to(torch.float8_e4m3fn)
+            b = (torch.randn((N, K), generator=g) * 0.05).to(torch.float8_e4m3fn)
+            sa = torch.rand(M, generator=g) * 0.09 + 0.01 if scaled else None
+            sb = torch.rand(N, generator=g) * 0.9 + 0.1 if scaled else None
+        out = gemm_rs_intra_node(a.to(cuda), b.to(cuda), ctx, row_scale=None if sa is None else sa.to(cuda),
+                                 col_scale=None if sb is None else sb.to(cuda))
+        torch.cuda.synchronize()
+        assert out.shape == (m_per, N) and out.dtype == torch.bfloat16
+        full = golden.fp8_scaled_gemm_fp32(a, sa, b, sb)
+        for o in range(W):
+            blk = ctx.scatter_bufs[o][rank * m_per:(rank + 1) * m_per].cpu()
+            want = full[o * m_per:(o + 1) * m_per]
+            if integer:
+                assert torch.equal(blk, want.to(torch.bfloat16)), "owner %d" % o
+            else:
+                assert golden.max_rel_err(blk.float(), want) <= 1e-2, "owner %d" % o
+        stored = ctx.scatter_bufs[rank][:M].cpu().view(W, m_per, N)
+        assert torch.equal(out.cpu().view(torch.int16), golden.reduce_slices_ordered(stored, (rank + 1) % W).view(torch.int16))
+    with pytest.raises(TypeError):
+        f16ctx = create_gemm_rs_intra_node_context(M, N, torch.float16, rank, W, None)
+        gemm_rs_intra_node(a.to(cuda), b.to(cuda), f16ctx)
+
+
 def test_gemm_rs_config2_full_size(cuda):
     """BASELINE config 2: A [8192, 3584] x B [3584, 8192] (stored [8192, 3584]), rank 0 of 8, 7 synthetic peers."""
     from triton_dist.kernels.amd import create_gemm_rs_intra_node_context, gemm_rs_intra_node

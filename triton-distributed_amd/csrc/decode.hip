@@ -49,6 +49,7 @@ struct DecodeParams {
   float sm_scale;
   float soft_cap;
   int B, Hq, Hkv, S;
+  int d_valid;  // kernels compiled for a padded head dimension: the real one (a multiple of 8), else unused
   int page_size;
   // n / page_size for 0 <= n < 2^31 as (n * page_magic) >> page_shift with
   // page_shift = 31 + ceil(log2 page_size), page_magic = ceil(2^page_shift / page_size)  (exact, Granlund-Montgomery)
@@ -98,6 +99,9 @@ struct MmaF16 {
 };
 
 constexpr int kTableSlots = 8;  // ring of page-table rows per wave (>= 2P+2)
+
+// what the DMA lanes of a padded head dimension read for the dimensions that do not exist
+static __device__ __align__(16) const unsigned char kZeroChunk[16] = {0};
 
 // KEYS = keys per block (16 or 32): one or two groups of 16 keys, a group being one MFMA tile of scores.
 // DM = value dimension = power-of-two part of the key dimension; DPE = the extra key dimensions (0 or 64).
@@ -165,11 +169,18 @@ __device__ __forceinline__ void store_partial(float* p, float v) {
   else *p = v;
 }
 
-template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse>
+// kPadded: the head dimension is prm.d_valid <= D (key and value alike, a multiple of 8): the rows in the LDS are D
+// wide, the 16-byte pieces beyond the real row are fetched from a page of zeros (so that the MFMA blocks see exact
+// zeros there: the reference masks the same dimensions, kernels/nvidia/flash_decode.py:771-772 with BLOCK_DPE), and
+// results are stored d_valid wide.
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded>
 __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   typedef DecodeCfg<D, DPE, KEYS, NST> C;
   constexpr int G = C::kGroups;
   constexpr int DK = D + DPE;  // key (and query) dimensions; D is the value dimension
+  static_assert(!kPadded || DPE == 0, "padded rows have no extra key dimensions");
+  const int Dout = kPadded ? prm.d_valid : D;          // width of the stored results
+  const int valid_chunks = kPadded ? prm.d_valid >> 3 : D / 8;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   // kv heads vary fastest over the grid: workgroups that run together then read the neighbouring 2*D-byte
@@ -193,13 +204,13 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   const int start = per * split;
   const int end = min(start + per, len);
 
-  float* out_base = prm.out + (((int64_t)b * prm.Hq + h0) * prm.S + split) * D;
+  float* out_base = prm.out + (((int64_t)b * prm.Hq + h0) * prm.S + split) * Dout;
   float* lse_base = prm.lse + ((int64_t)b * prm.Hq + h0) * prm.S + split;
   if (end <= start) {
     // empty split: zeros and LSE = -inf so that any merge gives it weight 0
-    for (int i = threadIdx.x; i < nvalid * D; i += NW * 64) {
-      const int h = i / D, d = i - h * D;
-      store_partial<kFuse>(out_base + (int64_t)h * prm.S * D + d, 0.f);
+    for (int i = threadIdx.x; i < nvalid * Dout; i += NW * 64) {
+      const int h = i / Dout, d = i - h * Dout;
+      store_partial<kFuse>(out_base + (int64_t)h * prm.S * Dout + d, 0.f);
     }
     if (threadIdx.x < nvalid) store_partial<kFuse>(lse_base + (int64_t)threadIdx.x * prm.S, -INFINITY);
     return;
@@ -221,7 +232,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
 #pragma unroll
     for (int s = 0; s < DK / 32; ++s) {
       int4v raw = {0, 0, 0, 0};
-      if (x < nvalid) raw = *(const int4v*)(qrow + (32 * s + 8 * g) * 2);
+      if (x < nvalid && (!kPadded || 4 * s + g < valid_chunks)) raw = *(const int4v*)(qrow + (32 * s + 8 * g) * 2);
       qf[s] = __builtin_bit_cast(typename MMA::frag8, raw);
     }
   }
@@ -295,6 +306,10 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
                                   (in_page * (uint32_t)prm.k_st + (uint32_t)kvh * (uint32_t)prm.k_sh + ((chunk ^ C::kswz(key)) << 4));
       const unsigned char* vsrc = prm.v + (uint64_t)page * (uint64_t)prm.v_sp +
                                   (in_page * (uint32_t)prm.v_st + (uint32_t)kvh * (uint32_t)prm.v_sh + ((chunk ^ C::vswz(key)) << 4));
+      if constexpr (kPadded) {
+        if ((chunk ^ C::kswz(key)) >= valid_chunks) ksrc = kZeroChunk;
+        if ((chunk ^ C::vswz(key)) >= valid_chunks) vsrc = kZeroChunk;
+      }
       __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)ksrc, (TDIST_AS3 void*)(kst + i * 1024), 16, 0, TDIST_KV_AUX);
       __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)vsrc, (TDIST_AS3 void*)(vst + i * 1024), 16, 0, TDIST_KV_AUX);
     }
@@ -433,8 +448,8 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
     for (int i = 0; i < 4; ++i) s_acc[(16 * d + 4 * g + i) * 16 + x] = acc[d][i];
   __syncthreads();
   constexpr float kLn2 = 0.6931471805599453f;
-  for (int idx = threadIdx.x; idx < nvalid * D; idx += NW * 64) {
-    const int h = idx / D, dv = idx - h * D;
+  for (int idx = threadIdx.x; idx < nvalid * Dout; idx += NW * 64) {
+    const int h = idx / Dout, dv = idx - h * Dout;
     float M = -INFINITY;
 #pragma unroll
     for (int w = 0; w < NW; ++w) M = fmaxf(M, ((const TDIST_AS3 float*)(smem3 + w * C::kWaveBytes))[h]);
@@ -447,7 +462,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
       L += wm[16 + h] * sc;
       O += wm[32 + dv * 16 + h] * sc;
     }
-    store_partial<kFuse>(out_base + (int64_t)h * prm.S * D + dv, O / L);
+    store_partial<kFuse>(out_base + (int64_t)h * prm.S * Dout + dv, O / L);
     if (dv == 0) store_partial<kFuse>(lse_base + (int64_t)h * prm.S, (M + log2f(L)) * kLn2);
   }
 }
@@ -542,8 +557,9 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams
 // Fused tail: publishes this workgroup's partial result; the last of the S workgroups of a (sequence, head block)
 // to get here merges their partials (same arithmetic, in the same order, as decode_combine_kernel in mode 1) and
 // puts the counter back to zero for the next launch.
-template <int D, int NW>
+template <int DM, int NW, bool kPadded>
 __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
+  const int D = kPadded ? prm.d_valid : DM;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   TDIST_AS3 int* const s_last = (TDIST_AS3 int*)smem;
   const int group = prm.Hq / prm.Hkv;
@@ -575,7 +591,7 @@ __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
 
   const float* lse_p = prm.lse + ((int64_t)b * prm.Hq + h0) * prm.S;
   const float* out_p = prm.out + ((int64_t)b * prm.Hq + h0) * prm.S * D;
-  constexpr int kVecs = D / 4;
+  const int kVecs = D / 4;
   for (int idx = threadIdx.x; idx < nvalid * kVecs; idx += NW * 64) {
     const int h = idx / kVecs, dv = (idx - h * kVecs) * 4;
     const float* l = lse_p + (int64_t)h * prm.S;
@@ -601,19 +617,19 @@ __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
   }
 }
 
-template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse>
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded>
 __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodeParams prm) {
-  decode_split_body<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse>(prm);
-  if constexpr (kFuse) decode_fused_merge<D, NW>(prm);
+  decode_split_body<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse, kPadded>(prm);
+  if constexpr (kFuse) decode_fused_merge<D, NW, kPadded>(prm);
 }
 
-template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse>
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded>
 static int launch_decode_cfg(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
   typedef DecodeCfg<D, DPE, KEYS, NST> C;
   static_assert((32 + D * 16) * 4 <= C::kWaveBytes, "merge scratch must fit in a wave's ring");
   const size_t lds = (size_t)NW * C::kWaveBytes;
   static_assert((size_t)NW * C::kWaveBytes <= 160 * 1024, "LDS of one CU");
-  auto kern = decode_split_kv_kernel<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse>;
+  auto kern = decode_split_kv_kernel<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse, kPadded>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -625,14 +641,14 @@ static int launch_decode_cfg(const DecodeParams& prm, int head_blocks, hipStream
   return launch_status(kFuse ? "tdist_decode_fused" : "tdist_decode_split_kv");
 }
 
-template <typename MMA, int D, int DPE, int KEYS, int NW, int NST>
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kPadded = false>
 static int launch_decode(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
   const bool fuse = prm.counters != nullptr;
   if (prm.soft_cap > 0.f)
-    return fuse ? launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, true, true>(prm, head_blocks, stream)
-                : launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, true, false>(prm, head_blocks, stream);
-  return fuse ? launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, false, true>(prm, head_blocks, stream)
-              : launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, false, false>(prm, head_blocks, stream);
+    return fuse ? launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, true, true, kPadded>(prm, head_blocks, stream)
+                : launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, true, false, kPadded>(prm, head_blocks, stream);
+  return fuse ? launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, false, true, kPadded>(prm, head_blocks, stream)
+              : launch_decode_cfg<MMA, D, DPE, KEYS, NW, NST, false, false, kPadded>(prm, head_blocks, stream);
 }
 
 }  // namespace tdist
@@ -678,11 +694,12 @@ static int run_decode(const DecodeCall& c, bool fuse) {
   if (c.dtype != TDIST_BF16 && c.dtype != TDIST_F16)
     return fail(TDIST_ERR_UNSUPPORTED, "%s: dtype %d (bf16 and f16 only)", who, c.dtype);
   const int dk = c.head_dim, dv = c.head_dim_v;
+  const bool padded = dk == dv && dk > 0 && dk < 256 && dk % 8 == 0 && dk != 64 && dk != 128;
   const bool dims_ok = (dk == dv && (dk == 64 || dk == 128 || dk == 256)) || (dk == 192 && dv == 128) ||
-                       (dk == 576 && dv == 512);
+                       (dk == 576 && dv == 512) || padded;
   if (!dims_ok)
-    return fail(TDIST_ERR_UNSUPPORTED, "%s: head dims (%d, %d): (64,64), (128,128), (256,256), (192,128), (576,512) only",
-                who, dk, dv);
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: head dims (%d, %d): equal ones that are a multiple of 8 up to 256, (192,128) "
+                "and (576,512) only", who, dk, dv);
   if (!aligned16(c.q) || !aligned16(c.k_cache) || !aligned16(c.v_cache) || (c.q_stride_b % 8) || (c.q_stride_h % 8) ||
       (c.k_stride_page % 8) || (c.k_stride_token % 8) || (c.k_stride_head % 8) || (c.v_stride_page % 8) ||
       (c.v_stride_token % 8) || (c.v_stride_head % 8))
@@ -702,6 +719,7 @@ static int run_decode(const DecodeCall& c, bool fuse) {
   prm.Hq = c.q_heads;
   prm.Hkv = c.kv_heads;
   prm.S = c.num_splits;
+  prm.d_valid = dk;
   prm.page_size = c.page_size;
   int lg = 0;
   while ((1ll << lg) < c.page_size) ++lg;
@@ -746,26 +764,26 @@ static int run_decode(const DecodeCall& c, bool fuse) {
 #define TDIST_DEC(D_, DPE_, KEYS_, NW_, NST_)                                             \
   return bf ? launch_decode<MmaBF16, D_, DPE_, KEYS_, NW_, NST_>(prm, head_blocks, st)   \
             : launch_decode<MmaF16, D_, DPE_, KEYS_, NW_, NST_>(prm, head_blocks, st);
+#define TDIST_DEC_PADDED(D_, KEYS_, NW_, NST_)                                                 \
+  return bf ? launch_decode<MmaBF16, D_, 0, KEYS_, NW_, NST_, true>(prm, head_blocks, st)     \
+            : launch_decode<MmaF16, D_, 0, KEYS_, NW_, NST_, true>(prm, head_blocks, st);
+  if (padded) {
+    // any other head dimension: the shape of the next power of two, rows filled up with zeros on their way in
+    if (dk < 64) TDIST_DEC_PADDED(64, 32, 4, 4)
+    if (dk < 128) TDIST_DEC_PADDED(128, 16, 3, 3)
+    TDIST_DEC_PADDED(256, 16, 2, 3)
+  }
   switch (dk) {
     case 64: TDIST_DEC(64, 0, 32, 4, 4)
-    case 128: {
-      // TDIST_DECODE_VARIANT picks another compiled shape (measurement aid). Default: 16-key blocks, 3 waves,
-      // 3 stages = 72 KB of LDS, so two workgroups share a CU and two thirds of the ring are in flight.
-      int variant = 0;
-      if (const char* v = getenv("TDIST_DECODE_VARIANT")) variant = atoi(v);
-      switch (variant) {
-        case 1: TDIST_DEC(128, 0, 32, 4, 2)
-        case 2: TDIST_DEC(128, 0, 32, 3, 3)
-        case 3: TDIST_DEC(128, 0, 16, 8, 2)
-        case 4: TDIST_DEC(128, 0, 16, 4, 2)
-        default: TDIST_DEC(128, 0, 16, 3, 3)
-      }
-    }
+    // 16-key blocks, 3 waves, 3 stages = 72 KB of LDS: two workgroups share a CU and two thirds of the ring are
+    // in flight
+    case 128: TDIST_DEC(128, 0, 16, 3, 3)
     case 192: TDIST_DEC(128, 64, 16, 2, 3)   // 61 KB: two workgroups per CU
     case 256: TDIST_DEC(256, 0, 16, 2, 3)
     default: TDIST_DEC(512, 64, 16, 2, 2)    // 576 = 512 + 64: 136 KB
   }
 #undef TDIST_DEC
+#undef TDIST_DEC_PADDED
 }
 
 }  // namespace tdist

@@ -1686,12 +1686,13 @@ int tdist_gemm_chunk_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
 
 static int gemm_rs_scatter(GemmElem elem, const void* A, int64_t lda, const void* B, int64_t ldb,
                            void* const* scatter_bufs, int64_t ldc, int M, int N, int K, int rank, int world_size,
-                           void* sk_workspace, int64_t sk_workspace_bytes, void* stream, const char* who) {
+                           void* sk_workspace, int64_t sk_workspace_bytes, void* stream, const char* who,
+                           const float* row_scale = nullptr, const float* col_scale = nullptr) {
   if (!scatter_bufs) return fail(TDIST_ERR_INVALID, "%s: null scatter_bufs", who);
   GemmCall c;
   c.A = A; c.lda = lda; c.A_local = nullptr; c.lda_local = 0; c.local_row_begin = 0; c.local_rows = 0;
   c.B = B; c.ldb = ldb; c.C = nullptr; c.scatter_bufs = scatter_bufs; c.ldc = ldc; c.M = M; c.N = N; c.K = K;
-  c.row_scale = nullptr; c.col_scale = nullptr; c.flags = nullptr; c.m_per_chunk = 0; c.wait_value = 0;
+  c.row_scale = row_scale; c.col_scale = col_scale; c.flags = nullptr; c.m_per_chunk = 0; c.wait_value = 0;
   c.chunk_order = nullptr; c.rank = rank; c.world_size = world_size; c.spin_limit = 0; c.status = nullptr;
   c.max_workgroups = 0; c.sk_workspace = sk_workspace; c.sk_workspace_bytes = sk_workspace_bytes;
   c.stream = (hipStream_t)stream; c.who = who;
@@ -1710,6 +1711,13 @@ int tdist_gemm_rs_scatter_f16(const void* A, int64_t lda, const void* B, int64_t
                               int64_t sk_workspace_bytes, void* stream) {
   return gemm_rs_scatter(kElemF16, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, sk_workspace,
                          sk_workspace_bytes, stream, "tdist_gemm_rs_scatter_f16");
+}
+
+int tdist_gemm_rs_scatter_fp8e4m3(const void* A, int64_t lda, const void* B, int64_t ldb, void* const* scatter_bufs,
+                                  int64_t ldc, int M, int N, int K, const float* row_scale, const float* col_scale,
+                                  int rank, int world_size, void* sk_workspace, int64_t sk_workspace_bytes, void* stream) {
+  return gemm_rs_scatter(kElemFP8, A, lda, B, ldb, scatter_bufs, ldc, M, N, K, rank, world_size, sk_workspace,
+                         sk_workspace_bytes, stream, "tdist_gemm_rs_scatter_fp8e4m3", row_scale, col_scale);
 }
 
 #define TDIST_GROUP_GEMM_BODY(ELEM, WHO)                                                                              \

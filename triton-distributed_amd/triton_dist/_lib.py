@@ -41,6 +41,7 @@ PROTOTYPES = {
     "tdist_flag_fill": (_I, [_P, _I, _I, _P]),
     "tdist_gemm_rs_scatter_bf16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P]),
     "tdist_gemm_rs_scatter_f16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P]),
+    "tdist_gemm_rs_scatter_fp8e4m3": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _P, _I, _I, _P, _L, _P]),
     "tdist_reduce_slices": (_I, [_P, _L, _I, _I, _L, _P, _I, _P]),
     "tdist_moe_workspace_bytes": (_L, [_L, _I]),
     "tdist_moe_splits_cumsum": (_I, [_P, _L, _I, _P, _P, _P, _L, _P]),

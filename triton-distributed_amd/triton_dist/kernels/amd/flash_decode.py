@@ -15,7 +15,14 @@ from triton_dist import _lib
 DEFAULT_KV_SPLITS = 32  # reference :777, :861
 
 
-SUPPORTED_HEAD_DIMS = ((64, 64), (128, 128), (256, 256), (192, 128), (576, 512))  # (q/k head dim, v head dim)
+# (q/k head dim, v head dim) with compiled shapes of their own; beside them every equal pair that is a multiple of 8
+# up to 256 runs on the shape of the next power of two (the reference splits a head into BLOCK_DMODEL + BLOCK_DPE and
+# masks, kernels/nvidia/flash_decode.py:771-772)
+SUPPORTED_HEAD_DIMS = ((64, 64), (128, 128), (256, 256), (192, 128), (576, 512))
+
+
+def head_dims_supported(dk, dv):
+    return (dk, dv) in SUPPORTED_HEAD_DIMS or (dk == dv and 0 < dk <= 256 and dk % 8 == 0)
 
 
 def _check_inputs(q, k_cache, v_cache, kv_lens, block_table):
@@ -25,8 +32,9 @@ def _check_inputs(q, k_cache, v_cache, kv_lens, block_table):
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
     v_head_dim = v_cache.shape[-1]
     assert q_heads % kv_heads == 0
-    if (q_head_dim, v_head_dim) not in SUPPORTED_HEAD_DIMS:
-        raise NotImplementedError("head dims (%d, %d); supported: %s" % (q_head_dim, v_head_dim, SUPPORTED_HEAD_DIMS))
+    if not head_dims_supported(q_head_dim, v_head_dim):
+        raise NotImplementedError("head dims (%d, %d); supported: equal ones that are a multiple of 8 up to 256 and %s" %
+                                  (q_head_dim, v_head_dim, SUPPORTED_HEAD_DIMS[3:]))
     if q.dtype != k_cache.dtype or q.dtype != v_cache.dtype:
         raise TypeError("q, k_cache and v_cache must share one dtype")
     if q.stride(-1) != 1 or k_cache.stride(-1) != 1 or v_cache.stride(-1) != 1:

@@ -77,14 +77,16 @@ def create_gemm_rs_intra_node_context(max_M, N, output_dtype, rank, num_ranks, t
     )
 
 
-_SCATTER_ENTRY = {torch.bfloat16: "tdist_gemm_rs_scatter_bf16", torch.float16: "tdist_gemm_rs_scatter_f16"}
+_SCATTER_ENTRY = {torch.bfloat16: "tdist_gemm_rs_scatter_bf16", torch.float16: "tdist_gemm_rs_scatter_f16",
+                  torch.float8_e4m3fn: "tdist_gemm_rs_scatter_fp8e4m3"}
 
 
 def matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weight, ldc=None, stream=None,
-                        strict_alignment=True, sk_workspace=None):
+                        strict_alignment=True, sk_workspace=None, row_scale=None, col_scale=None):
     """GEMM with the scatter epilogue (reference :289-314). ``b`` is [N, K]. ``strict_alignment`` keeps the
     reference's assertion (M, N, K multiples of 256); without it the library's own limits apply (M / num_ranks a
-    multiple of 128, K rows a multiple of 64 bytes)."""
+    multiple of 128, K rows a multiple of 16 bytes). e4m3 inputs write bf16 partial results and take optional fp32
+    ``row_scale`` [M] / ``col_scale`` [N]."""
     if transpose_weight:
         raise NotImplementedError()
     assert a.shape[1] == b.shape[1], "Incompatible dimensions"
@@ -95,8 +97,13 @@ def matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weigh
     assert not strict_alignment or (M % alignment == 0 and N % alignment == 0 and K % alignment == 0)
     if a.dtype not in _SCATTER_ENTRY:
         raise TypeError("unsupported GEMM-RS dtype %s" % a.dtype)
+    scales = []
+    if a.dtype == torch.float8_e4m3fn:
+        scales = [_lib.ptr(row_scale), _lib.ptr(col_scale)]
+    elif row_scale is not None or col_scale is not None:
+        raise ValueError("scales are only defined for fp8 inputs")
     _lib.call(_SCATTER_ENTRY[a.dtype], a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
-              scatter_bufs_ptr.data_ptr(), N if ldc is None else ldc, M, N, K, rank, num_ranks,
+              scatter_bufs_ptr.data_ptr(), N if ldc is None else ldc, M, N, K, *scales, rank, num_ranks,
               *_lib.workspace_args(sk_workspace), _lib.stream_ptr(stream))
 
 
@@ -113,7 +120,7 @@ def ring_reduce_after_scatter(rank, num_ranks, scatter_out, stream):
 
 
 def gemm_rs_intra_node_op(a, b, output_dtype, rank, num_ranks, scatter_bufs, scatter_bufs_ptr, sync_bufs_ptr,
-                          fuse_scatter=True, transpose_weight=False, sk_workspace=None):
+                          fuse_scatter=True, transpose_weight=False, sk_workspace=None, row_scale=None, col_scale=None):
     """gemm reduce scatter for intra-node (reference :317-365)."""
     if not fuse_scatter:
         raise NotImplementedError()
@@ -124,28 +131,32 @@ def gemm_rs_intra_node_op(a, b, output_dtype, rank, num_ranks, scatter_bufs, sca
     N, weight_local_K = b.shape
     assert weight_local_K == local_K
     assert a.dtype == b.dtype
-    if scatter_bufs[rank].dtype != a.dtype:
-        raise TypeError("the scatter buffers hold the GEMM's input dtype (reference :217-218): ctx was created "
-                        "for %s, inputs are %s" % (scatter_bufs[rank].dtype, a.dtype))
+    partial_dtype = torch.bfloat16 if a.dtype == torch.float8_e4m3fn else a.dtype
+    if scatter_bufs[rank].dtype != partial_dtype:
+        raise TypeError("the scatter buffers hold the GEMM's input dtype (reference :217-218; bf16 for e4m3 inputs): "
+                        "ctx was created for %s, inputs are %s" % (scatter_bufs[rank].dtype, a.dtype))
     current_stream = torch.cuda.current_stream()
     matmul_fuse_scatter(a, b, scatter_bufs_ptr, rank, num_ranks, transpose_weight=transpose_weight,
-                        ldc=scatter_bufs[rank].stride(0), stream=current_stream, sk_workspace=sk_workspace)
+                        ldc=scatter_bufs[rank].stride(0), stream=current_stream, sk_workspace=sk_workspace,
+                        row_scale=row_scale, col_scale=col_scale)
     scatter_out = scatter_bufs[rank][:M]
     output = ring_reduce_after_scatter(rank, num_ranks, scatter_out, current_stream)
     return output
 
 
-def gemm_rs_intra_node(a, b, ctx):
+def gemm_rs_intra_node(a, b, ctx, *, row_scale=None, col_scale=None):
     """GEMM Reduce-Scatter for Intra-Node (reference :429-446)
 
     Args:
-        a (torch.Tensor<bfloat16/float16>): local matmul A matrix. shape: [M, local_K]
-        b (torch.Tensor<bfloat16/float16>): local matmul B matrix. shape: [N, local_K]
+        a (torch.Tensor<bfloat16/float16/float8_e4m3fn>): local matmul A matrix. shape: [M, local_K]
+        b (torch.Tensor, same dtype): local matmul B matrix. shape: [N, local_K]
         ctx (GEMMReduceScatterTensorParallelContext)
+        row_scale / col_scale: e4m3 inputs only: fp32 scales per row of a ([M]) and per row of b ([N]); no
+            counterpart in the reference. The context of an e4m3 call is created with output_dtype bfloat16.
 
     Returns:
         c (torch.Tensor<bfloat16/float16>): shape [M // world_size, N]
     """
     return gemm_rs_intra_node_op(a, b, ctx.output_dtype, ctx.rank, ctx.num_ranks, ctx.scatter_bufs,
                                  ctx.scatter_bufs_ptr, ctx.sync_bufs_ptr, ctx.fuse_scatter, ctx.transpose_weight,
-                                 sk_workspace=ctx.sk_workspace)
+                                 sk_workspace=ctx.sk_workspace, row_scale=row_scale, col_scale=col_scale)
