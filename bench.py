@@ -449,7 +449,15 @@ def bench_copy(dev, steps, warmup):
     src = torch.empty(n, dtype=torch.uint8, device=dev)
     dst = torch.empty(n, dtype=torch.uint8, device=dev)
     s = time_launches(lambda: _lib.bench_call("tdist_copy_bytes", dst.data_ptr(), src.data_ptr(), n, _lib.stream_ptr()), steps, warmup)
-    return roof("hbm", 2 * n, s, "hbm")
+    r = roof("hbm", 2 * n, s, "hbm")
+    # the one-directional streams over the same 1 GiB (four times the memory-side cache): what HBM sustains for
+    # writes alone (the MoE dispatch writes 8 bytes per byte it reads) and for reads alone (combine, decode)
+    sink = torch.zeros(256, dtype=torch.int32, device=dev)
+    w = time_launches(lambda: _lib.bench_call("tdist_fill_bytes", dst.data_ptr(), n, _lib.stream_ptr()), steps, warmup)
+    rd = time_launches(lambda: _lib.bench_call("tdist_read_bytes", src.data_ptr(), n, sink.data_ptr(), _lib.stream_ptr()), steps, warmup)
+    r["write_only"] = {"achieved_GBps": round(n / w / 1e9, 1), "frac": round(n / w / PEAK["hbm"], 4)}
+    r["read_only"] = {"achieved_GBps": round(n / rd / 1e9, 1), "frac": round(n / rd / PEAK["hbm"], 4)}
+    return r
 
 
 def bench_mfma_ceiling(dev, steps, warmup):

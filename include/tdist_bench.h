@@ -21,6 +21,14 @@ const char* tdist_bench_last_error_string(void);
  * ------------------------------------------------------------------------------------------- */
 int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
 
+/* Measurement helpers: the one-directional streams. tdist_fill_bytes writes nbytes (16-byte vectors, non-temporal
+ * stores, no reads); tdist_read_bytes reads nbytes (non-temporal loads) and writes nothing unless the XOR of a lane's
+ * words hits one magic value (sink: 256 words). On buffers larger than the 256 MB memory-side cache they give the
+ * rates HBM sustains for writes and for reads alone: the ceilings of a write-dominated kernel (the MoE dispatch:
+ * 8 bytes written per byte read) and of a read-dominated one (the combine, the decode). */
+int tdist_fill_bytes(void* dst, int64_t nbytes, void* stream);
+int tdist_read_bytes(const void* src, int64_t nbytes, int32_t* sink, void* stream);
+
 /* Measurement helper: the MFMA rate this chip sustains with no memory traffic at all. One workgroup of four waves per
  * compute unit runs iters (even) K steps of a 128 x 128 wave tile on register operands, in the GEMM kernel's order (a B
  * fragment against every A fragment in turn, 256 accumulators per lane): 4 x 4 MFMAs of 32x32x16 (bf16, K step 16) or

@@ -51,18 +51,22 @@ def test_preprocess_repeated_ids_and_skewed_load(cuda):
         assert torch.equal(a.cpu(), b)
 
 
-@pytest.mark.parametrize("launches", ["one", "three"])
+@pytest.mark.parametrize("launches", ["one", "one with rendezvous", "three"])
 def test_preprocess_paths_sizes_in_turn_and_context_buffers(cuda, monkeypatch, launches):
-    """The one-launch index build and the three-launch form it falls back to (forced here through the library's
-    switch; taken by itself beyond one block per compute unit, as the 560 000 ids below do): calls of different sizes
-    in turn on the same cached scratch, ids outside [0, G) (dropped: scatter index -1), and the context-owned result
-    tensors, two sets used in turn."""
+    """The one-launch index build in both of its forms (up to 32 blocks every block counts all the ids itself; beyond,
+    or forced here through the library's switch, the blocks exchange their histograms) and the three-launch form it
+    falls back to (forced likewise; taken by itself beyond one block per compute unit, as the 560 000 ids below do):
+    calls of different sizes in turn on the same cached scratch, id counts that are no multiple of four, ids outside
+    [0, G) (dropped: scatter index -1), and the context-owned result tensors, two sets used in turn."""
     from triton_dist.kernels.amd import create_all_to_all_context, moe_dispatch_preprocess
     if launches == "three":
         monkeypatch.setenv("TDIST_MOE_INDEX_LAUNCHES", "3")
+    if launches == "one with rendezvous":
+        monkeypatch.setenv("TDIST_MOE_INDEX_RENDEZVOUS", "1")
     announce("moe preprocess paths (%s launch)" % launches)
     g = torch.Generator().manual_seed(9)
-    for T, topk, G in [(4096, 8, 256), (300, 4, 2048), (70000, 8, 64), (1000, 8, 256), (5, 3, 4096)]:
+    for T, topk, G in [(4096, 8, 256), (300, 4, 2048), (70000, 8, 64), (1000, 8, 256), (5, 3, 4096), (333, 3, 100),
+                       (3001, 5, 300), (20000, 8, 128), (8191, 8, 3500)]:
         ids = torch.randint(0, G, (T, topk), generator=g).to(torch.int32)
         out = moe_dispatch_preprocess(ids.to(cuda), G, want_topk_index=True)
         torch.cuda.synchronize()

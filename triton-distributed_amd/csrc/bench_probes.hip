@@ -41,6 +41,30 @@ __global__ __launch_bounds__(256) void copy_bytes_kernel(int4v* __restrict__ dst
   }
 }
 
+// one-directional streams: a fill (writes only) and a sum (reads only; every lane's partial sum goes to sink)
+__global__ __launch_bounds__(256) void fill_bytes_kernel(int4v* __restrict__ dst, int64_t n16) {
+  int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+  const int4v v = {(int)threadIdx.x, (int)blockIdx.x, 3, 4};
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    int64_t j = i + u * 256;
+    if (j < n16) __builtin_nontemporal_store(v, dst + j);
+  }
+}
+__global__ __launch_bounds__(256) void read_bytes_kernel(const int4v* __restrict__ src, int64_t n16, int* __restrict__ sink) {
+  int64_t i = (int64_t)blockIdx.x * 4096 + threadIdx.x;
+  int4v v[16];
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    int64_t j = i + u * 256;
+    v[u] = j < n16 ? __builtin_nontemporal_load(src + j) : int4v{0, 0, 0, 0};
+  }
+  int acc = 0;
+#pragma unroll
+  for (int u = 0; u < 16; ++u) acc += v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+  if (acc == 0x5a5a5a5a) sink[threadIdx.x] = acc;   // (keeps the loads alive; practically never taken)
+}
+
 // MFMA-only loop for the rate yardstick: the K loop of a 128 x 128 wave tile with no memory traffic at all. 256
 // accumulators, eight A and eight B operand fragments in registers, and the GEMM kernel's order of use: a B fragment
 // serves a row of MFMAs against every A fragment in turn. kRandom fills the fragments with hashed bit patterns (random
@@ -129,6 +153,26 @@ int tdist_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
   hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (int4v*)dst,
                      (const int4v*)src, n16);
   return launch_status("tdist_copy_bytes");
+}
+
+int tdist_fill_bytes(void* dst, int64_t nbytes, void* stream) {
+  if (!dst || nbytes < 0 || (nbytes & 15) || !aligned16(dst))
+    return fail(TDIST_ERR_INVALID, "tdist_fill_bytes: pointer and size must be 16-byte aligned");
+  if (nbytes == 0) return TDIST_OK;
+  const int64_t n16 = nbytes / 16, blocks = ceil_div(n16, 1024);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_fill_bytes: too large");
+  hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (int4v*)dst, n16);
+  return launch_status("tdist_fill_bytes");
+}
+
+int tdist_read_bytes(const void* src, int64_t nbytes, int32_t* sink, void* stream) {
+  if (!src || !sink || nbytes < 0 || (nbytes & 15) || !aligned16(src))
+    return fail(TDIST_ERR_INVALID, "tdist_read_bytes: pointer and size must be 16-byte aligned, sink of 256 words");
+  if (nbytes == 0) return TDIST_OK;
+  const int64_t n16 = nbytes / 16, blocks = ceil_div(n16, 4096);
+  if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_read_bytes: too large");
+  hipLaunchKernelGGL(read_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const int4v*)src, n16, sink);
+  return launch_status("tdist_read_bytes");
 }
 
 static int mfma_rate_probe(const char* who, bool narrow, int dtype, int random_operands, int iters, float* sink, void* stream) {

@@ -235,7 +235,17 @@ __global__ __launch_bounds__(kMoeThreads) void moe_rank_kernel(const int32_t* __
 constexpr int kFusedSpinLimit = 1 << 22;
 constexpr int kFusedThreads = 512, kFusedPerWave = 256, kFusedItems = kFusedThreads / 64 * kFusedPerWave;
 
-template <int kThreads, int kPerWave>
+// kRecount (few ids): no rendezvous and no histogram rows in memory at all. Every block counts, beside its own ids,
+// everybody else's (the ids in front of its range and those behind it, into two more rows of LDS counters): reading
+// all the ids once more per block (131 KB out of the L2 for a decode step's 32768) is cheaper than the three trips
+// through memory of the rendezvous, and with nothing to wait for the blocks can be small (512 or 1024 ids: one or two
+// ranking passes per wave). Measured for 32768 ids, launch to launch: 8.7 us with 64 blocks of 512 ids (10.5 with 16
+// blocks of 2048) against 12.3 with the rendezvous, of which 2.2 us are the first trip to memory, 2.4 the counting
+// (64 LDS atomics per thread), 1.9 column sums and scan, 1.0 the ranking; an empty launch is 3.3 us of the total.
+// The work grows with blocks x ids, so the host takes this form up to kRecountMaxBlocks blocks of 1024 ids only.
+constexpr int kRecountMaxBlocks = 64;
+
+template <int kThreads, int kPerWave, bool kRecount>
 __global__ __launch_bounds__(kThreads) void moe_index_fused_kernel(const int32_t* __restrict__ ids, int64_t n, int topk,
                                                                   int G, int nbits, int32_t* hist, int32_t* ctrl,
                                                                   int32_t* __restrict__ splits,
@@ -244,15 +254,16 @@ __global__ __launch_bounds__(kThreads) void moe_index_fused_kernel(const int32_t
                                                                   int32_t* __restrict__ gather_idx,
                                                                   int32_t* __restrict__ topk_idx) {
   constexpr int kWaves = kThreads / 64, kItems = kWaves * kPerWave, kPasses = kPerWave / 64;
-  extern __shared__ int32_t s_mem[];  // [kWaves][G] wave counters, [G] column sums
+  extern __shared__ int32_t s_mem[];  // [kWaves][G] wave counters, [G] column sums, kRecount: [2][G] ids before / behind
   int32_t* const s_cnt = s_mem;
   int32_t* const s_col = s_mem + kWaves * G;
+  int32_t* const s_out = s_col + G;
   __shared__ int32_t s_part[kWaves];
   __shared__ int s_flag;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int B = gridDim.x, b = blockIdx.x;
   int gen0 = 0;
-  if (B > 1 && threadIdx.x == 0) gen0 = __hip_atomic_load(ctrl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (!kRecount && B > 1 && threadIdx.x == 0) gen0 = __hip_atomic_load(ctrl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   // the wave's ids first: the loads are in flight while the counters are cleared
   const int64_t wbase = (int64_t)b * kItems + (int64_t)wave * kPerWave;
   int e_of[kPasses];
@@ -261,7 +272,40 @@ __global__ __launch_bounds__(kThreads) void moe_index_fused_kernel(const int32_t
     const int64_t i = wbase + u * 64 + lane;
     e_of[u] = i < n ? ids[i] : -1;
   }
-  for (int g = threadIdx.x; g < kWaves * G; g += kThreads) s_cnt[g] = 0;
+  // kRecount: the other blocks' ids, four per load, kVecBatch loads in flight (the ranges are multiples of four ids,
+  // so a vector lies on one side of this block's range or inside it). The first batch (all of a decode step's ids)
+  // goes out here, together with the block's own ids, so that there is one wait for memory and not two.
+  constexpr int kVecBatch = kRecount ? 16 : 1;
+  const int64_t own_lo = (int64_t)b * kItems, own_hi = own_lo + kItems;
+  const int64_t n_vec = (n + 3) / 4;
+  int4v q[kVecBatch];
+  auto load_others = [&](int64_t v0) {
+#pragma unroll
+    for (int u = 0; u < kVecBatch; ++u) {
+      const int64_t vi = v0 + (int64_t)u * kThreads;
+      const bool mine = vi * 4 >= own_lo && vi * 4 < own_hi;
+      q[u] = int4v{-1, -1, -1, -1};
+      if (vi < n_vec && !mine) {
+        if (vi * 4 + 3 < n) q[u] = ((const int4v*)ids)[vi];
+        else
+          for (int j = 0; j < 4; ++j) q[u][j] = vi * 4 + j < n ? ids[vi * 4 + j] : -1;
+      }
+    }
+  };
+  auto count_others = [&](int64_t v0) {
+#pragma unroll
+    for (int u = 0; u < kVecBatch; ++u) {
+      const int64_t vi = v0 + (int64_t)u * kThreads;
+      int32_t* const row = s_out + (vi * 4 < own_lo ? 0 : G);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (q[u][j] >= 0 && q[u][j] < G) atomicAdd(&row[q[u][j]], 1);
+    }
+  };
+  if constexpr (kRecount) {
+    if (B > 1) load_others(threadIdx.x);
+  }
+  for (int g = threadIdx.x; g < (kWaves + (kRecount ? 3 : 0)) * G; g += kThreads) s_cnt[g] = 0;
   __syncthreads();
   // 1. per-wave counts
   int32_t* const my_cnt = s_cnt + wave * G;
@@ -270,8 +314,17 @@ __global__ __launch_bounds__(kThreads) void moe_index_fused_kernel(const int32_t
     if (e_of[u] < 0 || e_of[u] >= G) e_of[u] = -1;
     if (e_of[u] >= 0) atomicAdd(&my_cnt[e_of[u]], 1);
   }
+  if constexpr (kRecount) {
+    if (B > 1) {
+      count_others(threadIdx.x);
+      for (int64_t v0 = threadIdx.x + (int64_t)kVecBatch * kThreads; v0 < n_vec; v0 += (int64_t)kVecBatch * kThreads) {
+        load_others(v0);
+        count_others(v0);
+      }
+    }
+  }
   __syncthreads();
-  if (B > 1) {
+  if (!kRecount && B > 1) {
     for (int g = threadIdx.x; g < G; g += kThreads) {
       int32_t t = 0;
 #pragma unroll
@@ -310,7 +363,12 @@ __global__ __launch_bounds__(kThreads) void moe_index_fused_kernel(const int32_t
   // 3. column sums: s_col[g] = ids of expert g in all blocks; the blocks before this one go into wave 0's start
   for (int g = threadIdx.x; g < G; g += kThreads) {
     int32_t total = 0, before = 0;
-    if (B > 1) {
+    if (kRecount && B > 1) {
+      before = s_out[g];
+      total = before + s_out[G + g];
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) total += s_cnt[w * G + g];
+    } else if (B > 1) {
       for (int r = 0; r < B; ++r) {
         const int32_t h = __hip_atomic_load(hist + (int64_t)r * G + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         total += h;
@@ -930,15 +988,29 @@ static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, 
   const DeviceInfo& di = device_info();
   const int64_t fused_blocks = ceil_div(n_ids > 0 ? n_ids : 1, kFusedItems);
   if (di.ok == 1 && fused_blocks <= di.num_cus && getenv("TDIST_MOE_INDEX_LAUNCHES") == nullptr) {
-    auto kern = moe_index_fused_kernel<kFusedThreads, kFusedPerWave>;
-    static bool attr_set = false;
-    if (!attr_set) {
-      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (kFusedThreads / 64 + 1) * kMoeMaxExperts * 4) != hipSuccess)
+    // few ids: every block counts all of them itself and nothing is exchanged (TDIST_MOE_INDEX_RENDEZVOUS keeps the
+    // exchange, for tests and measurements)
+    constexpr int kLdsLimit = 160 * 1024 - 256;          // (the kernel has a few static words of its own)
+    constexpr int kRowsPlain = kFusedThreads / 64 + 1;   // wave counters, column sums
+    constexpr int kRowsRecount = kRowsPlain + 2;         // and the ids before / behind the block
+    constexpr int kSmall = kFusedThreads;                // ids per block of the recounting forms: 512, or 1024
+    const int64_t n1 = n_ids > 0 ? n_ids : 1;
+    const bool can_recount = kRowsRecount * G * 4 <= kLdsLimit && aligned16(ids) && getenv("TDIST_MOE_INDEX_RENDEZVOUS") == nullptr;
+    // 0: blocks of 2048 ids that exchange their histograms; 1 / 2: blocks of 512 / 1024 ids that count everything
+    const int form = !can_recount ? 0 : ceil_div(n1, kSmall) <= kRecountMaxBlocks ? 1 : ceil_div(n1, 2 * kSmall) <= kRecountMaxBlocks ? 2 : 0;
+    auto kern = form == 1 ? moe_index_fused_kernel<kFusedThreads, kSmall / 8, true>
+              : form == 2 ? moe_index_fused_kernel<kFusedThreads, kSmall / 4, true>
+                          : moe_index_fused_kernel<kFusedThreads, kFusedPerWave, false>;
+    const int64_t blocks = form == 1 ? ceil_div(n1, kSmall) : form == 2 ? ceil_div(n1, 2 * kSmall) : fused_blocks;
+    const int rows = form != 0 ? kRowsRecount : kRowsPlain;
+    static bool attr_set[3] = {false, false, false};
+    if (!attr_set[form]) {
+      const int most = rows * kMoeMaxExperts * 4 < kLdsLimit ? rows * kMoeMaxExperts * 4 : kLdsLimit;
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess)
         return fail(TDIST_ERR_LAUNCH, "%s: cannot reserve LDS for the index kernel", who);
-      attr_set = true;
+      attr_set[form] = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)fused_blocks), dim3(kFusedThreads), (size_t)(kFusedThreads / 64 + 1) * G * 4, stream,
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kFusedThreads), (size_t)rows * G * 4, stream,
                        ids, n_ids, want_index ? topk : 1, G, id_bits(G), hist, scan_counter, splits, cumsum,
                        want_index ? scatter_idx : nullptr, gather_idx, topk_idx);
     return launch_status(who);

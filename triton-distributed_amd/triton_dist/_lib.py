@@ -72,6 +72,8 @@ BENCH_LIB_PATH = os.path.join(_HERE, "_lib", "libtdist_bench.so")
 BENCH_PROTOTYPES = {
     "tdist_bench_last_error_string": (c_char_p, []),
     "tdist_copy_bytes": (_I, [_P, _P, _L, _P]),
+    "tdist_fill_bytes": (_I, [_P, _L, _P]),
+    "tdist_read_bytes": (_I, [_P, _L, _P, _P]),
     "tdist_mfma_rate_probe": (_I, [_I, _I, _I, _P, _P]),
     "tdist_mfma_rate_probe_16row": (_I, [_I, _I, _I, _P, _P]),
 }

@@ -80,6 +80,7 @@ class AllToAllContext:
         self.MOD_VALUE = 1000000
         # index tensors of moe_dispatch_preprocess(..., ctx=self): two sets, allocated on first use for a shape
         self.index_sets, self.index_key, self.index_calls = None, None, 0
+        self.index_workspace, self.index_args = None, None
 
 
 def create_all_to_all_context(
@@ -133,6 +134,17 @@ def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_to
     One kernel launch. With ``ctx`` the five tensors are the context's own (allocated on the first call for a shape,
     two sets used in turn like the receive buffers, so a result stays valid until the call after next) and the call
     allocates nothing. Returns (splits, split_cumsum, scatter_idx, gather_idx[, topk_idx])."""
+    if ctx is not None and ctx.index_key == (exp_indices.shape[0], exp_indices.shape[1], num_experts, exp_indices.device) \
+            and exp_indices.dtype == torch.int32 and exp_indices.is_contiguous():
+        # the context has seen this shape: its tensors' addresses are at hand and the host does next to nothing
+        # (the index kernel takes ~9 us on the device; the general path below costs more than that on the host)
+        which = ctx.index_calls % 2
+        ctx.index_calls += 1
+        out = ctx.index_sets[which]
+        head, tail = ctx.index_args[which]
+        _lib.call("tdist_moe_scatter_index", exp_indices.data_ptr(), *head, _lib.ptr(out[4] if want_topk_index else None),
+                  *tail, _lib.stream_ptr())
+        return out if want_topk_index else out[:4]
     _lib.require_cuda(exp_indices)
     if exp_indices.dtype != torch.int32:
         exp_indices = exp_indices.to(torch.int32)
@@ -148,18 +160,21 @@ def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_to
                 torch.empty(n, dtype=torch.int32, device=dev),
                 torch.empty(n, dtype=torch.int32, device=dev))
 
+    ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
     if ctx is not None:
-        key = (T, topk, num_experts, dev)
-        if ctx.index_key != key:
-            ctx.index_sets, ctx.index_key, ctx.index_calls = [alloc(), alloc()], key, 0
-        splits, cumsum, scatter_idx, gather_idx, topk_idx = ctx.index_sets[ctx.index_calls % 2]
-        ctx.index_calls += 1
+        # (a new shape: two sets of result tensors and a zeroed workspace of the context's own; the calls of one
+        # context are ordered on its stream, so they may share it)
+        ctx.index_sets, ctx.index_key, ctx.index_calls = [alloc(), alloc()], (T, topk, num_experts, dev), 1
+        ctx.index_workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+        ctx.index_args = [((n, topk, num_experts, t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), t[3].data_ptr()),
+                           (ctx.index_workspace.data_ptr(), ws_bytes)) for t in ctx.index_sets]
+        splits, cumsum, scatter_idx, gather_idx, topk_idx = ctx.index_sets[0]
+        workspace = ctx.index_workspace
     else:
         splits, cumsum, scatter_idx, gather_idx, topk_idx = alloc()
+        workspace = _lib.zeroed_scratch(ws_bytes, dev)
     if not want_topk_index:
         topk_idx = None
-    ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
-    workspace = _lib.zeroed_scratch(ws_bytes, dev)
     _lib.call("tdist_moe_scatter_index", exp_indices.data_ptr(), n, topk, num_experts, splits.data_ptr(),
               cumsum.data_ptr(), scatter_idx.data_ptr(), gather_idx.data_ptr(), _lib.ptr(topk_idx),
               workspace.data_ptr(), workspace.numel(), _lib.stream_ptr())
