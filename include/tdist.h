@@ -142,6 +142,14 @@ int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int 
 int tdist_producer_mark(uint64_t* stamp, void* stream);
 int tdist_producer_wait_until(const uint64_t* stamp, int64_t offset_ns, void* stream);
 
+/* A gated GEMM whose bounded flag wait expires writes TDIST_ERR_TIMEOUT and the chunk into its status words, and
+ * while status[0] is non-zero every later wait of a launch on the same words gives up after one poll: that is what
+ * lets all workgroups of the failing launch leave quickly, and it would make the next launch skip its gated tiles as
+ * well. This call, queued in front of the next launch, confines it to one launch: it moves a non-zero status into
+ * first_error[0..1] (unless that already holds an earlier one; NULL: dropped) and clears status. No counterpart in
+ * the reference, whose waits are unbounded. Safe to record into a HIP graph. */
+int tdist_status_retire(int32_t* status, int32_t* first_error, void* stream);
+
 /* Stream-ordered store of `value` into *flag by a one-thread kernel (release, system scope).
  *   replaces set_signal  kernels/amd/common_ops.py:97-112 */
 int tdist_flag_set(int32_t* flag, int value, void* stream);

@@ -167,6 +167,44 @@ def test_gate_holds_and_times_out(cuda):
     assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
 
 
+def test_a_timeout_slows_down_one_call_and_is_not_forgotten(cuda):
+    """The op after a call whose flag wait expired runs normally (the status words are retired in front of every
+    launch: an expired wait makes the waits of ITS launch give up at once, not those of the next), and check_status
+    still reports the first expired wait, however many calls followed; tdist_status_retire by itself on the C-ABI."""
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import ag_gemm_intra_node, create_ag_gemm_intra_node_context
+    announce("ag-gemm timeout retired by the next call")
+    world, rank, mpr, K, N = 4, 0, 256, 256, 384
+    shards, b = make_ag_case(world, mpr, K, N, torch.bfloat16, seed=17)
+    ctx = create_ag_gemm_intra_node_context(world * mpr, N, K, torch.bfloat16, torch.bfloat16, rank, world, None, M_PER_CHUNK=256)
+    ctx.set_peer_shards({r: s.to(cuda) for r, s in enumerate(shards) if r != rank})
+    a_d, b_d = shards[rank].to(cuda), b.to(cuda)
+    ref = golden.ag_gemm_fp32(shards, b)
+    ctx.held_chunks, ctx.spin_limit = (2, ), 200
+    ag_gemm_intra_node(a_d, b_d, False, ctx)
+    torch.cuda.synchronize()
+    assert ctx.status.tolist()[:2] == [_lib.TDIST_ERR_TIMEOUT, 2]
+    ctx.held_chunks, ctx.spin_limit = (), 0
+    for _ in range(2):
+        c = ag_gemm_intra_node(a_d, b_d, False, ctx)
+        torch.cuda.synchronize()
+        assert golden.max_rel_err(c.float().cpu(), ref) <= 1e-2
+        assert ctx.status.tolist() == [0, 0, _lib.TDIST_ERR_TIMEOUT, 2]
+    with pytest.raises(_lib.TdistError, match="chunk 2"):
+        ctx.check_status()
+    assert ctx.status.tolist() == [0, 0, 0, 0]
+    ctx.check_status()
+    # the entry point: a later error does not replace the first one; a null first_error drops the status
+    words = torch.tensor([_lib.TDIST_ERR_TIMEOUT, 5, _lib.TDIST_ERR_TIMEOUT, 2], dtype=torch.int32, device=cuda)
+    _lib.call("tdist_status_retire", words.data_ptr(), words.data_ptr() + 8, None)
+    torch.cuda.synchronize()
+    assert words.tolist() == [0, 0, _lib.TDIST_ERR_TIMEOUT, 2]
+    words[0], words[1] = 7, 9
+    _lib.call("tdist_status_retire", words.data_ptr(), None, None)
+    torch.cuda.synchronize()
+    assert words.tolist() == [0, 0, _lib.TDIST_ERR_TIMEOUT, 2]
+
+
 def test_gate_released_by_a_stream_while_the_gemm_waits(cuda):
     """Flags are set by a second stream while the GEMM waits for them (explicit chunk order, last chunk first)."""
     from triton_dist import _lib

@@ -66,6 +66,18 @@ __global__ void flag_fill_kernel(int32_t* flags, int n, int value) {
   if (i < n) __hip_atomic_store(flags + i, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// status[0..1] of the launch before → first_error[0..1] if that is still clear; status cleared for the next launch
+__global__ void status_retire_kernel(int32_t* status, int32_t* first_error) {
+  if (threadIdx.x != 0) return;
+  const int32_t code = status[0];
+  if (code != 0 && first_error != nullptr && first_error[0] == 0) {
+    first_error[1] = status[1];
+    first_error[0] = code;
+  }
+  status[1] = 0;
+  status[0] = 0;
+}
+
 // Link pacing of the one-GPU producer: a time stamp of the constant-rate wall clock, and a one-wave kernel that
 // holds its stream until that clock has moved `ticks` past the stamp. The loop ends by itself: the clock only
 // moves forward, a stamp from the future makes the unsigned difference huge, and `ticks` is capped by the host.
@@ -203,6 +215,12 @@ int tdist_flag_set(int32_t* flag, int value, void* stream) {
   if (!flag) return fail(TDIST_ERR_INVALID, "tdist_flag_set: null flag");
   hipLaunchKernelGGL(flag_fill_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, flag, 1, value);
   return launch_status("tdist_flag_set");
+}
+
+int tdist_status_retire(int32_t* status, int32_t* first_error, void* stream) {
+  if (!status) return fail(TDIST_ERR_INVALID, "tdist_status_retire: null status");
+  hipLaunchKernelGGL(status_retire_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, status, first_error);
+  return launch_status("tdist_status_retire");
 }
 
 int tdist_producer_push_chunk(void* dst, const void* src, int64_t nbytes, int32_t* flag, const int32_t* one,

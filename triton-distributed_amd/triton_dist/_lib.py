@@ -38,6 +38,7 @@ PROTOTYPES = {
     "tdist_producer_mark": (_I, [_P, _P]),
     "tdist_producer_wait_until": (_I, [_P, _L, _P]),
     "tdist_flag_set": (_I, [_P, _I, _P]),
+    "tdist_status_retire": (_I, [_P, _P, _P]),
     "tdist_flag_fill": (_I, [_P, _I, _I, _P]),
     "tdist_gemm_rs_scatter_bf16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P]),
     "tdist_gemm_rs_scatter_f16": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P]),

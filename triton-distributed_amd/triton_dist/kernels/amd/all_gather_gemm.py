@@ -122,7 +122,9 @@ class AllGatherGEMMTensorParallelContext:
     arrival_order: Optional[List[Tuple[int, int]]] = None
     held_chunks: Tuple[int, ...] = ()
     spin_limit: int = 0          # 0 = library default (seconds of polling)
-    status: Optional[torch.Tensor] = None  # int32[2]: error code, chunk that timed out
+    # int32[4]: [0:2] error code and chunk of the current call's expired flag wait, [2:4] the first one of earlier
+    # calls that nobody has looked at yet (every call retires its predecessor's, so a timeout slows down one launch)
+    status: Optional[torch.Tensor] = None
     # True: chunk copies go to the copy engines (hipMemcpyDeviceToDeviceNoCU), as the reference's cp-engine
     # producer does across GPUs. On one GPU the engines move ~55 GB/s each, far below a kernel copy inside HBM, so
     # the default is the blit path.
@@ -178,9 +180,12 @@ class AllGatherGEMMTensorParallelContext:
         self.peer_ptrs = torch.tensor(ptrs, dtype=torch.int64).to(self.one.device)
 
     def check_status(self):
-        """Synchronises and raises TdistError if a bounded flag wait expired in an earlier call."""
+        """Synchronises and raises TdistError if a bounded flag wait expired in an earlier call (the earliest one
+        since the last check)."""
         torch.cuda.synchronize()
-        code, chunk = self.status.tolist()
+        code, chunk, first_code, first_chunk = self.status.tolist()
+        if first_code != 0:
+            code, chunk = first_code, first_chunk
         if code != 0:
             self.status.zero_()
             raise _lib.TdistError(code, "flag wait expired for chunk %d" % chunk)
@@ -222,7 +227,7 @@ def create_ag_gemm_intra_node_context(max_M, N, K, input_dtype, output_dtype, ra
     _ag_streams = [torch.cuda.Stream() for _ in range(min(num_ranks, 2))] if ag_streams is None else ag_streams
     _gemm_stream = current_stream if gemm_stream is None else gemm_stream
     one = torch.ones((1024, ), dtype=torch.int32, device=device)
-    status = torch.zeros((2, ), dtype=torch.int32, device=device)
+    status = torch.zeros((4, ), dtype=torch.int32, device=device)
     start_stamp = torch.zeros((1, ), dtype=torch.int64, device=device)
     torch.cuda.synchronize()
 
@@ -351,6 +356,9 @@ def ag_gemm_intra_node_op(a, b, c, rank, num_ranks, workspace_tensors, one, barr
         local = None
 
     def call_gemm(max_wgs):
+        if ctx is not None:
+            # the launch before may have given up on a flag: keep what it reported, start this one clean
+            _lib.call("tdist_status_retire", ctx.status.data_ptr(), ctx.status.data_ptr() + 8, gemm_stream.cuda_stream)
         if local is None:
             if not a.is_contiguous():
                 raise ValueError("the local shard must be contiguous")

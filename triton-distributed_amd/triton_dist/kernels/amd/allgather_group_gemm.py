@@ -158,8 +158,12 @@ class MoE_AllGatherGroupGEMMTensorParallelContext:
         self.peer_shards = {r: t for r, t in shards.items() if r != self.rank}
 
     def check_status(self):
+        """Synchronises and raises TdistError if a bounded flag wait expired in an earlier call (the earliest one
+        since the last check; status[0:2] is the current call's, [2:4] the first of the calls before it)."""
         torch.cuda.synchronize()
-        code, segment = self.status.tolist()
+        code, segment, first_code, first_segment = self.status.tolist()
+        if first_code != 0:
+            code, segment = first_code, first_segment
         if code != 0:
             self.status.zero_()
             raise _lib.TdistError(code, "flag wait expired for rank segment %d" % segment)
@@ -203,7 +207,7 @@ def create_ag_group_gemm_intra_node_context(tp_pg, tensor_A, tensor_B, full_topk
         ag_stream=torch.cuda.Stream() if ag_stream is None else ag_stream,
         group_gemm_stream=group_gemm_stream, BLOCK_M=BLOCK_M, BLOCK_N=BLOCK_N, BLOCK_K=BLOCK_K,
         GROUP_SIZE_M=GROUP_SIZE_M, stages=stages, warps=warps, rank_block_num=rank_block_num, first_block=first_block,
-        one=torch.ones((16, ), dtype=torch.int32, device=device), status=torch.zeros((2, ), dtype=torch.int32, device=device),
+        one=torch.ones((16, ), dtype=torch.int32, device=device), status=torch.zeros((4, ), dtype=torch.int32, device=device),
         sk_workspace=_lib.new_split_k_workspace(device) if split_k else None)
 
 
@@ -252,6 +256,8 @@ def ag_group_gemm_intra_node(a, b, ctx=None, full_topk_ids=None, num_experts=Non
         _lib.call("tdist_producer_push_chunk", workspace.data_ptr() + r * nbytes, ctx.peer_shards[r].data_ptr(), nbytes,
                   barrier.data_ptr() + 4 * r, ctx.one.data_ptr(), 0, ctx.ag_stream.cuda_stream)
     max_wgs = max(1, _lib.load().tdist_num_cus() - ctx.producer_cus) if (W > 1 and ctx.producer_cus > 0) else 0
+    # the launch before may have given up on a flag: keep what it reported, start this one clean
+    _lib.call("tdist_status_retire", ctx.status.data_ptr(), ctx.status.data_ptr() + 8, gemm_stream.cuda_stream)
     # (the launch names its stream; nothing here runs on torch's current stream)
     group_gemm_gated(workspace[:M_per_rank * W], a, rank * M_per_rank, b_nk, C, ctx.sorted_topk_ids,
                      ctx.aligned_expert_ids, ctx.aligned_barrier_ids, ctx.aligned_num_tokens, ctx.BLOCK_M,
