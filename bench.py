@@ -221,7 +221,7 @@ def bench_c1(dev, steps, warmup):
     full = torch.cat(shards).to(dev)
     flags = torch.ones(world, dtype=torch.int32, device=dev)
     out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
-    pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 1024, rank, world), steps, warmup)
+    pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 1024, rank, world, sk_workspace=ctx.sk_workspace), steps, warmup)
     r = roof("mfma", flops, pre_s, "bf16", MEASURED_TRAFFIC_BYTES["c1_gemm"])
     cs, cores = cpu_time(lambda: golden.torch_ag_gemm(shards, b))
     r["cpu_baseline"] = {"value": round(flops / cs / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
@@ -263,7 +263,8 @@ def bench_c3(dev, steps, warmup):
     full = torch.cat([s.view(torch.uint8) for s in shards]).to(dev).view(torch.float8_e4m3fn)
     flags = torch.ones(world, dtype=torch.int32, device=dev)
     out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
-    pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 2048, rank, world, row_scale=sa, col_scale=sb),
+    pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 2048, rank, world, row_scale=sa, col_scale=sb,
+                                             sk_workspace=ctx.sk_workspace),
                           steps, warmup)
     r = roof("mfma", flops, pre_s, "fp8", MEASURED_TRAFFIC_BYTES["c3_gemm"])
     sa_c, sb_c = sa.cpu(), sb.cpu()
@@ -435,7 +436,7 @@ def bench_group_gemm(dev, steps, warmup):
     pre_s = time_launches(
         lambda: group_gemm_gated(full, None, 0, w_nk, out, ctx.sorted_topk_ids, ctx.aligned_expert_ids,
                                  ctx.aligned_barrier_ids, ctx.aligned_num_tokens, block, ctx.full_num_tokens, topk, mpr,
-                                 ctx.first_block, flags, rank), steps, warmup)
+                                 ctx.first_block, flags, rank, sk_workspace=ctx.sk_workspace), steps, warmup)
     r = roof("mfma", flops, pre_s, "bf16")
     r["workload"] = "8192 tokens x top-2 of 8 experts, K 14336, N 512 per rank, row blocks of 128 (128 x 256 tiles)"
     r["with_live_producer_us"] = round(live_s * 1e6, 2) if live_s is not None else None
