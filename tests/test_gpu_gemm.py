@@ -618,6 +618,32 @@ def test_k_ending_inside_a_k_tile(cuda, dtype, K):
         gated_gemm(a_d[:, :K - 4 // esz], None, 0, b_d[:, :K - 4 // esz], c, None, 0, 0, 1)
 
 
+@pytest.mark.parametrize("dtype,K", [(torch.bfloat16, 2056), (torch.float8_e4m3fn, 4112)])
+def test_ragged_chunks_k_tail_and_split_round_together(cuda, dtype, K):
+    """Chunks of 200 rows, a K that ends 16 bytes into its last K tile and a last round cut along K (21 tiles of
+    128 x 128 on 256 workgroups: four pieces each, the last piece holding the ragged K tile), three launches in a row
+    on one workspace: exact on integer-valued inputs."""
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import gated_gemm
+    announce("gemm ragged chunks + K tail + split round %s" % dtype)
+    world, mpc, rank, N = 4, 200, 2, 328
+    M = world * mpc
+    ws = _lib.new_split_k_workspace(cuda)
+    status = torch.zeros(2, dtype=torch.int32, device=cuda)
+    flags = torch.ones(world, dtype=torch.int32, device=cuda)
+    for launch in range(3):
+        g = torch.Generator().manual_seed(K + launch)
+        a = torch.randint(-2, 3, (M, K), generator=g).float()
+        b = torch.randint(-2, 3, (N, K), generator=g).float()
+        c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+        gated_gemm(a.to(dtype).to(cuda), None, 0, b.to(dtype).to(cuda), c, flags, mpc, rank, world, status=status, sk_workspace=ws)
+        torch.cuda.synchronize()
+        assert status.tolist() == [0, 0]
+        assert torch.equal(c, (a.to(cuda) @ b.to(cuda).T).to(torch.bfloat16)), "launch %d" % launch
+    # (the split form really ran: the workspace's epoch word has moved)
+    assert int(ws.view(torch.int32)[0]) != 0
+
+
 @pytest.mark.parametrize("world,mpc,rank", [(4, 200, 1), (8, 72, 7), (2, 1000, 0), (3, 130, 2)])
 def test_chunks_that_are_no_whole_tiles(cuda, world, mpc, rank):
     """m_per_chunk of any size: a 128-row tile waits for every flag its rows touch. With every flag but one released,
