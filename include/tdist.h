@@ -301,8 +301,11 @@ int tdist_moe_dispatch_tokens_quant(const void* tokens_bf16, int hidden, int gro
  * reference's dtype), one segment of n_per_iteration entries per rank ("iteration"). Per segment, in order, the
  * entries are grouped by expert keeping their flat order, every group is padded to a multiple of block_size, and the
  * padded groups are laid end to end, segment after segment:
- *   sorted_token_ids[pos] = flat index of the entry (positions of padding keep what the caller pre-filled, the
- *                           reference fills with n_total); capacity n_total + num_experts*num_iterations*(block_size-1)
+ *   sorted_token_ids[pos] = flat index of the entry; capacity n_total + num_experts*num_iterations*(block_size-1).
+ *                           Positions of padding keep what was there before: with sorted_fill > 0 the call itself first
+ *                           stores n_total into sorted_token_ids[0 .. sorted_fill) (the reference's
+ *                           sorted_ids.fill_(numel) in front of its op, allgather_group_gemm.py:103), with 0 the caller
+ *                           has pre-filled the array
  *   expert_ids[b], block_barrier_ids[b] = expert and segment of block b; at most
  *                           n_total / block_size + num_experts * num_iterations blocks are written (the reference
  *                           allocates n_total + num_experts * num_iterations entries)
@@ -311,9 +314,10 @@ int tdist_moe_dispatch_tokens_quant(const void* tokens_bf16, int hidden, int gro
  * first 256 bytes are control words, ZERO on first use and left zero by every call (see tdist_moe_workspace_bytes). */
 int64_t tdist_moe_align_workspace_bytes(int64_t n_total, int num_experts, int num_iterations);
 int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_total, int num_experts,
-                               int num_iterations, int64_t n_per_iteration, int block_size, int32_t* sorted_token_ids,
-                               int32_t* expert_ids, int32_t* block_barrier_ids, int32_t* rank_block_num,
-                               int32_t* total_tokens_post_pad, void* workspace, int64_t workspace_bytes, void* stream);
+                               int num_iterations, int64_t n_per_iteration, int block_size,
+                               int32_t* sorted_token_ids, int64_t sorted_fill, int32_t* expert_ids,
+                               int32_t* block_barrier_ids, int32_t* rank_block_num, int32_t* total_tokens_post_pad,
+                               void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Chunk-gated grouped GEMM of the MoE tensor-parallel path: the consumer of the align / sort step.
  *   replaces kernel_consumer_m_parallel_scatter_group_gemm   kernels/nvidia/allgather_group_gemm.py:238-314

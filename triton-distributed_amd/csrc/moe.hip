@@ -901,25 +901,35 @@ __global__ __launch_bounds__(kCombineWaves * 64) void moe_combine_kernel(
 // the padded layout is its position in the unpadded sorted order moved by the padding in front of its group.
 
 // keys[i] = (i / per_iter) * E + ids[i], or -1 for an id outside [0, E)
+// Also pre-fills sorted_ids[0 .. fill_n) with n (the value padding positions keep; fill_n = 0: the caller has done it).
 __global__ __launch_bounds__(256) void moe_align_keys_kernel(const void* __restrict__ ids, int ids_int64, int64_t n,
-                                                            int64_t per_iter, int E, int32_t* __restrict__ keys) {
+                                                            int64_t per_iter, int E, int32_t* __restrict__ keys,
+                                                            int32_t* __restrict__ sorted_ids, int64_t fill_n) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < fill_n) sorted_ids[i] = (int32_t)n;
   if (i >= n) return;
   const int64_t id = ids_int64 ? ((const int64_t*)ids)[i] : (int64_t)((const int32_t*)ids)[i];
   keys[i] = (id >= 0 && id < E) ? (int32_t)((i / per_iter) * E + id) : -1;
 }
 
-// One workgroup: padded exclusive prefix over the G = R * E group sizes, the per-block expert / segment ids, the
-// blocks per segment and the padded total.
-__global__ __launch_bounds__(kScanThreads) void moe_align_pad_kernel(const int32_t* __restrict__ splits, int G, int E,
-                                                                    int R, int block_size,
-                                                                    int32_t* __restrict__ pad_cum,
-                                                                    int32_t* __restrict__ expert_ids,
-                                                                    int32_t* __restrict__ block_barrier_ids,
-                                                                    int32_t* __restrict__ rank_block_num,
-                                                                    int32_t* __restrict__ total_post_pad) {
-  __shared__ int32_t s_part[kScanThreads];
-  const int per = (G + kScanThreads - 1) / kScanThreads;  // consecutive groups per thread
+// Padding and placement in one launch. Every workgroup works out the padded exclusive prefix over the G = R * E group
+// sizes for itself (G <= 4096 values through LDS: cheaper than a launch of its own and the wait for it), then places
+// its 256 entries: an entry's position in the padded layout is its position in the unpadded sorted order moved by the
+// padding in front of its group. Workgroup 0 also writes the per-block expert / segment ids, the blocks per segment
+// and the padded total.
+constexpr int kPlaceThreads = 256;
+__global__ __launch_bounds__(kPlaceThreads) void moe_align_place_kernel(
+    const int32_t* __restrict__ keys, const int32_t* __restrict__ scatter_idx, const int32_t* __restrict__ splits,
+    const int32_t* __restrict__ cumsum, int64_t n, int G, int E, int R, int block_size, int32_t* __restrict__ sorted_ids,
+    int32_t* __restrict__ expert_ids, int32_t* __restrict__ block_barrier_ids, int32_t* __restrict__ rank_block_num,
+    int32_t* __restrict__ total_post_pad) {
+  extern __shared__ int32_t s_pad[];  // [G + 1] padded exclusive prefix
+  __shared__ int32_t s_part[kPlaceThreads];
+  // the entry's own loads first: they do not depend on the prefix
+  const int64_t i = (int64_t)blockIdx.x * kPlaceThreads + threadIdx.x;
+  const int32_t k = i < n ? keys[i] : -1;
+  const int32_t rank_in_group = k >= 0 ? scatter_idx[i] - cumsum[k] : 0;
+  const int per = (G + kPlaceThreads - 1) / kPlaceThreads;  // consecutive groups per thread
   const int g0 = threadIdx.x * per;
   int32_t local_total = 0;
   for (int j = 0; j < per; ++j) {
@@ -928,42 +938,34 @@ __global__ __launch_bounds__(kScanThreads) void moe_align_pad_kernel(const int32
   }
   s_part[threadIdx.x] = local_total;
   __syncthreads();
-  for (int off = 1; off < kScanThreads; off <<= 1) {
+  for (int off = 1; off < kPlaceThreads; off <<= 1) {
     const int32_t v = (threadIdx.x >= off) ? s_part[threadIdx.x - off] : 0;
     __syncthreads();
     s_part[threadIdx.x] += v;
     __syncthreads();
   }
   int32_t run = s_part[threadIdx.x] - local_total;
-  if (threadIdx.x == 0) pad_cum[0] = 0;
+  if (threadIdx.x == 0) s_pad[0] = 0;
   for (int j = 0; j < per; ++j) {
     const int g = g0 + j;
     if (g < G) {
       const int32_t padded = (splits[g] + block_size - 1) / block_size * block_size;
-      for (int32_t b = run / block_size; b < (run + padded) / block_size; ++b) {
-        expert_ids[b] = g % E;
-        block_barrier_ids[b] = g / E;
+      if (blockIdx.x == 0) {
+        for (int32_t b = run / block_size; b < (run + padded) / block_size; ++b) {
+          expert_ids[b] = g % E;
+          block_barrier_ids[b] = g / E;
+        }
       }
       run += padded;
-      pad_cum[g + 1] = run;
+      s_pad[g + 1] = run;
     }
   }
-  __threadfence_block();  // pad_cum was written by this workgroup and is read back below
   __syncthreads();
-  for (int r = threadIdx.x; r < R; r += kScanThreads)
-    rank_block_num[r] = (pad_cum[(r + 1) * E] - pad_cum[r * E]) / block_size;
-  if (threadIdx.x == 0) *total_post_pad = pad_cum[G];
-}
-
-__global__ __launch_bounds__(256) void moe_align_place_kernel(const int32_t* __restrict__ keys,
-                                                             const int32_t* __restrict__ scatter_idx,
-                                                             const int32_t* __restrict__ cumsum,
-                                                             const int32_t* __restrict__ pad_cum, int64_t n,
-                                                             int32_t* __restrict__ sorted_ids) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  const int32_t k = keys[i];
-  if (k >= 0) sorted_ids[pad_cum[k] + (scatter_idx[i] - cumsum[k])] = (int32_t)i;
+  if (blockIdx.x == 0) {
+    for (int r = threadIdx.x; r < R; r += kPlaceThreads) rank_block_num[r] = (s_pad[(r + 1) * E] - s_pad[r * E]) / block_size;
+    if (threadIdx.x == 0) *total_post_pad = s_pad[G];
+  }
+  if (k >= 0) sorted_ids[s_pad[k] + rank_in_group] = (int32_t)i;
 }
 
 static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, int32_t* splits, int32_t* cumsum,
@@ -1239,14 +1241,15 @@ int64_t tdist_moe_align_workspace_bytes(int64_t n_total, int num_experts, int nu
   if (n_total < 0 || num_experts <= 0 || num_iterations <= 0) return 0;
   const int64_t G = (int64_t)num_experts * num_iterations;
   if (G > kMoeMaxExperts) return 0;
-  // keys, scatter index, gather index; group sizes, two prefix rows; then the index build's own scratch
+  // the index build's own scratch; then keys, scatter index, gather index, group sizes and their prefix
   return (3 * n_total + 3 * (G + 1)) * 4 + tdist_moe_workspace_bytes(n_total, (int)G);
 }
 
 int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_total, int num_experts,
                                int num_iterations, int64_t n_per_iteration, int block_size, int32_t* sorted_token_ids,
-                               int32_t* expert_ids, int32_t* block_barrier_ids, int32_t* rank_block_num,
-                               int32_t* total_tokens_post_pad, void* workspace, int64_t workspace_bytes, void* stream) {
+                               int64_t sorted_fill, int32_t* expert_ids, int32_t* block_barrier_ids,
+                               int32_t* rank_block_num, int32_t* total_tokens_post_pad, void* workspace,
+                               int64_t workspace_bytes, void* stream) {
   const char* who = "tdist_moe_align_block_size";
   if (!topk_ids || !sorted_token_ids || !expert_ids || !block_barrier_ids || !rank_block_num || !total_tokens_post_pad)
     return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
@@ -1257,6 +1260,7 @@ int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_to
   if (G > kMoeMaxExperts)
     return fail(TDIST_ERR_UNSUPPORTED, "%s: num_experts * num_iterations = %lld > %d", who, (long long)G, kMoeMaxExperts);
   if (n_total + G * (int64_t)(block_size - 1) > 0x7fffffffll) return fail(TDIST_ERR_UNSUPPORTED, "%s: too many entries", who);
+  if (sorted_fill < 0 || sorted_fill > 0x7fffffffll) return fail(TDIST_ERR_INVALID, "%s: sorted_fill %lld", who, (long long)sorted_fill);
   const int64_t need = tdist_moe_align_workspace_bytes(n_total, num_experts, num_iterations);
   if (!workspace || workspace_bytes < need)
     return fail(TDIST_ERR_WORKSPACE, "%s: workspace %lld B < %lld B", who, (long long)workspace_bytes, (long long)need);
@@ -1269,19 +1273,18 @@ int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_to
   int32_t* gather = scatter + n_total;
   int32_t* splits = gather + n_total;
   int32_t* cumsum = splits + (G + 1);
-  int32_t* pad_cum = cumsum + (G + 1);
   const int64_t blocks = ceil_div(n_total > 0 ? n_total : 1, 256);
-  if (n_total > 0)
-    hipLaunchKernelGGL(moe_align_keys_kernel, dim3((unsigned)blocks), dim3(256), 0, st, topk_ids, ids_int64, n_total,
-                       n_per_iteration > 0 ? n_per_iteration : 1, num_experts, keys);
+  // three launches: keys (and the pre-fill of the padding positions), the stable index on the keys, padding + placement
+  const int64_t key_items = n_total > sorted_fill ? n_total : sorted_fill;
+  if (key_items > 0)
+    hipLaunchKernelGGL(moe_align_keys_kernel, dim3((unsigned)ceil_div(key_items, 256)), dim3(256), 0, st, topk_ids, ids_int64,
+                       n_total, n_per_iteration > 0 ? n_per_iteration : 1, num_experts, keys, sorted_token_ids, sorted_fill);
   int rc = moe_index_common(keys, n_total, 1, (int)G, splits, cumsum, scatter, gather, nullptr, index_ws,
                             tdist_moe_workspace_bytes(n_total, (int)G), st, true, who);
   if (rc != TDIST_OK) return rc;
-  hipLaunchKernelGGL(moe_align_pad_kernel, dim3(1), dim3(kScanThreads), 0, st, splits, (int)G, num_experts, num_iterations,
-                     block_size, pad_cum, expert_ids, block_barrier_ids, rank_block_num, total_tokens_post_pad);
-  if (n_total > 0)
-    hipLaunchKernelGGL(moe_align_place_kernel, dim3((unsigned)blocks), dim3(256), 0, st, keys, scatter, cumsum, pad_cum,
-                       n_total, sorted_token_ids);
+  hipLaunchKernelGGL(moe_align_place_kernel, dim3((unsigned)blocks), dim3(kPlaceThreads), (size_t)(G + 1) * 4, st, keys, scatter,
+                     splits, cumsum, n_total, (int)G, num_experts, num_iterations, block_size, sorted_token_ids, expert_ids,
+                     block_barrier_ids, rank_block_num, total_tokens_post_pad);
   return launch_status(who);
 }
 

@@ -55,7 +55,7 @@ PROTOTYPES = {
     "tdist_quant_e4m3_groups": (_I, [_P, _L, _I, _I, _P, _P, _P]),
     "tdist_moe_dispatch_tokens_quant": (_I, [_P, _I, _I, _P, _I, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_align_workspace_bytes": (_L, [_L, _I, _I]),
-    "tdist_moe_align_block_size": (_I, [_P, _I, _L, _I, _I, _L, _I, _P, _P, _P, _P, _P, _P, _L, _P]),
+    "tdist_moe_align_block_size": (_I, [_P, _I, _L, _I, _I, _L, _I, _P, _L, _P, _P, _P, _P, _P, _L, _P]),
     "tdist_group_gemm_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
     "tdist_group_gemm_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
     "tdist_group_gemm_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _L, _P, _L, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),

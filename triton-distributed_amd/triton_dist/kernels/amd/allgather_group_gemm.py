@@ -46,20 +46,23 @@ def sort_topk_ids_align_block_size(
     n_per = num_tokens_per_rank * num_topk
     n_total = topk_ids.numel()
     assert n_total == n_per * num_ranks, "topk_ids must hold num_ranks * num_tokens_per_rank tokens"
-    sorted_ids = torch.empty(((n_per + num_experts * (block_size - 1)) * num_ranks, ), dtype=torch.int32, device=dev)
-    expert_ids = torch.empty(((n_per + num_experts) * num_ranks, ), dtype=torch.int32, device=dev)
-    block_barrier_ids = torch.empty(((n_per + num_experts) * num_ranks, ), dtype=torch.int32, device=dev)
-    rank_block_num = torch.empty(num_ranks, dtype=torch.int32, device=dev)
-    num_tokens_post_pad = torch.empty((1), dtype=torch.int32, device=dev)
+    # the five results are views of one allocation (sizes as in the reference, :100-121; every view 16-byte aligned)
+    n_sorted = (n_per + num_experts * (block_size - 1)) * num_ranks
+    n_blocks = (n_per + num_experts) * num_ranks
+    up4 = lambda n: (n + 3) // 4 * 4
+    flat = torch.empty(up4(n_sorted) + 2 * up4(n_blocks) + up4(num_ranks) + 4, dtype=torch.int32, device=dev)
+    sorted_ids, expert_ids, block_barrier_ids, rank_block_num, num_tokens_post_pad = (
+        t[:n] for t, n in zip(flat.split([up4(n_sorted), up4(n_blocks), up4(n_blocks), up4(num_ranks), 4]),
+                              (n_sorted, n_blocks, n_blocks, num_ranks, 1)))
     ws_bytes = _lib.load().tdist_moe_align_workspace_bytes(n_total, num_experts, num_ranks)
     if ws_bytes == 0:
         raise _lib.TdistError(_lib.TDIST_ERR_UNSUPPORTED,
                               "num_experts * num_ranks = %d is above what the align kernel handles" % (num_experts * num_ranks))
     def launch(stream):
         workspace = _lib.zeroed_scratch(ws_bytes, dev)   # (cached per stream: current is `stream` here)
-        sorted_ids.fill_(n_total)
+        # (sorted_ids.fill_(numel) of the reference, :103, is done by the call's first kernel)
         _lib.call("tdist_moe_align_block_size", topk_ids.data_ptr(), 1 if topk_ids.dtype == torch.int64 else 0, n_total,
-                  num_experts, num_ranks, n_per, block_size, sorted_ids.data_ptr(), expert_ids.data_ptr(),
+                  num_experts, num_ranks, n_per, block_size, sorted_ids.data_ptr(), n_sorted, expert_ids.data_ptr(),
                   block_barrier_ids.data_ptr(), rank_block_num.data_ptr(), num_tokens_post_pad.data_ptr(),
                   workspace.data_ptr(), ws_bytes, stream.cuda_stream)
 
