@@ -1276,9 +1276,9 @@ static int launch_gemm_cfg(const GemmParams& prm, int grid, hipStream_t stream, 
 }
 
 // ---- split-K workspace (the caller's, per call) ------------------------------------------------------------
-// [0, kSkHeaderBytes): control words, one flag and one acknowledgement word per workgroup, the scheduler's decision
-// records; then one fp32 tile per workgroup. The memory must be zero when it is first used; the kernels keep it
-// consistent from then on (tags, never cleared flags).
+// [0, kSkHeaderBytes): control words (epoch, done counter), one flag and one acknowledgement word per workgroup; then
+// one fp32 tile per workgroup. The memory must be zero when it is first used; the kernels keep it consistent from then
+// on (tags, never cleared flags).
 
 // 0 = off, 1 = on wherever the workspace allows, -1 = by the cost estimate
 static int sk_env() {
