@@ -178,7 +178,9 @@ def new_split_k_workspace(device=None):
     bytes: 64 MiB + 12 KiB on MI355X). Every context owns one: launches that share a workspace must be ordered, and
     contexts may run on streams of their own. Returns a uint8 tensor."""
     import torch
-    dev = torch.cuda.current_device() if device is None else torch.device(device).index
+    dev = None if device is None else torch.device(device).index
+    if dev is None:   # (no device, or "cuda" without an index: the current one)
+        dev = torch.cuda.current_device()
     with torch.cuda.device(dev):
         nbytes = load().tdist_gemm_split_k_workspace_bytes()
         if nbytes <= 0:
@@ -196,6 +198,8 @@ def zeroed_scratch(nbytes, device):
     one stream are ordered and may share it; launches on different streams never do."""
     import torch
     device = torch.device(device)
+    if device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
     buf = _zero_scratch.get(key)
     if buf is None or buf.numel() < nbytes:
