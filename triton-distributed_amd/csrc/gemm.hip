@@ -222,9 +222,13 @@ struct GemmCfg {
   static constexpr int kDmaPerStep = (kLoadsPerTile + kKSteps - 1) / kKSteps;
   // epilogue staging: per wave kWaveM rows of kWaveN 16-bit outputs; 16-byte chunk c of row r sits at
   // position c ^ (r & kEpiSwz) so that the 32 rows one store instruction touches spread over the banks
-  static constexpr int kEpiPitch = kWaveN * 2;
+  // (a row of 16-byte pieces whose number is no power of two, the 96 columns of the 128 x 192 tile's waves, is
+  // staged at the pitch of the next power of two, so that the XOR stays inside the row)
+  static constexpr int kRowPieces = kWaveN * 2 / 16;
+  static constexpr int kEpiChunks = kRowPieces <= 4 ? 4 : kRowPieces <= 8 ? 8 : kRowPieces <= 16 ? 16 : 32;
+  static constexpr int kEpiPitch = kEpiChunks * 16;
   static constexpr int kEpiBytes = kWaveM * kEpiPitch;
-  static constexpr int kEpiSwz = (kEpiPitch / 16 < 16 ? kEpiPitch / 16 : 16) - 1;
+  static constexpr int kEpiSwz = (kEpiChunks < 16 ? kEpiChunks : 16) - 1;
   // MFMAs of a tile's last K step issued before the barrier
   static constexpr int kLeadMfma = (kTM * kTN >= 8) ? 2 : 1;
   // n-th operand fragment (A fragments are 0..kTM-1, B fragments kTM..) in the order in which the MFMA sequence
@@ -295,9 +299,10 @@ constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
     TDIST_A10(19), TDIST_A10(20), TDIST_A10(21), TDIST_A10(22), TDIST_A10(23), TDIST_A10(24), "a250", "a251", "a252", "a253", "a254", "a255"
 template <int kN>
 __device__ __forceinline__ void acc_reserve() {
-  static_assert(kN == 128 || kN == 256, "accumulators of a 128 x 64 or a 128 x 128 wave tile");
+  static_assert(kN == 96 || kN == 128 || kN == 256, "accumulators of a 64 x 96, a 128 x 64 or a 128 x 128 wave tile");
   if constexpr (kN == 256) asm volatile("" ::: TDIST_A_0_99, TDIST_A_100_127, TDIST_A_128_255);
-  else asm volatile("" ::: TDIST_A_0_99, TDIST_A_100_127);
+  else if constexpr (kN == 128) asm volatile("" ::: TDIST_A_0_99, TDIST_A_100_127);
+  else asm volatile("" ::: TDIST_A_0_99);   // (a96 .. a99 go unused)
 }
 template <int kN>
 __device__ __forceinline__ void acc_clear() {
@@ -860,7 +865,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       Cbase = p.C;
       crow0 = m0;
     }
-    constexpr int kLanesPerRow = C::kWaveN * 2 / 16;  // 16-byte vectors per staged row
+    constexpr int kLanesPerRow = C::kEpiChunks;  // lanes per staged row: one per 16-byte piece, the last ones idle
+                                                 // where the row is no power of two wide
+    constexpr bool kFullRows = C::kRowPieces == C::kEpiChunks;
     constexpr int kRowsPerPass = 64 / kLanesPerRow;
     const int er = e_lane / kLanesPerRow, ec = e_lane % kLanesPerRow;
     const bool n_vec_ok = (p.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(Cbase) & 15) == 0);
@@ -926,7 +933,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 #pragma unroll 4
       for (int pass = 0; pass < nrows / kRowsPerPass; ++pass) {
         const int mrow = row0 + pass * kRowsPerPass + er;
-        store_piece_at(mrow, ec, staged_piece_at(mrow, ec));
+        if (kFullRows || ec < C::kRowPieces) store_piece_at(mrow, ec, staged_piece_at(mrow, ec));
       }
     };
     static_assert(32 % kRowsPerPass == 0, "a 32-row block is a whole number of store passes");
@@ -1085,7 +1092,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // per lane for the whole tile (uniform base + constant row step) and no per-store bounds arithmetic. The scales
     // of the whole wave tile are fetched up front, in one round trip.
     bool stored = false;
-    if constexpr (C::kWaves <= 4 && !kGrouped) {
+    if constexpr (C::kWaves <= 4 && !kGrouped && kFullRows) {
       if (m0 + BM <= p.M && n0 + BN <= p.N && n_vec_ok) {
         stored = true;
         constexpr int kPasses = 32 / kRowsPerPass;
@@ -1335,8 +1342,10 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
 
   // Tile configuration. The 256-row tiles (256x256 and 256x128, both on the split ring) need the call's row blocks
   // (chunks, rank slices, the local shard) to be multiples of 256 rows and K to be a multiple of 128 bytes; the
-  // 128x128 tile takes everything else. Among the admissible ones the cheapest estimate wins: rounds of the grid
-  // times the tile's work over its measured relative efficiency.
+  // 128x192 tile (split ring as well, waves of 64 x 96: three quarters of a 256x128 tile's work, for shapes whose
+  // large tiles would leave a quarter of the chip without one) needs whole 128-byte K tiles; the 128x128 tile takes
+  // everything else. Among the admissible ones the cheapest estimate wins: rounds of the grid times the tile's work
+  // over its measured relative efficiency.
   bool rows256 = true;
   if (c.scatter_bufs && c.world_size > 0 && (c.M % c.world_size != 0 || (c.M / c.world_size) % 256 != 0)) rows256 = false;
   if (!c.scatter_bufs && c.flags && c.m_per_chunk % 256 != 0) rows256 = false;
@@ -1346,7 +1355,14 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   int cap_wgs = di.num_cus;
   if (c.max_workgroups > 0 && c.max_workgroups < cap_wgs) cap_wgs = c.max_workgroups;
   struct TileChoice { int bm, bn; double eff; };
-  static const TileChoice kChoices[3] = {{256, 256, 1.0}, {256, 128, 0.9}, {128, 128, 0.6}};
+  constexpr int kNumChoices = 4;
+  // (rates relative to the 256x256 tile, measured on 8192 x 6144 x 3584 bf16: 1425, 1255, 774 and 1078 TFLOP/s; the
+  // 128x192 tile is entered below its multi-round rate because a tile's prologue and epilogue weigh more the smaller
+  // it is: one round of 256 of them takes 50.5 us on 4096 x 1536 x 4096 where 192 tiles of 256x128 take 48.3)
+  static const TileChoice kChoices[kNumChoices] = {{256, 256, 1.0}, {256, 128, 0.88}, {128, 128, 0.54}, {128, 192, 0.65}};
+  const bool k128 = ((int64_t)c.K * esz) % 128 == 0;
+  auto admissible = [&](int t) { return kChoices[t].bm == 256 ? rows256 : (kChoices[t].bn != 192 || k128); };
+  auto k_tile_bytes = [&](int t) { return kChoices[t].bm == 256 || kChoices[t].bn == 192 ? 128 : 64; };
   // With a workspace, a last round that fills at most half of the grid is split along K (see GemmParams): it then
   // costs 1/s of a round plus one exchange of the tile's accumulators, and that form is taken where it beats whole
   // tiles by a margin.
@@ -1354,32 +1370,33 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   int pick = 2;
   bool use_sk = false;
   double best = 0;
-  for (int t = 0; t < 3; ++t) {
-    if (kChoices[t].bm == 256 && !rows256) continue;
+  for (int t = 0; t < kNumChoices; ++t) {
+    if (!admissible(t)) continue;
     const int bm = kChoices[t].bm, bn = kChoices[t].bn;
     const int64_t tiles = ceil_div(c.M, bm) * ceil_div(c.N, bn);
-    const int64_t kt = ceil_div((int64_t)c.K * esz, bm == 256 ? 128 : 64);
+    const int64_t kt = ceil_div((int64_t)c.K * esz, k_tile_bytes(t));
     const double per_k_tile = (double)bm * bn / kChoices[t].eff;
     const double cost = (double)ceil_div(tiles, cap_wgs) * kt * per_k_tile;
     if (best == 0 || cost < best) best = cost, pick = t, use_sk = false;
     const int64_t tail = tiles % cap_wgs;
     const int split = tail > 0 ? sk_split_for(cap_wgs, (int)tail, (int)(kt < 0x7fffffff ? kt : 0x7fffffff)) : 1;
-    if (sk_mode != 0 && split >= 2 && sk_workspace_fits(c.sk_workspace, c.sk_workspace_bytes, cap_wgs, bm, bn)) {
+    // (the exchange of the split form is written for staged rows of a power-of-two width: not for the 128x192 tile)
+    if (sk_mode != 0 && split >= 2 && bn != 192 && sk_workspace_fits(c.sk_workspace, c.sk_workspace_bytes, cap_wgs, bm, bn)) {
       const double cost_sk = ((double)(tiles / cap_wgs) * kt + (double)kt / split + sk_handover_k_tiles(bm, bn)) * per_k_tile;
       if (cost_sk < 0.95 * best || (sk_mode == 1 && (!use_sk || cost_sk < best))) best = cost_sk, pick = t, use_sk = true;
     }
   }
-  // TDIST_GEMM_TILE forces a tile (test and measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128; a 256-row tile
-  // that the call's row blocks do not admit is not taken.
+  // TDIST_GEMM_TILE forces a tile (test and measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128, 3 = 128x192; a
+  // tile that the call's row blocks or K do not admit is not taken.
   if (const char* v = getenv("TDIST_GEMM_TILE")) {
     const int t = atoi(v);
-    if (t >= 0 && t < 3 && (kChoices[t].bm != 256 || rows256)) {
+    if (t >= 0 && t < kNumChoices && admissible(t)) {
       pick = t;
       // (the split is re-derived for the forced tile)
       const int64_t tiles = ceil_div(c.M, kChoices[t].bm) * ceil_div(c.N, kChoices[t].bn);
-      const int64_t kt = ceil_div((int64_t)c.K * esz, kChoices[t].bm == 256 ? 128 : 64);
+      const int64_t kt = ceil_div((int64_t)c.K * esz, k_tile_bytes(t));
       const int64_t tail = tiles % cap_wgs;
-      use_sk = sk_mode != 0 && use_sk && tail > 0 && sk_split_for(cap_wgs, (int)tail, (int)kt) >= 2 &&
+      use_sk = sk_mode != 0 && use_sk && kChoices[t].bn != 192 && tail > 0 && sk_split_for(cap_wgs, (int)tail, (int)kt) >= 2 &&
                sk_workspace_fits(c.sk_workspace, c.sk_workspace_bytes, cap_wgs, kChoices[t].bm, kChoices[t].bn);
     }
   }
@@ -1496,6 +1513,15 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       default:
         return scales ? launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, true>(p, grid, c.stream, who)
                       : launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+    }
+  }
+  if (BN == 192) {  // 128 x 192: waves of 64 x 96 on the split ring
+    switch (elem) {
+      case kElemBF16: return launch_gemm_cfg<ElemBF16N, 128, 192, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      case kElemF16: return launch_gemm_cfg<ElemF16N, 128, 192, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      default:
+        return scales ? launch_gemm_cfg<ElemFP8N, 128, 192, 128, 2, 2, 5, true>(p, grid, c.stream, who)
+                      : launch_gemm_cfg<ElemFP8N, 128, 192, 128, 2, 2, 5, false>(p, grid, c.stream, who);
     }
   }
   // the 128 x 128 tile on a four-stage ring of 64-byte K tiles, 32-row MFMA blocks: every shape
