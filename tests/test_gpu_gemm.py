@@ -447,10 +447,10 @@ def test_randomised_shapes_gating_and_layouts(cuda):
         assert torch.equal(c, ref), "case %d differs" % case
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
 def test_each_tile_configuration_forced(cuda, monkeypatch, tile, dtype):
-    """Every compiled tile (256x256, 256x128, 128x128, 128x192) forced through the library's measurement switch on the same
+    """Every compiled tile (256x256, 256x128, 128x128, 128x192, 128x256) forced through the library's measurement switch on the same
     ragged, padded, gated and scaled cases; integer-valued inputs, so only the final rounding remains."""
     from triton_dist.kernels.amd import gated_gemm
     monkeypatch.setenv("TDIST_GEMM_TILE", str(tile))

@@ -1,4 +1,4 @@
-"""The split-ring GEMM tiles (256 x 256, 256 x 128, 128 x 192) run on the 16-row MFMA blocks (16x16x32 for bf16/f16,
+"""The split-ring GEMM tiles (256 x 256, 256 x 128, 128 x 256, 128 x 192) run on the 16-row MFMA blocks (16x16x32 for bf16/f16,
 16x16x128 for e4m3) with their accumulators in fixed registers; the 128 x 128 tile runs on the 32-row blocks (32x32x16
 / 32x32x64) with accumulators the compiler places. Each form is held against the exact result on integer-valued inputs (every partial sum is an
 integer that fp32 holds) over the K-loop's corner cases, and on random inputs to max relative error <= 1e-2 of fp32 and
@@ -36,12 +36,12 @@ def run_tile(cuda, a, b, out_dtype, tile, **kw):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("M,N,K", [(512, 512, 128), (768, 512, 384), (300, 200, 640), (1024, 1280, 1152), (640, 1536, 256)])
 def test_exact_on_integer_inputs(cuda, tile_env, dtype, tile, M, N, K):
     """One K tile (e4m3) or two; an odd number of K tiles (the e4m3 loop works in pairs of tiles); a ragged shape (the
     bounds-checked epilogue); several tiles per workgroup row; a width that is whole 192-column tiles. tile 0 = 256x256,
-    1 = 256x128, 2 = 128x128, 3 = 128x192."""
+    1 = 256x128, 2 = 128x128, 3 = 128x192, 4 = 128x256."""
     announce("mfma shapes exact %s tile %d %dx%dx%d" % (dtype, tile, M, N, K))
     g = torch.Generator().manual_seed(M + N + K + tile)
     a = torch.randint(-2, 3, (M, K), generator=g).float().to(dtype).to(cuda)
@@ -64,7 +64,7 @@ def test_random_inputs_close_in_every_form(cuda, tile_env, dtype):
         kw["row_scale"] = (torch.rand(M, generator=g) * 0.09 + 0.01).to(cuda)
         kw["col_scale"] = (torch.rand(N, generator=g) * 0.9 + 0.1).to(cuda)
         ref = ref * kw["row_scale"][:, None] * kw["col_scale"][None, :]
-    out = [run_tile(cuda, a, b, torch.bfloat16, tile, **kw) for tile in (0, 1, 2, 3)]
+    out = [run_tile(cuda, a, b, torch.bfloat16, tile, **kw) for tile in (0, 1, 2, 3, 4)]
     for c in out:
         rel = (c.float() - ref).abs().max() / ref.abs().max()
         assert rel.item() <= 1e-2

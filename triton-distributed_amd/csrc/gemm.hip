@@ -1342,9 +1342,9 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
 
   // Tile configuration. The 256-row tiles (256x256 and 256x128, both on the split ring) need the call's row blocks
   // (chunks, rank slices, the local shard) to be multiples of 256 rows and K to be a multiple of 128 bytes; the
-  // 128x192 tile (split ring as well, waves of 64 x 96: three quarters of a 256x128 tile's work, for shapes whose
-  // large tiles would leave a quarter of the chip without one) needs whole 128-byte K tiles; the 128x128 tile takes
-  // everything else. Among the admissible ones the cheapest estimate wins: rounds of the grid times the tile's work
+  // 128x256 and 128x192 tiles (split ring as well, waves of 64 x 128 and 64 x 96: for row blocks of 128·odd rows, and
+  // three quarters of a 256x128 tile's work for shapes whose larger tiles would leave a quarter of the chip without
+  // one) need whole 128-byte K tiles; the 128x128 tile takes everything else. Among the admissible ones the cheapest estimate wins: rounds of the grid times the tile's work
   // over its measured relative efficiency.
   bool rows256 = true;
   if (c.scatter_bufs && c.world_size > 0 && (c.M % c.world_size != 0 || (c.M / c.world_size) % 256 != 0)) rows256 = false;
@@ -1355,14 +1355,15 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   int cap_wgs = di.num_cus;
   if (c.max_workgroups > 0 && c.max_workgroups < cap_wgs) cap_wgs = c.max_workgroups;
   struct TileChoice { int bm, bn; double eff; };
-  constexpr int kNumChoices = 4;
-  // (rates relative to the 256x256 tile, measured on 8192 x 6144 x 3584 bf16: 1425, 1255, 774 and 1078 TFLOP/s; the
-  // 128x192 tile is entered below its multi-round rate because a tile's prologue and epilogue weigh more the smaller
-  // it is: one round of 256 of them takes 50.5 us on 4096 x 1536 x 4096 where 192 tiles of 256x128 take 48.3)
-  static const TileChoice kChoices[kNumChoices] = {{256, 256, 1.0}, {256, 128, 0.88}, {128, 128, 0.54}, {128, 192, 0.65}};
+  constexpr int kNumChoices = 5;
+  // (rates relative to the 256x256 tile, measured on 8192 x 6144 x 3584 bf16: 1425, 1255, 774, 1078 and 1178
+  // TFLOP/s; the 128x192 tile is entered below its multi-round rate because a tile's prologue and epilogue weigh
+  // more the smaller it is: one round of 256 of them takes 50.5 us on 4096 x 1536 x 4096 where 192 tiles of 256x128
+  // take 48.3 and 192 tiles of 128x256 53.1)
+  static const TileChoice kChoices[kNumChoices] = {{256, 256, 1.0}, {256, 128, 0.88}, {128, 128, 0.54}, {128, 192, 0.65}, {128, 256, 0.8}};
   const bool k128 = ((int64_t)c.K * esz) % 128 == 0;
-  auto admissible = [&](int t) { return kChoices[t].bm == 256 ? rows256 : (kChoices[t].bn != 192 || k128); };
-  auto k_tile_bytes = [&](int t) { return kChoices[t].bm == 256 || kChoices[t].bn == 192 ? 128 : 64; };
+  auto admissible = [&](int t) { return kChoices[t].bm == 256 ? rows256 : (kChoices[t].bn == 128 || k128); };
+  auto k_tile_bytes = [&](int t) { return kChoices[t].bm == 256 || kChoices[t].bn != 128 ? 128 : 64; };
   // With a workspace, a last round that fills at most half of the grid is split along K (see GemmParams): it then
   // costs 1/s of a round plus one exchange of the tile's accumulators, and that form is taken where it beats whole
   // tiles by a margin.
@@ -1386,8 +1387,8 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       if (cost_sk < 0.95 * best || (sk_mode == 1 && (!use_sk || cost_sk < best))) best = cost_sk, pick = t, use_sk = true;
     }
   }
-  // TDIST_GEMM_TILE forces a tile (test and measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128, 3 = 128x192; a
-  // tile that the call's row blocks or K do not admit is not taken.
+  // TDIST_GEMM_TILE forces a tile (test and measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128, 3 = 128x192,
+  // 4 = 128x256; a tile that the call's row blocks or K do not admit is not taken.
   if (const char* v = getenv("TDIST_GEMM_TILE")) {
     const int t = atoi(v);
     if (t >= 0 && t < kNumChoices && admissible(t)) {
@@ -1513,6 +1514,15 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       default:
         return scales ? launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, true>(p, grid, c.stream, who)
                       : launch_gemm_cfg<ElemFP8N, 256, 128, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+    }
+  }
+  if (BM == 128 && BN == 256) {  // 128 x 256: waves of 64 x 128 on the split ring
+    switch (elem) {
+      case kElemBF16: return launch_gemm_cfg<ElemBF16N, 128, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      case kElemF16: return launch_gemm_cfg<ElemF16N, 128, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
+      default:
+        return scales ? launch_gemm_cfg<ElemFP8N, 128, 256, 128, 2, 2, 5, true>(p, grid, c.stream, who)
+                      : launch_gemm_cfg<ElemFP8N, 128, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
     }
   }
   if (BN == 192) {  // 128 x 192: waves of 64 x 96 on the split ring
