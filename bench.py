@@ -496,6 +496,30 @@ def bench_library_gemm(dev, steps, warmup):
     return roof("mfma", 2.0 * M * N * K, s, "bf16")
 
 
+def bench_library_fp8_gemm(dev, steps, warmup):
+    """Yardstick, not product: the vendor library's e4m3 GEMM (torch._scaled_mm) on the C3 shape and the same seeded
+    operands and scales: with one scale per row of A and per row of B (what the C3 kernel applies), and with one
+    scale per tensor."""
+    import torch
+    M, N, K = 16384, 7168, 8192
+    g = torch.Generator().manual_seed(3 + 2)
+    a = torch.randn((M, K), generator=g).to(torch.float8_e4m3fn).to(dev)
+    b = torch.randn((N, K), generator=g).to(torch.float8_e4m3fn).to(dev)
+    sa = (torch.rand(M, generator=g) * 0.09 + 0.01).to(dev)
+    sb = (torch.rand(N, generator=g) * 0.009 + 0.001).to(dev)
+    one = torch.ones((), device=dev)
+    out = {}
+    for name, scale_a, scale_b in (("row_scales", sa.view(M, 1), sb.view(1, N)), ("tensor_scales", one, one)):
+        try:
+            call = lambda: torch._scaled_mm(a, b.t(), scale_a=scale_a, scale_b=scale_b, out_dtype=torch.bfloat16)
+            call()
+            r = roof("mfma", 2.0 * M * N * K, time_launches(call, max(steps // 2, 1), warmup), "fp8")
+            out[name] = {k: r[k] for k in ("achieved", "frac", "us_per_launch")}
+        except Exception as exc:   # (a library without this form of the call)
+            out[name] = {"unavailable": repr(exc)[:120]}
+    return out
+
+
 def main():
     global LIVE_PRODUCER, SETTLE_SECONDS
     ap = argparse.ArgumentParser()
@@ -554,6 +578,8 @@ def main():
     if "library" in want:
         kernels["hipblaslt_matmul_c2_shape_yardstick"] = bench_library_gemm(dev, args.steps, args.warmup)
         log("library", kernels["hipblaslt_matmul_c2_shape_yardstick"])
+        kernels["hipblaslt_scaled_mm_c3_shape_yardstick"] = bench_library_fp8_gemm(dev, args.steps, args.warmup)
+        log("library fp8", kernels["hipblaslt_scaled_mm_c3_shape_yardstick"])
 
     flops = 2.0 * 8192 * 8192 * 3584
     line = {
