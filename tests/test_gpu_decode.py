@@ -335,3 +335,53 @@ def test_head_dimensions_that_are_no_power_of_two(cuda, D, num_heads, kv_lens, S
     exact, _ = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, scale, soft_cap)
     eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
     assert ((got.cpu().double() - exact).abs() <= ATOL + eps * exact.abs()).all()
+
+
+@pytest.mark.parametrize("D,num_heads,force", [(128, (64, 8), 2), (128, (16, 16), 2), (128, (32, 8), 2), (64, (64, 8), 4),
+                                               (64, (24, 8), 2), (64, (16, 16), 4), (64, (64, 4), 2), (256, (32, 8), 2),
+                                               (256, (12, 4), 2)])
+@pytest.mark.parametrize("kv_lens,S,block_size", [([1320, 18, 463], 4, 16), ([1, 54, 293, 70], 8, 1), ([777, 0, 5, 2047], 3, 16),
+                                                  ([100, 31], 1, 16)])
+@pytest.mark.parametrize("dtype,soft_cap", [(torch.bfloat16, 0), (torch.float16, 30)])
+def test_a_kv_head_per_wave(cuda, monkeypatch, D, num_heads, force, kv_lens, S, block_size, dtype, soft_cap):
+    """The form in which every wave of a workgroup takes a kv head of its own (chosen by itself only for grids that
+    fill the chip; forced here on small cases): per-split partials and LSE against the oracle, the one-launch form bit
+    for bit against split + combine with the counters back at zero, and both within the oracle's bar of the other
+    form's results."""
+    from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine, decode_fused
+    announce("decode, a kv head per wave (%d): D=%d heads=%s kv_lens=%s S=%d page=%d %s cap=%s" % (force, D, num_heads, kv_lens, S, block_size, dtype, soft_cap))
+    q, k_cache, v_cache, table = build_case(kv_lens, num_heads, D, block_size, dtype, seed=D + S + num_heads[0])
+    scale = D**-0.5
+    B, Hq = len(kv_lens), num_heads[0]
+    lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
+    qd, kd, vd, td = q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), table.to(cuda)
+    monkeypatch.setenv("TDIST_DECODE_WAVE_HEADS", "0")
+    other_out, other_lse, _ = _split_kv(qd, kd, vd, lens_dev, td, scale, soft_cap, S)
+    monkeypatch.setenv("TDIST_DECODE_WAVE_HEADS", str(force))   # 2: eight waves where the heads allow, 4: four
+    out_split, lse_split, _ = _split_kv(qd, kd, vd, lens_dev, td, scale, soft_cap, S)
+    torch.cuda.synchronize()
+    w_out, w_lse = golden.decode_split_exact(q, k_cache, v_cache, kv_lens, table, scale, S, soft_cap)
+    got_lse = lse_split.cpu().double()
+    empty = torch.isinf(w_lse)
+    assert torch.equal(torch.isinf(got_lse), empty)
+    assert (got_lse[~empty] - w_lse[~empty]).abs().max() <= ATOL
+    assert (out_split.cpu().double() - w_out).abs().max() <= ATOL
+    assert (out_split.cpu()[empty] == 0).all()
+    assert (out_split - other_out).abs().max() <= ATOL
+    want = torch.empty((B, Hq, D), dtype=dtype, device=cuda)
+    want_lse = torch.empty((B, Hq), dtype=torch.float32, device=cuda)
+    decode_combine(out_split, lse_split, S, 1, lens_dev, B, Hq, D,
+                   (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
+                   (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), want, want_lse)
+    counters = torch.zeros(1024, dtype=torch.int32, device=cuda)
+    for _ in range(2):   # twice on the same counters
+        got = torch.full((B, Hq, D), float("nan"), dtype=dtype, device=cuda)
+        got_lse = torch.full((B, Hq), float("nan"), dtype=torch.float32, device=cuda)
+        decode_fused(qd, kd, vd, lens_dev, td, scale, soft_cap, S, got, got_lse, workspace=counters)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        assert torch.equal(got_lse.view(torch.int32), want_lse.view(torch.int32))
+        assert int(counters.abs().sum()) == 0
+    exact, _ = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, scale, soft_cap)
+    eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    assert ((got.cpu().double() - exact).abs() <= ATOL + eps * exact.abs()).all()

@@ -173,7 +173,11 @@ __device__ __forceinline__ void store_partial(float* p, float v) {
 // wide, the 16-byte pieces beyond the real row are fetched from a page of zeros (so that the MFMA blocks see exact
 // zeros there: the reference masks the same dimensions, kernels/nvidia/flash_decode.py:771-772 with BLOCK_DPE), and
 // results are stored d_valid wide.
-template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded>
+// kWaveHeads: the NW waves of a workgroup take NW neighbouring kv heads (one each, all keys of the split) instead of
+// sharing one kv head's keys: together they read whole stretches of the token rows (NW * 2 * D bytes of every row) at
+// the same time, and no wave waits for another: each writes its own heads' results. For at most 16 query heads per kv
+// head and a number of kv heads that is a multiple of NW.
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded, bool kWaveHeads>
 __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   typedef DecodeCfg<D, DPE, KEYS, NST> C;
   constexpr int G = C::kGroups;
@@ -188,14 +192,16 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   const int split = blockIdx.y;
   const int group = prm.Hq / prm.Hkv;
   const int head_blocks = (group + 15) >> 4;
-  const int kvh = blockIdx.x / head_blocks;
-  const int hb = blockIdx.x - kvh * head_blocks;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform for the compiler too
+  const int lane = threadIdx.x & 63;
+  const int kvh = kWaveHeads ? blockIdx.x * NW + wave : blockIdx.x / head_blocks;
+  const int hb = kWaveHeads ? 0 : blockIdx.x - kvh * head_blocks;
   const int b = blockIdx.z;
   const int h0 = kvh * group + hb * 16;
   const int nvalid = min(16, group - hb * 16);
-
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform for the compiler too
-  const int lane = threadIdx.x & 63;
+  // threads that share the work of one (kv head, head block): the workgroup, or the wave
+  const int team_tid = kWaveHeads ? lane : (int)threadIdx.x;
+  constexpr int kTeam = kWaveHeads ? 64 : NW * 64;
   const int g = lane >> 4;   // lane group 0..3
   const int x = lane & 15;   // head (score column) / dv within tile (V^T row) / key (K row)
 
@@ -208,11 +214,11 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   float* lse_base = prm.lse + ((int64_t)b * prm.Hq + h0) * prm.S + split;
   if (end <= start) {
     // empty split: zeros and LSE = -inf so that any merge gives it weight 0
-    for (int i = threadIdx.x; i < nvalid * Dout; i += NW * 64) {
+    for (int i = team_tid; i < nvalid * Dout; i += kTeam) {
       const int h = i / Dout, d = i - h * Dout;
       store_partial<kFuse>(out_base + (int64_t)h * prm.S * Dout + d, 0.f);
     }
-    if (threadIdx.x < nvalid) store_partial<kFuse>(lse_base + (int64_t)threadIdx.x * prm.S, -INFINITY);
+    if (team_tid < nvalid) store_partial<kFuse>(lse_base + (int64_t)team_tid * prm.S, -INFINITY);
     return;
   }
 
@@ -223,7 +229,8 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   lds_u8 const tbl_base = wbase + NST * C::kStageBytes;
 
   const int nb_total = (end - start + KEYS - 1) / KEYS;
-  const int n_w = nb_total > wave ? (nb_total - wave + NW - 1) / NW : 0;  // this wave's blocks
+  // this wave's blocks: every NW-th one of the kv head's, or all of its own kv head's
+  const int n_w = kWaveHeads ? nb_total : (nb_total > wave ? (nb_total - wave + NW - 1) / NW : 0);
 
   // ---- Q fragments (B operand of the score MFMA): head x, dims 32s + 8g .. +8 -------------------
   typename MMA::frag8 qf[DK / 32];
@@ -272,7 +279,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
     }
 
   // first key of the wave's j-th block
-  auto block_key0 = [&](int j) { return start + (wave + j * NW) * KEYS; };
+  auto block_key0 = [&](int j) { return kWaveHeads ? start + j * KEYS : start + (wave + j * NW) * KEYS; };
 
   // page-table row of block j → table ring slot j % kTableSlots (one entry per key)
   auto issue_table = [&](int j) {
@@ -434,7 +441,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   l_run += __shfl_xor(l_run, 16);
   l_run += __shfl_xor(l_run, 32);
   wait_vmcnt<0>();
-  __syncthreads();  // every wave is done with its ring; reuse it
+  if constexpr (!kWaveHeads) __syncthreads();  // every wave is done with its ring; reuse it
   TDIST_AS3 float* s_m = (TDIST_AS3 float*)(wbase);  // [16]
   TDIST_AS3 float* s_l = s_m + 16;                   // [16]
   TDIST_AS3 float* s_acc = s_l + 16;                 // [D][16]
@@ -446,8 +453,21 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   for (int d = 0; d < D / 16; ++d)
 #pragma unroll
     for (int i = 0; i < 4; ++i) s_acc[(16 * d + 4 * g + i) * 16 + x] = acc[d][i];
-  __syncthreads();
   constexpr float kLn2 = 0.6931471805599453f;
+  if constexpr (kWaveHeads) {
+    // the wave's own heads: its state through its own LDS rows (a wave's LDS instructions run in order), transposed so
+    // that consecutive lanes store consecutive value dimensions
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    for (int idx = lane; idx < nvalid * Dout; idx += 64) {
+      const int h = idx / Dout, dv = idx - h * Dout;
+      const float L = s_l[h];
+      store_partial<kFuse>(out_base + (int64_t)h * prm.S * Dout + dv, s_acc[dv * 16 + h] / L);
+      if (dv == 0) store_partial<kFuse>(lse_base + (int64_t)h * prm.S, (s_m[h] + log2f(L)) * kLn2);
+    }
+    return;
+  }
+  __syncthreads();
   for (int idx = threadIdx.x; idx < nvalid * Dout; idx += NW * 64) {
     const int h = idx / Dout, dv = idx - h * Dout;
     float M = -INFINITY;
@@ -554,45 +574,61 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams
   if (prm.lse_out && lane == 0) prm.lse_out[bh] = L > 0.f ? M + logf(L) : -INFINITY;
 }
 
-// Fused tail: publishes this workgroup's partial result; the last of the S workgroups of a (sequence, head block)
-// to get here merges their partials (same arithmetic, in the same order, as decode_combine_kernel in mode 1) and
-// puts the counter back to zero for the next launch.
-template <int DM, int NW, bool kPadded>
+// Fused tail: publishes this team's partial result (the workgroup's, or with kWaveHeads the wave's); the last of the
+// S teams of a (sequence, head block) to get here merges their partials (same arithmetic, in the same order, as
+// decode_combine_kernel in mode 1) and puts the counter back to zero for the next launch.
+template <int DM, int NW, bool kPadded, bool kWaveHeads>
 __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
   const int D = kPadded ? prm.d_valid : DM;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   TDIST_AS3 int* const s_last = (TDIST_AS3 int*)smem;
   const int group = prm.Hq / prm.Hkv;
   const int head_blocks = (group + 15) >> 4;
-  const int kvh = blockIdx.x / head_blocks;
-  const int hb = blockIdx.x - kvh * head_blocks;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kvh = kWaveHeads ? blockIdx.x * NW + wave : blockIdx.x / head_blocks;
+  const int hb = kWaveHeads ? 0 : blockIdx.x - kvh * head_blocks;
   const int b = blockIdx.z;
   const int h0 = kvh * group + hb * 16;
   const int nvalid = min(16, group - hb * 16);
+  const int team_tid = kWaveHeads ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
+  constexpr int kTeam = kWaveHeads ? 64 : NW * 64;
+  // one counter per (sequence, kv head, head block)
+  int32_t* const ctr = prm.counters + ((int64_t)b * prm.Hkv + kvh) * head_blocks + hb;
 
   // This thread's partial results were stored write-through (store_partial): once the stores have completed they
-  // are visible to every XCD. The barrier then orders all of the workgroup's stores before thread 0's counter
-  // update. (A release fence here would write back the whole L2 once per wave: measured at 2x the kernel time.)
+  // are visible to every XCD. (A release fence here would write back the whole L2 once per wave: measured at 2x the
+  // kernel time.)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();   // (also: every wave is done with the merge scratch that s_last overlays)
-  if (threadIdx.x == 0) {
-    int32_t* ctr = prm.counters + (int64_t)b * gridDim.x + blockIdx.x;
-    const int old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const int last = old == prm.S - 1;
-    if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    *s_last = last;
+  if constexpr (kWaveHeads) {
+    // the wave's stores are complete: its first lane counts, and tells the others
+    int last = 0;
+    if (team_tid == 0) {
+      const int old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      last = old == prm.S - 1;
+      if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (!__builtin_amdgcn_readfirstlane(last)) return;
+  } else {
+    // the barrier orders all of the workgroup's stores before thread 0's counter update
+    __syncthreads();   // (also: every wave is done with the merge scratch that s_last overlays)
+    if (threadIdx.x == 0) {
+      const int old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int last = old == prm.S - 1;
+      if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *s_last = last;
+    }
+    __syncthreads();
+    if (!*s_last) return;
   }
-  __syncthreads();
-  if (!*s_last) return;
-  // The counter said S-1: every other workgroup's stores completed before its increment. Only the merging
-  // workgroup pays for an acquire (it drops this CU's and this XCD's possibly stale lines; the K/V stream is
-  // non-temporal and loses nothing by it), after which plain vector loads may read the partial results.
+  // The counter said S-1: every other team's stores completed before its increment. Only the merging team pays
+  // for an acquire (it drops this CU's and this XCD's possibly stale lines; the K/V stream is non-temporal and
+  // loses nothing by it), after which plain vector loads may read the partial results.
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 
   const float* lse_p = prm.lse + ((int64_t)b * prm.Hq + h0) * prm.S;
   const float* out_p = prm.out + ((int64_t)b * prm.Hq + h0) * prm.S * D;
   const int kVecs = D / 4;
-  for (int idx = threadIdx.x; idx < nvalid * kVecs; idx += NW * 64) {
+  for (int idx = team_tid; idx < nvalid * kVecs; idx += kTeam) {
     const int h = idx / kVecs, dv = (idx - h * kVecs) * 4;
     const float* l = lse_p + (int64_t)h * prm.S;
     float M = -INFINITY;
@@ -617,26 +653,26 @@ __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
   }
 }
 
-template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded>
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded, bool kWaveHeads = false>
 __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodeParams prm) {
-  decode_split_body<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse, kPadded>(prm);
-  if constexpr (kFuse) decode_fused_merge<D, NW, kPadded>(prm);
+  decode_split_body<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse, kPadded, kWaveHeads>(prm);
+  if constexpr (kFuse) decode_fused_merge<D, NW, kPadded, kWaveHeads>(prm);
 }
 
-template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded>
+template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded, bool kWaveHeads = false>
 static int launch_decode_cfg(const DecodeParams& prm, int head_blocks, hipStream_t stream) {
   typedef DecodeCfg<D, DPE, KEYS, NST> C;
   static_assert((32 + D * 16) * 4 <= C::kWaveBytes, "merge scratch must fit in a wave's ring");
   const size_t lds = (size_t)NW * C::kWaveBytes;
   static_assert((size_t)NW * C::kWaveBytes <= 160 * 1024, "LDS of one CU");
-  auto kern = decode_split_kv_kernel<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse, kPadded>;
+  auto kern = decode_split_kv_kernel<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse, kPadded, kWaveHeads>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail(TDIST_ERR_LAUNCH, "decode: cannot reserve %zu B of LDS: %s", lds, hipGetErrorString(e));
     attr_set = true;
   }
-  dim3 grid(prm.Hkv * head_blocks, prm.S, prm.B);
+  dim3 grid(kWaveHeads ? prm.Hkv / NW : prm.Hkv * head_blocks, prm.S, prm.B);
   hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, prm);
   return launch_status(kFuse ? "tdist_decode_fused" : "tdist_decode_split_kv");
 }
@@ -773,16 +809,50 @@ static int run_decode(const DecodeCall& c, bool fuse) {
     if (dk < 128) TDIST_DEC_PADDED(128, 16, 3, 3)
     TDIST_DEC_PADDED(256, 16, 2, 3)
   }
+  // A kv head per wave (8 waves of 2 stages or 4 waves of 4, 130-136 KB: one workgroup per CU) where the heads allow it and the grid
+  // fills the CUs in whole rounds or in many: such a workgroup is NW_ times the work of one of the other form,
+  // whose small workgroups fill a small grid's CUs better. TDIST_DECODE_WAVE_HEADS=0 never takes this form, 2 takes
+  // it wherever the heads allow it, 4 likewise but only its 4-wave workgroups.
+  const char* wh_env = getenv("TDIST_DECODE_WAVE_HEADS");
+  const int wh_mode = wh_env ? atoi(wh_env) : 1;
+  auto wave_heads = [&](int nw) {
+    if (wh_mode == 0 || head_blocks != 1 || c.kv_heads % nw != 0 || (wh_mode == 4 && nw != 4)) return false;
+    if (wh_mode > 1) return true;
+    const int64_t teams = (int64_t)(c.kv_heads / nw) * c.num_splits * c.batch;
+    const int cus = device_info().num_cus > 0 ? device_info().num_cus : 256;
+    const int64_t rounds = (teams + cus - 1) / cus;
+    return teams >= cus && rounds * cus * 3 <= teams * 4;   // at most a quarter of the last round's slots idle
+  };
+#define TDIST_DEC_WH_(MMA_, D_, KEYS_, NW_, NST_, CAP_, FUSE_) \
+  launch_decode_cfg<MMA_, D_, 0, KEYS_, NW_, NST_, CAP_, FUSE_, false, true>(prm, head_blocks, st)
+#define TDIST_DEC_WH(D_, KEYS_, NW_, NST_)                                                                              \
+  if (wave_heads(NW_)) {                                                                                             \
+    if (prm.soft_cap > 0.f) {                                                                                        \
+      if (fuse) return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, true) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, true);     \
+      return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, false) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, false);             \
+    }                                                                                                                \
+    if (fuse) return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, true) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, true);     \
+    return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, false) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, false);             \
+  }
   switch (dk) {
-    case 64: TDIST_DEC(64, 0, 32, 4, 4)
+    case 64:
+      TDIST_DEC_WH(64, 32, 8, 2)
+      TDIST_DEC_WH(64, 32, 4, 4)
+      TDIST_DEC(64, 0, 32, 4, 4)
     // 16-key blocks, 3 waves, 3 stages = 72 KB of LDS: two workgroups share a CU and two thirds of the ring are
     // in flight
-    case 128: TDIST_DEC(128, 0, 16, 3, 3)
+    case 128:
+      TDIST_DEC_WH(128, 16, 8, 2)   // (four waves of four stages: no faster than the form below)
+      TDIST_DEC(128, 0, 16, 3, 3)
     case 192: TDIST_DEC(128, 64, 16, 2, 3)   // 61 KB: two workgroups per CU
-    case 256: TDIST_DEC(256, 0, 16, 2, 3)
+    case 256:
+      TDIST_DEC_WH(256, 16, 4, 2)
+      TDIST_DEC(256, 0, 16, 2, 3)
     default: TDIST_DEC(512, 64, 16, 2, 2)    // 576 = 512 + 64: 136 KB
   }
 #undef TDIST_DEC
+#undef TDIST_DEC_WH
+#undef TDIST_DEC_WH_
 #undef TDIST_DEC_PADDED
 }
 
