@@ -49,6 +49,7 @@ struct DecodeParams {
   float sm_scale;
   float soft_cap;
   int B, Hq, Hkv, S;
+  int splits_per_team;  // kWaveHeads: consecutive splits of a sequence that one workgroup streams through (>= 1)
   int d_valid;  // kernels compiled for a padded head dimension: the real one (a multiple of 8), else unused
   int page_size;
   // n / page_size for 0 <= n < 2^31 as (n * page_magic) >> page_shift with
@@ -98,6 +99,8 @@ struct MmaF16 {
   }
 };
 
+// kWaveHeads: splits one workgroup may stream through (the results of all but the last wait in registers: D / 4 each)
+constexpr int decode_max_splits_per_team(int d) { return d <= 64 ? 4 : d <= 128 ? 3 : 2; }
 constexpr int kTableSlots = 8;  // ring of page-table rows per wave (>= 2P+2)
 
 // what the DMA lanes of a padded head dimension read for the dimensions that do not exist
@@ -168,6 +171,16 @@ __device__ __forceinline__ void store_partial(float* p, float v) {
   if constexpr (kCoherent) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   else *p = v;
 }
+// Four consecutive floats (16-byte aligned) the same way: one 16-byte vector store, written through at agent scope
+// (the sc1 bit, which is what the 4-byte atomic store above carries) where the merge reads them in the same launch.
+// A store of more than 8 bytes reads its data registers one cycle after it issues: the s_nop keeps the next
+// instruction, which the compiler may let write those registers, out of that cycle (for its own stores the compiler
+// does this itself; it does not look into the asm).
+template <bool kCoherent>
+__device__ __forceinline__ void store_partial4(float* p, float4v v) {
+  if constexpr (kCoherent) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0" ::"v"(p), "v"(v) : "memory");
+  else *(float4v*)p = v;
+}
 
 // kPadded: the head dimension is prm.d_valid <= D (key and value alike, a multiple of 8): the rows in the LDS are D
 // wide, the 16-byte pieces beyond the real row are fetched from a page of zeros (so that the MFMA blocks see exact
@@ -189,7 +202,6 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
 
   // kv heads vary fastest over the grid: workgroups that run together then read the neighbouring 2*D-byte
   // pieces of the same token rows
-  const int split = blockIdx.y;
   const int group = prm.Hq / prm.Hkv;
   const int head_blocks = (group + 15) >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform for the compiler too
@@ -207,18 +219,23 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
 
   const int len = prm.lens[b];
   const int per = (len + prm.S - 1) / prm.S;
+  // kWaveHeads: the team streams through splits split .. split + n_splits - 1 of its sequence, one after the other
+  const int split = kWaveHeads ? blockIdx.y * prm.splits_per_team : blockIdx.y;
+  const int n_splits = kWaveHeads ? min(prm.splits_per_team, prm.S - split) : 1;
   const int start = per * split;
   const int end = min(start + per, len);
 
   float* out_base = prm.out + (((int64_t)b * prm.Hq + h0) * prm.S + split) * Dout;
   float* lse_base = prm.lse + ((int64_t)b * prm.Hq + h0) * prm.S + split;
   if (end <= start) {
-    // empty split: zeros and LSE = -inf so that any merge gives it weight 0
-    for (int i = team_tid; i < nvalid * Dout; i += kTeam) {
-      const int h = i / Dout, d = i - h * Dout;
-      store_partial<kFuse>(out_base + (int64_t)h * prm.S * Dout + d, 0.f);
+    // empty split (and with it every later one): zeros and LSE = -inf so that any merge gives it weight 0
+    for (int sp = 0; sp < n_splits; ++sp) {
+      for (int i = team_tid; i < nvalid * Dout; i += kTeam) {
+        const int h = i / Dout, d = i - h * Dout;
+        store_partial<kFuse>(out_base + ((int64_t)h * prm.S + sp) * Dout + d, 0.f);
+      }
+      if (team_tid < nvalid) store_partial<kFuse>(lse_base + (int64_t)team_tid * prm.S + sp, -INFINITY);
     }
-    if (team_tid < nvalid) store_partial<kFuse>(lse_base + (int64_t)team_tid * prm.S, -INFINITY);
     return;
   }
 
@@ -229,8 +246,14 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   lds_u8 const tbl_base = wbase + NST * C::kStageBytes;
 
   const int nb_total = (end - start + KEYS - 1) / KEYS;
-  // this wave's blocks: every NW-th one of the kv head's, or all of its own kv head's
-  const int n_w = kWaveHeads ? nb_total : (nb_total > wave ? (nb_total - wave + NW - 1) / NW : 0);
+  // this wave's blocks: every NW-th one of the kv head's; or all of its own kv head's, split after split (an empty
+  // split at the sequence's end runs one block with every key masked, which writes its zeros)
+  auto blocks_of = [&](int lo, int hi) { return max(1, (hi - lo + KEYS - 1) / KEYS); };
+  int n_w = nb_total > wave ? (nb_total - wave + NW - 1) / NW : 0;
+  if constexpr (kWaveHeads) {
+    n_w = 0;
+    for (int sp = 0; sp < n_splits; ++sp) n_w += blocks_of(start + sp * per, min(start + (sp + 1) * per, len));
+  }
 
   // ---- Q fragments (B operand of the score MFMA): head x, dims 32s + 8g .. +8 -------------------
   typename MMA::frag8 qf[DK / 32];
@@ -278,15 +301,33 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
       voff[q][d] = C::kTensorBytes + key * C::kRowBytes + ((chunk ^ C::vswz(key)) << 4) + (x & 1) * 8;
     }
 
-  // first key of the wave's j-th block
-  auto block_key0 = [&](int j) { return kWaveHeads ? start + j * KEYS : start + (wave + j * NW) * KEYS; };
+  // A block: its first key and the key range [lo, hi) of its split. Keys outside the range are read as the nearest
+  // key inside (and, for a split that is empty, as the sequence's last key) and masked in the scores.
+  struct Block { int key0, lo, hi; };
+  auto clamp_key = [&](int n, const Block& blk) {
+    n = max(min(n, blk.hi - 1), blk.lo);
+    if constexpr (kWaveHeads) n = min(n, len - 1);
+    return n;
+  };
+  // first key of the wave's j-th block where the workgroup shares one split
+  auto shared_block = [&](int j) { return Block{start + (wave + j * NW) * KEYS, start, end}; };
+  // kWaveHeads: a cursor over the team's blocks in order
+  struct Cursor { Block blk; int left; };   // left: blocks of this split still to come, this one included
+  auto cursor_begin = [&]() { return Cursor{Block{start, start, end}, blocks_of(start, end)}; };
+  auto cursor_next = [&](Cursor& c) {
+    c.blk.key0 += KEYS;
+    if (--c.left == 0) {
+      c.blk.lo += per;
+      c.blk.hi = min(c.blk.lo + per, len);
+      c.blk.key0 = c.blk.lo;
+      c.left = blocks_of(c.blk.lo, c.blk.hi);
+    }
+  };
 
   // page-table row of block j → table ring slot j % kTableSlots (one entry per key)
-  auto issue_table = [&](int j) {
+  auto issue_table = [&](int j, const Block& blk) {
     if (lane < KEYS) {
-      int n = block_key0(j) + lane;
-      n = min(n, end - 1);
-      n = max(n, start);
+      const int n = clamp_key(blk.key0 + lane, blk);
       const int e = (int)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift);
       const int32_t* src = prm.table + (int64_t)b * prm.t_s + e;
       __builtin_amdgcn_global_load_lds((const TDIST_AS1 void*)src,
@@ -295,8 +336,8 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   };
 
   // K and V rows of block j → stage j % NST
-  auto issue_rows = [&](int j) {
-    const int key0 = block_key0(j);
+  auto issue_rows = [&](int j, const Block& blk) {
+    const int key0 = blk.key0;
     const volatile TDIST_AS3 int32_t* tbl =
         (const volatile TDIST_AS3 int32_t*)(tbl_base + (j % kTableSlots) * C::kTableSlotBytes);
     lds_u8 const kst = wbase + (j % NST) * C::kStageBytes;
@@ -305,8 +346,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
 #pragma unroll
     for (int i = 0; i < C::kInstrPerTensor; ++i) {
       const int key = i * C::kRowsPerInstr + lane / C::kLanesPerRow;
-      int n = min(key0 + key, end - 1);
-      n = max(n, start);
+      const int n = clamp_key(key0 + key, blk);
       const uint32_t page = (uint32_t)tbl[key];
       const uint32_t in_page = (uint32_t)n - (uint32_t)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift) * (uint32_t)prm.page_size;
       const unsigned char* ksrc = prm.k + (uint64_t)page * (uint64_t)prm.k_sp +
@@ -326,8 +366,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
 #pragma unroll
       for (int i = 0; i < C::kPeInstr; ++i) {
         const int key = i * C::kPeRowsPerInstr + lane / C::kPeLanesPerRow;
-        int n = min(key0 + key, end - 1);
-        n = max(n, start);
+        const int n = clamp_key(key0 + key, blk);
         const uint32_t page = (uint32_t)tbl[key];
         const uint32_t in_page = (uint32_t)n - (uint32_t)(((uint64_t)(uint32_t)n * prm.page_magic) >> prm.page_shift) * (uint32_t)prm.page_size;
         const unsigned char* psrc = prm.k + (uint64_t)page * (uint64_t)prm.k_sp +
@@ -338,8 +377,8 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
     }
   };
 
-  auto compute = [&](int j) {
-    const int key0 = block_key0(j);
+  auto compute = [&](int j, const Block& blk) {
+    const int key0 = blk.key0;
     lds_u8 const st = wbase + (j % NST) * C::kStageBytes;
     // scores: A = K rows (key x of group q, dims 32s+8g..), B = Q  →  sc[q][i]: key 16q+4g+i, head x
     float4v sc[G];
@@ -364,7 +403,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
         } else {
           v = sc[q][i] * scale_log2;
         }
-        const bool valid = key0 + 16 * q + 4 * g + i < end;
+        const bool valid = key0 + 16 * q + 4 * g + i < blk.hi;
         t[q][i] = valid ? v : -INFINITY;
         mx = fmaxf(mx, t[q][i]);
       }
@@ -416,24 +455,112 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
     }
   };
 
+  constexpr float kLn2 = 0.6931471805599453f;
+  if constexpr (kWaveHeads) {
+    static_assert(!kPadded && !C::kWaitFirst, "a kv head per wave: plain rows, several groups in flight");
+    // One pipeline over all blocks of the team's splits: the loads of the next split's first blocks are in flight
+    // while the last blocks of this one are computed. The results go out of the registers (no LDS: the ring belongs
+    // to the loads in flight) when the stream has ended.
+    Cursor c_tbl = cursor_begin(), c_rows = cursor_begin(), c_cmp = cursor_begin();
+    int j_tbl = 0;
+    for (; j_tbl <= C::kP; ++j_tbl) {
+      issue_table(j_tbl, c_tbl.blk);
+      cursor_next(c_tbl);
+    }
+    wait_vmcnt<0>();
+    for (int gi = 0; gi < C::kP; ++gi) {
+      if (gi < n_w) {
+        issue_table(j_tbl++, c_tbl.blk);
+        cursor_next(c_tbl);
+        issue_rows(gi, c_rows.blk);
+        cursor_next(c_rows);
+      }
+    }
+    // results of the splits before the team's last one, held until the stream ends
+    constexpr int kMaxHeld = decode_max_splits_per_team(D) - 1;
+    float4v held[kMaxHeld][D / 16];
+    float held_lse[kMaxHeld];
+#pragma unroll
+    for (int u = 0; u < kMaxHeld; ++u) {
+      held_lse[u] = 0.f;
+#pragma unroll
+      for (int d = 0; d < D / 16; ++d) held[u][d] = float4v{0.f, 0.f, 0.f, 0.f};
+    }
+    int sp = 0;
+    for (int i = 0; i < n_w; ++i) {
+      if (i + C::kP < n_w) {
+        issue_table(j_tbl++, c_tbl.blk);
+        cursor_next(c_tbl);
+        issue_rows(i + C::kP, c_rows.blk);
+        cursor_next(c_rows);
+      }
+      wait_groups<C::kLoadsPerGroup>(min(C::kP, n_w - 1 - i));
+      compute(i, c_cmp.blk);
+      if (c_cmp.left == 1) {
+        // the split's last block: this lane holds dimensions 16d + 4g .. + 3 of head x
+        float L = l_run + __shfl_xor(l_run, 16);
+        L += __shfl_xor(L, 32);
+        float4v r[D / 16];
+#pragma unroll
+        for (int d = 0; d < D / 16; ++d)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) r[d][e] = L > 0.f ? acc[d][e] / L : 0.f;
+        const float r_lse = L > 0.f ? (m_run + log2f(L)) * kLn2 : -INFINITY;
+        auto store_split = [&](int which, const float4v(&val)[D / 16], float val_lse) {
+          if (x < nvalid) {
+            float* o = out_base + ((int64_t)x * prm.S + which) * Dout + 4 * g;
+#pragma unroll
+            for (int d = 0; d < D / 16; ++d) store_partial4<kFuse>(o + 16 * d, val[d]);
+            if (g == 0) store_partial<kFuse>(lse_base + (int64_t)x * prm.S + which, val_lse);
+          }
+        };
+        if (i == n_w - 1) {
+          // the team's last split: everything goes out now
+#pragma unroll
+          for (int u = 0; u < kMaxHeld; ++u)
+            if (u < sp) store_split(u, held[u], held_lse[u]);
+          store_split(sp, r, r_lse);
+        } else {
+          // Not yet: stores count on the same counter as the loads, so the next wait for a block would also wait for
+          // these stores, which take tens of microseconds to be acknowledged while the read stream runs (measured:
+          // 40 us per launch at 8 stores per wave). The result waits in registers for the end of the stream.
+#pragma unroll
+          for (int u = 0; u < kMaxHeld; ++u)
+            if (sp == u) {
+#pragma unroll
+              for (int d = 0; d < D / 16; ++d) held[u][d] = r[d];
+              held_lse[u] = r_lse;
+            }
+        }
+        ++sp;
+        m_run = -INFINITY;
+        l_run = 0.f;
+#pragma unroll
+        for (int d = 0; d < D / 16; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
+      }
+      cursor_next(c_cmp);
+    }
+    return;
+  }
+
   if (n_w > 0) {
     // page-table rows of the first P+1 blocks, then the first P row groups
-    for (int j = 0; j <= C::kP; ++j) issue_table(j);
+    for (int j = 0; j <= C::kP; ++j) issue_table(j, shared_block(j));
     wait_vmcnt<0>();
     for (int gi = -C::kP; gi < 0; ++gi) {
       if (gi + C::kP < n_w) {
-        issue_table(gi + 2 * C::kP + 1);
-        issue_rows(gi + C::kP);
+        issue_table(gi + 2 * C::kP + 1, shared_block(gi + 2 * C::kP + 1));
+        issue_rows(gi + C::kP, shared_block(gi + C::kP));
       }
     }
     for (int i = 0; i < n_w; ++i) {
       if constexpr (C::kWaitFirst) wait_vmcnt<0>();
       if (i + C::kP < n_w) {
-        issue_table(i + 2 * C::kP + 1);
-        issue_rows(i + C::kP);
+        issue_table(i + 2 * C::kP + 1, shared_block(i + 2 * C::kP + 1));
+        issue_rows(i + C::kP, shared_block(i + C::kP));
       }
       if constexpr (!C::kWaitFirst) wait_groups<C::kLoadsPerGroup>(min(C::kP, n_w - 1 - i));
-      compute(i);
+      compute(i, shared_block(i));
     }
   }
 
@@ -441,7 +568,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   l_run += __shfl_xor(l_run, 16);
   l_run += __shfl_xor(l_run, 32);
   wait_vmcnt<0>();
-  if constexpr (!kWaveHeads) __syncthreads();  // every wave is done with its ring; reuse it
+  __syncthreads();  // every wave is done with its ring; reuse it
   TDIST_AS3 float* s_m = (TDIST_AS3 float*)(wbase);  // [16]
   TDIST_AS3 float* s_l = s_m + 16;                   // [16]
   TDIST_AS3 float* s_acc = s_l + 16;                 // [D][16]
@@ -453,20 +580,6 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
   for (int d = 0; d < D / 16; ++d)
 #pragma unroll
     for (int i = 0; i < 4; ++i) s_acc[(16 * d + 4 * g + i) * 16 + x] = acc[d][i];
-  constexpr float kLn2 = 0.6931471805599453f;
-  if constexpr (kWaveHeads) {
-    // the wave's own heads: its state through its own LDS rows (a wave's LDS instructions run in order), transposed so
-    // that consecutive lanes store consecutive value dimensions
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_wave_barrier();
-    for (int idx = lane; idx < nvalid * Dout; idx += 64) {
-      const int h = idx / Dout, dv = idx - h * Dout;
-      const float L = s_l[h];
-      store_partial<kFuse>(out_base + (int64_t)h * prm.S * Dout + dv, s_acc[dv * 16 + h] / L);
-      if (dv == 0) store_partial<kFuse>(lse_base + (int64_t)h * prm.S, (s_m[h] + log2f(L)) * kLn2);
-    }
-    return;
-  }
   __syncthreads();
   for (int idx = threadIdx.x; idx < nvalid * Dout; idx += NW * 64) {
     const int h = idx / Dout, dv = idx - h * Dout;
@@ -601,10 +714,12 @@ __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if constexpr (kWaveHeads) {
     // the wave's stores are complete: its first lane counts, and tells the others
+    // (its team brought n_mine of the S splits)
+    const int n_mine = min(prm.splits_per_team, prm.S - (int)blockIdx.y * prm.splits_per_team);
     int last = 0;
     if (team_tid == 0) {
-      const int old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      last = old == prm.S - 1;
+      const int old = __hip_atomic_fetch_add(ctr, n_mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      last = old + n_mine == prm.S;
       if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (!__builtin_amdgcn_readfirstlane(last)) return;
@@ -620,7 +735,7 @@ __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
     __syncthreads();
     if (!*s_last) return;
   }
-  // The counter said S-1: every other team's stores completed before its increment. Only the merging team pays
+  // The counter has reached S: every other team's stores completed before its increment. Only the merging team pays
   // for an acquire (it drops this CU's and this XCD's possibly stale lines; the K/V stream is non-temporal and
   // loses nothing by it), after which plain vector loads may read the partial results.
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -672,7 +787,8 @@ static int launch_decode_cfg(const DecodeParams& prm, int head_blocks, hipStream
     if (e != hipSuccess) return fail(TDIST_ERR_LAUNCH, "decode: cannot reserve %zu B of LDS: %s", lds, hipGetErrorString(e));
     attr_set = true;
   }
-  dim3 grid(kWaveHeads ? prm.Hkv / NW : prm.Hkv * head_blocks, prm.S, prm.B);
+  dim3 grid(kWaveHeads ? prm.Hkv / NW : prm.Hkv * head_blocks,
+            kWaveHeads ? (prm.S + prm.splits_per_team - 1) / prm.splits_per_team : prm.S, prm.B);
   hipLaunchKernelGGL(kern, grid, dim3(NW * 64), lds, stream, prm);
   return launch_status(kFuse ? "tdist_decode_fused" : "tdist_decode_split_kv");
 }
@@ -756,6 +872,7 @@ static int run_decode(const DecodeCall& c, bool fuse) {
   prm.Hkv = c.kv_heads;
   prm.S = c.num_splits;
   prm.d_valid = dk;
+  prm.splits_per_team = 1;
   prm.page_size = c.page_size;
   int lg = 0;
   while ((1ll << lg) < c.page_size) ++lg;
@@ -817,11 +934,25 @@ static int run_decode(const DecodeCall& c, bool fuse) {
   const int wh_mode = wh_env ? atoi(wh_env) : 1;
   auto wave_heads = [&](int nw) {
     if (wh_mode == 0 || head_blocks != 1 || c.kv_heads % nw != 0 || (wh_mode == 4 && nw != 4)) return false;
-    if (wh_mode > 1) return true;
-    const int64_t teams = (int64_t)(c.kv_heads / nw) * c.num_splits * c.batch;
+    if (!aligned16(c.out_split)) return false;   // its partial results go out as 16-byte vectors
+    // Splits per workgroup: the count that needs the least time in units of (one split on every CU): rounds of
+    // workgroups x splits in each; of equal ones the larger, which starts fewer workgroups.
+    const int64_t heads_seqs = (int64_t)(c.kv_heads / nw) * c.batch;
     const int cus = device_info().num_cus > 0 ? device_info().num_cus : 256;
-    const int64_t rounds = (teams + cus - 1) / cus;
-    return teams >= cus && rounds * cus * 3 <= teams * 4;   // at most a quarter of the last round's slots idle
+    int64_t best_cost = 0;
+    int best_w = 1;
+    const int max_w = std::min(c.num_splits, decode_max_splits_per_team(dv));
+    for (int w = 1; w <= max_w; ++w) {
+      const int64_t teams = heads_seqs * ((c.num_splits + w - 1) / w);
+      const int64_t cost = ((teams + cus - 1) / cus) * w;
+      if (w == 1 || cost <= best_cost) best_cost = cost, best_w = w;
+    }
+    const char* spt = getenv("TDIST_DECODE_SPLITS_PER_TEAM");
+    if (spt && atoi(spt) >= 1) best_w = std::min(atoi(spt), max_w);
+    prm.splits_per_team = best_w;
+    if (wh_mode > 1) return true;
+    // against the time that work spread evenly over the CUs would need: at most a third more
+    return best_cost * cus * 3 <= heads_seqs * c.num_splits * 4;
   };
 #define TDIST_DEC_WH_(MMA_, D_, KEYS_, NW_, NST_, CAP_, FUSE_) \
   launch_decode_cfg<MMA_, D_, 0, KEYS_, NW_, NST_, CAP_, FUSE_, false, true>(prm, head_blocks, st)
