@@ -33,7 +33,7 @@ PEAK = {"bf16": 2.5e15, "fp8": 5.0e15, "hbm": 8.0e12}  # MI355X published dense 
 # the summaries are kept under profiles/.
 MEASURED_TRAFFIC_BYTES = {
     "c2_gemm": 839.2e6, "c2_reduce": 151.0e6, "c1_gemm": 130.3e6, "c3_gemm": 1646.6e6, "c4_dispatch": 265.8e6,
-    "c4_combine": 296.7e6, "c5_split_kv": 4315.7e6,
+    "c4_combine": 296.7e6, "c5_split_kv": 4316.1e6,
 }
 LIVE_PRODUCER = True  # --no-live-producer clears it
 METRIC = "AG-GEMM/GEMM-RS TFLOPS (% MFMA peak); decode & A2A GB/s (% HBM peak)"
