@@ -349,6 +349,21 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   const int wm = wave / WN, wn = wave % WN;
   const int lrow = lane % E::kRows, lgrp = lane / E::kRows;
 
+  // Per-lane parts of the operand fragment reads (16-row MFMA blocks: 16-byte piece lgrp or lgrp + 4 of row lrow of the
+  // wave's rows; the swizzle term does not depend on the 16-row block): A rows, A rows + 64 KB (the offset field of
+  // an LDS read ends at 64 KB), B rows with the start of the B stages folded in. Opaque to the compiler, which would
+  // otherwise re-associate them with the constants of the K loop.
+  uint32_t frag_lane_a[2] = {0, 0}, frag_lane_a_hi[2] = {0, 0}, frag_lane_b[2] = {0, 0};
+  if constexpr (E::kRows == 16) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int ra = wm * C::kWaveM + lrow, rb = wn * C::kWaveN + lrow;
+      frag_lane_a[q] = ra * KB + (((lgrp + 4 * q) ^ swz<KB>(ra)) << 4);
+      frag_lane_a_hi[q] = frag_lane_a[q] + 65536;
+      frag_lane_b[q] = C::kAStages * C::kABytes + rb * KB + (((lgrp + 4 * q) ^ swz<KB>(rb)) << 4);
+      asm volatile("" : "+v"(frag_lane_a[q]), "+v"(frag_lane_a_hi[q]), "+v"(frag_lane_b[q]));
+    }
+  }
   const int num_pid_m = (p.M + BM - 1) / BM;
   const int num_pid_n = (p.N + BN - 1) / BN;
   const int cm = p.m_per_chunk / BM;                 // row tiles per chunk
@@ -563,7 +578,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // operand fragments of the K step being multiplied (cur) and of the one after it (nxt)
     typename E::frag a_cur[C::kTM], b_cur[C::kTN], a_nxt[C::kTM], b_nxt[C::kTN];
     // f-th operand fragment (A fragments first) of K step ks of tile kt
-    auto load_frag = [&](int kt, int ks, int f, typename E::frag* af, typename E::frag* bf) {
+    // (a_st, b_st: the stages that hold the K tile's A and B rows)
+    auto load_frag_from = [&](lds_u8 a_st, lds_u8 b_st, int ks, int f, typename E::frag* af, typename E::frag* bf) {
       // 16-byte chunks of this lane's K bytes (c1 == c0 for 16-byte fragments). With four lane groups and two chunks
       // per lane, group g takes chunks g and g + 4 rather than 2g and 2g + 1: any assignment of K bytes to lanes gives
       // the same product as long as A and B share it, and only with the four groups of one read on consecutive chunks
@@ -573,14 +589,62 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       const int c1 = kStridedPieces ? lgrp + 4 : c0 + C::kFragVecs - 1;
       if (f < C::kTM) {
         const int r = wm * C::kWaveM + f * E::kRows + lrow;
-        lds_u8 const row = a_stage(kt) + r * KB;
+        lds_u8 const row = a_st + r * KB;
         af[f] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
       } else {
         const int j = f - C::kTM;
         const int r = wn * C::kWaveN + j * E::kRows + lrow;
-        lds_u8 const row = b_stage(kt) + r * KB;
+        lds_u8 const row = b_st + r * KB;
         bf[j] = E::load(row + ((c0 ^ swz<KB>(r)) << 4), row + ((c1 ^ swz<KB>(r)) << 4));
       }
+    };
+    auto load_frag = [&](int kt, int ks, int f, typename E::frag* af, typename E::frag* bf) {
+      load_frag_from(a_stage(kt), b_stage(kt), ks, f, af, bf);
+    };
+    // The same read with the stages as constants (split ring, 16-row MFMA blocks): the address is one of a few per-lane
+    // bases (frag_lane_*, set up once per kernel: everything that depends on the lane) plus a constant that fits the
+    // instruction's 16-bit offset field, so the K loop holds no address arithmetic for its LDS reads.
+    auto load_frag_c = [&](auto sa_c, auto sb_c, auto ks_c, auto f_c, typename E::frag* af, typename E::frag* bf) {
+      constexpr int SA = decltype(sa_c)::value % C::kAStages, SB = decltype(sb_c)::value % C::kBStages;
+      constexpr int ks = decltype(ks_c)::value, f = decltype(f_c)::value;
+      constexpr bool kStridedPieces = C::kLaneGroups == 4 && C::kFragVecs == 2;
+      static_assert(kStridedPieces || (C::kLaneGroups == 4 && C::kFragVecs == 1 && C::kKSteps == 2), "pieces lgrp and lgrp + 4");
+      constexpr int q0 = kStridedPieces ? 0 : ks, q1 = kStridedPieces ? 1 : ks;
+      if constexpr (f < C::kTM) {
+        constexpr int off = SA * C::kABytes + f * E::kRows * KB;
+        constexpr bool hi = off >= 65536;
+        lds_u8 const p0 = smem + (hi ? frag_lane_a_hi[q0] : frag_lane_a[q0]) + (hi ? off - 65536 : off);
+        lds_u8 const p1 = smem + (hi ? frag_lane_a_hi[q1] : frag_lane_a[q1]) + (hi ? off - 65536 : off);
+        af[f] = E::load(p0, p1);
+      } else {
+        constexpr int j = f - C::kTM;
+        constexpr int off = SB * C::kBBytes + j * E::kRows * KB;
+        static_assert(off < 65536, "B stages within reach of the offset field");
+        bf[j] = E::load(smem + frag_lane_b[q0] + off, smem + frag_lane_b[q1] + off);
+      }
+    };
+    // Split ring, K loop unrolled over the six (A stage, B stage) pairs: stage S of either ring as a constant address
+    auto a_stage_c = [&](auto s_c) -> lds_u8 { return smem + (decltype(s_c)::value % C::kAStages) * C::kABytes; };
+    auto b_stage_c = [&](auto s_c) -> lds_u8 {
+      return smem + C::kAStages * C::kABytes + (decltype(s_c)::value % C::kBStages) * C::kBBytes;
+    };
+    // The LDS address of such a load is a constant plus the wave's share of the stage; added inside the assembly, so
+    // that the compiler does not keep the sum of every (stage, instruction) pair in a scalar register of its own
+    // (there are more pairs than registers, and a spilled one comes back through the vector ALU).
+    auto dma16_at = [&](const unsigned char* sbase, uint32_t voff, lds_u8 dst_const, uint32_t dst_wave) {
+      const uint32_t lds_addr = (uint32_t)(uintptr_t)dst_const;
+      asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr),
+                   "s"(dst_wave)
+                   : "memory", "scc");
+    };
+    const uint32_t a_wave_off = __builtin_amdgcn_readfirstlane(wave * C::kAInstr * 1024);
+    const uint32_t b_wave_off = __builtin_amdgcn_readfirstlane(wave * C::kBInstr * 1024);
+    // K tile kt_src's rows into the given stage
+    auto issue_a_to = [&](lds_u8 st, int kt_src, int t) {
+      dma16_at(a_base + (int64_t)min(kt_src, KTp - 1) * KB, a_off[t], st + t * 1024, a_wave_off);
+    };
+    auto issue_b_to = [&](lds_u8 st, int kt_src, int u) {
+      dma16_at(b_base + (int64_t)min(kt_src, KTp - 1) * KB, b_off[u], st + u * 1024, b_wave_off);
     };
     auto load_frags = [&](int kt, int ks, typename E::frag* af, typename E::frag* bf) {
 #pragma unroll
@@ -648,10 +712,20 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
 #pragma unroll
       for (int f = 0; f < kHB; ++f) load_frag(0, 0, C::kTM + f, a_cur, b_cur);   // lower B half
       __builtin_amdgcn_sched_barrier(0);
-      // one tile; kOdd: the B halves in the order (upper, lower)
-      auto tile = [&](auto odd_c, int kt) {
-        constexpr int kOdd = decltype(odd_c)::value;
-        const int kt_next = min(kt + 1, KTp - 1);
+      // one tile; kOdd: the B halves in the order (upper, lower); SA, SB: the stages of its A and B rows (the tile
+      // after it sits in the next stage of either ring: behind the last K tile that is a stage nobody needs, read all
+      // the same, so that every trip runs the same instructions)
+      auto tile = [&](auto odd_c, auto sa_c, auto sb_c, int kt) {
+        constexpr int kOdd = decltype(odd_c)::value, SA = decltype(sa_c)::value, SB = decltype(sb_c)::value;
+        lds_u8 const a_now = a_stage_c(std::integral_constant<int, SA>{});
+        lds_u8 const b_now = b_stage_c(std::integral_constant<int, SB>{}), b_nx = b_stage_c(std::integral_constant<int, SB + 1>{});
+        // entry q of the list begun at this tile's barrier ([B(kt+2), A(kt+3)]: the stages of this tile's own rows) or
+        // of the one before ([B(kt+1), A(kt+2)])
+        auto issue_entry = [&](auto own_c, int q) {
+          constexpr bool own = decltype(own_c)::value;
+          if (q < C::kBInstr) issue_b_to(own ? b_now : b_nx, own ? kt + 2 : kt + 1, q);
+          else issue_a_to(own ? a_now : a_stage_c(std::integral_constant<int, SA + 2>{}), own ? kt + 3 : kt + 2, q - C::kBInstr);
+        };
         static_for<kMfmaPerStep>([&](auto u_c) {
           constexpr int u = decltype(u_c)::value;
           constexpr int quarter = u / kQuarter, w = u % kQuarter;
@@ -669,20 +743,26 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
           constexpr int stride = (kQuarter - 2) / n_reads;
           if constexpr (w >= 2 && (w - 2) % stride == 0 && (w - 2) / stride < n_reads) {
             constexpr int f = (w - 2) / stride;
-            if constexpr (quarter == 0) load_frag(kt, 0, C::kTM + kHB * (1 ^ kOdd) + f, a_cur, b_cur);
-            if constexpr (quarter == 1) load_frag(kt, 0, kHA + f, a_cur, b_cur);
-            if constexpr (quarter == 2) load_frag(kt_next, 0, f, a_cur, b_cur);
-            if constexpr (quarter == 3) load_frag(kt_next, 0, C::kTM + kHB * (1 ^ kOdd) + f, a_cur, b_cur);
+            using Z = std::integral_constant<int, 0>;
+            using NowA = std::integral_constant<int, SA>; using NowB = std::integral_constant<int, SB>;
+            using NxA = std::integral_constant<int, SA + 1>; using NxB = std::integral_constant<int, SB + 1>;
+            if constexpr (quarter == 0) load_frag_c(NowA{}, NowB{}, Z{}, std::integral_constant<int, C::kTM + kHB * (1 ^ kOdd) + f>{}, a_cur, b_cur);
+            if constexpr (quarter == 1) load_frag_c(NowA{}, NowB{}, Z{}, std::integral_constant<int, kHA + f>{}, a_cur, b_cur);
+            if constexpr (quarter == 2) load_frag_c(NxA{}, NxB{}, Z{}, std::integral_constant<int, f>{}, a_cur, b_cur);
+            if constexpr (quarter == 3) load_frag_c(NxA{}, NxB{}, Z{}, std::integral_constant<int, C::kTM + kHB * (1 ^ kOdd) + f>{}, a_cur, b_cur);
           }
           constexpr int since = (u - kBar + kMfmaPerStep) % kMfmaPerStep;  // slots since the last barrier
           constexpr int due = dma_due(since);
-          if constexpr (due >= 0) issue_list(u >= kBar ? kt : kt - 1, due);
+          if constexpr (due >= 0) issue_entry(std::integral_constant<bool, (u >= kBar)>{}, due);
           __builtin_amdgcn_sched_barrier(0);
         });
       };
-      for (int kt = 0; kt < KTp; kt += 2) {
-        tile(std::integral_constant<int, 0>{}, kt);
-        if (kt + 1 < KTp) tile(std::integral_constant<int, 1>{}, kt + 1);
+      for (int kt = 0; kt < KTp; kt += 6) {
+        static_for<6>([&](auto n_c) {
+          constexpr int n = decltype(n_c)::value;
+          if (kt + n < KTp)
+            tile(std::integral_constant<int, n % 2>{}, std::integral_constant<int, n % 3>{}, std::integral_constant<int, n % 2>{}, kt + n);
+        });
       }
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the last MFMAs' results: 8 passes + 3 cycles after issue
     } else if constexpr (C::kSplit && E::kRows == 16) {
@@ -710,16 +790,30 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       wait_tiles_and_barrier<C::kAInstr + C::kDmaPerStep>();
       load_frags(0, 0, a_cur, b_cur);
       __builtin_amdgcn_sched_barrier(0);
-      for (int kt = 0; kt < KTp; ++kt) {
-        const int kt_next = min(kt + 1, KTp - 1);
+      // K tile kt, its A rows in stage SA and its B rows in stage SB (the tile after it sits in the next stage of either
+      // ring: behind the last K tile that is a stage nobody needs, read all the same, so that every trip runs the same
+      // instructions)
+      auto k_tile = [&](auto sa_c, auto sb_c, int kt) {
+        constexpr int SA = decltype(sa_c)::value, SB = decltype(sb_c)::value;
+        lds_u8 const st_a = a_stage_c(std::integral_constant<int, SA>{});
+        lds_u8 const st_b = b_stage_c(std::integral_constant<int, SB>{}), st_b_nx = b_stage_c(std::integral_constant<int, SB + 1>{});
+        // entry q of this tile's own refill list ([B(kt+2), A(kt+3)]: into the stages of its own rows) or of the one
+        // before ([B(kt+1), A(kt+2)])
+        auto issue_entry = [&](auto own_c, int q) {
+          constexpr bool own = decltype(own_c)::value;
+          if (q < C::kBInstr) issue_b_to(own ? st_b : st_b_nx, own ? kt + 2 : kt + 1, q);
+          else issue_a_to(own ? st_a : a_stage_c(std::integral_constant<int, SA + 2>{}), own ? kt + 3 : kt + 2, q - C::kBInstr);
+        };
         auto step = [&](auto ks_c, typename E::frag* a_now, typename E::frag* a_new) {
           constexpr int ks = decltype(ks_c)::value;
           constexpr bool last = ks == C::kKSteps - 1;
           constexpr int first = last ? kLead : 0;
           constexpr int nslots = kMfmaPerStep - first;
           constexpr int pos = (ks + 1) % C::kKSteps;
-          const int r_kt = last ? kt_next : kt;   // tile and K step the reads of this step fetch
-          constexpr int r_ks = last ? 0 : ks + 1;
+          // stages and K step the reads of this step fetch
+          using RA = std::integral_constant<int, last ? SA + 1 : SA>;
+          using RB = std::integral_constant<int, last ? SB + 1 : SB>;
+          using RKs = std::integral_constant<int, last ? 0 : ks + 1>;
           static_for<kMfmaPerStep>([&](auto idx_c) {
             constexpr int idx = decltype(idx_c)::value;
             constexpr int j = idx / C::kTM, i = idx % C::kTM;
@@ -729,20 +823,27 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
               wait_tiles_and_barrier<C::kAInstr>();
               __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (i == C::kTM - 1) load_frag(r_kt, r_ks, C::kTM + j, a_new, b_cur);  // B fragment j, in place
+            if constexpr (i == C::kTM - 1) load_frag_c(RA{}, RB{}, RKs{}, std::integral_constant<int, C::kTM + j>{}, a_new, b_cur);  // B fragment j, in place
             if constexpr (idx > kLead && (idx - kLead - 1) % kAStride == 0 && (idx - kLead - 1) / kAStride < C::kTM)
-              load_frag(r_kt, r_ks, (idx - kLead - 1) / kAStride, a_new, b_cur);
+              load_frag_c(RA{}, RB{}, RKs{}, std::integral_constant<int, (idx - kLead - 1) / kAStride>{}, a_new, b_cur);
             if constexpr (idx >= first) {
               constexpr int slot = idx - first;
 #pragma unroll
               for (int d = 0; d < C::kDmaPerStep; ++d)
-                if (slot == (d * nslots) / C::kDmaPerStep) issue_list(last ? kt : kt - 1, pos * C::kDmaPerStep + d);
+                if (slot == (d * nslots) / C::kDmaPerStep) issue_entry(std::integral_constant<bool, last>{}, pos * C::kDmaPerStep + d);
             }
             __builtin_amdgcn_sched_barrier(0);
           });
         };
         step(std::integral_constant<int, 0>{}, a_cur, a_nxt);
         step(std::integral_constant<int, 1>{}, a_nxt, a_cur);
+      };
+      // unrolled over the six (A stage, B stage) pairs: every LDS address in the loop is a constant
+      for (int kt = 0; kt < KTp; kt += 6) {
+        static_for<6>([&](auto n_c) {
+          constexpr int n = decltype(n_c)::value;
+          if (kt + n < KTp) k_tile(std::integral_constant<int, n % 3>{}, std::integral_constant<int, n % 2>{}, kt + n);
+        });
       }
       // the last MFMAs' results are readable 4 passes + 3 cycles after issue
       asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
