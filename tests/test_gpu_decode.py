@@ -339,7 +339,7 @@ def test_head_dimensions_that_are_no_power_of_two(cuda, D, num_heads, kv_lens, S
 
 @pytest.mark.parametrize("D,num_heads,force", [(128, (64, 8), 2), (128, (16, 16), 2), (128, (32, 8), 2), (64, (64, 8), 4),
                                                (64, (24, 8), 2), (64, (16, 16), 4), (64, (64, 4), 2), (256, (32, 8), 2),
-                                               (256, (12, 4), 2)])
+                                               (256, (12, 4), 2), (96, (64, 8), 2), (80, (16, 16), 2), (112, (24, 8), 2)])
 @pytest.mark.parametrize("kv_lens,S,block_size", [([1320, 18, 463], 4, 16), ([1, 54, 293, 70], 8, 1), ([777, 0, 5, 2047], 3, 16),
                                                   ([100, 31], 1, 16)])
 @pytest.mark.parametrize("dtype,soft_cap", [(torch.bfloat16, 0), (torch.float16, 30)])

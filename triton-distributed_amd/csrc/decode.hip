@@ -457,7 +457,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
 
   constexpr float kLn2 = 0.6931471805599453f;
   if constexpr (kWaveHeads) {
-    static_assert(!kPadded && !C::kWaitFirst, "a kv head per wave: plain rows, several groups in flight");
+    static_assert(!C::kWaitFirst, "a kv head per wave: several groups in flight");
     // One pipeline over all blocks of the team's splits: the loads of the next split's first blocks are in flight
     // while the last blocks of this one are computed. The results go out of the registers (no LDS: the ring belongs
     // to the loads in flight) when the stream has ended.
@@ -510,7 +510,8 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
           if (x < nvalid) {
             float* o = out_base + ((int64_t)x * prm.S + which) * Dout + 4 * g;
 #pragma unroll
-            for (int d = 0; d < D / 16; ++d) store_partial4<kFuse>(o + 16 * d, val[d]);
+            for (int d = 0; d < D / 16; ++d)
+              if (!kPadded || 16 * d + 4 * g < Dout) store_partial4<kFuse>(o + 16 * d, val[d]);
             if (g == 0) store_partial<kFuse>(lse_base + (int64_t)x * prm.S + which, val_lse);
           }
         };
@@ -920,12 +921,6 @@ static int run_decode(const DecodeCall& c, bool fuse) {
 #define TDIST_DEC_PADDED(D_, KEYS_, NW_, NST_)                                                 \
   return bf ? launch_decode<MmaBF16, D_, 0, KEYS_, NW_, NST_, true>(prm, head_blocks, st)     \
             : launch_decode<MmaF16, D_, 0, KEYS_, NW_, NST_, true>(prm, head_blocks, st);
-  if (padded) {
-    // any other head dimension: the shape of the next power of two, rows filled up with zeros on their way in
-    if (dk < 64) TDIST_DEC_PADDED(64, 32, 4, 4)
-    if (dk < 128) TDIST_DEC_PADDED(128, 16, 3, 3)
-    TDIST_DEC_PADDED(256, 16, 2, 3)
-  }
   // A kv head per wave (8 waves of 2 stages or 4 waves of 4, 130-136 KB: one workgroup per CU) where the heads allow it and the grid
   // fills the CUs in whole rounds or in many: such a workgroup is NW_ times the work of one of the other form,
   // whose small workgroups fill a small grid's CUs better. TDIST_DECODE_WAVE_HEADS=0 never takes this form, 2 takes
@@ -954,16 +949,26 @@ static int run_decode(const DecodeCall& c, bool fuse) {
     // against the time that work spread evenly over the CUs would need: at most a third more
     return best_cost * cus * 3 <= heads_seqs * c.num_splits * 4;
   };
-#define TDIST_DEC_WH_(MMA_, D_, KEYS_, NW_, NST_, CAP_, FUSE_) \
-  launch_decode_cfg<MMA_, D_, 0, KEYS_, NW_, NST_, CAP_, FUSE_, false, true>(prm, head_blocks, st)
-#define TDIST_DEC_WH(D_, KEYS_, NW_, NST_)                                                                              \
+#define TDIST_DEC_WH_(MMA_, D_, KEYS_, NW_, NST_, CAP_, FUSE_, PAD_) \
+  launch_decode_cfg<MMA_, D_, 0, KEYS_, NW_, NST_, CAP_, FUSE_, PAD_, true>(prm, head_blocks, st)
+#define TDIST_DEC_WH(D_, KEYS_, NW_, NST_) TDIST_DEC_WH_P(D_, KEYS_, NW_, NST_, false)
+#define TDIST_DEC_WH_P(D_, KEYS_, NW_, NST_, PAD_)                                                                              \
   if (wave_heads(NW_)) {                                                                                             \
     if (prm.soft_cap > 0.f) {                                                                                        \
-      if (fuse) return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, true) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, true);     \
-      return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, false) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, false);             \
+      if (fuse) return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, true, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, true, PAD_);     \
+      return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, false, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, false, PAD_);             \
     }                                                                                                                \
-    if (fuse) return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, true) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, true);     \
-    return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, false) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, false);             \
+    if (fuse) return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, true, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, true, PAD_);     \
+    return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, false, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, false, PAD_);             \
+  }
+  if (padded) {
+    // any other head dimension: the shape of the next power of two, rows filled up with zeros on their way in
+    if (dk < 64) TDIST_DEC_PADDED(64, 32, 4, 4)
+    if (dk < 128) {
+      TDIST_DEC_WH_P(128, 16, 8, 2, true)
+      TDIST_DEC_PADDED(128, 16, 3, 3)
+    }
+    TDIST_DEC_PADDED(256, 16, 2, 3)
   }
   switch (dk) {
     case 64:
@@ -983,6 +988,7 @@ static int run_decode(const DecodeCall& c, bool fuse) {
   }
 #undef TDIST_DEC
 #undef TDIST_DEC_WH
+#undef TDIST_DEC_WH_P
 #undef TDIST_DEC_WH_
 #undef TDIST_DEC_PADDED
 }
