@@ -52,6 +52,24 @@ def test_exact_on_integer_inputs(cuda, tile_env, dtype, tile, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
+@pytest.mark.parametrize("tile", [0, 1, 3, 4])
+def test_every_k_tile_count_from_one_to_thirteen(cuda, tile_env, dtype, tile):
+    """The split ring's K loop is unrolled over its six (A stage, B stage) pairs: every number of 128-byte K tiles
+    from 1 to 13 leaves the loop after a different pair, twice over. Two tiles of C per workgroup column so that a
+    second tile starts on a ring the first one has used. Exact on integer-valued inputs."""
+    esz = 1 if dtype == torch.float8_e4m3fn else 2
+    out_dtype = torch.bfloat16 if dtype == torch.float8_e4m3fn else dtype
+    for kt in range(1, 14):
+        M, N, K = 512, 768, kt * 128 // esz
+        announce("mfma shapes k tiles %s tile %d kt %d (%dx%dx%d)" % (dtype, tile, kt, M, N, K))
+        g = torch.Generator().manual_seed(kt + 100 * tile)
+        a = torch.randint(-2, 3, (M, K), generator=g).float().to(dtype).to(cuda)
+        b = torch.randint(-2, 3, (N, K), generator=g).float().to(dtype).to(cuda)
+        ref = (a.float() @ b.float().T).to(out_dtype)
+        assert torch.equal(run_tile(cuda, a, b, out_dtype, tile, max_workgroups=2), ref), "kt = %d" % kt
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
 def test_random_inputs_close_in_every_form(cuda, tile_env, dtype):
     M, N, K = 1536, 1024, 4224
     announce("mfma shapes random %s %dx%dx%d" % (dtype, M, N, K))
