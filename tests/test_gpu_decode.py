@@ -389,3 +389,51 @@ def test_a_kv_head_per_wave(cuda, monkeypatch, D, num_heads, force, kv_lens, S, 
     exact, _ = golden.decode_exact(q, k_cache, v_cache, kv_lens, table, scale, soft_cap)
     eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
     assert ((got.cpu().double() - exact).abs() <= ATOL + eps * exact.abs()).all()
+
+
+@pytest.mark.parametrize("kind", ["even", "one long", "random"])
+def test_form_follows_the_sequence_lengths(cuda, monkeypatch, kind):
+    """A grid that fills the chip gets two launches: the form with a kv head per wave, which runs if the sequence
+    lengths are even (mean >= 0.8 max, decided on the device by every wave from the same loads), and the form with a
+    kv head per workgroup behind it, which runs if they are not. Exactly one of them must have written every partial
+    result (the buffers start as NaN), for even and uneven batches alike, split and one-launch forms."""
+    from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine, decode_fused
+    monkeypatch.delenv("TDIST_DECODE_WAVE_HEADS", raising=False)
+    monkeypatch.delenv("TDIST_DECODE_SPLITS_PER_TEAM", raising=False)
+    B, heads, D, page, S = 32, (8, 8), 64, 16, 8      # 32 x 8 (sequence, split) pairs on one head group: 256 workgroups
+    g = torch.Generator().manual_seed(5)
+    if kind == "even":
+        kv_lens = [2048] * B
+    elif kind == "one long":
+        kv_lens = [2048] + [64] * (B - 1)
+    else:
+        kv_lens = torch.randint(1, 2049, (B,), generator=g).tolist()
+    announce("decode form by lengths: %s (sum %d, max %d)" % (kind, sum(kv_lens), max(kv_lens)))
+    q, k_cache, v_cache, table = build_case(kv_lens, heads, D, page, torch.bfloat16, seed=9)
+    scale = D**-0.5
+    lens_dev = torch.tensor(kv_lens, dtype=torch.int32, device=cuda)
+    qd, kd, vd, td = q.to(cuda), k_cache.to(cuda), v_cache.to(cuda), table.to(cuda)
+    out_split = torch.full((B, heads[0], S, D), float("nan"), dtype=torch.float32, device=cuda)
+    lse_split = torch.full((B, heads[0], S), float("nan"), dtype=torch.float32, device=cuda)
+    _split_kv(qd, kd, vd, lens_dev, td, scale, 0.0, S, out_split, lse_split)
+    torch.cuda.synchronize()
+    w_out, w_lse = golden.decode_split_exact(q, k_cache, v_cache, kv_lens, table, scale, S)
+    got_lse = lse_split.cpu().double()
+    empty = torch.isinf(w_lse)
+    assert not torch.isnan(out_split).any() and not torch.isnan(lse_split).any()
+    assert torch.equal(torch.isinf(got_lse), empty)
+    assert (got_lse[~empty] - w_lse[~empty]).abs().max() <= ATOL
+    assert (out_split.cpu().double() - w_out).abs().max() <= ATOL
+    want = torch.empty((B, heads[0], D), dtype=torch.bfloat16, device=cuda)
+    want_lse = torch.empty((B, heads[0]), dtype=torch.float32, device=cuda)
+    decode_combine(out_split, lse_split, S, 1, lens_dev, B, heads[0], D,
+                   (out_split.stride(2), out_split.stride(0), out_split.stride(1)),
+                   (lse_split.stride(2), lse_split.stride(0), lse_split.stride(1)), want, want_lse)
+    counters = torch.zeros(1024, dtype=torch.int32, device=cuda)
+    got = torch.full((B, heads[0], D), float("nan"), dtype=torch.bfloat16, device=cuda)
+    got_lse = torch.full((B, heads[0]), float("nan"), dtype=torch.float32, device=cuda)
+    decode_fused(qd, kd, vd, lens_dev, td, scale, 0.0, S, got, got_lse, workspace=counters)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(got_lse.view(torch.int32), want_lse.view(torch.int32))
+    assert int(counters.abs().sum()) == 0

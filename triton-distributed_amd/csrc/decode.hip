@@ -49,6 +49,7 @@ struct DecodeParams {
   float sm_scale;
   float soft_cap;
   int B, Hq, Hkv, S;
+  int when_lens;        // 0: run; 1: run only if the sequence lengths are even (decode_lens_even), 2: only if not
   int splits_per_team;  // kWaveHeads: consecutive splits of a sequence that one workgroup streams through (>= 1)
   int d_valid;  // kernels compiled for a padded head dimension: the real one (a multiple of 8), else unused
   int page_size;
@@ -180,6 +181,29 @@ template <bool kCoherent>
 __device__ __forceinline__ void store_partial4(float* p, float4v v) {
   if constexpr (kCoherent) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0" ::"v"(p), "v"(v) : "memory");
   else *(float4v*)p = v;
+}
+
+// Are the B sequence lengths even enough for the form that hands a workgroup 8 kv heads of one (sequence, split)?
+// Its time goes with the longest sequence, the other form's (eight times as many, smaller workgroups) with the
+// sum: even means mean >= 0.8 max (measured: the one form is 7-11 % faster from mean = 0.9 max on, the other 11 % at
+// 0.57 and 6 x with one long sequence among short ones). Every wave computes the same answer from the same loads, so
+// two launches, one of each form, can each ask and exactly one of them does the work.
+__device__ __forceinline__ bool decode_lens_even(const int32_t* lens, int B) {
+  const int lane = threadIdx.x & 63;
+  long long sum = 0;
+  int mx = 0;
+  for (int i = lane; i < B; i += 64) {
+    const int l = lens[i];
+    sum += l;
+    mx = max(mx, l);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const unsigned int lo = __shfl_xor((unsigned int)sum, o), hi = __shfl_xor((unsigned int)(sum >> 32), o);
+    sum += (long long)(((unsigned long long)hi << 32) | lo);
+    mx = max(mx, __shfl_xor(mx, o));
+  }
+  return sum * 5 >= (long long)mx * B * 4;
 }
 
 // kPadded: the head dimension is prm.d_valid <= D (key and value alike, a multiple of 8): the rows in the LDS are D
@@ -771,6 +795,7 @@ __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
 
 template <typename MMA, int D, int DPE, int KEYS, int NW, int NST, bool kSoftCap, bool kFuse, bool kPadded, bool kWaveHeads = false>
 __global__ __launch_bounds__(NW * 64) void decode_split_kv_kernel(const DecodeParams prm) {
+  if (prm.when_lens != 0 && decode_lens_even(prm.lens, prm.B) != (prm.when_lens == 1)) return;
   decode_split_body<MMA, D, DPE, KEYS, NW, NST, kSoftCap, kFuse, kPadded, kWaveHeads>(prm);
   if constexpr (kFuse) decode_fused_merge<D, NW, kPadded, kWaveHeads>(prm);
 }
@@ -874,6 +899,7 @@ static int run_decode(const DecodeCall& c, bool fuse) {
   prm.S = c.num_splits;
   prm.d_valid = dk;
   prm.splits_per_team = 1;
+  prm.when_lens = 0;
   prm.page_size = c.page_size;
   int lg = 0;
   while ((1ll << lg) < c.page_size) ++lg;
@@ -952,14 +978,21 @@ static int run_decode(const DecodeCall& c, bool fuse) {
 #define TDIST_DEC_WH_(MMA_, D_, KEYS_, NW_, NST_, CAP_, FUSE_, PAD_) \
   launch_decode_cfg<MMA_, D_, 0, KEYS_, NW_, NST_, CAP_, FUSE_, PAD_, true>(prm, head_blocks, st)
 #define TDIST_DEC_WH(D_, KEYS_, NW_, NST_) TDIST_DEC_WH_P(D_, KEYS_, NW_, NST_, false)
-#define TDIST_DEC_WH_P(D_, KEYS_, NW_, NST_, PAD_)                                                                              \
-  if (wave_heads(NW_)) {                                                                                             \
+#define TDIST_DEC_WH_P(D_, KEYS_, NW_, NST_, PAD_)                                                                      \
+  if (prm.when_lens == 0 && wave_heads(NW_)) {                                                                       \
+    /* chosen for the grid: it runs if the sequence lengths are even, and the other form, launched behind it, if   \
+       they are not (forced by the environment: unconditionally, alone) */                                          \
+    prm.when_lens = wh_mode > 1 ? 0 : 1;                                                                             \
+    int rc_;                                                                                                         \
     if (prm.soft_cap > 0.f) {                                                                                        \
-      if (fuse) return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, true, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, true, PAD_);     \
-      return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, false, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, false, PAD_);             \
+      if (fuse) rc_ = bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, true, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, true, PAD_);     \
+      else rc_ = bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, false, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, false, PAD_);         \
+    } else {                                                                                                         \
+      if (fuse) rc_ = bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, true, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, true, PAD_);   \
+      else rc_ = bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, false, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, false, PAD_);       \
     }                                                                                                                \
-    if (fuse) return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, true, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, true, PAD_);     \
-    return bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, false, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, false, PAD_);             \
+    if (rc_ != TDIST_OK || wh_mode > 1) return rc_;                                                                  \
+    prm.when_lens = 2;                                                                                               \
   }
   if (padded) {
     // any other head dimension: the shape of the next power of two, rows filled up with zeros on their way in
