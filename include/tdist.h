@@ -404,7 +404,11 @@ int64_t tdist_gemm_split_k_workspace_bytes(void);
  * to 256 ((64,64), (128,128) and (256,256) on shapes of their own, the others, e.g. 80, 96 and 160, on the shape of
  * the next power of two with the missing dimensions read as zeros: the reference's BLOCK_DMODEL + BLOCK_DPE split
  * with masks, flash_decode.py:771-772), and the heads whose keys carry 64 dimensions more than their values:
- * (192,128), (576,512); dtype bf16 / f16. */
+ * (192,128), (576,512); dtype bf16 / f16.
+ * A call is one kernel launch, or two where the grid is large enough for the form that gives every wave a kv head of
+ * its own: that form runs if the sequence lengths are even (mean >= 0.8 max), the other one, launched behind it, if
+ * not; the kernels decide from kv_lens on the device, and the one that does not run returns at once. Kernels only:
+ * the call can be captured into a HIP graph. */
 int tdist_decode_split_kv(const void* q, const void* k_cache, const void* v_cache, float* out_split,
                           float* lse_split, float sm_scale, float soft_cap, const int32_t* block_table,
                           const int32_t* kv_lens, int batch, int q_heads, int kv_heads, int head_dim,
