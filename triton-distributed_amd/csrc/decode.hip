@@ -947,10 +947,13 @@ static int run_decode(const DecodeCall& c, bool fuse) {
 #define TDIST_DEC_PADDED(D_, KEYS_, NW_, NST_)                                                 \
   return bf ? launch_decode<MmaBF16, D_, 0, KEYS_, NW_, NST_, true>(prm, head_blocks, st)     \
             : launch_decode<MmaF16, D_, 0, KEYS_, NW_, NST_, true>(prm, head_blocks, st);
-  // A kv head per wave (8 waves of 2 stages or 4 waves of 4, 130-136 KB: one workgroup per CU) where the heads allow it and the grid
-  // fills the CUs in whole rounds or in many: such a workgroup is NW_ times the work of one of the other form,
-  // whose small workgroups fill a small grid's CUs better. TDIST_DECODE_WAVE_HEADS=0 never takes this form, 2 takes
-  // it wherever the heads allow it, 4 likewise but only its 4-wave workgroups.
+  // A kv head per wave (8 waves of 2 stages or 4 waves of 4, 130-136 KB: one workgroup per CU) where the heads allow
+  // it, the grid fills the CUs in whole rounds or in many (such a workgroup is NW_ times the work of one of the other
+  // form, whose small workgroups fill a small grid's CUs better) and the cache is large enough for a tenth of the
+  // kernel's time to outweigh a second launch: the form's time goes with the longest sequence, so the other form is
+  // launched behind it and the kernels decide by the sequence lengths which of the two runs (decode_lens_even).
+  // TDIST_DECODE_WAVE_HEADS=0 never takes this form; 2 takes it wherever the heads allow it, alone and whatever the
+  // lengths; 4 likewise but only its 4-wave workgroups.
   const char* wh_env = getenv("TDIST_DECODE_WAVE_HEADS");
   const int wh_mode = wh_env ? atoi(wh_env) : 1;
   auto wave_heads = [&](int nw) {
@@ -972,6 +975,9 @@ static int run_decode(const DecodeCall& c, bool fuse) {
     if (spt && atoi(spt) >= 1) best_w = std::min(atoi(spt), max_w);
     prm.splits_per_team = best_w;
     if (wh_mode > 1) return true;
+    // the most that the block table lets the call read: below 256 MB (40 us) the form's gain is less than a launch
+    const double cap_bytes = (double)c.batch * c.kv_heads * (double)c.table_stride * c.page_size * (dk + dv) * 2.0;
+    if (cap_bytes < 256e6) return false;
     // against the time that work spread evenly over the CUs would need: at most a third more
     return best_cost * cus * 3 <= heads_seqs * c.num_splits * 4;
   };
@@ -982,7 +988,7 @@ static int run_decode(const DecodeCall& c, bool fuse) {
   if (prm.when_lens == 0 && wave_heads(NW_)) {                                                                       \
     /* chosen for the grid: it runs if the sequence lengths are even, and the other form, launched behind it, if   \
        they are not (forced by the environment: unconditionally, alone) */                                          \
-    prm.when_lens = wh_mode > 1 ? 0 : 1;                                                                             \
+    prm.when_lens = (wh_mode > 1 || c.batch == 1) ? 0 : 1;   /* (one sequence: even by definition) */               \
     int rc_;                                                                                                         \
     if (prm.soft_cap > 0.f) {                                                                                        \
       if (fuse) rc_ = bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, true, true, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, true, true, PAD_);     \
@@ -991,7 +997,7 @@ static int run_decode(const DecodeCall& c, bool fuse) {
       if (fuse) rc_ = bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, true, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, true, PAD_);   \
       else rc_ = bf ? TDIST_DEC_WH_(MmaBF16, D_, KEYS_, NW_, NST_, false, false, PAD_) : TDIST_DEC_WH_(MmaF16, D_, KEYS_, NW_, NST_, false, false, PAD_);       \
     }                                                                                                                \
-    if (rc_ != TDIST_OK || wh_mode > 1) return rc_;                                                                  \
+    if (rc_ != TDIST_OK || prm.when_lens == 0) return rc_;                                                           \
     prm.when_lens = 2;                                                                                               \
   }
   if (padded) {
