@@ -192,10 +192,19 @@ __device__ __forceinline__ bool decode_lens_even(const int32_t* lens, int B) {
   const int lane = threadIdx.x & 63;
   long long sum = 0;
   int mx = 0;
-  for (int i = lane; i < B; i += 64) {
-    const int l = lens[i];
-    sum += l;
-    mx = max(mx, l);
+  // sixteen loads in flight per lane: one round trip for up to 1024 sequences
+  for (int i0 = 0; i0 < B; i0 += 64 * 16) {
+    int l[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int i = i0 + u * 64 + lane;
+      l[u] = i < B ? lens[i] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      sum += max(l[u], 0);
+      mx = max(mx, l[u]);
+    }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
