@@ -660,6 +660,11 @@ __device__ __forceinline__ void store_elem(unsigned char* base, int64_t idx, int
 }
 
 // One wave per (b,h); lanes stride over Dv. Partial j is weighted by exp(lse_j - max).
+// Lane j holds the LSE of partial j (one load per lane instead of a loop of loads in every lane; -inf where the
+// partial is skipped), the maximum is a wave reduction, and the partial rows of up to 32 / kPerLane partials are in
+// flight together: two round trips to memory for a merge of 16 partials. The sums run over the partials in index
+// order, whatever the batching.
+template <int kPerLane>
 __global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams prm) {
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -678,43 +683,51 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const CombineParams
     return false;
   };
   const float* lse = prm.lse + (int64_t)b * prm.l_sb + (int64_t)h * prm.l_sh;
+  // LSE of partial j0 + lane
+  auto lse_of_lane = [&](int j0) -> float {
+    const int j = j0 + lane;
+    return (j < prm.P && !skipped(j)) ? lse[(int64_t)j * prm.l_sp] : -INFINITY;
+  };
   float M = -INFINITY;
-  for (int j = 0; j < prm.P; ++j)
-    if (!skipped(j)) M = fmaxf(M, lse[(int64_t)j * prm.l_sp]);
+  for (int j0 = 0; j0 < prm.P; j0 += 64) M = fmaxf(M, lse_of_lane(j0));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
   float L = 0.f;
-  constexpr int kMaxPerLane = 8;  // Dv <= 512
-  float acc[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const int per_lane = (prm.Dv + 63) >> 6;
+  float acc[kPerLane];
+#pragma unroll
+  for (int q = 0; q < kPerLane; ++q) acc[q] = 0.f;
   if (M != -INFINITY) {
-    // four partials at a time: their loads are issued together, the sums stay in partial order
-    constexpr int kBatch = 4;
-    for (int j0 = 0; j0 < prm.P; j0 += kBatch) {
-      float w[kBatch];
-      float x[kBatch][kMaxPerLane];
+    constexpr int kBatch = 32 / kPerLane;
+    for (int c0 = 0; c0 < prm.P; c0 += 64) {
+      const float l_lane = lse_of_lane(c0);
+      const int n_here = min(64, prm.P - c0);
+      for (int j0 = 0; j0 < n_here; j0 += kBatch) {
+        float w[kBatch];
+        float x[kBatch][kPerLane];
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        const int j = j0 + u;
-        float lj = -INFINITY;
-        if (j < prm.P && !skipped(j)) lj = lse[(int64_t)j * prm.l_sp];
-        w[u] = lj == -INFINITY ? 0.f : __expf(lj - M);
-        const int64_t base = (int64_t)min(j, prm.P - 1) * prm.p_sp + (int64_t)b * prm.p_sb + (int64_t)h * prm.p_sh;
+        for (int u = 0; u < kBatch; ++u) {
+          const int jj = j0 + u;   // (within the chunk; lanes beyond it hold -inf)
+          const float lj = jj < 64 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l_lane), jj & 63)) : -INFINITY;
+          w[u] = lj == -INFINITY ? 0.f : __expf(lj - M);
+          const int64_t base = (int64_t)min(c0 + jj, prm.P - 1) * prm.p_sp + (int64_t)b * prm.p_sb + (int64_t)h * prm.p_sh;
 #pragma unroll
-        for (int q = 0; q < kMaxPerLane; ++q) {
-          const int d = lane + q * 64;
-          x[u][q] = (q < per_lane && d < prm.Dv && lj != -INFINITY) ? load_elem(prm.part, base + d, prm.part_dtype) : 0.f;
+          for (int q = 0; q < kPerLane; ++q) {
+            const int d = lane + q * 64;
+            x[u][q] = (d < prm.Dv && lj != -INFINITY) ? load_elem(prm.part, base + d, prm.part_dtype) : 0.f;
+          }
         }
-      }
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        L += w[u];   // a skipped, empty or out-of-range partial has w = 0 and x = 0: it adds nothing
+        for (int u = 0; u < kBatch; ++u) {
+          L += w[u];   // a skipped, empty or out-of-range partial has w = 0 and x = 0: it adds nothing
 #pragma unroll
-        for (int q = 0; q < kMaxPerLane; ++q) acc[q] += w[u] * x[u][q];
+          for (int q = 0; q < kPerLane; ++q) acc[q] += w[u] * x[u][q];
+        }
       }
     }
   }
   const int64_t obase = (int64_t)b * prm.o_sb + (int64_t)h * prm.o_sh;
 #pragma unroll
-  for (int u = 0; u < kMaxPerLane; ++u) {
+  for (int u = 0; u < kPerLane; ++u) {
     const int d = lane + u * 64;
     if (d < prm.Dv) store_elem(prm.out, obase + d, prm.out_dtype, L > 0.f ? acc[u] / L : 0.f);
   }
@@ -780,19 +793,39 @@ __device__ __forceinline__ void decode_fused_merge(const DecodeParams& prm) {
   for (int idx = team_tid; idx < nvalid * kVecs; idx += kTeam) {
     const int h = idx / kVecs, dv = (idx - h * kVecs) * 4;
     const float* l = lse_p + (int64_t)h * prm.S;
+    // sixteen splits at a time: their LSEs, then their rows, are in flight together (two round trips for 16 splits);
+    // the sums run over the splits in order
+    constexpr int kBatch = 16;
     float M = -INFINITY;
-    for (int j = 0; j < prm.S; ++j) M = fmaxf(M, l[j]);
+    for (int j0 = 0; j0 < prm.S; j0 += kBatch) {
+      float lj[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) lj[u] = j0 + u < prm.S ? l[j0 + u] : -INFINITY;
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) M = fmaxf(M, lj[u]);
+    }
     float L = 0.f;
     float4v acc = {0.f, 0.f, 0.f, 0.f};
     if (M != -INFINITY) {
       // an empty split has LSE = -inf and zeros: weight exp(-inf) = 0 adds nothing, as skipping it would
-#pragma unroll 4
-      for (int j = 0; j < prm.S; ++j) {
-        const float w = __expf(l[j] - M);
-        L += w;
-        const float4v x = *(const float4v*)(out_p + ((int64_t)h * prm.S + j) * D + dv);
+      for (int j0 = 0; j0 < prm.S; j0 += kBatch) {
+        float lj[kBatch];
+        float4v x[kBatch];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] += w * x[e];
+        for (int u = 0; u < kBatch; ++u) {
+          const int j = min(j0 + u, prm.S - 1);
+          lj[u] = l[j];
+          x[u] = *(const float4v*)(out_p + ((int64_t)h * prm.S + j) * D + dv);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          if (j0 + u < prm.S) {
+            const float w = __expf(lj[u] - M);
+            L += w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += w * x[u][e];
+          }
+        }
       }
     }
     const int64_t o = (int64_t)b * prm.fo_sb + (int64_t)(h0 + h) * prm.fo_sh + dv;
@@ -1114,7 +1147,8 @@ int tdist_decode_combine(const void* part, int part_dtype, const float* lse, int
   prm.o_sh = out_stride_h;
   const int64_t blocks = ceil_div((int64_t)batch * q_heads, 4);
   if (blocks > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "tdist_decode_combine: grid too large");
-  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, prm);
+  auto kern = head_dim_v <= 128 ? decode_combine_kernel<2> : head_dim_v <= 256 ? decode_combine_kernel<4> : decode_combine_kernel<8>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, prm);
   return launch_status("tdist_decode_combine");
 }
 
