@@ -399,7 +399,23 @@ def bench_c5(dev, steps, warmup):
     r["split_then_combine_us"] = round(both_s * 1e6, 2)
     r["fused_split_and_combine_us"] = round(fused_s * 1e6, 2)
     r["inter_rank_combine_us"] = round(rank_s * 1e6, 2)
-    return r
+    # the reference layer's defaults (layers/nvidia/sp_flash_decode_layer.py:45,61): 32 splits, and pages of one token
+    # (the same caches seen as 1 048 576 pages of one token each, every token of a sequence at a random place: 2 KB
+    # gather granules per cache and a 4.19 MB block table)
+    S32 = 32
+    out32 = torch.empty((B, Hq, S32, D), dtype=torch.float32, device=dev)
+    lse32 = torch.empty((B, Hq, S32), dtype=torch.float32, device=dev)
+    s32_s = time_launches(lambda: _split_kv(q, k, v, lens, table, scale, 0.0, S32, out32, lse32), steps, warmup)
+    r32 = roof("hbm", kv_bytes + q.numel() * 2 + table.numel() * 4 + out32.numel() * 4 + lse32.numel() * 4, s32_s, "hbm")
+    r32["workload"] = "C5 with 32 splits (page 16)"
+    k1p, v1p = k.view(num_pages * page, 1, Hkv, D), v.view(num_pages * page, 1, Hkv, D)
+    table1 = torch.randperm(B * L, generator=torch.Generator().manual_seed(7)).view(B, L).int().to(dev)
+    p1_s = time_launches(lambda: _split_kv(q, k1p, v1p, lens, table1, scale, 0.0, S, out_split, lse_split), steps, warmup)
+    rp1 = roof("hbm", kv_bytes + q.numel() * 2 + table1.numel() * 4 + out_split.numel() * 4 + lse_split.numel() * 4, p1_s, "hbm")
+    rp1["workload"] = "C5 with pages of one token (16 splits), tokens at random places"
+    p1s32_s = time_launches(lambda: _split_kv(q, k1p, v1p, lens, table1, scale, 0.0, S32, out32, lse32), steps, warmup)
+    rp1["with_32_splits_us"] = round(p1s32_s * 1e6, 2)
+    return r, r32, rp1
 
 
 def bench_group_gemm(dev, steps, warmup):
@@ -563,8 +579,8 @@ def main():
         kernels["c4_moe_dispatch_fp8"], kernels["c4_moe_combine"] = d, c
         log("c4", d, c)
     if "c5" in want:
-        kernels["c5_decode_split_kv_bf16"] = bench_c5(dev, args.steps, args.warmup)
-        log("c5", kernels["c5_decode_split_kv_bf16"])
+        kernels["c5_decode_split_kv_bf16"], kernels["c5_decode_32splits"], kernels["c5_decode_page1"] = bench_c5(dev, args.steps, args.warmup)
+        log("c5", kernels["c5_decode_split_kv_bf16"], kernels["c5_decode_32splits"], kernels["c5_decode_page1"])
     if "moe_gemm" in want:
         kernels["ag_group_gemm_bf16_mixtral_8x7b_tp8"] = bench_group_gemm(dev, args.steps, args.warmup)
         log("moe_gemm", kernels["ag_group_gemm_bf16_mixtral_8x7b_tp8"])

@@ -8,6 +8,8 @@
  *   - pointers are DEVICE pointers unless the parameter name ends in _host;
  *   - `stream` is a hipStream_t passed as void* (NULL = the legacy default stream);
  *   - no entry point allocates or frees memory; scratch comes from the caller (see *_workspace_bytes);
+ *   - nothing is read from the environment; the only process-wide state is the cached device properties
+ *     (tdist_init) and the test switches of tdist_debug_set, which default to "the library decides";
  *   - leading dimensions (lda, ldb, ...) are in ELEMENTS, sizes in elements unless named *_bytes;
  *   - launches are asynchronous on `stream`; a non-zero return means nothing was launched.
  *
@@ -46,10 +48,35 @@ typedef enum tdist_dtype {
 int tdist_version(void);
 const char* tdist_last_error_string(void);
 /* Caches properties of the current device (CU count, XCD count) and the device address of the library's built-in
- * scratch (tdist_moe_scatter_index_static). Optional: every entry point does its part lazily. Returns
- * TDIST_ERR_DEVICE when the current device is not gfx950. */
+ * scratch (tdist_moe_scatter_index_static), and checks once, with a small grid whose workgroups read their XCD id from
+ * the hardware (one launch on the NULL stream and a synchronous 4 KiB copy back; no allocation), that workgroup i
+ * of a grid runs on XCD i mod 8. Optional: every entry point does the first two lazily. Without the call, or when the
+ * check does not hold (another partition mode, a CU mask), the GEMMs' split-round exchange (sk_workspace) goes through
+ * device-coherent stores instead of staying within one XCD's L2: slower by a few microseconds, never wrong.
+ * Returns TDIST_ERR_DEVICE when the current device is not gfx950. */
 int tdist_init(void);
 int tdist_num_cus(void);
+
+/* Test and measurement switches. Process-wide, read by the host side of the entry points at call time; every key
+ * starts at -1 = "the library decides" and a negative value puts it back. They select among kernels that all give
+ * the documented results; a serving process has no reason to touch them. No counterpart in the reference (its
+ * kernels take their variants from autotune configs, e.g. kernels/amd/all_gather_gemm.py:103-137). */
+typedef enum tdist_debug_key {
+  TDIST_DEBUG_GEMM_TILE = 0,       /* 0..4: force the 256x256, 256x128, 128x128, 128x192 or 128x256 tile where the
+                                      call's row blocks and K admit it */
+  TDIST_DEBUG_GEMM_SPLIT_K = 1,    /* 0: whole tiles only; 1: split a last round wherever the workspace allows */
+  TDIST_DEBUG_GEMM_SK_COHERENT = 2,/* 1: the split-round exchange always through device-coherent stores */
+  TDIST_DEBUG_GEMM_SCHEDULE = 3,   /* 0: tiles in the static chunk-major order; 1: in arrival order (the default
+                                      for gated calls, see tdist_gemm_chunk_gated_bf16) */
+  TDIST_DEBUG_DECODE_WAVE_HEADS = 4,      /* 0: never the kv-head-per-wave form; 2: wherever the heads allow it, whatever
+                                             the lengths; 4: likewise, its 4-wave workgroups only */
+  TDIST_DEBUG_DECODE_SPLITS_PER_TEAM = 5, /* >= 1: splits one workgroup of that form streams through */
+  TDIST_DEBUG_MOE_INDEX_FORM = 6,  /* 2: one launch whose blocks exchange histograms (needs every block resident at
+                                      once: see tdist_moe_scatter_index); 3: always three launches */
+  TDIST_DEBUG_NUM_KEYS = 8
+} tdist_debug_key;
+int tdist_debug_set(int key, int value);
+int tdist_debug_get(int key);
 
 /* ---------------------------------------------------------------------------------------------
  * (a) chunk-gated tile GEMM — the AG-GEMM consumer.
@@ -127,12 +154,16 @@ int tdist_producer_push_chunk(void* dst, const void* src, int64_t nbytes, int32_
  * (test hook for the consumer's bounded wait). stamp + ns_per_chunk > 0: the pace of one link per peer: chunk c of
  * every peer is copied from c*ns_per_chunk after the stamp (tdist_producer_mark) on and its flag is released no
  * earlier than (c+1)*ns_per_chunk after it, when a link of that rate would have delivered the chunk's last byte; the
- * total must stay within 100 ms. The kernel needs 32 registers per lane and no LDS, so its waves fit on a SIMD beside a
- * resident wave of the consumer GEMM; nothing in it waits for another workgroup. */
+ * total must stay within 100 ms. max_delay_ns > 0: race provocation, as the reference's producer sleeps with probability
+ * 0.7 when run "for correctness" (kernels/nvidia/allgather.py:72-77,118-121): about 7 of 10 (peer, chunk) pairs,
+ * chosen by a hash of delay_seed and the chunk, are held back by a pseudo-random time below max_delay_ns before they
+ * are copied (max_delay_ns x chunks per rank within 100 ms). The kernel is held to 24 registers per lane and uses no
+ * LDS, so its waves fit on a SIMD beside a resident wave of the consumer GEMM; nothing in it waits for another
+ * workgroup, and every wait in it is bounded by the device's wall clock. */
 int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int world_size, int rank,
                               int64_t rank_bytes, int64_t chunk_bytes, int32_t* flags, int flag_value,
                               int32_t* counters, const int32_t* held, const uint64_t* stamp, int64_t ns_per_chunk,
-                              int workgroups_per_peer, void* stream);
+                              uint32_t delay_seed, int64_t max_delay_ns, int workgroups_per_peer, void* stream);
 
 /* Link pacing for the one-GPU producer (no counterpart in the reference, whose chunks arrive over xGMI at the
  * link's rate: ~153 GB/s per peer). tdist_producer_mark stores the device's constant-rate wall clock into *stamp
@@ -220,7 +251,14 @@ int tdist_moe_splits_cumsum(const int32_t* ids, int64_t n_ids, int num_experts, 
  *                    (argsort(stable).argsort(), calc_scatter_index_stable, test_all_to_all.py:95-96)
  *   gather_idx[p]  = token (i / topk) of the entry sorted to position p (calc_gather_index, :49-92)
  *   topk_idx[p]    = i % topk of that entry (may be NULL)
- * all int32; splits may be NULL. */
+ * all int32; splits may be NULL.
+ * Up to 65536 ids: one launch in which every workgroup counts all ids itself; beyond: three launches. No workgroup of
+ * either form waits for another one, so both are safe beside kernels that hold compute units (a persistent GEMM
+ * spinning on flags). A third form (one launch, workgroups of 2048 ids that exchange histograms and wait for each
+ * other) runs only when tdist_debug_set(TDIST_DEBUG_MOE_INDEX_FORM, 2) asks for it: its wait ends only if all its
+ * workgroups are resident at once, which is the caller's to guarantee. If that bounded wait expires, the workgroup
+ * writes no index rows, cumsum[0] reads -1 unless workgroup 0 got through later, and word 2 of the workspace's
+ * control words is set to 1 and stays so until the caller clears it. */
 int tdist_moe_scatter_index(const int32_t* ids, int64_t n_ids, int topk, int num_experts, int32_t* splits,
                             int32_t* cumsum, int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx,
                             void* workspace, int64_t workspace_bytes, void* stream);
@@ -381,7 +419,12 @@ int tdist_group_gemm_gated_fp8e4m3(const void* A, int64_t lda, const void* A_loc
  * launches that share one must be ordered (same stream, or events). A workspace that is misaligned or smaller than
  * the header plus one 128 x 128 tile is rejected (TDIST_ERR_WORKSPACE); one too small for the call's tiles and grid
  * is left unused.
- * TDIST_GEMM_SPLIT_K=0 in the environment turns the split off, =1 takes it wherever a last round can be split. */
+ * Where the s workgroups of a tile are expected on one XCD (s divides the workgroups per XCD) and tdist_init has
+ * seen the dispatch order hold, the partials stay in that XCD's L2 (plain stores, first-level invalidate on the
+ * reading side). Every piece also publishes the XCD it ran on, and a reader that finds a partner on another XCD
+ * reports {TDIST_ERR_DEVICE, -1 - workgroup} through status and does not store the tile, rather than sum stale slots.
+ * tdist_debug_set(TDIST_DEBUG_GEMM_SPLIT_K, 0) turns the split off, 1 takes it wherever a last round can be split;
+ * TDIST_DEBUG_GEMM_SK_COHERENT = 1 keeps the exchange device-coherent. */
 int64_t tdist_gemm_split_k_workspace_bytes(void);
 
 /* ---------------------------------------------------------------------------------------------

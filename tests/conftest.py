@@ -26,3 +26,25 @@ def cuda():
 def announce(msg):
     """Print and flush the case about to touch the GPU, so that a fault names its test."""
     print("[gpu-case] " + msg, flush=True)
+
+
+@pytest.fixture
+def switches():
+    """``switches(key, value)`` sets one of the library's test and measurement switches (tdist_debug_set; None = the
+    library decides again); all of them are put back when the test ends, after the GPU has drained."""
+    from triton_dist import _lib
+    lib = _lib.load()
+    saved = {}
+
+    def set_switch(key, value):
+        saved.setdefault(key, lib.tdist_debug_get(key))
+        _lib.check(lib.tdist_debug_set(key, -1 if value is None else int(value)))
+
+    yield set_switch
+    try:
+        import torch
+        if torch.cuda.is_available():
+            torch.cuda.synchronize()
+    finally:
+        for key, old in saved.items():
+            lib.tdist_debug_set(key, old)

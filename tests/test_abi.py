@@ -99,6 +99,34 @@ def test_null_pointers_are_rejected_without_touching_the_gpu():
     assert lib.tdist_moe_workspace_bytes(32768, 256) == (128 + 1) * 256 * 4 + 256
 
 
+def test_debug_switches_default_to_automatic_and_ignore_the_environment(monkeypatch):
+    """The library's test and measurement switches: -1 (the library decides) until tdist_debug_set says otherwise,
+    a negative value puts a key back, unknown keys are rejected, and nothing is read from the environment."""
+    lib = _lib.load()
+    for name in ("TDIST_GEMM_TILE", "TDIST_GEMM_SPLIT_K", "TDIST_DECODE_WAVE_HEADS", "TDIST_MOE_INDEX_LAUNCHES"):
+        monkeypatch.setenv(name, "2")
+    keys = [_lib.TDIST_DEBUG_GEMM_TILE, _lib.TDIST_DEBUG_GEMM_SPLIT_K, _lib.TDIST_DEBUG_GEMM_SK_COHERENT,
+            _lib.TDIST_DEBUG_GEMM_SCHEDULE, _lib.TDIST_DEBUG_DECODE_WAVE_HEADS, _lib.TDIST_DEBUG_DECODE_SPLITS_PER_TEAM,
+            _lib.TDIST_DEBUG_MOE_INDEX_FORM]
+    assert [lib.tdist_debug_get(k) for k in keys] == [-1] * len(keys)
+    with _lib.debug_switch(_lib.TDIST_DEBUG_GEMM_TILE, 3):
+        assert lib.tdist_debug_get(_lib.TDIST_DEBUG_GEMM_TILE) == 3
+        assert lib.tdist_debug_get(_lib.TDIST_DEBUG_GEMM_SPLIT_K) == -1
+    assert lib.tdist_debug_get(_lib.TDIST_DEBUG_GEMM_TILE) == -1
+    assert lib.tdist_debug_set(_lib.TDIST_DEBUG_GEMM_TILE, -7) == 0 and lib.tdist_debug_get(_lib.TDIST_DEBUG_GEMM_TILE) == -1
+    assert lib.tdist_debug_set(99, 1) == _lib.TDIST_ERR_INVALID and lib.tdist_debug_set(-1, 1) == _lib.TDIST_ERR_INVALID
+    assert lib.tdist_debug_get(99) == -1
+    # the header's key values are the binding's
+    text = open(HEADER).read()
+    for name in ("GEMM_TILE", "GEMM_SPLIT_K", "GEMM_SK_COHERENT", "GEMM_SCHEDULE", "DECODE_WAVE_HEADS",
+                 "DECODE_SPLITS_PER_TEAM", "MOE_INDEX_FORM"):
+        m = re.search(r"TDIST_DEBUG_%s\s*=\s*(\d+)" % name, text)
+        assert m and int(m.group(1)) == getattr(_lib, "TDIST_DEBUG_" + name), name
+    import glob
+    for src in glob.glob(os.path.join(ROOT, "triton-distributed_amd", "csrc", "*")):
+        assert "getenv" not in open(src).read(), "%s reads the environment" % src
+
+
 def test_ops_fail_loudly_without_gpu():
     import torch
     if torch.cuda.is_available():

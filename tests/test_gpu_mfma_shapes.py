@@ -3,7 +3,6 @@
 / 32x32x64) with accumulators the compiler places. Each form is held against the exact result on integer-valued inputs (every partial sum is an
 integer that fp32 holds) over the K-loop's corner cases, and on random inputs to max relative error <= 1e-2 of fp32 and
 to each other within the rounding of the output."""
-import os
 
 import pytest
 import torch
@@ -14,19 +13,17 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture
-def tile_env():
-    old = os.environ.get("TDIST_GEMM_TILE")
+def tile_env(switches):
+    """Puts the forced tile back to "the library decides" when the test ends."""
+    from triton_dist import _lib
+    switches(_lib.TDIST_DEBUG_GEMM_TILE, None)
     yield
-    torch.cuda.synchronize()
-    if old is None:
-        os.environ.pop("TDIST_GEMM_TILE", None)
-    else:
-        os.environ["TDIST_GEMM_TILE"] = old
 
 
 def run_tile(cuda, a, b, out_dtype, tile, **kw):
+    from triton_dist import _lib
     from triton_dist.kernels.amd import gated_gemm
-    os.environ["TDIST_GEMM_TILE"] = str(tile)
+    _lib.check(_lib.load().tdist_debug_set(_lib.TDIST_DEBUG_GEMM_TILE, tile))
     c = torch.full((a.shape[0], b.shape[0]), float("nan"), dtype=out_dtype, device=cuda)
     status = torch.zeros(2, dtype=torch.int32, device=cuda)
     gated_gemm(a, None, 0, b, c, None, 0, 0, 1, status=status, **kw)

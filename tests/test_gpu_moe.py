@@ -52,17 +52,18 @@ def test_preprocess_repeated_ids_and_skewed_load(cuda):
 
 
 @pytest.mark.parametrize("launches", ["one", "one with rendezvous", "three"])
-def test_preprocess_paths_sizes_in_turn_and_context_buffers(cuda, monkeypatch, launches):
+def test_preprocess_paths_sizes_in_turn_and_context_buffers(cuda, switches, launches):
     """The one-launch index build in both of its forms (up to 32 blocks every block counts all the ids itself; beyond,
     or forced here through the library's switch, the blocks exchange their histograms) and the three-launch form it
     falls back to (forced likewise; taken by itself beyond one block per compute unit, as the 560 000 ids below do):
     calls of different sizes in turn on the same cached scratch, id counts that are no multiple of four, ids outside
     [0, G) (dropped: scatter index -1), and the context-owned result tensors, two sets used in turn."""
     from triton_dist.kernels.amd import create_all_to_all_context, moe_dispatch_preprocess
+    from triton_dist import _lib
     if launches == "three":
-        monkeypatch.setenv("TDIST_MOE_INDEX_LAUNCHES", "3")
+        switches(_lib.TDIST_DEBUG_MOE_INDEX_FORM, 3)
     if launches == "one with rendezvous":
-        monkeypatch.setenv("TDIST_MOE_INDEX_RENDEZVOUS", "1")
+        switches(_lib.TDIST_DEBUG_MOE_INDEX_FORM, 2)
     announce("moe preprocess paths (%s launch)" % launches)
     g = torch.Generator().manual_seed(9)
     for T, topk, G in [(4096, 8, 256), (300, 4, 2048), (70000, 8, 64), (1000, 8, 256), (5, 3, 4096), (333, 3, 100),
@@ -101,6 +102,19 @@ def test_preprocess_paths_sizes_in_turn_and_context_buffers(cuda, monkeypatch, l
         assert torch.equal(a.cpu(), b)
     out_c = moe_dispatch_preprocess(ids_a.to(cuda), 16, ctx=ctx)
     assert out_c[2].data_ptr() == out_a[2].data_ptr() and out_c[2].data_ptr() != out_b[2].data_ptr()
+    # int64 ids (what torch.topk returns) on a shape the context has seen: converted into the context's own int32
+    # staging tensor, the same two result sets in turn, nothing allocated
+    ids64 = ids_b.long().to(cuda)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    out_d = moe_dispatch_preprocess(ids64, 16, ctx=ctx)
+    out_e = moe_dispatch_preprocess(ids64.t().contiguous().t(), 16, ctx=ctx)    # and a non-contiguous view
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert out_d[2].data_ptr() == out_b[2].data_ptr() and out_e[2].data_ptr() == out_a[2].data_ptr()
+    for got in (out_d, out_e):
+        for a, b in zip(got, golden.moe_preprocess(ids_b, 16)[:4]):
+            assert torch.equal(a.cpu(), b)
 
 
 def test_splits_cumsum_entry_point(cuda):

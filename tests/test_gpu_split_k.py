@@ -3,7 +3,6 @@ K into 2, 4 or 8 equal pieces, one per workgroup; the pieces go through the call
 up and stores its share of the tile) against the oracle and against the whole-tile form.
 Bar: exact on integer-valued inputs (every partial sum is an integer that fp32 holds), max relative error <= 1e-2 on
 random inputs; a piece that never arrives ends in TDIST_ERR_TIMEOUT, not in a hang."""
-import os
 
 import pytest
 import torch
@@ -15,18 +14,12 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture
-def split_k(cuda):
+def split_k(cuda, switches):
     """A workspace of this test's own, with the split forced wherever it is possible (whatever the cost estimate says)."""
     from triton_dist import _lib
     ws = _lib.new_split_k_workspace()
-    old = os.environ.get("TDIST_GEMM_SPLIT_K")
-    os.environ["TDIST_GEMM_SPLIT_K"] = "1"
+    switches(_lib.TDIST_DEBUG_GEMM_SPLIT_K, 1)
     yield ws
-    torch.cuda.synchronize()
-    if old is None:
-        del os.environ["TDIST_GEMM_SPLIT_K"]
-    else:
-        os.environ["TDIST_GEMM_SPLIT_K"] = old
 
 
 def ints(shape, g, dtype, lo=-2, hi=3):
@@ -52,6 +45,31 @@ def test_exact_on_integer_inputs(cuda, split_k, dtype, M, N, K, wgs):
     assert status.tolist() == [0, 0]
     ref = (a.float() @ b.float().T).to(out_dtype)
     assert torch.equal(c.cpu(), ref)
+
+
+def test_exchange_within_an_xcd_and_through_memory_agree(cuda, split_k, switches):
+    """The pieces of a tile exchange their partial sums through the L2 of the XCD they share (only where tdist_init has
+    seen workgroup i land on XCD i mod 8: on this device it must have) or through device-coherent stores (forced here
+    through the library's switch): the same bits either way, exact on integer-valued inputs, and no piece reports a
+    partner on another XCD."""
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import gated_gemm
+    M, N, K = 512, 640, 2048          # 6 tiles of 256 x 256 on 256 workgroups: eight pieces each, all on one XCD
+    announce("split-k exchange paths %dx%dx%d" % (M, N, K))
+    g = torch.Generator().manual_seed(77)
+    a, b = ints((M, K), g, torch.bfloat16), ints((N, K), g, torch.bfloat16)
+    ref = (a.float() @ b.float().T).to(torch.bfloat16)
+    outs = []
+    for coherent in (0, 1, 0):
+        switches(_lib.TDIST_DEBUG_GEMM_SK_COHERENT, coherent)
+        c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+        status = torch.zeros(2, dtype=torch.int32, device=cuda)
+        gated_gemm(a.to(cuda), None, 0, b.to(cuda), c, None, 0, 0, 1, status=status, sk_workspace=split_k)
+        torch.cuda.synchronize()
+        assert status.tolist() == [0, 0], "a piece found its partner on another XCD (or timed out): %s" % status.tolist()
+        assert torch.equal(c.cpu(), ref)
+        outs.append(c)
+    assert int(split_k.view(torch.int32)[0]) != 0   # (the split form really ran: the workspace's epoch word has moved)
 
 
 def test_random_inputs_match_the_whole_tile_form(cuda, split_k):

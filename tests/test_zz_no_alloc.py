@@ -33,9 +33,9 @@ def run_both(cuda, ids, G):
 
 
 @pytest.mark.parametrize("launches", ["one", "three"])
-def test_static_scratch_entry_matches_the_workspace_entry(cuda, monkeypatch, launches):
+def test_static_scratch_entry_matches_the_workspace_entry(cuda, switches, launches):
     if launches == "three":
-        monkeypatch.setenv("TDIST_MOE_INDEX_LAUNCHES", "3")
+        switches(_lib.TDIST_DEBUG_MOE_INDEX_FORM, 3)
     g = torch.Generator().manual_seed(21)
     # BASELINE's MoE config first, then smaller ones: the second call finds the first call's leftovers in the scratch
     for T, topk, G in [(4096, 8, 256), (500, 8, 256), (37, 2, 16), (4096, 8, 256)]:

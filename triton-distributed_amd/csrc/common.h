@@ -14,7 +14,11 @@ namespace tdist {
 struct DeviceInfo {
   int ok;        // 1 once probed successfully
   int num_cus;   // compute units of the current device
-  int num_xcds;  // accelerator complex dies; workgroup i is dispatched to XCD i % num_xcds
+  int num_xcds;  // accelerator complex dies; workgroup i is expected on XCD i % num_xcds (see xcd_round_robin)
+  // 1 once tdist_init has SEEN a one-workgroup-per-CU grid land that way on this device (every workgroup read its
+  // XCD id from the hardware register and the host compared); 0 = not checked or not so. Only with 1 may a kernel
+  // let workgroups that it expects on one XCD exchange data through that XCD's L2 alone.
+  int xcd_round_robin;
 };
 
 // Records a printf-style message for tdist_last_error_string() and returns `code`.
@@ -22,6 +26,11 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 // hipGetLastError() → TDIST_OK or TDIST_ERR_LAUNCH (message recorded).
 int launch_status(const char* what);
 const DeviceInfo& device_info();
+// The dispatch-order check behind DeviceInfo::xcd_round_robin; run by tdist_init (it allocates and synchronises, so it
+// is never run lazily from an entry point).
+int probe_xcd_round_robin();
+// Test and measurement switches (tdist_debug_set): the value of `key`, -1 = the library decides.
+int debug_get(int key);
 // Looks up, once per device and with that device current, the device address of the built-in scratch of
 // tdist_moe_scatter_index_static (moe.hip). Called by tdist_init and, lazily, by that entry point.
 int moe_static_scratch_init();
@@ -110,6 +119,13 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Id of the accelerator complex die (XCD) this wave runs on, from the hardware register (bits 3:0 of XCC_ID).
+__device__ __forceinline__ int xcc_id() {
+  int v;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID, 0, 4)" : "=s"(v));
+  return v;
 }
 
 __device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0)); }

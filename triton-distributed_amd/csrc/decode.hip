@@ -994,10 +994,10 @@ static int run_decode(const DecodeCall& c, bool fuse) {
   // form, whose small workgroups fill a small grid's CUs better) and the cache is large enough for a tenth of the
   // kernel's time to outweigh a second launch: the form's time goes with the longest sequence, so the other form is
   // launched behind it and the kernels decide by the sequence lengths which of the two runs (decode_lens_even).
-  // TDIST_DECODE_WAVE_HEADS=0 never takes this form; 2 takes it wherever the heads allow it, alone and whatever the
-  // lengths; 4 likewise but only its 4-wave workgroups.
-  const char* wh_env = getenv("TDIST_DECODE_WAVE_HEADS");
-  const int wh_mode = wh_env ? atoi(wh_env) : 1;
+  // tdist_debug_set(TDIST_DEBUG_DECODE_WAVE_HEADS, 0) never takes this form; 2 takes it wherever the heads allow it,
+  // alone and whatever the lengths; 4 likewise but only its 4-wave workgroups.
+  const int wh_dbg = debug_get(TDIST_DEBUG_DECODE_WAVE_HEADS);
+  const int wh_mode = wh_dbg >= 0 ? wh_dbg : 1;
   auto wave_heads = [&](int nw) {
     if (wh_mode == 0 || head_blocks != 1 || c.kv_heads % nw != 0 || (wh_mode == 4 && nw != 4)) return false;
     if (!aligned16(c.out_split)) return false;   // its partial results go out as 16-byte vectors
@@ -1013,8 +1013,8 @@ static int run_decode(const DecodeCall& c, bool fuse) {
       const int64_t cost = ((teams + cus - 1) / cus) * w;
       if (w == 1 || cost <= best_cost) best_cost = cost, best_w = w;
     }
-    const char* spt = getenv("TDIST_DECODE_SPLITS_PER_TEAM");
-    if (spt && atoi(spt) >= 1) best_w = std::min(atoi(spt), max_w);
+    const int spt = debug_get(TDIST_DEBUG_DECODE_SPLITS_PER_TEAM);
+    if (spt >= 1) best_w = std::min(spt, max_w);
     prm.splits_per_team = best_w;
     if (wh_mode > 1) return true;
     // the most that the block table lets the call read: below 256 MB (40 us) the form's gain is less than a launch

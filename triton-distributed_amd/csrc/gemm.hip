@@ -84,6 +84,8 @@ struct GemmParams {
   int32_t* sk_ctrl;
   float* sk_partials;
   int sk_mode;
+  int sk_l2_local;   // 1: workgroup i has been seen to run on XCD i mod num_xcds (tdist_init), so pieces that the
+                     // schedule puts on one XCD may exchange through that XCD's L2 alone
 };
 
 // Workspace header, in int32 words
@@ -95,6 +97,8 @@ constexpr int kSkAcksOff = 2048;         // [kSkMaxWorkgroups] readers that are 
 constexpr int kSkHeaderWords = 3072;
 constexpr int64_t kSkHeaderBytes = (int64_t)kSkHeaderWords * 4;
 constexpr int kSkTagStride = 16;         // tags per launch (rounds that may be split)
+// a flag word is the tag (low 27 bits) with the XCD the piece ran on above it
+constexpr int kSkTagBits = 27, kSkTagMask = (1 << kSkTagBits) - 1, kSkTagWrap = kSkTagMask - 0x10000;
 static_assert(kSkHeaderBytes % 256 == 0, "the partial slots start 256-byte aligned");
 
 // Operand fragment of one lane: K bytes [0, kLaneBytes) of one row; chunk0 / chunk1 are LDS addresses of its
@@ -387,7 +391,10 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   int32_t* const sk_acks = p.sk_ctrl + kSkAcksOff;
   // the workgroups of one XCD hold a contiguous range of positions (see wg_pos): pieces of a tile share an XCD when
   // the pieces per tile (2, 4 or 8) divide the workgroups per XCD
-  const bool sk_xcd_local = p.num_xcds > 1 && G % p.num_xcds == 0 && (G / p.num_xcds) % kSkMaxSplit == 0;
+  // (only where that dispatch order has been checked on this device; each piece also publishes the XCD it really ran
+  // on and the readers compare, so a launch that lands differently reports it instead of summing stale slots)
+  const bool sk_xcd_local = p.sk_l2_local != 0 && p.num_xcds > 1 && G % p.num_xcds == 0 && (G / p.num_xcds) % kSkMaxSplit == 0;
+  const int my_xcc = p.sk_mode != 0 ? __builtin_amdgcn_readfirstlane(xcc_id()) : 0;
   int tag_base = 0;   // tags of this launch are tag_base + 1 + round
   int sk_need = 0;    // value of this workgroup's ack word once every reader of its last partial is done
   if (p.sk_mode != 0) {
@@ -1088,30 +1095,35 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         });
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (threadIdx.x == 0) __hip_atomic_store(sk_flags + wg_pos, sk_tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0)
+          __hip_atomic_store(sk_flags + wg_pos, sk_tag | (my_xcc << kSkTagBits), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
 
       // (3) all pieces of the tile: thread i waits for the flag of piece i. (The full limit even after an error
       // elsewhere: these pieces are being computed, not awaited from outside; if a workgroup gave its piece up at a
       // chunk flag, the wait runs out and the tile is not stored.)
       if (threadIdx.x < 64) {
-        int ok = 1;
+        int ok = 1, same_xcd = 1;
         if ((int)threadIdx.x < sk_s) {
           ok = 0;
           for (int it = 0; it < p.spin_limit; ++it) {
-            if (__hip_atomic_load(sk_flags + w0 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == sk_tag) {
+            const int f = __hip_atomic_load(sk_flags + w0 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((f & kSkTagMask) == sk_tag) {
               ok = 1;
+              same_xcd = (f >> kSkTagBits) == my_xcc;
               break;
             }
             __builtin_amdgcn_s_sleep(2);
           }
         }
         const int all_ok = __ballot(ok != 0) == ~0ull;
+        // partials that stayed in another XCD's L2 cannot be read from here
+        const int reach_ok = !sk_xcd_local || __ballot(same_xcd != 0) == ~0ull;
         if (threadIdx.x == 0) {
-          if (!(all_ok && slot_ok) && p.status != nullptr) {
-            if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = -1 - wg_pos;
+          if (!(all_ok && slot_ok && reach_ok) && p.status != nullptr) {
+            if (atomicCAS(p.status, 0, all_ok && slot_ok ? TDIST_ERR_DEVICE : TDIST_ERR_TIMEOUT) == 0) p.status[1] = -1 - wg_pos;
           }
-          *s_gate = all_ok && slot_ok;
+          *s_gate = all_ok && slot_ok && reach_ok;
         }
       }
       __syncthreads();
@@ -1330,7 +1342,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     if (__hip_atomic_fetch_add(done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == G - 1) {
       __hip_atomic_store(done, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       int next = tag_base + kSkTagStride;
-      if (next > 0x3fff0000) {
+      if (next > kSkTagWrap) {
         // tags start over: no word may still hold a value that a tag will take again
         next = 0;
         for (int i = 0; i < kSkMaxWorkgroups; ++i) __hip_atomic_store(sk_flags + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1390,8 +1402,8 @@ static int launch_gemm_cfg(const GemmParams& prm, int grid, hipStream_t stream, 
 
 // 0 = off, 1 = on wherever the workspace allows, -1 = by the cost estimate
 static int sk_env() {
-  if (const char* v = getenv("TDIST_GEMM_SPLIT_K")) return atoi(v) != 0 ? 1 : 0;
-  return -1;
+  const int v = debug_get(TDIST_DEBUG_GEMM_SPLIT_K);
+  return v < 0 ? -1 : (v != 0 ? 1 : 0);
 }
 
 static bool sk_workspace_fits(const void* ws, int64_t bytes, int workgroups, int bm, int bn) {
@@ -1411,6 +1423,7 @@ static void sk_attach(GemmParams& p, void* ws, int mode) {
   p.sk_ctrl = (int32_t*)ws;
   p.sk_partials = (float*)((unsigned char*)ws + kSkHeaderBytes);
   p.sk_mode = mode;
+  p.sk_l2_local = device_info().xcd_round_robin == 1 && debug_get(TDIST_DEBUG_GEMM_SK_COHERENT) != 1;
 }
 
 // cost of handing a tile's pieces through the workspace, in K tiles of that tile's work (one compute unit writes the
@@ -1488,10 +1501,10 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       if (cost_sk < 0.95 * best || (sk_mode == 1 && (!use_sk || cost_sk < best))) best = cost_sk, pick = t, use_sk = true;
     }
   }
-  // TDIST_GEMM_TILE forces a tile (test and measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128, 3 = 128x192,
+  // TDIST_DEBUG_GEMM_TILE forces a tile (test and measurement aid): 0 = 256x256, 1 = 256x128, 2 = 128x128, 3 = 128x192,
   // 4 = 128x256; a tile that the call's row blocks or K do not admit is not taken.
-  if (const char* v = getenv("TDIST_GEMM_TILE")) {
-    const int t = atoi(v);
+  {
+    const int t = debug_get(TDIST_DEBUG_GEMM_TILE);
     if (t >= 0 && t < kNumChoices && admissible(t)) {
       pick = t;
       // (the split is re-derived for the forced tile)
@@ -1538,6 +1551,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   p.sk_ctrl = nullptr;
   p.sk_partials = nullptr;
   p.sk_mode = 0;
+  p.sk_l2_local = 0;
   p.k_tail_bytes = k_tail_bytes;
 
   if (c.scatter_bufs) {
@@ -1736,6 +1750,7 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   p.sk_ctrl = nullptr;
   p.sk_partials = nullptr;
   p.sk_mode = 0;
+  p.sk_l2_local = 0;
   p.gate_rows = p.m_per_chunk;
   p.k_tail_bytes = 0;
 

@@ -4,6 +4,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "common.h"
@@ -26,8 +27,22 @@ int launch_status(const char* what) {
   return TDIST_OK;
 }
 
-static DeviceInfo g_info = {0, 0, 0};
+static DeviceInfo g_info = {0, 0, 0, 0};
 static std::mutex g_info_mu;
+
+// Test and measurement switches: -1 = the library decides. Set through tdist_debug_set only (nothing is read from the
+// environment), read by the host side of the entry points at call time.
+static std::atomic<int> g_debug[TDIST_DEBUG_NUM_KEYS];
+static std::once_flag g_debug_once;
+static void debug_init() {
+  std::call_once(g_debug_once, [] {
+    for (auto& v : g_debug) v.store(-1, std::memory_order_relaxed);
+  });
+}
+int debug_get(int key) {
+  debug_init();
+  return key >= 0 && key < TDIST_DEBUG_NUM_KEYS ? g_debug[key].load(std::memory_order_relaxed) : -1;
+}
 
 const DeviceInfo& device_info() {
   std::lock_guard<std::mutex> lk(g_info_mu);
@@ -45,6 +60,41 @@ const DeviceInfo& device_info() {
     }
   }
   return g_info;
+}
+
+// Every workgroup of a grid writes down the XCD it runs on. The ids land in a small array of the library's own (one
+// copy per GPU; its device address comes from hipGetSymbolAddress), so the check allocates nothing.
+constexpr int kProbeMaxWorkgroups = 4096;
+static __device__ int32_t g_probe_ids[kProbeMaxWorkgroups];
+__global__ void xcd_probe_kernel(int32_t* out) {
+  if (threadIdx.x == 0) out[blockIdx.x] = xcc_id();
+}
+
+int probe_xcd_round_robin() {
+  const DeviceInfo& di = device_info();
+  if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "tdist_init: current device is not a gfx950 GPU");
+  {
+    std::lock_guard<std::mutex> lk(g_info_mu);
+    if (g_info.xcd_round_robin != 0) return TDIST_OK;   // checked before (1 = holds, -1 = does not)
+  }
+  if (di.num_xcds <= 1) return TDIST_OK;
+  // four workgroups per compute unit: workgroups i and j must share an XCD exactly when i = j (mod num_xcds)
+  const int n = 4 * di.num_cus < kProbeMaxWorkgroups ? 4 * di.num_cus : kProbeMaxWorkgroups;
+  int32_t* dev_ids = nullptr;
+  bool ok = hipGetSymbolAddress((void**)&dev_ids, HIP_SYMBOL(g_probe_ids)) == hipSuccess && dev_ids != nullptr;
+  int32_t* ids = new int32_t[n];
+  if (ok) {
+    hipLaunchKernelGGL(xcd_probe_kernel, dim3(n), dim3(256), 0, (hipStream_t) nullptr, dev_ids);
+    ok = hipMemcpy(ids, dev_ids, (size_t)n * 4, hipMemcpyDeviceToHost) == hipSuccess;
+  }
+  if (!ok) (void)hipGetLastError();   // not verified: the kernels keep to device-coherent exchanges
+  for (int i = 0; ok && i < n; ++i) ok = ids[i] == ids[i % di.num_xcds];
+  for (int i = 0; ok && i < di.num_xcds; ++i)
+    for (int j = 0; ok && j < i; ++j) ok = ids[i] != ids[j];
+  delete[] ids;
+  std::lock_guard<std::mutex> lk(g_info_mu);
+  g_info.xcd_round_robin = ok ? 1 : -1;
+  return TDIST_OK;
 }
 
 static int wall_clock_khz() {
@@ -109,9 +159,22 @@ struct PushParams {
   const int32_t* held;                   // optional [world * chunks_per_rank]: non-zero = never deliver (test hook)
   const unsigned long long* stamp;       // optional: wall-clock stamp of the op's start
   unsigned long long ticks_per_chunk;
+  unsigned long long max_delay_ticks;    // > 0: seeded random extra delay per (peer, chunk), see producer_delay_ticks
+  uint32_t delay_seed;
   long long chunk_bytes, rank_bytes;
   int world, rank, chunks_per_rank, flag_value;
 };
+
+// Race provocation (the reference sleeps in front of its producer with probability 0.7 when it runs "for
+// correctness", kernels/nvidia/allgather.py:72-77,118-121): chunk `chunk_pos` is held back by a pseudo-random time
+// below max_ticks in about 7 of 10 cases, by none otherwise. A function of (seed, chunk) alone, so every workgroup of a
+// peer's block row holds the chunk for the same time and a run can be repeated.
+__device__ __forceinline__ unsigned long long producer_delay_ticks(uint32_t seed, int chunk_pos, unsigned long long max_ticks) {
+  uint32_t h = seed ^ (0x9e3779b9u * (uint32_t)(chunk_pos + 1));
+  h ^= h >> 16; h *= 0x7feb352du; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+  if ((h & 1023u) >= 717u) return 0;
+  return (unsigned long long)(h >> 10) % max_ticks;
+}
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(24))) void producer_push_kernel(const PushParams p) {
   const int r = (p.rank + 1 + (int)blockIdx.y) % p.world;
@@ -136,6 +199,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(24))) void prod
           if (now - t0 >= due || now - begin >= due) break;
           __builtin_amdgcn_s_sleep(16);
         }
+      }
+      __syncthreads();
+    }
+    if (p.max_delay_ticks != 0) {
+      if (threadIdx.x == 0) {
+        const unsigned long long hold = producer_delay_ticks(p.delay_seed, chunk_pos, p.max_delay_ticks);
+        const unsigned long long from = wall_clock64();
+        while (wall_clock64() - from < hold) __builtin_amdgcn_s_sleep(16);   // (ends by itself: the clock only moves forward)
       }
       __syncthreads();
     }
@@ -194,10 +265,22 @@ const char* tdist_last_error_string(void) { return g_err; }
 int tdist_init(void) {
   const DeviceInfo& di = device_info();
   if (di.ok != 1) return fail(TDIST_ERR_DEVICE, "tdist_init: current device is not a gfx950 GPU");
+  // where the workgroups of a grid land (the split-round exchange of the GEMMs stays within one XCD's L2 only when
+  // this has been seen to hold on this device)
+  if (int rc = probe_xcd_round_robin()) return rc;
   // the address of the current device's copy of the library's built-in scratch (tdist_moe_scatter_index_static), so
   // that a caller that may not run set-up work later (under graph capture) finds it ready
   return moe_static_scratch_init();
 }
+
+int tdist_debug_set(int key, int value) {
+  if (key < 0 || key >= TDIST_DEBUG_NUM_KEYS) return fail(TDIST_ERR_INVALID, "tdist_debug_set: key %d outside [0, %d)", key, TDIST_DEBUG_NUM_KEYS);
+  debug_init();
+  g_debug[key].store(value < 0 ? -1 : value, std::memory_order_relaxed);
+  return TDIST_OK;
+}
+
+int tdist_debug_get(int key) { return debug_get(key); }
 
 int tdist_num_cus(void) {
   const DeviceInfo& di = device_info();
@@ -260,7 +343,7 @@ int tdist_producer_wait_until(const uint64_t* stamp, int64_t offset_ns, void* st
 int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int world_size, int rank,
                               int64_t rank_bytes, int64_t chunk_bytes, int32_t* flags, int flag_value,
                               int32_t* counters, const int32_t* held, const uint64_t* stamp, int64_t ns_per_chunk,
-                              int workgroups_per_peer, void* stream) {
+                              uint32_t delay_seed, int64_t max_delay_ns, int workgroups_per_peer, void* stream) {
   const char* who = "tdist_producer_push_peers";
   if (!workspace || !peer_src || !flags || !counters) return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
   if (world_size < 1 || rank < 0 || rank >= world_size) return fail(TDIST_ERR_INVALID, "%s: rank %d / world_size %d", who, rank, world_size);
@@ -289,6 +372,15 @@ int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int 
     if (khz <= 0) return fail(TDIST_ERR_DEVICE, "%s: cannot read the wall clock rate", who);
     p.stamp = (const unsigned long long*)stamp;
     p.ticks_per_chunk = (unsigned long long)((double)ns_per_chunk * 1e-6 * (double)khz);
+  }
+  p.max_delay_ticks = 0;
+  p.delay_seed = delay_seed;
+  if (max_delay_ns < 0 || max_delay_ns * cpr > 100000000)
+    return fail(TDIST_ERR_INVALID, "%s: max_delay_ns %lld x %lld chunks outside [0, 100 ms]", who, (long long)max_delay_ns, (long long)cpr);
+  if (max_delay_ns > 0) {
+    const int khz = wall_clock_khz();
+    if (khz <= 0) return fail(TDIST_ERR_DEVICE, "%s: cannot read the wall clock rate", who);
+    p.max_delay_ticks = (unsigned long long)((double)max_delay_ns * 1e-6 * (double)khz);
   }
   p.chunk_bytes = chunk_bytes;
   p.rank_bytes = rank_bytes;

@@ -223,7 +223,9 @@ __global__ __launch_bounds__(kMoeThreads) void moe_rank_kernel(const int32_t* __
 //      wait for each other. That is safe because the host only takes this path when the grid is at most one block per
 //      compute unit, i.e. co-resident (ctrl[0] counts arrivals and is put back to zero by the last one, ctrl[1] is a
 //      generation number that the last arrival bumps; the wait is bounded all the same: if it ran out, the block leaves
-//      without writing and cumsum[0] is set to -1 instead of 0);
+//      without writing, cumsum[0] is set to -1 instead of 0 and ctrl[2] to 1, where it stays). Co-residency is the
+//      caller's to guarantee (nothing else on the GPU may hold compute units for good, e.g. a persistent GEMM that
+//      waits for flags), so the host takes this form only on request (TDIST_DEBUG_MOE_INDEX_FORM = 2);
 //   3. every block adds up the histogram columns (all rows: the split of the expert; rows before its own: its offset
 //      within the expert), scans the splits into cumsum, and turns its waves' counters into start positions;
 //   4. ranking as in moe_rank_kernel.
@@ -356,7 +358,12 @@ __global__ __launch_bounds__(kThreads) void moe_index_fused_kernel(const int32_t
     }
     __syncthreads();
     if (!s_flag) {
-      if (threadIdx.x == 0) cumsum[0] = -1;
+      // Reported in a word nobody else writes (block 0, if it gets through later, puts cumsum[0] back to 0): ctrl[2]
+      // stays non-zero from the first expiry on until the caller clears it.
+      if (threadIdx.x == 0) {
+        __hip_atomic_store(ctrl + 2, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        cumsum[0] = -1;
+      }
       return;
     }
   }
@@ -985,21 +992,24 @@ static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, 
   int32_t* scan_counter = (int32_t*)workspace;
   int32_t* hist = scan_counter + 64;
   int32_t* splits_buf = splits ? splits : hist + (int64_t)num_blocks * G;
-  // One launch when every block of it is resident at once (one per compute unit at most): the blocks wait for each
-  // other's histograms. Its histogram rows (one per 2048 ids) fit the rows the workspace holds (one per 256 ids).
+  // One launch for few ids (up to 65536): every block counts all of them itself and nothing is exchanged. Beyond
+  // that, three launches. A one-launch form whose blocks (2048 ids each, at most one per compute unit) wait for each
+  // other's histograms exists too, but its wait only ends if every block is resident at once, which the library
+  // cannot know when other streams hold compute units: it is taken on request only (TDIST_DEBUG_MOE_INDEX_FORM = 2,
+  // for tests and measurements; 3 = always three launches). Its histogram rows (one per 2048 ids) fit the rows the
+  // workspace holds (one per 256 ids).
   const DeviceInfo& di = device_info();
   const int64_t fused_blocks = ceil_div(n_ids > 0 ? n_ids : 1, kFusedItems);
-  if (di.ok == 1 && fused_blocks <= di.num_cus && getenv("TDIST_MOE_INDEX_LAUNCHES") == nullptr) {
-    // few ids: every block counts all of them itself and nothing is exchanged (TDIST_MOE_INDEX_RENDEZVOUS keeps the
-    // exchange, for tests and measurements)
-    constexpr int kLdsLimit = 160 * 1024 - 256;          // (the kernel has a few static words of its own)
-    constexpr int kRowsPlain = kFusedThreads / 64 + 1;   // wave counters, column sums
-    constexpr int kRowsRecount = kRowsPlain + 2;         // and the ids before / behind the block
-    constexpr int kSmall = kFusedThreads;                // ids per block of the recounting forms: 512, or 1024
-    const int64_t n1 = n_ids > 0 ? n_ids : 1;
-    const bool can_recount = kRowsRecount * G * 4 <= kLdsLimit && aligned16(ids) && getenv("TDIST_MOE_INDEX_RENDEZVOUS") == nullptr;
-    // 0: blocks of 2048 ids that exchange their histograms; 1 / 2: blocks of 512 / 1024 ids that count everything
-    const int form = !can_recount ? 0 : ceil_div(n1, kSmall) <= kRecountMaxBlocks ? 1 : ceil_div(n1, 2 * kSmall) <= kRecountMaxBlocks ? 2 : 0;
+  const int form_dbg = debug_get(TDIST_DEBUG_MOE_INDEX_FORM);
+  constexpr int kLdsLimit = 160 * 1024 - 256;          // (the kernel has a few static words of its own)
+  constexpr int kRowsPlain = kFusedThreads / 64 + 1;   // wave counters, column sums
+  constexpr int kRowsRecount = kRowsPlain + 2;         // and the ids before / behind the block
+  constexpr int kSmall = kFusedThreads;                // ids per block of the recounting forms: 512, or 1024
+  const int64_t n1 = n_ids > 0 ? n_ids : 1;
+  const bool can_recount = form_dbg != 2 && kRowsRecount * G * 4 <= kLdsLimit && aligned16(ids);
+  // 0: blocks of 2048 ids that exchange their histograms; 1 / 2: blocks of 512 / 1024 ids that count everything
+  const int form = !can_recount ? 0 : ceil_div(n1, kSmall) <= kRecountMaxBlocks ? 1 : ceil_div(n1, 2 * kSmall) <= kRecountMaxBlocks ? 2 : 0;
+  if (di.ok == 1 && fused_blocks <= di.num_cus && form_dbg != 3 && (form != 0 || form_dbg == 2)) {
     auto kern = form == 1 ? moe_index_fused_kernel<kFusedThreads, kSmall / 8, true>
               : form == 2 ? moe_index_fused_kernel<kFusedThreads, kSmall / 4, true>
                           : moe_index_fused_kernel<kFusedThreads, kFusedPerWave, false>;

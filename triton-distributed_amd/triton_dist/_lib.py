@@ -19,6 +19,15 @@ TDIST_F16 = 1
 TDIST_F8E4M3 = 2
 TDIST_F32 = 3
 
+# tdist_debug_key (include/tdist.h): test and measurement switches, -1 = the library decides
+TDIST_DEBUG_GEMM_TILE = 0
+TDIST_DEBUG_GEMM_SPLIT_K = 1
+TDIST_DEBUG_GEMM_SK_COHERENT = 2
+TDIST_DEBUG_GEMM_SCHEDULE = 3
+TDIST_DEBUG_DECODE_WAVE_HEADS = 4
+TDIST_DEBUG_DECODE_SPLITS_PER_TEAM = 5
+TDIST_DEBUG_MOE_INDEX_FORM = 6
+
 _P = c_void_p
 _I = c_int
 _L = c_int64
@@ -30,11 +39,13 @@ PROTOTYPES = {
     "tdist_last_error_string": (c_char_p, []),
     "tdist_init": (_I, []),
     "tdist_num_cus": (_I, []),
+    "tdist_debug_set": (_I, [_I, _I]),
+    "tdist_debug_get": (_I, [_I]),
     "tdist_gemm_chunk_gated_bf16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
     "tdist_gemm_chunk_gated_f16": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
     "tdist_gemm_chunk_gated_fp8e4m3": (_I, [_P, _L, _P, _L, _I, _I, _P, _L, _P, _L, _I, _I, _I, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _I, _P, _L, _P]),
     "tdist_producer_push_chunk": (_I, [_P, _P, _L, _P, _P, _I, _P]),
-    "tdist_producer_push_peers": (_I, [_P, _P, _I, _I, _L, _L, _P, _I, _P, _P, _P, _L, _I, _P]),
+    "tdist_producer_push_peers": (_I, [_P, _P, _I, _I, _L, _L, _P, _I, _P, _P, _P, _L, ctypes.c_uint32, _L, _I, _P]),
     "tdist_producer_mark": (_I, [_P, _P]),
     "tdist_producer_wait_until": (_I, [_P, _L, _P]),
     "tdist_flag_set": (_I, [_P, _I, _P]),
@@ -120,6 +131,23 @@ def check(code):
 def call(name, *args):
     """Calls an entry point that returns a tdist_status and raises TdistError on failure."""
     check(getattr(load(), name)(*args))
+
+
+class debug_switch:
+    """``with debug_switch(key, value): ...`` sets one of the library's test and measurement switches
+    (tdist_debug_set) and puts the previous value back on exit."""
+
+    def __init__(self, key, value):
+        self.key, self.value = key, value
+
+    def __enter__(self):
+        self.old = load().tdist_debug_get(self.key)
+        check(load().tdist_debug_set(self.key, -1 if self.value is None else int(self.value)))
+        return self
+
+    def __exit__(self, *exc):
+        check(load().tdist_debug_set(self.key, self.old))
+        return False
 
 
 def ptr(t):

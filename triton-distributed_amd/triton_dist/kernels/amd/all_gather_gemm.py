@@ -92,10 +92,15 @@ def kernel_producer_all_gather_push(rank, num_ranks, ctx, workspace, M_PER_CHUNK
     ctx.held_mask = held   # stays alive until the next call replaces it
     paced = ctx.link_gbps > 0
     nbytes = M_PER_CHUNK * K * esz
+    # race provocation: a new seed per call, so every call sees another pattern of late chunks
+    delay_ns = int(ctx.random_delay_us * 1000)
+    if delay_ns > 0:
+        ctx.delay_calls += 1
+    seed = (ctx.delay_seed * 0x9E3779B1 + ctx.delay_calls) & 0xFFFFFFFF
     _lib.call("tdist_producer_push_peers", workspace.data_ptr(), ctx.peer_ptrs.data_ptr(), num_ranks, rank,
               M_per_rank * K * esz, nbytes, barrier.data_ptr(), 1, ctx.producer_counters.data_ptr(), _lib.ptr(held),
               ctx.start_stamp.data_ptr() if paced else None, int(nbytes / ctx.link_gbps) if paced else 0,
-              int(ctx.producer_workgroups), stream.cuda_stream)
+              seed, delay_ns, int(ctx.producer_workgroups), stream.cuda_stream)
 
 
 @dataclasses.dataclass
@@ -139,6 +144,13 @@ class AllGatherGEMMTensorParallelContext:
     # (producer_cus is ignored) and the host queues three launches per call, however many chunks there are.
     producer_kernel: bool = False
     producer_workgroups: int = 8   # workgroups per peer of that kernel
+    # > 0 (kernel producer only): about 7 of 10 chunks, chosen by a hash of (delay_seed, call number, chunk), are held
+    # back by a pseudo-random time below this many microseconds before they are copied: the reference's race
+    # provocation (its producer sleeps with probability 0.7 when run "for correctness",
+    # kernels/nvidia/allgather.py:72-77,118-121), seeded so that a failing pattern can be replayed.
+    random_delay_us: float = 0.0
+    delay_seed: int = 0
+    delay_calls: int = 0
     producer_counters: Optional[torch.Tensor] = None
     peer_ptrs: Optional[torch.Tensor] = None   # int64[num_ranks] device array of the peer shards' addresses
     held_mask: Optional[torch.Tensor] = None

@@ -78,16 +78,19 @@ def _split_kv(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_sp
 _fused_counters = {}   # (device index, stream handle) -> zero-initialised int32 counters (the kernel leaves them zero)
 
 
-def _counters_for(q, kv_heads, workspace):
-    """Arrival counters of the fused launch: a caller's ``workspace`` when it is a contiguous int32 tensor on the
-    device that is large enough (it must be ALL ZERO; the kernel leaves it zero), else a buffer cached per
+def _counters_for(q, kv_heads, counters):
+    """Arrival counters of the fused launch. ``counters`` (an explicit opt-in of this module's own callers: the layer,
+    the tests): a contiguous int32 device tensor of at least tdist_decode_fused_counters(...) entries that is ALL ZERO
+    and shared with no launch that may overlap this one; the kernel leaves it zero. None: a zeroed buffer cached per
     (device, current stream): launches on one stream are ordered, so they may share it, and launches on different
     streams never do."""
     batch, q_heads, _ = q.shape
     need = _lib.load().tdist_decode_fused_counters(batch, q_heads, kv_heads)
-    if (isinstance(workspace, torch.Tensor) and workspace.is_cuda and workspace.dtype == torch.int32
-            and workspace.is_contiguous() and workspace.numel() >= need):
-        return workspace, workspace.numel()
+    if counters is not None:
+        if not (isinstance(counters, torch.Tensor) and counters.is_cuda and counters.dtype == torch.int32
+                and counters.is_contiguous() and counters.numel() >= need):
+            raise ValueError("counters: a contiguous int32 device tensor of at least %d zeroed entries" % need)
+        return counters, counters.numel()
     key = (q.device.index, torch.cuda.current_stream(q.device).cuda_stream)
     buf = _fused_counters.get(key)
     if buf is None or buf.numel() < need:
@@ -99,7 +102,8 @@ def _counters_for(q, kv_heads, workspace):
 def decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, out, lse_out=None,
                  workspace=None, out_split=None, lse_split=None):
     """tdist_decode_fused: split-KV decode and the merge of the splits in one launch. ``out`` [B,Hq,Dv]
-    (bf16 / f16 / fp32), ``lse_out`` fp32 [B,Hq] or None. Returns (out, out_split, lse_split)."""
+    (bf16 / f16 / fp32), ``lse_out`` fp32 [B,Hq] or None. ``workspace``: None, or zeroed arrival counters of the
+    caller's own (see _counters_for; anything else is an error). Returns (out, out_split, lse_split)."""
     kv_lens, block_table = _check_inputs(q, k_cache, v_cache, kv_lens, block_table)
     out_split, lse_split = _split_buffers(q, v_cache, num_splits, out_split, lse_split)
     assert out.stride(-1) == 1 and (lse_out is None or (lse_out.dtype == torch.float32 and lse_out.is_contiguous()))
@@ -146,25 +150,26 @@ def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_l
                                     output_split=None, output_combine=None, kv_split=-1):
     """Same result as gqa_fwd_batch_decode in one launch (reference :931-1004: split-KV, a grid barrier on
     ``workspace``, then the combine). Here the last workgroup to finish a (sequence, head block) merges its splits.
-    The arrival counters live in ``workspace`` when it is a zero-filled contiguous int32 device tensor of at least
-    tdist_decode_fused_counters(batch, q_heads, kv_heads) entries (the reference's barrier workspace is such a
-    tensor; the kernel leaves it zero), else in a zeroed buffer cached per (device, stream). ``output_split`` is
-    ignored (partials are fp32 internally)."""
+    ``workspace`` (the reference's barrier buffer) and ``q_lens`` are accepted and unused: nothing says what a
+    caller's buffer holds or who else uses it, and a counter that does not start at zero makes a merge fire early or
+    never, so the arrival counters are the library's own (zeroed, cached per device and stream, left zero by every
+    call). ``output_split`` is ignored (partials are fp32 internally)."""
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
     batch, q_heads, _ = q.shape
     if output_combine is None:
         output_combine = torch.empty((batch, q_heads, v_cache.shape[-1]), dtype=q.dtype, device=q.device)
-    decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, output_combine,
-                 workspace=workspace)
+    decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, output_combine)
     return output_combine
 
 
 def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
-                                    output_split=None, output_combine=None, kv_split=-1, return_lse=False):
+                                    output_split=None, output_combine=None, kv_split=-1, return_lse=False, counters=None):
     """One rank's KV shard: split-KV decode, then the merge of its splits keeping the LSE (reference
     :847-928). Returns ``output_combine`` [B,Hq,Dv+1] with the LSE in column Dv, fp32 unless the caller
     passes a buffer of another dtype (the reference uses q's dtype). With ``return_lse`` also returns the
-    fp32 (out [B,Hq,Dv], lse [B,Hq]) pair the merge produced."""
+    fp32 (out [B,Hq,Dv], lse [B,Hq]) pair the merge produced. ``workspace`` and ``q_lens`` are accepted and unused, as
+    in the reference; ``counters`` (keyword only in spirit: an addition) hands in zeroed arrival counters of the
+    caller's own, see _counters_for."""
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
     batch, q_heads, _ = q.shape
     dv = v_cache.shape[-1]
@@ -174,7 +179,7 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
     lse32 = torch.empty((batch, q_heads), dtype=torch.float32, device=q.device)
     # split-KV and the merge of the splits (keeping the LSE) in one launch
     decode_fused(q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap, num_splits, out32, lse32,
-                 workspace=workspace)
+                 workspace=counters)
     output_combine[..., :dv].copy_(out32)
     output_combine[..., dv].copy_(lse32)
     if return_lse:

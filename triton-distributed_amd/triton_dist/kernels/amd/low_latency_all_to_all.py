@@ -80,7 +80,7 @@ class AllToAllContext:
         self.MOD_VALUE = 1000000
         # index tensors of moe_dispatch_preprocess(..., ctx=self): two sets, allocated on first use for a shape
         self.index_sets, self.index_key, self.index_calls = None, None, 0
-        self.index_workspace, self.index_args = None, None
+        self.index_workspace, self.index_args, self.index_ids = None, None, None
 
 
 def create_all_to_all_context(
@@ -134,21 +134,7 @@ def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_to
     One kernel launch. With ``ctx`` the five tensors are the context's own (allocated on the first call for a shape,
     two sets used in turn like the receive buffers, so a result stays valid until the call after next) and the call
     allocates nothing. Returns (splits, split_cumsum, scatter_idx, gather_idx[, topk_idx])."""
-    if ctx is not None and ctx.index_key == (exp_indices.shape[0], exp_indices.shape[1], num_experts, exp_indices.device) \
-            and exp_indices.dtype == torch.int32 and exp_indices.is_contiguous():
-        # the context has seen this shape: its tensors' addresses are at hand and the host does next to nothing
-        # (the index kernel takes ~9 us on the device; the general path below costs more than that on the host)
-        which = ctx.index_calls % 2
-        ctx.index_calls += 1
-        out = ctx.index_sets[which]
-        head, tail = ctx.index_args[which]
-        _lib.call("tdist_moe_scatter_index", exp_indices.data_ptr(), *head, _lib.ptr(out[4] if want_topk_index else None),
-                  *tail, _lib.stream_ptr())
-        return out if want_topk_index else out[:4]
     _lib.require_cuda(exp_indices)
-    if exp_indices.dtype != torch.int32:
-        exp_indices = exp_indices.to(torch.int32)
-    exp_indices = exp_indices.contiguous()
     T, topk = exp_indices.shape
     n = T * topk
     dev = exp_indices.device
@@ -160,19 +146,37 @@ def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_to
                 torch.empty(n, dtype=torch.int32, device=dev),
                 torch.empty(n, dtype=torch.int32, device=dev))
 
-    ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
     if ctx is not None:
-        # (a new shape: two sets of result tensors and a zeroed workspace of the context's own; the calls of one
-        # context are ordered on its stream, so they may share it)
-        ctx.index_sets, ctx.index_key, ctx.index_calls = [alloc(), alloc()], (T, topk, num_experts, dev), 1
-        ctx.index_workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
-        ctx.index_args = [((n, topk, num_experts, t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), t[3].data_ptr()),
-                           (ctx.index_workspace.data_ptr(), ws_bytes)) for t in ctx.index_sets]
-        splits, cumsum, scatter_idx, gather_idx, topk_idx = ctx.index_sets[0]
-        workspace = ctx.index_workspace
-    else:
-        splits, cumsum, scatter_idx, gather_idx, topk_idx = alloc()
-        workspace = _lib.zeroed_scratch(ws_bytes, dev)
+        if ctx.index_key != (T, topk, num_experts, dev):
+            # a new shape: two sets of result tensors, a zeroed workspace and an int32 staging tensor for ids of
+            # another dtype, all the context's own (the calls of one context are ordered on its stream, so they may
+            # share them)
+            ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
+            ctx.index_sets, ctx.index_key, ctx.index_calls = [alloc(), alloc()], (T, topk, num_experts, dev), 0
+            ctx.index_workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+            ctx.index_ids = torch.empty((T, topk), dtype=torch.int32, device=dev)
+            ctx.index_args = [((n, topk, num_experts, t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), t[3].data_ptr()),
+                               (ctx.index_workspace.data_ptr(), ws_bytes)) for t in ctx.index_sets]
+        # the context has seen this shape: its tensors' addresses are at hand and the host does next to nothing (the
+        # index kernel takes ~9 us on the device; a general path costs more than that on the host). Ids that are not
+        # contiguous int32 (torch.topk gives int64) are converted into the context's staging tensor: one copy kernel,
+        # no allocation.
+        if exp_indices.dtype != torch.int32 or not exp_indices.is_contiguous():
+            ctx.index_ids.copy_(exp_indices)
+            exp_indices = ctx.index_ids
+        which = ctx.index_calls % 2
+        ctx.index_calls += 1
+        out = ctx.index_sets[which]
+        head, tail = ctx.index_args[which]
+        _lib.call("tdist_moe_scatter_index", exp_indices.data_ptr(), *head, _lib.ptr(out[4] if want_topk_index else None),
+                  *tail, _lib.stream_ptr())
+        return out if want_topk_index else out[:4]
+    if exp_indices.dtype != torch.int32:
+        exp_indices = exp_indices.to(torch.int32)
+    exp_indices = exp_indices.contiguous()
+    ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
+    splits, cumsum, scatter_idx, gather_idx, topk_idx = alloc()
+    workspace = _lib.zeroed_scratch(ws_bytes, dev)
     if not want_topk_index:
         topk_idx = None
     _lib.call("tdist_moe_scatter_index", exp_indices.data_ptr(), n, topk, num_experts, splits.data_ptr(),

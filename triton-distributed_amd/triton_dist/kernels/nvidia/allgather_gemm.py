@@ -15,19 +15,25 @@ def create_ag_gemm_intra_node_context(tensor_A, tensor_B, rank, num_ranks, max_M
                                       gemm_stream=None, serial=False, autotune=False):
     """tensor_A [M_per_rank, K], tensor_B [N_per_rank, K]. One flag per rank segment, as in the reference
     (barriers of shape [num_ranks], :817); M_per_rank may be any number of rows (a tile of the GEMM waits for every
-    rank segment its rows touch, as the reference's consumer does, :222-224). ``max_blocks`` and ``for_correctness`` are accepted and unused (no
-    block-level barrier buffer here; delayed arrivals are a context option: ``ctx.link_gbps``)."""
+    rank segment its rows touch, as the reference's consumer does, :222-224). ``max_blocks`` is accepted and unused (no
+    block-level barrier buffer here). ``for_correctness``: the reference's producer then sleeps with probability 0.7
+    before it copies (allgather.py:72-77,118-121), to show a consumer that does not wait; here the peers' rows then
+    come from the one-launch producer with seeded random delays of up to 200 us per rank segment
+    (``ctx.random_delay_us``, ``ctx.delay_seed``)."""
     M_per_rank, K = tensor_A.shape
     assert tensor_B.shape[1] == K, "tensor_B should have shape [N_per_rank, %d], got %s" % (K, tuple(tensor_B.shape))
     assert tensor_A.dtype == tensor_B.dtype
     M = M_per_rank * num_ranks
     assert M <= max_M
     out_dtype = tensor_A.dtype if tensor_A.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
-    return _amd.create_ag_gemm_intra_node_context(M, tensor_B.shape[0], K, tensor_A.dtype, out_dtype, rank, num_ranks, None,
-                                                  ag_streams=None if ag_stream is None else [ag_stream],
-                                                  gemm_stream=gemm_stream, M_PER_CHUNK=M_per_rank, BLOCK_M=BLOCK_M,
-                                                  BLOCK_N=BLOCK_N, BLOCK_K=BLOCK_K, stages=stages, serial=serial,
-                                                  autotune=autotune, ragged_chunks=True)
+    ctx = _amd.create_ag_gemm_intra_node_context(M, tensor_B.shape[0], K, tensor_A.dtype, out_dtype, rank, num_ranks, None,
+                                                 ag_streams=None if ag_stream is None else [ag_stream],
+                                                 gemm_stream=gemm_stream, M_PER_CHUNK=M_per_rank, BLOCK_M=BLOCK_M,
+                                                 BLOCK_N=BLOCK_N, BLOCK_K=BLOCK_K, stages=stages, serial=serial,
+                                                 autotune=autotune, ragged_chunks=True)
+    if for_correctness:
+        ctx.producer_kernel, ctx.random_delay_us = True, 200.0
+    return ctx
 
 
 def ag_gemm_intra_node(a, b, ctx=None, rank=None, num_ranks=None, persistent=True):

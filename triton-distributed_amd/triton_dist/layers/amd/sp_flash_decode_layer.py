@@ -53,10 +53,10 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         if self.workspace is None or self.workspace.device != q.device:
             n = _lib.load().tdist_decode_fused_counters(self.max_allowed_batch, self.num_q_heads, self.num_kv_heads)
             self.workspace = torch.zeros(max(int(n), 1), dtype=torch.int32, device=q.device)
-        _, out32, lse32 = gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, self.workspace, [1] * batch,
+        _, out32, lse32 = gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, None, [1] * batch,
                                                           global_kv_lens[self.rank], block_table, self.scale,
                                                           soft_cap=self.soft_cap, kv_split=self.kv_split,
-                                                          return_lse=True)
+                                                          return_lse=True, counters=self.workspace)
         if self.num_ranks == 1:
             all_out, all_lse = out32.unsqueeze(0), lse32.unsqueeze(0)
         else:
