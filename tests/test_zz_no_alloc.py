@@ -34,6 +34,7 @@ def run_both(cuda, ids, G):
 
 @pytest.mark.parametrize("launches", ["one", "three"])
 def test_static_scratch_entry_matches_the_workspace_entry(cuda, switches, launches):
+    from triton_dist import _lib
     if launches == "three":
         switches(_lib.TDIST_DEBUG_MOE_INDEX_FORM, 3)
     g = torch.Generator().manual_seed(21)
