@@ -93,8 +93,12 @@ def paced_ag_gemm(make_call, world, rank, mpr, N, K, in_dtype, peer_shards, chun
     """AG-GEMM with every peer's chunks held back to the pace of one xGMI link per peer (the one-GPU producer kernel
     copies chunk c of every peer no earlier than (c+1) chunk times of a link after the call started), for several
     chunk sizes. Overlap efficiency = time with every flag pre-set / time with paced arrivals; the time includes
-    the host's queueing of the call (three streams, their events), which is what bounds the small config."""
+    the host's queueing of the call (three streams, their events), which is what bounds the small config.
+    ``straggler``: on top of the pacing, the peer that the static order expects first is late, so that chunks arrive out
+    of the order the static schedule walks them in: timed with the tiles taken in arrival order (the default) and in
+    the static order."""
     import torch
+    from triton_dist import _lib
     from triton_dist.kernels.amd import create_ag_gemm_intra_node_context
     out = {}
     for rows in chunk_rows:
@@ -108,6 +112,22 @@ def paced_ag_gemm(make_call, world, rank, mpr, N, K, in_dtype, peer_shards, chun
         out["m_per_chunk_%d" % rows] = {"us": round(s * 1e6, 2), "order": order,
                                         "overlap_efficiency": round(pre_s / s, 4),
                                         "last_chunk_arrives_us": round(arrive_us, 1)}
+        if rows == chunk_rows[-1]:
+            # a straggler: the peer the static order expects first delivers its first chunk `late` us late (a third of
+            # the call's time with every flag set), its other chunks behind it
+            late = round(pre_s * 1e6 / 3)
+            ctx.late_chunks_us = {((rank + 1) % world) * (mpr // rows): late}
+            res = {"first_peer_late_by_us": late}
+            for name, static in (("arrival_order", False), ("static_order", True)):
+                old = _lib.load().tdist_debug_get(_lib.TDIST_DEBUG_GEMM_SCHEDULE)
+                if static:
+                    _lib.check(_lib.load().tdist_debug_set(_lib.TDIST_DEBUG_GEMM_SCHEDULE, 0))
+                try:
+                    js, _ = time_live_ag_gemm(make_call(ctx), ctx, max(steps // 2, 1), warmup)
+                finally:
+                    _lib.check(_lib.load().tdist_debug_set(_lib.TDIST_DEBUG_GEMM_SCHEDULE, old))
+                res[name + "_us"] = round(js * 1e6, 2)
+            out["m_per_chunk_%d" % rows]["straggler"] = res
     return out
 
 
@@ -548,6 +568,9 @@ def main():
     ap.add_argument("--no-live-producer", action="store_true",
                     help="skip the AG-GEMM legs in which a copy stream releases the flags while the GEMM spins: a "
                     "counter-collecting profiler serialises dispatches, so the producer could never run beside it")
+    ap.add_argument("--static-schedule", action="store_true",
+                    help="gated GEMMs walk their tiles in the static chunk-major order instead of in arrival order "
+                    "(the library's TDIST_DEBUG_GEMM_SCHEDULE switch): the comparison leg of the overlap figures")
     args = ap.parse_args()
     LIVE_PRODUCER = not args.no_live_producer
     SETTLE_SECONDS = args.settle_seconds
@@ -561,6 +584,8 @@ def main():
         sys.exit(1)
     from triton_dist import _lib
     _lib.check(_lib.load().tdist_init())
+    if args.static_schedule:
+        _lib.check(_lib.load().tdist_debug_set(_lib.TDIST_DEBUG_GEMM_SCHEDULE, 0))
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     want = set(x for x in args.only.split(",") if x) or {"c1", "c2", "c3", "c4", "c5", "moe_gemm", "copy", "mfma", "library"}

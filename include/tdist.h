@@ -150,8 +150,9 @@ int tdist_producer_push_chunk(void* dst, const void* src, int64_t nbytes, int32_
  * last of them has stored its part of chunk c it stores flag_value into flags[r*chunks_per_rank + c] (release,
  * system scope) — the data-then-flag protocol of kernels/amd/all_gather_gemm.py:80-100.
  * peer_src: device array of world_size device pointers (entry `rank` unused). counters: int32
- * [world_size*chunks_per_rank], zero on entry, left zero. held: optional int32 mask of chunks never to deliver
- * (test hook for the consumer's bounded wait). stamp + ns_per_chunk > 0: the pace of one link per peer: chunk c of
+ * [world_size*chunks_per_rank], zero on entry, left zero. held: optional int32 per chunk: > 0 = never deliver
+ * (test hook for the consumer's bounded wait), < 0 = copy it that many microseconds late, at most 100 000 (a straggler;
+ * the peer's later chunks follow behind it). stamp + ns_per_chunk > 0: the pace of one link per peer: chunk c of
  * every peer is copied from c*ns_per_chunk after the stamp (tdist_producer_mark) on and its flag is released no
  * earlier than (c+1)*ns_per_chunk after it, when a link of that rate would have delivered the chunk's last byte; the
  * total must stay within 100 ms. max_delay_ns > 0: race provocation, as the reference's producer sleeps with probability

@@ -235,6 +235,73 @@ def test_gate_released_by_a_stream_while_the_gemm_waits(cuda):
     assert golden.max_rel_err(c.float().cpu(), golden.ag_gemm_fp32([a], b)) <= 1e-2
 
 
+@pytest.mark.parametrize("schedule", ["arrival", "static"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn])
+def test_tiles_in_arrival_order(cuda, switches, schedule, dtype):
+    """More than one round of tiles (384 tiles of 256 x 256 on 256 workgroups), so that gated calls with a workspace take
+    their tiles in arrival order (first round static, then one draw per tile from the XCD's list, tiles of chunks that
+    have not arrived put aside): flags released late and out of the expected order by a second stream, a straggler
+    behind the kernel producer, and a chunk that never arrives (every other row right, the held chunk's rows
+    untouched, TDIST_ERR_TIMEOUT naming it, the ticket counters back at zero so that the next launch is clean). The
+    static order, forced through the library's switch, must give the same bits."""
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import ag_gemm_intra_node, create_ag_gemm_intra_node_context, gated_gemm
+    from triton_dist.kernels.amd.common_ops import set_signal
+    announce("gemm tiles in %s order %s" % (schedule, dtype))
+    if schedule == "static":
+        switches(_lib.TDIST_DEBUG_GEMM_SCHEDULE, 0)
+    world, mpc, N, K = 8, 512, 6144, 256
+    M = world * mpc
+    g = torch.Generator().manual_seed(31)
+    a = torch.randint(-2, 3, (M, K), generator=g).float()
+    b = torch.randint(-2, 3, (N, K), generator=g).float()
+    want = golden.ag_gemm_fp32([a], b).to(torch.bfloat16)
+    a_d, b_d = a.to(dtype).to(cuda), b.to(dtype).to(cuda)
+    ws = _lib.new_split_k_workspace(cuda)
+    sched_words = ws.view(torch.int32)[16:16 + 16 + 8 * 16]   # the schedule's done counter and draw counters
+    status = torch.zeros(2, dtype=torch.int32, device=cuda)
+    # (1) flags released 200 us into the launch, last chunk first, by a second stream (queued before the GEMM)
+    flags = torch.zeros(world, dtype=torch.int32, device=cuda)
+    flags[3] = 1
+    c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+    side = torch.cuda.Stream()
+    stamp = torch.zeros(1, dtype=torch.int64, device=cuda)
+    torch.cuda.synchronize()
+    _lib.call("tdist_producer_mark", stamp.data_ptr(), side.cuda_stream)
+    _lib.call("tdist_producer_wait_until", stamp.data_ptr(), 200000, side.cuda_stream)
+    for chunk in (7, 6, 5, 4, 2, 1, 0):
+        set_signal(flags.data_ptr() + 4 * chunk, 1, side)
+    gated_gemm(a_d, None, 0, b_d, c, flags, mpc, 3, world, status=status, sk_workspace=ws)
+    torch.cuda.synchronize()
+    assert status.tolist() == [0, 0]
+    assert torch.equal(c.cpu(), want)
+    assert int(sched_words.abs().sum()) == 0, "the schedule's counters must be left at zero"
+    # (2) a chunk that never arrives
+    flags.fill_(1)
+    flags[5] = 0
+    c.fill_(-7.0)
+    gated_gemm(a_d, None, 0, b_d, c, flags, mpc, 3, world, spin_limit=50, status=status, sk_workspace=ws)
+    torch.cuda.synchronize()
+    assert status.tolist() == [_lib.TDIST_ERR_TIMEOUT, 5]
+    got = c.cpu()
+    assert (got[5 * mpc:6 * mpc] == -7.0).all(), "rows of the held chunk were written"
+    keep = torch.ones(M, dtype=torch.bool)
+    keep[5 * mpc:6 * mpc] = False
+    assert torch.equal(got[keep], want[keep])
+    assert int(sched_words.abs().sum()) == 0
+    # (3) the op with the kernel producer and a straggler: rank 2's first chunk 300 us late, its second one behind it
+    rank = 1
+    shards = [a[r * mpc:(r + 1) * mpc] for r in range(world)]
+    ctx = create_ag_gemm_intra_node_context(M, N, K, dtype, torch.bfloat16, rank, world, None, M_PER_CHUNK=256)
+    ctx.set_peer_shards({r: s_.to(dtype).to(cuda) for r, s_ in enumerate(shards) if r != rank})
+    ctx.producer_kernel, ctx.late_chunks_us = True, {2 * 2: 300}
+    for _ in range(3):
+        ctx.workspace_tensors[rank].view(torch.uint8).fill_(0x7B if dtype != torch.float8_e4m3fn else 0x7F)
+        out = ag_gemm_intra_node(shards[rank].to(dtype).to(cuda), b_d, False, ctx)
+        ctx.check_status()
+        assert torch.equal(out.cpu(), want)
+
+
 def test_gemm_rs_small_and_owner_mapping(cuda):
     from triton_dist.kernels.amd import create_gemm_rs_intra_node_context, gemm_rs_intra_node
     announce("gemm_rs small")

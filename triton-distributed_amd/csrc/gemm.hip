@@ -86,6 +86,24 @@ struct GemmParams {
   int sk_mode;
   int sk_l2_local;   // 1: workgroup i has been seen to run on XCD i mod num_xcds (tdist_init), so pieces that the
                      // schedule puts on one XCD may exchange through that XCD's L2 alone
+  // Tiles in arrival order (sched_ctrl != NULL; gated calls with whole-tile chunks, at most kSchedMaxChunks of them, and
+  // more than one round of tiles). The static schedule parks a workgroup on the flag of the chunk its position names,
+  // also while rows of other chunks have long arrived, and gives every workgroup a fixed list of tiles whatever
+  // happens (the reference orders its tiles by expected arrival for the same reason,
+  // kernels/amd/all_gather_gemm.py:193-206). Here only the first round is static (workgroup w owns the tile at
+  // position w of the static order). From the second round on, the tiles that the static schedule gives to the
+  // workgroups of one XCD form that XCD's LIST, in the static order, and a workgroup that needs work draws the list's
+  // next tile with one atomic add on the XCD's counter (a workgroup whose own list has run out draws from the other
+  // XCDs' lists), so the workgroups of an XCD still work on neighbouring tiles and share operand panels in that
+  // XCD's L2. A tile whose chunk has not arrived is put aside (two per workgroup at most) and the next one is drawn;
+  // tiles put aside come first again as soon as their flag is up. With nothing to do, the workgroup polls the flags
+  // of what it holds, bounded as the static order's flag wait is. The draw and the look at the flags (wave 0, one
+  // lane per chunk) are issued when the current tile's epilogue begins and used when it ends, so in a call whose rows
+  // are all there the schedule costs no waiting at all. Every tile is computed whole and by one workgroup, so the
+  // result does not depend on who computes it or when.
+  // The counters live in spare words of the workspace header: zero between launches (the last workgroup out clears
+  // them), so launches that share a workspace must be ordered, as for the split rounds.
+  int32_t* sched_ctrl;
 };
 
 // Workspace header, in int32 words
@@ -96,6 +114,13 @@ constexpr int kSkFlagsOff = 1024;        // [kSkMaxWorkgroups] tag of the partia
 constexpr int kSkAcksOff = 2048;         // [kSkMaxWorkgroups] readers that are done with the slot, ever
 constexpr int kSkHeaderWords = 3072;
 constexpr int64_t kSkHeaderBytes = (int64_t)kSkHeaderWords * 4;
+// words [kSchedOff, kSkFlagsOff) of the header: the arrival-order schedule's done counter and, a cache line apart,
+// one draw counter per XCD
+constexpr int kSchedOff = 16, kSchedDone = 0, kSchedCounters = 16, kSchedCounterStride = 16;
+constexpr int kSchedMaxChunks = 64;      // one lane of the deciding wave per chunk
+constexpr int kSchedMaxXcds = 8;
+constexpr int kSchedAside = 2;           // tiles a workgroup may put aside
+static_assert(kSchedOff + kSchedCounters + kSchedMaxXcds * kSchedCounterStride <= 1024, "draw counters within the header's spare words");
 constexpr int kSkTagStride = 16;         // tags per launch (rounds that may be split)
 // a flag word is the tag (low 27 bits) with the XCD the piece ran on above it
 constexpr int kSkTagBits = 27, kSkTagMask = (1 << kSkTagBits) - 1, kSkTagWrap = kSkTagMask - 0x10000;
@@ -412,11 +437,170 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   int sk_split = 1;
   if (p.sk_mode == 1 && sk_tail_tiles > 0) sk_split = sk_split_for(G, sk_tail_tiles, KT);
 
+  // ---- tiles in arrival order (see GemmParams::sched_ctrl); everything here is wave 0's, one lane per chunk ----------
+  const bool arrival = !kGrouped && p.sched_ctrl != nullptr;
+  const int arr_nx = (p.num_xcds > 1 && p.num_xcds <= kSchedMaxXcds && G % p.num_xcds == 0) ? p.num_xcds : 1;
+  const int arr_gx = G / arr_nx;               // workgroups per XCD = tiles of a round in one XCD's list
+  const int arr_my_x = arr_nx > 1 ? blockIdx.x % arr_nx : 0;
+  bool arr_first = true, arr_decided = false;
+  // positions in the static order: the tile drawn but not yet begun, and the tiles put aside (-1 = none; kArrNone in
+  // arr_held once every list has run out)
+  constexpr int kArrNone = -2;
+  int arr_held = -1, arr_aside[kSchedAside] = {-1, -1};
+  int arr_dead = 0;                            // XCDs whose lists this workgroup has found empty
+  int arr_limit = p.spin_limit;                // looks a wait may take: 1 once any wait of the launch has expired
+  // draw t of XCD x's list → position in the static order (rounds from the second on), or -1 behind the list's end
+  auto arr_position = [&](int x, int t) {
+    const int sidx = (1 + t / arr_gx) * G + x * arr_gx + t % arr_gx;
+    return t >= 0 && sidx < total_sched ? sidx : -1;
+  };
+  auto arr_chunk_at = [&](int sidx) { return chunk_of(p, sidx / tiles_per_chunk); };
+  auto arr_is_local = [&](int ch) {
+    const int cm0 = ch * p.m_per_chunk;
+    return p.A_local != nullptr && cm0 >= p.local_row_begin && cm0 < p.local_row_begin + p.local_rows;
+  };
+  // One look: lane c loads chunk c's flag (system scope), lane x the draw counter of XCD x (device scope). Two
+  // independent loads with nothing branching around them: they go out at once and are waited for at their first use.
+  auto arr_look = [&](int& flag, int& cnt) {
+    int l = lane;
+    asm volatile("" : "+v"(l));   // (nothing of this is computed ahead and held across the K loop)
+    flag = __hip_atomic_load(p.flags + min(l, n_chunks - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    cnt = __hip_atomic_load(p.sched_ctrl + kSchedCounters + min(l, arr_nx - 1) * kSchedCounterStride, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+  };
+  // the draw: one lane's atomic add on XCD x's counter (the raw counter value, valid in every lane afterwards)
+  auto arr_draw = [&](int x) {
+    int t = 0;
+    if (lane == 0)
+      t = __hip_atomic_fetch_add(p.sched_ctrl + kSchedCounters + x * kSchedCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return t;
+  };
+  // The next tile of this workgroup, given a look (flag, cnt) and, if one was issued with it, a draw from the own
+  // XCD's list (drawn = true, t its raw result in lane 0). Returns the tile's position in the static order, or -1 when
+  // there is nothing left to do.
+  auto arr_next = [&](int flag, int cnt, bool drawn, int t_raw) -> int {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    if (drawn) {
+      const int pos = arr_position(arr_my_x, __shfl(t_raw, 0));
+      arr_held = pos >= 0 ? pos : -1;
+      if (pos < 0) arr_dead |= 1 << arr_my_x;
+    }
+    int looks = 0, next = -1;
+    for (;;) {
+      // chunk c has arrived (lane c's verdict); the lists that are empty by their counters (counters only grow)
+      const uint64_t arrived = __ballot(l < n_chunks && (flag == p.wait_value || arr_is_local(l)));
+      arr_dead |= (int)__ballot(l < arr_nx && arr_position(l, cnt) < 0);
+      auto ready = [&](int sidx) { return ((arrived >> arr_chunk_at(sidx)) & 1) != 0; };
+      // 1. a tile put aside whose chunk has arrived, the oldest first
+      bool took = false;
+#pragma unroll
+      for (int i = 0; i < kSchedAside; ++i) {
+        if (!took && arr_aside[i] >= 0 && ready(arr_aside[i])) {
+          next = arr_aside[i];
+#pragma unroll
+          for (int j = i; j + 1 < kSchedAside; ++j) arr_aside[j] = arr_aside[j + 1];
+          arr_aside[kSchedAside - 1] = -1;
+          took = true;
+        }
+      }
+      if (took) break;
+      // 2. the tile in hand, or a new draw: the own list first, then the other XCDs' while any has tiles left
+      if (arr_held == -1) {
+        for (int dx = 0; dx < arr_nx && arr_held == -1; ++dx) {
+          const int x = (arr_my_x + dx) % arr_nx;
+          if ((arr_dead >> x) & 1) continue;
+          const int pos = arr_position(x, __shfl(arr_draw(x), 0));
+          if (pos >= 0) arr_held = pos;
+          else arr_dead |= 1 << x;
+        }
+        if (arr_held == -1) arr_held = kArrNone;
+      }
+      if (arr_held >= 0) {
+        if (ready(arr_held)) {
+          next = arr_held;
+          arr_held = -1;
+          break;
+        }
+        if (arr_aside[kSchedAside - 1] < 0) {   // room to put it aside: do, and draw again
+#pragma unroll
+          for (int i = 0; i < kSchedAside; ++i) {
+            if (arr_aside[i] < 0) {
+              arr_aside[i] = arr_held;
+              break;
+            }
+          }
+          arr_held = -1;
+          continue;
+        }
+      } else if (arr_aside[0] < 0) {
+        break;   // every list is empty and nothing is put aside: done (next = -1)
+      }
+      // 3. everything this workgroup holds waits for a flag: look again, as the static order's flag wait does (bounded;
+      // once any wait of the launch has expired, one look is all the others get)
+      if (looks == 0 && p.status != nullptr && __hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) arr_limit = 1;
+      if (++looks >= arr_limit) {
+        // expired: the oldest tile is given up (skipped, as a tile whose flag wait expires is) and reported
+        const int lost = arr_aside[0] >= 0 ? arr_aside[0] : arr_held;
+        if (arr_aside[0] >= 0) {
+#pragma unroll
+          for (int j = 0; j + 1 < kSchedAside; ++j) arr_aside[j] = arr_aside[j + 1];
+          arr_aside[kSchedAside - 1] = -1;
+        } else {
+          arr_held = -1;
+        }
+        if (l == 0 && p.status != nullptr) {
+          if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = arr_chunk_at(lost);
+        }
+        arr_limit = 1;
+        looks = 0;
+        continue;
+      }
+      __builtin_amdgcn_s_sleep(4);
+      arr_look(flag, cnt);
+    }
+    if (next >= 0 && !arr_is_local(arr_chunk_at(next))) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    return next;
+  };
+
   int sbase = 0;
   for (;;) {
     // ---- next piece of work: K tiles [ka, kb) of tile `within` of chunk position oc, as piece sk_j of sk_s -----
     int oc, within, ka = 0, kb = KT, sk_s = 1, sk_j = 0, sk_tag = 0;
-    {
+    int arr_chunk = -1;   // arrival order: the chunk of the tile taken (its flag has been seen and acquired)
+    if (arrival) {
+      if (!arr_decided && wave == 0) {
+        // not decided while the last tile was stored: the first tile, or a position that turned out to hold no tile
+        int next = -1;
+        bool quick = false;
+        if (arr_first && wg_pos < total_sched) {
+          // the first round is static: this workgroup's own tile, which nobody else can take
+          arr_held = wg_pos;
+          const int ch = arr_chunk_at(wg_pos);
+          if (arr_is_local(ch) || __hip_atomic_load(p.flags + ch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == p.wait_value) {
+            if (!arr_is_local(ch)) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+            next = wg_pos;
+            arr_held = -1;
+            quick = true;
+          }
+        }
+        if (!quick) {
+          int flag, cnt;
+          arr_look(flag, cnt);
+          next = arr_next(flag, cnt, false, 0);
+        }
+        if (lane == 0) s_gate[0] = next;
+      }
+      arr_first = false;
+      arr_decided = false;
+      __syncthreads();
+      const int next = __builtin_amdgcn_readfirstlane(s_gate[0]);
+      __syncthreads();
+      if (next < 0) break;
+      oc = next / tiles_per_chunk;
+      within = next - oc * tiles_per_chunk;
+      arr_chunk = chunk_of(p, oc);
+    } else {
       int sidx;
       if (sbase >= total_sched) break;
       const int round_base = sbase;
@@ -439,7 +623,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       within = sidx - oc * tiles_per_chunk;
     }
     const int KTp = kb - ka;
-    const int chunk = kGrouped ? (oc + p.first_block) % n_chunks : chunk_of(p, oc);
+    const int chunk = kGrouped ? (oc + p.first_block) % n_chunks : arr_chunk >= 0 ? arr_chunk : chunk_of(p, oc);
     const int pid_m = chunk * cm + within % cm;
     const int pid_n = within / cm;
     if (pid_m >= num_pid_m) continue;
@@ -453,7 +637,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // ---- gate ---------------------------------------------------------------------------------
     const bool is_local = kGrouped ? (p.A_local != nullptr && segment == p.rank)
                                    : (p.A_local != nullptr && m0 >= p.local_row_begin && m0 < p.local_row_begin + p.local_rows);
-    if (p.flags != nullptr && !is_local) {
+    if (p.flags != nullptr && !is_local && arr_chunk < 0) {
       if (threadIdx.x == 0) {
         // the flags of the tile's rows: one (the tile lies inside a chunk), or, with ragged chunks, every flag from
         // the first row's to the last row's (the reference's NVIDIA-side kernel waits for a range of rank segments
@@ -934,6 +1118,15 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     constexpr int kRowBlocks = C::kWaveM / 32, kGroups = C::kWaveN / 8;
     constexpr bool kWide = E::kRows == 32;
     wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
+    // arrival order: the look for the next tile goes out now and is used when this tile has been stored
+    int arr_flag = 0, arr_cnt = 0, arr_t = 0;
+    bool arr_drawn = false;
+    if (arrival && wave == 0) {
+      arr_look(arr_flag, arr_cnt);
+      // and the draw, unless a tile is in hand already or the own list is known to be empty
+      arr_drawn = arr_held == -1 && ((arr_dead >> arr_my_x) & 1) == 0;
+      if (arr_drawn) arr_t = arr_draw(arr_my_x);
+    }
     lds_u8 const epi = smem + wave * C::kEpiBytes;
     // The epilogue's lane-dependent addresses are the same for every tile; computed from these opaque copies they are
     // rebuilt per tile (a few dozen instructions) instead of being held in ~100 registers across the K loop.
@@ -1333,10 +1526,29 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       store_rows(0, C::kWaveM);
     }
+    if (arrival) {
+      // the next tile, by the look taken when the epilogue began (wave 0 is done reading its staging rows, which is
+      // where the gate words lie)
+      if (wave == 0) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int next = arr_next(arr_flag, arr_cnt, arr_drawn, arr_t);
+        if (lane == 0) s_gate[0] = next;
+      }
+      arr_decided = true;
+    }
     // the next tile's prologue overwrites the ring: every wave must be done reading its staging area
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   }
-  // ---- leave: the last workgroup out advances the workspace's tag base for the next launch -------------------
+  // ---- leave: the last workgroup out puts the ticket counters back to zero for the next launch ------------------
+  if (!kGrouped && p.sched_ctrl != nullptr && threadIdx.x == 0) {
+    int32_t* const done = p.sched_ctrl + kSchedDone;
+    if (__hip_atomic_fetch_add(done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == G - 1) {
+      for (int x = 0; x < kSchedMaxXcds; ++x)
+        __hip_atomic_store(p.sched_ctrl + kSchedCounters + x * kSchedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(done, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  // ---- the last workgroup out advances the workspace's tag base for the next launch --------------------------
   if (p.sk_mode != 0 && threadIdx.x == 0) {
     int32_t* const done = p.sk_ctrl + kSkCtrlDone;
     if (__hip_atomic_fetch_add(done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == G - 1) {
@@ -1552,6 +1764,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   p.sk_partials = nullptr;
   p.sk_mode = 0;
   p.sk_l2_local = 0;
+  p.sched_ctrl = nullptr;
   p.k_tail_bytes = k_tail_bytes;
 
   if (c.scatter_bufs) {
@@ -1609,6 +1822,11 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (use_sk) {
     grid = cap_wgs;
     sk_attach(p, c.sk_workspace, 1);
+  } else if (c.flags && !c.scatter_bufs && !ragged && c.sk_workspace != nullptr && p.n_chunks <= kSchedMaxChunks &&
+             sched > grid && debug_get(TDIST_DEBUG_GEMM_SCHEDULE) != 0) {
+    // gated, whole-tile chunks, more than one round of tiles, a workspace for the ticket counters: tiles in arrival
+    // order (a single round is static either way: every workgroup owns its one tile)
+    p.sched_ctrl = (int32_t*)c.sk_workspace + kSchedOff;
   }
   const bool scales = elem == kElemFP8 && (c.row_scale || c.col_scale);
 
@@ -1751,6 +1969,7 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   p.sk_partials = nullptr;
   p.sk_mode = 0;
   p.sk_l2_local = 0;
+  p.sched_ctrl = nullptr;
   p.gate_rows = p.m_per_chunk;
   p.k_tail_bytes = 0;
 

@@ -156,10 +156,12 @@ struct PushParams {
   const unsigned char* const* peer_src;  // [world] device pointers; the entry of `rank` is not read
   int32_t* flags;
   int32_t* counters;                     // [world * chunks_per_rank], zero on entry, left zero
-  const int32_t* held;                   // optional [world * chunks_per_rank]: non-zero = never deliver (test hook)
+  const int32_t* held;                   // optional [world * chunks_per_rank]: > 0 = never deliver, < 0 = deliver that many
+                                         // microseconds late (test and measurement hooks)
   const unsigned long long* stamp;       // optional: wall-clock stamp of the op's start
   unsigned long long ticks_per_chunk;
   unsigned long long max_delay_ticks;    // > 0: seeded random extra delay per (peer, chunk), see producer_delay_ticks
+  unsigned long long ticks_per_us;       // wall-clock ticks per microsecond (for the per-chunk delays in `held`)
   uint32_t delay_seed;
   long long chunk_bytes, rank_bytes;
   int world, rank, chunks_per_rank, flag_value;
@@ -187,7 +189,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(24))) void prod
   }
   for (int c = 0; c < p.chunks_per_rank; ++c) {
     const int chunk_pos = r * p.chunks_per_rank + c;
-    if (p.held != nullptr && p.held[chunk_pos] != 0) continue;
+    const int hold = p.held != nullptr ? p.held[chunk_pos] : 0;
+    if (hold > 0) continue;
     // Pacing: over a link the last byte of the peer's chunk c lands (c+1) chunk times after the start. The rows
     // are therefore copied when their turn comes (they are "on the wire" once chunk c-1 is through) and the flag is
     // held back until the chunk's arrival time: what the consumer sees is a chunk that is complete at that time.
@@ -202,11 +205,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(24))) void prod
       }
       __syncthreads();
     }
-    if (p.max_delay_ticks != 0) {
+    if (p.max_delay_ticks != 0 || hold < 0) {
       if (threadIdx.x == 0) {
-        const unsigned long long hold = producer_delay_ticks(p.delay_seed, chunk_pos, p.max_delay_ticks);
+        unsigned long long wait = p.max_delay_ticks != 0 ? producer_delay_ticks(p.delay_seed, chunk_pos, p.max_delay_ticks) : 0;
+        if (hold < 0) wait += (unsigned long long)(-(long long)hold) * p.ticks_per_us;   // a straggler: this chunk is late by -hold us
         const unsigned long long from = wall_clock64();
-        while (wall_clock64() - from < hold) __builtin_amdgcn_s_sleep(16);   // (ends by itself: the clock only moves forward)
+        while (wall_clock64() - from < wait) __builtin_amdgcn_s_sleep(16);   // (ends by itself: the clock only moves forward)
       }
       __syncthreads();
     }
@@ -374,6 +378,12 @@ int tdist_producer_push_peers(void* workspace, const void* const* peer_src, int 
     p.ticks_per_chunk = (unsigned long long)((double)ns_per_chunk * 1e-6 * (double)khz);
   }
   p.max_delay_ticks = 0;
+  p.ticks_per_us = 0;
+  if (held != nullptr) {
+    const int khz = wall_clock_khz();
+    if (khz <= 0) return fail(TDIST_ERR_DEVICE, "%s: cannot read the wall clock rate", who);
+    p.ticks_per_us = (unsigned long long)khz / 1000ull;
+  }
   p.delay_seed = delay_seed;
   if (max_delay_ns < 0 || max_delay_ns * cpr > 100000000)
     return fail(TDIST_ERR_INVALID, "%s: max_delay_ns %lld x %lld chunks outside [0, 100 ms]", who, (long long)max_delay_ns, (long long)cpr);

@@ -85,11 +85,17 @@ def kernel_producer_all_gather_push(rank, num_ranks, ctx, workspace, M_PER_CHUNK
     if ctx.producer_counters is None or ctx.producer_counters.numel() < n_chunks:
         ctx.producer_counters = torch.zeros(n_chunks, dtype=torch.int32, device=some.device)
     held = None
-    if ctx.held_chunks:
-        held = torch.zeros(n_chunks, dtype=torch.int32)
-        held[list(int(c) for c in ctx.held_chunks)] = 1
-        held = held.to(some.device)
-    ctx.held_mask = held   # stays alive until the next call replaces it
+    if ctx.held_chunks or ctx.late_chunks_us:
+        key = (tuple(ctx.held_chunks), tuple(sorted(ctx.late_chunks_us.items())), n_chunks)
+        if ctx.held_mask_key != key:
+            held = torch.zeros(n_chunks, dtype=torch.int32)
+            for c, us in ctx.late_chunks_us.items():
+                held[int(c)] = -min(int(us), 100000)
+            held[list(int(c) for c in ctx.held_chunks)] = 1
+            ctx.held_mask, ctx.held_mask_key = held.to(some.device), key
+        held = ctx.held_mask
+    else:
+        ctx.held_mask, ctx.held_mask_key = None, None
     paced = ctx.link_gbps > 0
     nbytes = M_PER_CHUNK * K * esz
     # race provocation: a new seed per call, so every call sees another pattern of late chunks
@@ -154,6 +160,10 @@ class AllGatherGEMMTensorParallelContext:
     producer_counters: Optional[torch.Tensor] = None
     peer_ptrs: Optional[torch.Tensor] = None   # int64[num_ranks] device array of the peer shards' addresses
     held_mask: Optional[torch.Tensor] = None
+    held_mask_key: Optional[tuple] = None
+    # kernel producer only: global chunk id -> microseconds by which that chunk is copied late (a straggler: the same
+    # peer's later chunks follow behind it)
+    late_chunks_us: Dict[int, float] = dataclasses.field(default_factory=dict)
     # Compute units the gated GEMM leaves to the producer's copies. On one GPU those copies need compute
     # units of this GPU; measured on MI355X they make no progress next to a full-chip persistent grid
     # unless 32 units stay free. A peer's copy engine pushing over xGMI would need none.
