@@ -319,7 +319,9 @@ def bench_c4(dev, steps, warmup):
     def index_then_dispatch():
         _, cs, sc, _ = moe_dispatch_preprocess(ids_d, G, ctx=ctx)
         fast_all_to_all(ctx, q_d, cs, s_d, scatter_index=sc)
-    both_s = time_launches(index_then_dispatch, steps, warmup)
+    two_s = time_launches(index_then_dispatch, steps, warmup)
+    # the same from the raw ids in ONE launch: every workgroup of the dispatch counts the ids itself
+    both_s = time_launches(lambda: fast_all_to_all(ctx, q_d, None, s_d, expert_ids=ids_d), steps, warmup)
     _, recv, recv_scale = fast_all_to_all(ctx, q_d, cumsum, s_d, scatter_index=scatter)
     comb_s = time_launches(lambda: moe_weighted_combine(ctx, recv, recv_scale, scatter, w, cumsum), steps, warmup)
     n = T * topk
@@ -338,7 +340,8 @@ def bench_c4(dev, steps, warmup):
     # the dispatch end to end: splits / cumsum / scatter index from the raw expert ids (one launch, the context's own
     # tensors, no allocation), then the row movement; the ids' 131 KB are added to the bytes
     d["with_index_build"] = {"us": round(both_s * 1e6, 2), "achieved_GBps": round((disp_bytes + n * 4) / both_s / 1e9, 1),
-                             "frac": round((disp_bytes + n * 4) / both_s / PEAK["hbm"], 4)}
+                             "frac": round((disp_bytes + n * 4) / both_s / PEAK["hbm"], 4),
+                             "as_two_launches_us": round(two_s * 1e6, 2)}
     # the step after the dispatch: align / sort of the same ids for the grouped GEMM (8 rank segments, block 128)
     from triton_dist.kernels.amd import sort_topk_ids_align_block_size
     ids64 = ids_d.long()

@@ -295,6 +295,21 @@ int tdist_moe_dispatch_tokens(const void* tokens, int64_t row_bytes, const float
                               int world_size, int experts_per_rank, int max_m, void* slot_rows, float* slot_scales,
                               int32_t* splits_out, void* stream);
 
+/* tdist_moe_scatter_index and tdist_moe_dispatch_tokens in ONE launch, for a decode step's worth of tokens: the
+ * reference prepares the index tensors with several torch calls and then launches its kernel
+ * (test/nvidia/test_all_to_all.py:314-329, kernels/nvidia/low_latency_all_to_all.py:189-248); here every workgroup of
+ * the dispatch counts all ids itself while its rows are being fetched, so the rows are placed without a separate
+ * index launch and without a workspace. ids int32[n_tokens*topk] (values outside [0, G) take no place: scatter index
+ * -1, row not sent). Outputs: the slots as tdist_moe_dispatch_tokens writes them, splits_out (may be NULL), and the
+ * index tensors as tdist_moe_scatter_index writes them: splits int32[G] (may be NULL), cumsum int32[G+1], scatter_idx
+ * int32[n_tokens*topk], gather_idx int32[n_tokens*topk]. Limits (TDIST_ERR_UNSUPPORTED beyond them: use the two calls):
+ * n_tokens*topk <= 65536, rows of 1, 2, 4, 8 or 16 windows of 8 KB. */
+int tdist_moe_dispatch_tokens_from_ids(const void* tokens, int64_t row_bytes, const float* token_scales,
+                                       const int32_t* ids, int topk, int64_t n_tokens, int world_size,
+                                       int experts_per_rank, int max_m, void* slot_rows, float* slot_scales,
+                                       int32_t* splits_out, int32_t* splits, int32_t* cumsum, int32_t* scatter_idx,
+                                       int32_t* gather_idx, void* stream);
+
 /* Compaction of the slots into one [sum, row_bytes] tensor in destination order
  * (all_to_all_post_process, low_latency_all_to_all.py:251-270): output row p comes from slot row
  * d*max_m + (p - start_d) where start_d = sum of splits of destinations < d.

@@ -141,7 +141,9 @@ def test_splits_cumsum_entry_point(cuda):
                                                      (50, 3, 6, 2, 24, 40, "tokens"), (10, 2, 8, 8, 1024, 8, True),
                                                      (10, 2, 8, 8, 1024, 8, "tokens"), (33, 5, 8, 2, 12000, 128, "tokens"),
                                                      (21, 3, 4, 4, 52, 64, "tokens"), (300, 4, 128, 64, 64, 48, "tokens"),
-                                                     (300, 4, 126, 63, 64, 48, "tokens"), (300, 4, 160, 80, 64, 48, "tokens")])
+                                                     (300, 4, 126, 63, 64, 48, "tokens"), (300, 4, 160, 80, 64, 48, "tokens"),
+                                                     (4096, 8, 256, 32, 7168, 4096, "ids"), (96, 4, 16, 4, 48, 160, "ids"), (50, 3, 6, 2, 24, 40, "ids"), (10, 2, 8, 8, 1024, 8, "ids"), (33, 5, 8, 2, 12000, 128, "ids"), (21, 3, 4, 4, 52, 64, "ids"), (300, 4, 128, 64, 64, 48, "ids"), (300, 4, 126, 63, 64, 48, "ids"), (300, 4, 160, 80, 64, 48, "ids"), (33, 5, 8, 2, 20000, 128, "ids"), (77, 3, 12, 4, 40000, 64, "ids"), (100, 7, 30, 5, 200, 300, "ids"),
+                                                     (20, 2, 4, 2, 30000, 32, "ids"), (9000, 8, 64, 8, 64, 9100, "ids")])
 def test_dispatch_bytes_bit_exact_and_round_trip(cuda, T, topk, G, W, H, max_m, fused):
     from triton_dist.kernels.amd import (all_to_all_post_process, create_all_to_all_context, fast_all_to_all,
                                          moe_dispatch_preprocess)
@@ -152,7 +154,13 @@ def test_dispatch_bytes_bit_exact_and_round_trip(cuda, T, topk, G, W, H, max_m, 
     ctx.recv_buf.view(torch.uint8).fill_(0xAB)
     splits, cumsum, scatter, gather = moe_dispatch_preprocess(ids.to(cuda), G)
     dq, ds = q.to(cuda), s.to(cuda)
-    if fused == "tokens":
+    if fused == "ids":
+        # straight from the raw expert ids (int64, as torch.topk gives them): index build and dispatch in one launch
+        out_splits, recv, recv_scale = fast_all_to_all(ctx, dq, None, ds, expert_ids=ids.long().to(cuda))
+        torch.cuda.synchronize()
+        for got_t, want_t in zip(ctx.last_index, golden.moe_preprocess(ids, G)[:4]):
+            assert torch.equal(got_t.cpu(), want_t), "index tensors written by the dispatch"
+    elif fused == "tokens":
         out_splits, recv, recv_scale = fast_all_to_all(ctx, dq, cumsum, ds, scatter_index=scatter)
     elif fused:
         out_splits, recv, recv_scale = fast_all_to_all(ctx, dq, cumsum, ds, gather_index=gather)
@@ -178,6 +186,35 @@ def test_dispatch_bytes_bit_exact_and_round_trip(cuda, T, topk, G, W, H, max_m, 
         torch.cuda.synchronize()
         assert torch.equal(out.view(torch.uint8).cpu(), sorted_rows)
         assert torch.equal(out_scale.cpu(), sorted_scales)
+
+
+def test_dispatch_from_ids_matches_the_two_calls_with_ids_out_of_range(cuda):
+    """The one-launch form against index build + token-major dispatch on ids of which some lie outside [0, G) (they
+    take no place and their rows are not sent) and some repeat within a token: the same slot bytes, scales, splits and
+    index tensors; three calls in a row on one context (its two sets of index tensors and receive buffers in turn)."""
+    from triton_dist.kernels.amd import create_all_to_all_context, fast_all_to_all, moe_dispatch_preprocess
+    announce("moe dispatch from ids, ids out of range")
+    T, topk, G, W, H, max_m = 333, 6, 24, 4, 272, 700
+    g = torch.Generator().manual_seed(4)
+    ctx_a = create_all_to_all_context(max_m, H, 0, G, W, G // W, dtype=torch.float8_e4m3fn)
+    ctx_b = create_all_to_all_context(max_m, H, 0, G, W, G // W, dtype=torch.float8_e4m3fn)
+    for call in range(3):
+        ids = torch.randint(-2, G + 3, (T, topk), generator=g).to(torch.int32)
+        q, s_ = golden.quantize_per_token_e4m3(torch.randn((T, H), generator=g))
+        for ctx in (ctx_a, ctx_b):
+            ctx.recv_buf.view(torch.uint8).fill_(0xAB)
+            ctx.scale_recv_buf.fill_(-1.0)
+        dq, ds, dids = q.to(cuda), s_.to(cuda), ids.to(cuda)
+        splits, cumsum, scatter, gather = moe_dispatch_preprocess(dids, G, ctx=ctx_a)
+        want = fast_all_to_all(ctx_a, dq, cumsum, ds, scatter_index=scatter)
+        got = fast_all_to_all(ctx_b, dq, None, ds, expert_ids=dids)
+        torch.cuda.synchronize()
+        n_valid = int(cumsum[-1])
+        for a, b in zip(got, want):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), "call %d" % call
+        i_splits, i_cumsum, i_scatter, i_gather = ctx_b.last_index
+        assert torch.equal(i_splits, splits) and torch.equal(i_cumsum, cumsum) and torch.equal(i_scatter, scatter)
+        assert torch.equal(i_gather[:n_valid], gather[:n_valid])
 
 
 def test_dispatch_bf16_rows_without_scales_and_odd_row_bytes(cuda):

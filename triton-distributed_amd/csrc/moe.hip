@@ -654,6 +654,181 @@ __global__ __launch_bounds__(256) void moe_dispatch_tokens_kernel(const unsigned
   }
 }
 
+// ---- dispatch straight from the expert ids: index build and row movement in one launch ---------------------------
+// For a decode step's worth of ids (up to kFusedDispatchMaxIds) the index build is cheaper redone by everybody than
+// waited for: as in the recounting form of moe_index_fused_kernel, every workgroup counts ALL ids itself (its own
+// tokens' per wave, the ids in front of its range and behind it into two more rows of LDS counters), so it knows the
+// splits, their prefix sums and the rank of each of its own (token, k) entries without any exchange, and can place its
+// rows at once. The row loads go out before the counting starts, so the counting runs while they are in flight. As
+// by-products the workgroups write what tdist_moe_scatter_index writes: scatter_idx and gather_idx for their own
+// entries, workgroup 0 the splits and cumsum.
+// A workgroup is kFdWaves waves; wave w stands for (token, 8 KB window) unit w of the workgroup, as in
+// moe_dispatch_tokens_kernel. The window-0 wave of a token counts and ranks that token's ids.
+constexpr int kFdWaves = 16, kFdThreads = kFdWaves * 64;
+constexpr int64_t kFusedDispatchMaxIds = 65536;
+
+template <bool kVec16>
+__global__ __launch_bounds__(kFdThreads) void moe_dispatch_fused_kernel(
+    const unsigned char* __restrict__ tokens, int64_t row_bytes, const float* __restrict__ scales,
+    const int32_t* __restrict__ ids, int topk, int64_t n_tokens, int G, int nbits, int W, int Er, int max_m, int windows,
+    unsigned char* __restrict__ slot_rows, float* __restrict__ slot_scales, int32_t* __restrict__ splits_out,
+    int32_t* __restrict__ splits, int32_t* __restrict__ cumsum, int32_t* __restrict__ scatter_idx,
+    int32_t* __restrict__ gather_idx) {
+  // [3][G] counters: ids in front of this workgroup's range, its own, ids behind it; [G + 1] expert starts (cumsum);
+  // then this workgroup's own ids in flat order, padded to a multiple of four with -1
+  extern __shared__ int32_t s_fd[];
+  int32_t* const s_before = s_fd;
+  int32_t* const s_own = s_fd + G;
+  int32_t* const s_behind = s_fd + 2 * G;
+  int32_t* const s_start = s_fd + 3 * G;
+  int32_t* const s_ids = s_start + ((G + 1 + 3) & ~3);
+  __shared__ int32_t s_part[kFdWaves];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tokens_per_block = kFdWaves / windows;
+  const int64_t unit = (int64_t)blockIdx.x * kFdWaves + wave;
+  const int64_t t = unit / windows;
+  const int win = (int)(unit - t * windows);
+  const bool live = t < n_tokens;
+  // 1. this token's ids, and everybody else's four at a time
+  const int64_t n = n_tokens * topk;
+  const int own_n = tokens_per_block * topk;
+  const int64_t own_lo = (int64_t)blockIdx.x * own_n, own_hi = own_lo + own_n;
+  const int own_f = (wave / windows) * topk + lane;   // this lane's entry among the workgroup's own, in flat order
+  int e = -1;
+  if (live && lane < topk) e = ids[t * topk + lane];
+  if (e < 0 || e >= G) e = -1;
+  constexpr int kBatch = 8;
+  const int64_t n_vec = (n + 3) / 4;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(ids) & 15u) == 0;
+  int4v q[kBatch];
+  auto load_others = [&](int64_t v0) {
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t vi = v0 + (int64_t)u * kFdThreads;
+      q[u] = int4v{-1, -1, -1, -1};
+      if (vi < n_vec) {
+        if (vec_ok && vi * 4 + 3 < n) q[u] = ((const int4v*)ids)[vi];
+        else
+          for (int j = 0; j < 4; ++j) q[u][j] = vi * 4 + j < n ? ids[vi * 4 + j] : -1;
+      }
+    }
+  };
+  auto count_others = [&](int64_t v0) {
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t vi = v0 + (int64_t)u * kFdThreads;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t i = vi * 4 + j;
+        const int x = q[u][j];
+        if (x >= 0 && x < G && (i < own_lo || i >= own_hi)) atomicAdd(i < own_lo ? &s_before[x] : &s_behind[x], 1);
+      }
+    }
+  };
+  load_others(threadIdx.x);
+  // the row's loads go out behind the ids' (loads return in order, and the counting only needs the ids: it runs while
+  // the row is on its way)
+  const int n16 = (int)(row_bytes >> 4);
+  const int base = win * 512;
+  int4v v[8];
+  if (kVec16 && live) {
+    const int4v* s16 = (const int4v*)(tokens + t * row_bytes);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = base + j * 64 + lane;
+      if (c < n16) v[j] = s16[c];
+    }
+  }
+  for (int g = threadIdx.x; g < 3 * G; g += kFdThreads) s_fd[g] = 0;
+  if (win == 0 && lane < topk) s_ids[own_f] = e;
+  if (threadIdx.x < 4) s_ids[own_n + threadIdx.x] = -1;
+  __syncthreads();
+  if (e >= 0 && win == 0) atomicAdd(&s_own[e], 1);
+  count_others(threadIdx.x);
+  for (int64_t v0 = threadIdx.x + (int64_t)kBatch * kFdThreads; v0 < n_vec; v0 += (int64_t)kBatch * kFdThreads) {
+    load_others(v0);
+    count_others(v0);
+  }
+  __syncthreads();
+  // 3. the splits (ids in front + own + behind) and their exclusive scan over the experts: consecutive experts per
+  // thread, the threads' totals within the wave by shuffles, the waves' through LDS
+  const int per = (G + kFdThreads - 1) / kFdThreads;
+  const int g0 = threadIdx.x * per;
+  int32_t local_total = 0;
+  for (int j = 0; j < per; ++j)
+    if (g0 + j < G) local_total += s_before[g0 + j] + s_own[g0 + j] + s_behind[g0 + j];
+  int32_t incl = local_total;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int32_t up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) s_part[wave] = incl;
+  __syncthreads();
+  int32_t acc = incl - local_total;
+#pragma unroll
+  for (int w = 0; w < kFdWaves; ++w) acc += w < wave ? s_part[w] : 0;
+  if (threadIdx.x == 0 && blockIdx.x == 0) cumsum[0] = 0;
+  for (int j = 0; j < per; ++j) {
+    const int g = g0 + j;
+    if (g < G) {
+      const int32_t c = s_before[g] + s_own[g] + s_behind[g];
+      if (blockIdx.x == 0) {
+        if (splits) splits[g] = c;
+        if (splits_out) splits_out[g] = c;
+        cumsum[g + 1] = acc + c;
+      }
+      s_start[g] = acc;
+      acc += c;
+    }
+  }
+  __syncthreads();
+  if (!live) return;
+  // 4. the sorted position of this token's k-th entry (lane k): the expert's start, the ids in front of the workgroup's
+  // range, and the workgroup's own entries before this one in flat order; then its slot row
+  int32_t my_dst = -1;
+  if (e >= 0) {
+    int32_t earlier = 0;
+    for (int f = 0; f < own_f; f += 4) {
+      const int4v o = *(const int4v*)(s_ids + f);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) earlier += (f + j < own_f && o[j] == e) ? 1 : 0;
+    }
+    const int32_t p = s_start[e] + s_before[e] + earlier;
+    if (win == 0) {
+      scatter_idx[t * topk + lane] = p;
+      gather_idx[p] = (int32_t)t;
+    }
+    const int d = e / Er;
+    const int32_t in_slot = p - s_start[d * Er];
+    if (in_slot < max_m) my_dst = d * max_m + in_slot;
+    if (win == 0 && my_dst >= 0 && scales) slot_scales[my_dst] = scales[t];
+  } else if (lane < topk && win == 0) {
+    scatter_idx[t * topk + lane] = -1;
+  }
+  // 5. the copies
+  if (kVec16) {
+    for (int k = 0; k < topk; ++k) {
+      const int32_t dst_row = __shfl(my_dst, k);
+      if (dst_row < 0) continue;
+      int4v* d16 = (int4v*)(slot_rows + (int64_t)dst_row * row_bytes);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int c = base + j * 64 + lane;
+        if (c < n16) __builtin_nontemporal_store(v[j], d16 + c);
+      }
+    }
+  } else {
+    const unsigned char* src = tokens + t * row_bytes;
+    for (int k = 0; k < topk; ++k) {
+      const int32_t dst_row = __shfl(my_dst, k);
+      if (dst_row < 0) continue;
+      unsigned char* dst = slot_rows + (int64_t)dst_row * row_bytes;
+      for (int64_t c = (int64_t)win * 8192 + lane; c < row_bytes && c < (int64_t)(win + 1) * 8192; c += 64) dst[c] = src[c];
+    }
+  }
+}
+
 // ---- online e4m3 quantisation in groups of 128 columns -----------------------------------------------------
 // Follows _quant_kernel of the reference's tutorials/04-deepseek-infer-all2all.py (:309-329) and its fused form in
 // the dispatch kernel (:180-200): per group, scale = max|x| (as fp32) * fp32(1/448), q = e4m3(float(x) / scale).
@@ -1157,6 +1332,45 @@ int tdist_moe_dispatch_tokens(const void* tokens, int64_t row_bytes, const float
                      (const unsigned char*)tokens, row_bytes, token_scales, scatter_idx, topk, cumsum, n_tokens,
                      world_size, experts_per_rank, max_m, (unsigned char*)slot_rows, slot_scales, splits_out, windows);
   return launch_status("tdist_moe_dispatch_tokens");
+}
+
+int tdist_moe_dispatch_tokens_from_ids(const void* tokens, int64_t row_bytes, const float* token_scales,
+                                       const int32_t* ids, int topk, int64_t n_tokens, int world_size,
+                                       int experts_per_rank, int max_m, void* slot_rows, float* slot_scales,
+                                       int32_t* splits_out, int32_t* splits, int32_t* cumsum, int32_t* scatter_idx,
+                                       int32_t* gather_idx, void* stream) {
+  const char* who = "tdist_moe_dispatch_tokens_from_ids";
+  if (!tokens || !ids || !slot_rows || !cumsum || !scatter_idx || !gather_idx) return fail(TDIST_ERR_INVALID, "%s: null pointer", who);
+  if ((token_scales != nullptr) != (slot_scales != nullptr))
+    return fail(TDIST_ERR_INVALID, "%s: token_scales and slot_scales go together", who);
+  if (row_bytes <= 0 || n_tokens < 0 || world_size <= 0 || experts_per_rank <= 0 || max_m <= 0 || topk <= 0)
+    return fail(TDIST_ERR_INVALID, "%s: bad sizes", who);
+  if (topk > 64) return fail(TDIST_ERR_UNSUPPORTED, "%s: topk > 64", who);
+  const int64_t G64 = (int64_t)world_size * experts_per_rank;
+  if (G64 > kMoeMaxExperts) return fail(TDIST_ERR_UNSUPPORTED, "%s: num_experts %lld > %d", who, (long long)G64, kMoeMaxExperts);
+  if ((int64_t)world_size * max_m > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: world_size * max_m too large", who);
+  const int G = (int)G64;
+  const int windows = (int)ceil_div(row_bytes, 8192);
+  const int64_t lds = ((int64_t)3 * G + ((G + 1 + 3) & ~3) + kFdWaves * topk + 4) * 4;
+  if (n_tokens * topk > kFusedDispatchMaxIds || windows > kFdWaves || kFdWaves % windows != 0 || lds > 160 * 1024 - 256)
+    return fail(TDIST_ERR_UNSUPPORTED, "%s: more than %lld ids, rows above %d bytes (or no power-of-two number of 8 KB windows), or too "
+                "many experts for one workgroup's counters: use tdist_moe_scatter_index + tdist_moe_dispatch_tokens", who,
+                (long long)kFusedDispatchMaxIds, kFdWaves * 8192);
+  const int64_t units = (n_tokens > 0 ? n_tokens : 1) * windows;
+  const int64_t blocks = ceil_div(units, kFdWaves);
+  const bool vec = (row_bytes % 16 == 0) && aligned16(tokens) && aligned16(slot_rows);
+  auto kern = vec ? moe_dispatch_fused_kernel<true> : moe_dispatch_fused_kernel<false>;
+  static bool attr_set[2] = {false, false};
+  if (!attr_set[vec]) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256) != hipSuccess)
+      return fail(TDIST_ERR_LAUNCH, "%s: cannot reserve LDS", who);
+    attr_set[vec] = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kFdThreads), (size_t)lds, (hipStream_t)stream,
+                     (const unsigned char*)tokens, row_bytes, token_scales, ids, topk, n_tokens, G, id_bits(G), world_size,
+                     experts_per_rank, max_m, windows, (unsigned char*)slot_rows, slot_scales, splits_out, splits, cumsum,
+                     scatter_idx, gather_idx);
+  return launch_status(who);
 }
 
 int tdist_moe_post_process(const void* slot_rows, int64_t row_bytes, const float* slot_scales, const int32_t* splits,

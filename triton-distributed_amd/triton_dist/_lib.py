@@ -61,6 +61,7 @@ PROTOTYPES = {
     "tdist_moe_scatter_index_static": (_I, [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P]),
     "tdist_moe_dispatch": (_I, [_P, _L, _P, _P, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
     "tdist_moe_dispatch_tokens": (_I, [_P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _P, _P, _P, _P]),
+    "tdist_moe_dispatch_tokens_from_ids": (_I, [_P, _L, _P, _P, _I, _L, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]),
     "tdist_moe_post_process": (_I, [_P, _L, _P, _P, _L, _I, _I, _I, _P, _P, _P]),
     "tdist_moe_combine": (_I, [_P, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P, _P]),
     "tdist_quant_e4m3_groups": (_I, [_P, _L, _I, _I, _P, _P, _P]),

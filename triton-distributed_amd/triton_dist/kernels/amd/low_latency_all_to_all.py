@@ -81,6 +81,7 @@ class AllToAllContext:
         # index tensors of moe_dispatch_preprocess(..., ctx=self): two sets, allocated on first use for a shape
         self.index_sets, self.index_key, self.index_calls = None, None, 0
         self.index_workspace, self.index_args, self.index_ids = None, None, None
+        self.last_index = None   # (splits, split_cumsum, scatter_idx, gather_idx) of the last fast_all_to_all(expert_ids=)
 
 
 def create_all_to_all_context(
@@ -122,6 +123,39 @@ def splits_to_cumsum(splits: torch.Tensor):
     return out
 
 
+def _ensure_index_sets(ctx, T, topk, num_experts, dev):
+    """The context's own index tensors for a (T, topk, num_experts) shape: two sets of (splits, cumsum, scatter_idx,
+    gather_idx, topk_idx) used in turn, a zeroed workspace and an int32 staging tensor for ids of another dtype,
+    allocated when the shape is first seen (the calls of one context are ordered on its stream, so they may share
+    them)."""
+    if ctx.index_key == (T, topk, num_experts, dev):
+        return
+    n = T * topk
+
+    def alloc():
+        return (torch.empty(num_experts, dtype=torch.int32, device=dev),
+                torch.empty(num_experts + 1, dtype=torch.int32, device=dev),
+                torch.empty((T, topk), dtype=torch.int32, device=dev),
+                torch.empty(n, dtype=torch.int32, device=dev),
+                torch.empty(n, dtype=torch.int32, device=dev))
+
+    ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
+    ctx.index_sets, ctx.index_key, ctx.index_calls = [alloc(), alloc()], (T, topk, num_experts, dev), 0
+    ctx.index_workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+    ctx.index_ids = torch.empty((T, topk), dtype=torch.int32, device=dev)
+    ctx.index_args = [((n, topk, num_experts, t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), t[3].data_ptr()),
+                       (ctx.index_workspace.data_ptr(), ws_bytes)) for t in ctx.index_sets]
+
+
+def _staged_ids(ctx, exp_indices):
+    """Ids as contiguous int32: as they are, or converted into the context's staging tensor (torch.topk gives int64):
+    one copy kernel, no allocation."""
+    if exp_indices.dtype != torch.int32 or not exp_indices.is_contiguous():
+        ctx.index_ids.copy_(exp_indices)
+        return ctx.index_ids
+    return exp_indices
+
+
 def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_topk_index: bool = False,
                             ctx: Optional[AllToAllContext] = None):
     """GPU version of the reference test's index preparation (test/nvidia/test_all_to_all.py:314-320):
@@ -147,23 +181,12 @@ def moe_dispatch_preprocess(exp_indices: torch.Tensor, num_experts: int, want_to
                 torch.empty(n, dtype=torch.int32, device=dev))
 
     if ctx is not None:
-        if ctx.index_key != (T, topk, num_experts, dev):
-            # a new shape: two sets of result tensors, a zeroed workspace and an int32 staging tensor for ids of
-            # another dtype, all the context's own (the calls of one context are ordered on its stream, so they may
-            # share them)
-            ws_bytes = _lib.load().tdist_moe_workspace_bytes(n, num_experts)
-            ctx.index_sets, ctx.index_key, ctx.index_calls = [alloc(), alloc()], (T, topk, num_experts, dev), 0
-            ctx.index_workspace = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
-            ctx.index_ids = torch.empty((T, topk), dtype=torch.int32, device=dev)
-            ctx.index_args = [((n, topk, num_experts, t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(), t[3].data_ptr()),
-                               (ctx.index_workspace.data_ptr(), ws_bytes)) for t in ctx.index_sets]
+        _ensure_index_sets(ctx, T, topk, num_experts, dev)
         # the context has seen this shape: its tensors' addresses are at hand and the host does next to nothing (the
         # index kernel takes ~9 us on the device; a general path costs more than that on the host). Ids that are not
         # contiguous int32 (torch.topk gives int64) are converted into the context's staging tensor: one copy kernel,
         # no allocation.
-        if exp_indices.dtype != torch.int32 or not exp_indices.is_contiguous():
-            ctx.index_ids.copy_(exp_indices)
-            exp_indices = ctx.index_ids
+        exp_indices = _staged_ids(ctx, exp_indices)
         which = ctx.index_calls % 2
         ctx.index_calls += 1
         out = ctx.index_sets[which]
@@ -195,6 +218,7 @@ def fast_all_to_all(
     gather_index: Optional[torch.Tensor] = None,
     scatter_index: Optional[torch.Tensor] = None,
     online_quant_fp8: bool = False,
+    expert_ids: Optional[torch.Tensor] = None,
 ):
     """
     low-latency all-to-all communication (reference :189-248).
@@ -211,10 +235,20 @@ def fast_all_to_all(
     row is quantised to e4m3 in groups of 128 columns while it is dispatched, ``send_scale`` must be None and the
     scales returned are [W*max_m, hidden/128].
 
+    With ``expert_ids`` ([T, topk] integer tensor, an addition; ``send_split_cumsum`` may then be None) the call starts
+    from the router's raw expert ids: for up to 65536 of them the index build (moe_dispatch_preprocess) runs inside the
+    dispatch's one launch, beyond that in a launch of its own in front of it. ``send_tensor`` is the unsorted
+    [T, hidden] token tensor. The index tensors land in the context's own (two sets in turn, as the receive buffers)
+    and are kept as ``ctx.last_index`` = (splits, split_cumsum, scatter_idx, gather_idx) for the combine.
+
     Returns [splits int32[G], recv [W*max_m, hidden], scales [W*max_m] | None] — views into the context's
     buffers, valid until the call after next.
     """
-    _lib.require_cuda(send_tensor, send_split_cumsum, send_scale, gather_index, scatter_index)
+    _lib.require_cuda(send_tensor, send_split_cumsum, send_scale, gather_index, scatter_index, expert_ids)
+    if expert_ids is not None:
+        if online_quant_fp8 or gather_index is not None or scatter_index is not None:
+            raise ValueError("expert_ids replaces gather_index / scatter_index and does not combine with online_quant_fp8")
+        return _fast_all_to_all_from_ids(ctx, send_tensor, send_scale, expert_ids)
     if online_quant_fp8:
         return _fast_all_to_all_online_quant(ctx, send_tensor, send_split_cumsum, send_scale, scatter_index)
     if ctx.fp8_group_size:
@@ -260,6 +294,48 @@ def fast_all_to_all(
     out_lis = [splits, recv]
     out_lis.append(scale_recv if with_scale else None)
     return out_lis
+
+
+FUSED_INDEX_MAX_IDS = 65536   # tdist_moe_dispatch_tokens_from_ids takes up to this many ids
+
+
+def _fast_all_to_all_from_ids(ctx, send_tensor, send_scale, expert_ids):
+    if ctx.fp8_group_size:
+        raise ValueError("a context with group scales takes its rows through online_quant_fp8=True")
+    assert send_tensor.dim() == 2 and send_tensor.shape[1] == ctx.hidden and send_tensor.dtype == ctx.dtype
+    T, topk = expert_ids.shape
+    assert T == send_tensor.shape[0]
+    G = ctx.num_tot_experts
+    row_bytes = ctx.hidden * ctx.ele_size
+    windows = -(-row_bytes // 8192)
+    fused = (T * topk <= FUSED_INDEX_MAX_IDS and windows in (1, 2, 4, 8, 16) and topk <= 64
+             and (4 * G + 16 * topk + 8) * 4 <= 160 * 1024 - 256)
+    if not fused:
+        splits_i, cumsum, scatter, gather = moe_dispatch_preprocess(expert_ids, G, ctx=ctx)
+        ctx.last_index = (splits_i, cumsum, scatter, gather)
+        return fast_all_to_all(ctx, send_tensor, cumsum, send_scale, scatter_index=scatter)
+    _ensure_index_sets(ctx, T, topk, G, send_tensor.device)
+    ids = _staged_ids(ctx, expert_ids)
+    which = ctx.index_calls % 2
+    ctx.index_calls += 1
+    splits_i, cumsum, scatter, gather, _ = ctx.index_sets[which]
+    send_tensor = send_tensor.contiguous()
+    with_scale = send_scale is not None
+    if with_scale:
+        assert send_scale.dtype == torch.float32
+        send_scale = send_scale.contiguous()
+    act_pos = ctx.call_count % 2
+    rows = ctx.WORLD_SIZE * ctx.max_m
+    recv = ctx.recv_buf[act_pos * rows:(act_pos + 1) * rows, :]
+    scale_recv = ctx.scale_recv_buf[act_pos * rows:(act_pos + 1) * rows]
+    splits = ctx.split_recv_buf[act_pos * G:(act_pos + 1) * G]
+    _lib.call("tdist_moe_dispatch_tokens_from_ids", send_tensor.data_ptr(), row_bytes, _lib.ptr(send_scale), ids.data_ptr(),
+              topk, T, ctx.WORLD_SIZE, ctx.experts_per_rank, ctx.max_m, recv.data_ptr(),
+              scale_recv.data_ptr() if with_scale else None, splits.data_ptr(), splits_i.data_ptr(), cumsum.data_ptr(),
+              scatter.data_ptr(), gather.data_ptr(), _lib.stream_ptr())
+    ctx.last_index = (splits_i, cumsum, scatter, gather)
+    ctx.call_count = (ctx.call_count + 1) % ctx.MOD_VALUE
+    return [splits, recv, scale_recv if with_scale else None]
 
 
 def _fast_all_to_all_online_quant(ctx, send_tensor, send_split_cumsum, send_scale, scatter_index):
