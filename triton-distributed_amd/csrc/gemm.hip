@@ -247,6 +247,9 @@ struct GemmCfg {
   static constexpr bool kSplit = NST == 5;
   static constexpr int kAStages = kSplit ? 3 : NST, kBStages = kSplit ? 2 : NST;
   static constexpr int kLdsBytes = kSplit ? kAStages * kABytes + kBStages * kBBytes : NST * kStageBytes;
+  // split ring: byte offset of A stage s / B stage s (taken modulo the ring's length)
+  static constexpr int a_stage_off(int s) { return (s % kAStages) * kABytes; }
+  static constexpr int b_stage_off(int s) { return kAStages * kABytes + (s % kBStages) * kBBytes; }
   // split ring: DMA instructions issued per K step (list of one K tile: the B rows, then the A rows)
   static constexpr int kDmaPerStep = (kLoadsPerTile + kKSteps - 1) / kKSteps;
   // epilogue staging: per wave kWaveM rows of kWaveN 16-bit outputs; 16-byte chunk c of row r sits at
@@ -360,7 +363,9 @@ __device__ __forceinline__ int chunk_of(const GemmParams& p, int oc) {
   }
 }
 
-template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales, bool kGrouped = false>
+// kPlain: an instance for calls without flags and without a local shard (the GEMM-RS producer, plain GEMMs): no gating
+// code at all, and the next tile's first loads go out before the current tile's epilogue (see kEarly).
+template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales, bool kGrouped = false, bool kPlain = false>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams p) {
   typedef GemmCfg<E, BM, BN, KB, WM, WN, NST> C;
   typedef TDIST_AS3 unsigned char* lds_u8;
@@ -438,20 +443,32 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   if (p.sk_mode == 1 && sk_tail_tiles > 0) sk_split = sk_split_for(G, sk_tail_tiles, KT);
 
   // ---- tiles in arrival order (see GemmParams::sched_ctrl); everything here is wave 0's, one lane per chunk ----------
-  const bool arrival = !kGrouped && p.sched_ctrl != nullptr;
-  const int arr_nx = (p.num_xcds > 1 && p.num_xcds <= kSchedMaxXcds && G % p.num_xcds == 0) ? p.num_xcds : 1;
-  const int arr_gx = G / arr_nx;               // workgroups per XCD = tiles of a round in one XCD's list
-  const int arr_my_x = arr_nx > 1 ? blockIdx.x % arr_nx : 0;
+  const bool arrival = !kGrouped && !kPlain && p.sched_ctrl != nullptr;
+  // (small functions of the launch, recomputed where they are needed rather than held in scalar registers across the
+  // K loop, whose wave has no second wave to hide a reload behind)
+  auto arr_nx_f = [&]() { return (p.num_xcds > 1 && p.num_xcds <= kSchedMaxXcds && G % p.num_xcds == 0) ? p.num_xcds : 1; };
   bool arr_first = true, arr_decided = false;
-  // positions in the static order: the tile drawn but not yet begun, and the tiles put aside (-1 = none; kArrNone in
-  // arr_held once every list has run out)
+  // The schedule's state lives in ONE vector register, a word per lane (wave 0's copy is the one that counts), and is
+  // read and written with v_readlane / v_writelane where a tile is chosen: positions in the static order of the tile
+  // drawn but not yet begun (kArrHeld; -1 = none, kArrNone once every list has run out) and of the tiles put aside
+  // (-1 = none), the XCDs whose lists this workgroup has found empty (a bit each), and the looks a wait may take (1
+  // once any wait of the launch has expired).
   constexpr int kArrNone = -2;
-  int arr_held = -1, arr_aside[kSchedAside] = {-1, -1};
-  int arr_dead = 0;                            // XCDs whose lists this workgroup has found empty
-  int arr_limit = p.spin_limit;                // looks a wait may take: 1 once any wait of the launch has expired
+  enum { kArrHeld = 0, kArrAside0 = 1, kArrDead = 1 + kSchedAside, kArrLimit = 2 + kSchedAside };
+  int arr_v = -1;
+  asm volatile("" : "+v"(arr_v));
+  auto arr_get = [&](int i) { return __builtin_amdgcn_readlane(arr_v, i); };
+  // (the lane is an immediate: a second scalar operand would be one too many for the instruction)
+#define TDIST_ARR_SET(LANE, VAL) \
+  asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(arr_v) : "s"(__builtin_amdgcn_readfirstlane(VAL)), "n"(LANE))
+  if (arrival) {
+    TDIST_ARR_SET(kArrDead, 0);
+    TDIST_ARR_SET(kArrLimit, p.spin_limit);
+  }
   // draw t of XCD x's list → position in the static order (rounds from the second on), or -1 behind the list's end
   auto arr_position = [&](int x, int t) {
-    const int sidx = (1 + t / arr_gx) * G + x * arr_gx + t % arr_gx;
+    const int gx = G / arr_nx_f();               // workgroups per XCD = tiles of a round in one XCD's list
+    const int sidx = (1 + t / gx) * G + x * gx + t % gx;
     return t >= 0 && sidx < total_sched ? sidx : -1;
   };
   auto arr_chunk_at = [&](int sidx) { return chunk_of(p, sidx / tiles_per_chunk); };
@@ -465,7 +482,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     int l = lane;
     asm volatile("" : "+v"(l));   // (nothing of this is computed ahead and held across the K loop)
     flag = __hip_atomic_load(p.flags + min(l, n_chunks - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    cnt = __hip_atomic_load(p.sched_ctrl + kSchedCounters + min(l, arr_nx - 1) * kSchedCounterStride, __ATOMIC_RELAXED,
+    cnt = __hip_atomic_load(p.sched_ctrl + kSchedCounters + min(l, arr_nx_f() - 1) * kSchedCounterStride, __ATOMIC_RELAXED,
                             __HIP_MEMORY_SCOPE_AGENT);
   };
   // the draw: one lane's atomic add on XCD x's counter (the raw counter value, valid in every lane afterwards)
@@ -481,6 +498,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   auto arr_next = [&](int flag, int cnt, bool drawn, int t_raw) -> int {
     int l = lane;
     asm volatile("" : "+v"(l));
+    const int arr_nx = arr_nx_f(), arr_my_x = arr_nx > 1 ? (int)blockIdx.x % arr_nx : 0;
+    int arr_held = arr_get(kArrHeld), arr_dead = arr_get(kArrDead), arr_limit = arr_get(kArrLimit);
+    int arr_aside[kSchedAside];
+#pragma unroll
+    for (int i = 0; i < kSchedAside; ++i) arr_aside[i] = arr_get(kArrAside0 + i);
     if (drawn) {
       const int pos = arr_position(arr_my_x, __shfl(t_raw, 0));
       arr_held = pos >= 0 ? pos : -1;
@@ -559,8 +581,35 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       __builtin_amdgcn_s_sleep(4);
       arr_look(flag, cnt);
     }
+    TDIST_ARR_SET(kArrHeld, arr_held);
+    TDIST_ARR_SET(kArrDead, arr_dead);
+    TDIST_ARR_SET(kArrLimit, arr_limit);
+    static_assert(kSchedAside == 2, "one write per tile put aside");
+    TDIST_ARR_SET(kArrAside0, arr_aside[0]);
+    TDIST_ARR_SET(kArrAside0 + 1, arr_aside[1]);
     if (next >= 0 && !arr_is_local(arr_chunk_at(next))) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
     return next;
+  };
+
+  // ---- the next tile's first loads issued before this tile's epilogue ------------------------------------------------
+  // Plain tiles (whole, ungated, unsplit) followed by another plain tile of the same workgroup, on the 256 x 256 split
+  // ring: A(0), B(0) and B(1) of the next tile go out before this tile's epilogue, which then stages through the A
+  // stages 1 and 2 only (two 32-row blocks per wave, used in turn). The next tile's prologue has A(1) left to issue
+  // and waits for A(0) and B(0) alone: the epilogue's stores, issued behind those loads, are still on their way then
+  // and have the whole first K tile to be acknowledged (loads and stores retire in order through one counter, so a
+  // prologue that issues its loads behind the stores waits for every store of the tile before it).
+  constexpr bool kEarly = kPlain && C::kSplit && !kGrouped && kFixedAcc && C::kWaves <= 4 && C::kRowPieces == C::kEpiChunks &&
+                          2 * C::kABytes >= C::kWaves * 64 * C::kEpiPitch && C::kAInstr == C::kBInstr;
+  constexpr int kEpiStores = (C::kWaveM / 32) * 32 * C::kEpiChunks / 64;   // 16-byte stores per wave and tile
+  static_assert(!kEarly || C::kBInstr + kEpiStores + C::kAInstr < 64, "vmcnt is a 6-bit counter");
+  bool prefetched = false;   // this tile's A(0), B(0), B(1) were issued by the tile before
+  // tile of C behind schedule index sidx (ungated calls)
+  auto locate = [&](int sidx, int& tm0, int& tn0) -> bool {
+    const int toc = sidx / tiles_per_chunk, twithin = sidx - toc * tiles_per_chunk;
+    const int tpid_m = chunk_of(p, toc) * cm + twithin % cm;
+    tm0 = tpid_m * BM;
+    tn0 = (twithin / cm) * BN;
+    return tpid_m < num_pid_m;
   };
 
   int sbase = 0;
@@ -575,13 +624,13 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         bool quick = false;
         if (arr_first && wg_pos < total_sched) {
           // the first round is static: this workgroup's own tile, which nobody else can take
-          arr_held = wg_pos;
           const int ch = arr_chunk_at(wg_pos);
           if (arr_is_local(ch) || __hip_atomic_load(p.flags + ch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == p.wait_value) {
             if (!arr_is_local(ch)) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
             next = wg_pos;
-            arr_held = -1;
             quick = true;
+          } else {
+            TDIST_ARR_SET(kArrHeld, wg_pos);
           }
         }
         if (!quick) {
@@ -635,9 +684,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     }
 
     // ---- gate ---------------------------------------------------------------------------------
-    const bool is_local = kGrouped ? (p.A_local != nullptr && segment == p.rank)
+    const bool is_local = kPlain ? false : kGrouped ? (p.A_local != nullptr && segment == p.rank)
                                    : (p.A_local != nullptr && m0 >= p.local_row_begin && m0 < p.local_row_begin + p.local_rows);
-    if (p.flags != nullptr && !is_local && arr_chunk < 0) {
+    if (!kPlain && p.flags != nullptr && !is_local && arr_chunk < 0) {
       if (threadIdx.x == 0) {
         // the flags of the tile's rows: one (the tile lies inside a chunk), or, with ragged chunks, every flag from
         // the first row's to the last row's (the reference's NVIDIA-side kernel waits for a range of rank segments
@@ -708,6 +757,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       const int gr = min(n0 + r, p.N - 1);
       b_off[t] = (uint32_t)(gr - b_g0) * (uint32_t)p.ldb_b + (uint32_t)((dma_pos ^ swz<KB>(r)) << 4);
     }
+
 
     // DMA of K tile kt into stage kt % NST, one instruction at a time (kLoadsPerTile of them: A rows first, then
     // B rows). Past the last tile the last one is fetched again (into a stage nobody reads any more): every trip
@@ -816,25 +866,28 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     };
     // Split ring, K loop unrolled over the six (A stage, B stage) pairs: stage S of either ring as a constant address
     auto a_stage_c = [&](auto s_c) -> lds_u8 { return smem + (decltype(s_c)::value % C::kAStages) * C::kABytes; };
+    // (the same as byte offsets into the ring: C::a_stage_off(S), C::b_stage_off(S))
     auto b_stage_c = [&](auto s_c) -> lds_u8 {
       return smem + C::kAStages * C::kABytes + (decltype(s_c)::value % C::kBStages) * C::kBBytes;
     };
     // The LDS address of such a load is a constant plus the wave's share of the stage; added inside the assembly, so
     // that the compiler does not keep the sum of every (stage, instruction) pair in a scalar register of its own
     // (there are more pairs than registers, and a spilled one comes back through the vector ALU).
-    auto dma16_at = [&](const unsigned char* sbase, uint32_t voff, lds_u8 dst_const, uint32_t dst_wave) {
-      const uint32_t lds_addr = (uint32_t)(uintptr_t)dst_const;
-      asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr),
+    auto dma16_at = [&](const unsigned char* sbase, uint32_t voff, int dst_const, uint32_t dst_wave) {
+      // (the constant as a literal of the instruction: held in scalar registers, the forty of them are hoisted out of
+      // the K loop, spilled, and reloaded through the vector ALU inside it)
+      asm volatile("s_add_u32 m0, %3, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "n"(dst_const),
                    "s"(dst_wave)
                    : "memory", "scc");
     };
-    const uint32_t a_wave_off = __builtin_amdgcn_readfirstlane(wave * C::kAInstr * 1024);
-    const uint32_t b_wave_off = __builtin_amdgcn_readfirstlane(wave * C::kBInstr * 1024);
-    // K tile kt_src's rows into the given stage
-    auto issue_a_to = [&](lds_u8 st, int kt_src, int t) {
+    // start of the ring plus the wave's share of a stage
+    const uint32_t a_wave_off = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem + wave * C::kAInstr * 1024);
+    const uint32_t b_wave_off = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem + wave * C::kBInstr * 1024);
+    // K tile kt_src's rows into the stage at byte `st` of the ring
+    auto issue_a_to = [&](int st, int kt_src, int t) {
       dma16_at(a_base + (int64_t)min(kt_src, KTp - 1) * KB, a_off[t], st + t * 1024, a_wave_off);
     };
-    auto issue_b_to = [&](lds_u8 st, int kt_src, int u) {
+    auto issue_b_to = [&](int st, int kt_src, int u) {
       dma16_at(b_base + (int64_t)min(kt_src, KTp - 1) * KB, b_off[u], st + u * 1024, b_wave_off);
     };
     auto load_frags = [&](int kt, int ks, typename E::frag* af, typename E::frag* bf) {
@@ -889,15 +942,23 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         if (q < C::kBInstr) issue_b(cyc + 2, q);
         else issue_a(cyc + 3, q - C::kBInstr);
       };
+      static_assert(!kEarly || kProDma == C::kBInstr, "the prologue's share of the first list is B(1)");
+      if (kEarly && prefetched) {
+        // A(0), B(0) and B(1) went out before the last tile's epilogue; its stores are allowed to be still on their way
 #pragma unroll
-      for (int t = 0; t < C::kAInstr; ++t) issue_a(0, t);
+        for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+        wait_tiles_and_barrier<kEarly ? C::kBInstr + kEpiStores + C::kAInstr : 0>();
+      } else {
 #pragma unroll
-      for (int u = 0; u < C::kBInstr; ++u) issue_b(0, u);
+        for (int t = 0; t < C::kAInstr; ++t) issue_a(0, t);
 #pragma unroll
-      for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+        for (int u = 0; u < C::kBInstr; ++u) issue_b(0, u);
 #pragma unroll
-      for (int q = 0; q < kProDma; ++q) issue_list(-1, q);
-      wait_tiles_and_barrier<C::kAInstr + kProDma>();
+        for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+#pragma unroll
+        for (int q = 0; q < kProDma; ++q) issue_list(-1, q);
+        wait_tiles_and_barrier<C::kAInstr + kProDma>();
+      }
 #pragma unroll
       for (int f = 0; f < kHA; ++f) load_frag(0, 0, f, a_cur, b_cur);            // lower A half
 #pragma unroll
@@ -908,14 +969,14 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       // the same, so that every trip runs the same instructions)
       auto tile = [&](auto odd_c, auto sa_c, auto sb_c, int kt) {
         constexpr int kOdd = decltype(odd_c)::value, SA = decltype(sa_c)::value, SB = decltype(sb_c)::value;
-        lds_u8 const a_now = a_stage_c(std::integral_constant<int, SA>{});
-        lds_u8 const b_now = b_stage_c(std::integral_constant<int, SB>{}), b_nx = b_stage_c(std::integral_constant<int, SB + 1>{});
+        constexpr int a_now = C::a_stage_off(SA);
+        constexpr int b_now = C::b_stage_off(SB), b_nx = C::b_stage_off(SB + 1);
         // entry q of the list begun at this tile's barrier ([B(kt+2), A(kt+3)]: the stages of this tile's own rows) or
         // of the one before ([B(kt+1), A(kt+2)])
         auto issue_entry = [&](auto own_c, int q) {
           constexpr bool own = decltype(own_c)::value;
           if (q < C::kBInstr) issue_b_to(own ? b_now : b_nx, own ? kt + 2 : kt + 1, q);
-          else issue_a_to(own ? a_now : a_stage_c(std::integral_constant<int, SA + 2>{}), own ? kt + 3 : kt + 2, q - C::kBInstr);
+          else issue_a_to(own ? a_now : C::a_stage_off(SA + 2), own ? kt + 3 : kt + 2, q - C::kBInstr);
         };
         static_for<kMfmaPerStep>([&](auto u_c) {
           constexpr int u = decltype(u_c)::value;
@@ -970,15 +1031,23 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         if (q < C::kBInstr) issue_b(cyc + 2, q);
         else issue_a(cyc + 3, q - C::kBInstr);
       };
+      static_assert(!kEarly || C::kDmaPerStep == C::kBInstr, "the prologue's share of the first list is B(1)");
+      if (kEarly && prefetched) {
+        // A(0), B(0) and B(1) went out before the last tile's epilogue; its stores are allowed to be still on their way
 #pragma unroll
-      for (int t = 0; t < C::kAInstr; ++t) issue_a(0, t);
+        for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+        wait_tiles_and_barrier<kEarly ? C::kBInstr + kEpiStores + C::kAInstr : 0>();
+      } else {
 #pragma unroll
-      for (int u = 0; u < C::kBInstr; ++u) issue_b(0, u);
+        for (int t = 0; t < C::kAInstr; ++t) issue_a(0, t);
 #pragma unroll
-      for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+        for (int u = 0; u < C::kBInstr; ++u) issue_b(0, u);
 #pragma unroll
-      for (int q = 0; q < C::kDmaPerStep; ++q) issue_list(-1, q);
-      wait_tiles_and_barrier<C::kAInstr + C::kDmaPerStep>();
+        for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+#pragma unroll
+        for (int q = 0; q < C::kDmaPerStep; ++q) issue_list(-1, q);
+        wait_tiles_and_barrier<C::kAInstr + C::kDmaPerStep>();
+      }
       load_frags(0, 0, a_cur, b_cur);
       __builtin_amdgcn_sched_barrier(0);
       // K tile kt, its A rows in stage SA and its B rows in stage SB (the tile after it sits in the next stage of either
@@ -986,14 +1055,14 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       // instructions)
       auto k_tile = [&](auto sa_c, auto sb_c, int kt) {
         constexpr int SA = decltype(sa_c)::value, SB = decltype(sb_c)::value;
-        lds_u8 const st_a = a_stage_c(std::integral_constant<int, SA>{});
-        lds_u8 const st_b = b_stage_c(std::integral_constant<int, SB>{}), st_b_nx = b_stage_c(std::integral_constant<int, SB + 1>{});
+        constexpr int st_a = C::a_stage_off(SA);
+        constexpr int st_b = C::b_stage_off(SB), st_b_nx = C::b_stage_off(SB + 1);
         // entry q of this tile's own refill list ([B(kt+2), A(kt+3)]: into the stages of its own rows) or of the one
         // before ([B(kt+1), A(kt+2)])
         auto issue_entry = [&](auto own_c, int q) {
           constexpr bool own = decltype(own_c)::value;
           if (q < C::kBInstr) issue_b_to(own ? st_b : st_b_nx, own ? kt + 2 : kt + 1, q);
-          else issue_a_to(own ? st_a : a_stage_c(std::integral_constant<int, SA + 2>{}), own ? kt + 3 : kt + 2, q - C::kBInstr);
+          else issue_a_to(own ? st_a : C::a_stage_off(SA + 2), own ? kt + 3 : kt + 2, q - C::kBInstr);
         };
         auto step = [&](auto ks_c, typename E::frag* a_now, typename E::frag* a_new) {
           constexpr int ks = decltype(ks_c)::value;
@@ -1117,17 +1186,62 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     //   16-row MFMA blocks: acc[g/2][2*ib + g%2][0 ...], row 32*ib + 16*(g%2) + lrow,   column 16*(g/2) + 4*lgrp
     constexpr int kRowBlocks = C::kWaveM / 32, kGroups = C::kWaveN / 8;
     constexpr bool kWide = E::kRows == 32;
-    wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
+    // Is the next tile's start issued before this tile's epilogue? Both tiles whole and ungated, this one stored by
+    // the vector epilogue (the per-lane offsets of the operand loads are then the same for both, only the uniform bases differ). Decided here,
+    // behind the K loop, so that nothing of it is held in registers across the loop.
+    bool early = false;
+    const unsigned char* a_base_n = a_base;
+    const unsigned char* b_base_n = b_base;
+    if constexpr (kEarly) {
+      int nm0 = 0, nn0 = 0;
+      const bool next_whole_round = !arrival && sbase < total_sched && !(sk_split > 1 && sbase + G > total_sched) && sbase + wg_pos < total_sched;
+      if (p.flags == nullptr && p.A_local == nullptr && sk_s == 1 && KT >= 2 && next_whole_round && m0 + BM <= p.M &&
+          n0 + BN <= p.N && p.ldc % 8 == 0 && locate(sbase + wg_pos, nm0, nn0) && nm0 + BM <= p.M && nn0 + BN <= p.N) {
+        bool c_aligned = (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+        if (p.scatter_bufs != nullptr) c_aligned = (reinterpret_cast<uintptr_t>(p.scatter_bufs[m0 / p.m_per_rank]) & 15) == 0;
+        if (c_aligned) {
+          early = true;
+          a_base_n = p.A + (int64_t)nm0 * p.lda_b;
+          b_base_n = p.B + (int64_t)nn0 * p.ldb_b;
+        }
+      }
+      // (wave-uniform by construction; said so to the compiler, which otherwise carries them in vector registers)
+      auto uniform_ptr = [](const unsigned char* q) {
+        const uint64_t v = reinterpret_cast<uint64_t>(q);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return reinterpret_cast<const unsigned char*>(((uint64_t)hi << 32) | lo);
+      };
+      a_base_n = uniform_ptr(a_base_n);
+      b_base_n = uniform_ptr(b_base_n);
+    }
+    if (kEarly && early) {
+      // nobody reads the ring any more; then the next tile's A(0), B(0), B(1) go out into A stage 0 and the B stages,
+      // and once everything older than them has landed (the loads the K loop issued beyond the tile's end, which may
+      // point anywhere in the ring) the A stages 1 and 2 are free for staging
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+      for (int t = 0; t < C::kAInstr; ++t) dma16(a_base_n, a_off[t], smem + (wave * C::kAInstr + t) * 1024);
+#pragma unroll
+      for (int u = 0; u < C::kBInstr; ++u)
+        dma16(b_base_n, b_off[u], smem + C::kAStages * C::kABytes + (wave * C::kBInstr + u) * 1024);
+#pragma unroll
+      for (int u = 0; u < C::kBInstr; ++u)
+        dma16(b_base_n + KB, b_off[u], smem + C::kAStages * C::kABytes + C::kBBytes + (wave * C::kBInstr + u) * 1024);
+      wait_tiles_and_barrier<C::kAInstr + 2 * C::kBInstr>();
+    } else {
+      wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
+    }
     // arrival order: the look for the next tile goes out now and is used when this tile has been stored
     int arr_flag = 0, arr_cnt = 0, arr_t = 0;
     bool arr_drawn = false;
     if (arrival && wave == 0) {
       arr_look(arr_flag, arr_cnt);
       // and the draw, unless a tile is in hand already or the own list is known to be empty
-      arr_drawn = arr_held == -1 && ((arr_dead >> arr_my_x) & 1) == 0;
-      if (arr_drawn) arr_t = arr_draw(arr_my_x);
+      const int my_x = arr_nx_f() > 1 ? (int)blockIdx.x % arr_nx_f() : 0;
+      arr_drawn = arr_get(kArrHeld) == -1 && ((arr_get(kArrDead) >> my_x) & 1) == 0;
+      if (arr_drawn) arr_t = arr_draw(my_x);
     }
-    lds_u8 const epi = smem + wave * C::kEpiBytes;
+    lds_u8 const epi = (kEarly && early) ? smem + C::kABytes + wave * (64 * C::kEpiPitch) : smem + wave * C::kEpiBytes;
     // The epilogue's lane-dependent addresses are the same for every tile; computed from these opaque copies they are
     // rebuilt per tile (a few dozen instructions) instead of being held in ~100 registers across the K loop.
     int e_lane = lane;
@@ -1407,6 +1521,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         unsigned char* const tile_dst = Cbase + ((crow0 + wm * C::kWaveM) * p.ldc + n0 + wn * C::kWaveN) * 2;
         const uint32_t lane_off = (uint32_t)er * (uint32_t)row_bytes + (uint32_t)ec * 16u;
         const bool streaming = p.scatter_bufs == nullptr;
+        const bool blocks_in_turn = kEarly && early;   // two staging blocks per wave instead of one per row block
         float rs[kScales ? C::kTM : 1] = {1.f};
         // (the two groups of a 16-column block share their column scales)
         constexpr int kColSlots = kWide ? kGroups : kGroups / 2;
@@ -1437,13 +1552,13 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         auto stage_fast = [&](auto i_c, auto g_c) {
           constexpr int i = decltype(i_c)::value, g = decltype(g_c)::value;
           stage_vals(acc4(i_c, g_c), kScales ? rs[scale_slot(i, g)] : 1.f, cs[kScales ? (kWide ? g : g / 2) : 0],
-                     wbase[g] + i * 32 * C::kEpiPitch);
+                     wbase[g] + (blocks_in_turn ? i % 2 : i) * 32 * C::kEpiPitch);
         };
         static_for<kGroups>([&](auto g_c) { stage_fast(std::integral_constant<int, 0>{}, g_c); });
         __builtin_amdgcn_sched_barrier(0);
         int4v v[kPasses];
         auto read_piece = [&](int i, int u) {
-          v[u] = *(const TDIST_AS3 int4v*)(rbase[u % kReadPhases] + (32 * i + u * kRowsPerPass) * C::kEpiPitch);
+          v[u] = *(const TDIST_AS3 int4v*)(rbase[u % kReadPhases] + (32 * (blocks_in_turn ? i % 2 : i) + u * kRowsPerPass) * C::kEpiPitch);
         };
         auto store_fast = [&](int i, int u) {
           TDIST_AS1 int4v* dst = (TDIST_AS1 int4v*)(tile_dst + (int64_t)(32 * i + u * kRowsPerPass) * row_bytes + lane_off);
@@ -1538,6 +1653,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     }
     // the next tile's prologue overwrites the ring: every wave must be done reading its staging area
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if constexpr (kEarly) prefetched = early;
   }
   // ---- leave: the last workgroup out puts the ticket counters back to zero for the next launch ------------------
   if (!kGrouped && p.sched_ctrl != nullptr && threadIdx.x == 0) {
@@ -1593,10 +1709,10 @@ struct GemmCall {
   const char* who;
 };
 
-template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales, bool kGrouped = false>
+template <typename E, int BM, int BN, int KB, int WM, int WN, int NST, bool kScales, bool kGrouped = false, bool kPlain = false>
 static int launch_gemm_cfg(const GemmParams& prm, int grid, hipStream_t stream, const char* who) {
   typedef GemmCfg<E, BM, BN, KB, WM, WN, NST> C;
-  auto kern = gemm_kernel<E, BM, BN, KB, WM, WN, NST, kScales, kGrouped>;
+  auto kern = gemm_kernel<E, BM, BN, KB, WM, WN, NST, kScales, kGrouped, kPlain>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes);
@@ -1831,6 +1947,16 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   const bool scales = elem == kElemFP8 && (c.row_scale || c.col_scale);
 
   // 256-row tiles: 2 x 2 waves on the split ring (3 A stages + 2 B stages), 16-row MFMA blocks
+  if (BM == 256 && BN == 256 && p.flags == nullptr && p.A_local == nullptr) {
+    // no flags, no local shard: the instances without gating code (the GEMM-RS producer's, the headline shape's)
+    switch (elem) {
+      case kElemBF16: return launch_gemm_cfg<ElemBF16N, 256, 256, 128, 2, 2, 5, false, false, true>(p, grid, c.stream, who);
+      case kElemF16: return launch_gemm_cfg<ElemF16N, 256, 256, 128, 2, 2, 5, false, false, true>(p, grid, c.stream, who);
+      default:
+        return scales ? launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, true, false, true>(p, grid, c.stream, who)
+                      : launch_gemm_cfg<ElemFP8N, 256, 256, 128, 2, 2, 5, false, false, true>(p, grid, c.stream, who);
+    }
+  }
   if (BM == 256 && BN == 256) {
     switch (elem) {
       case kElemBF16: return launch_gemm_cfg<ElemBF16N, 256, 256, 128, 2, 2, 5, false>(p, grid, c.stream, who);
