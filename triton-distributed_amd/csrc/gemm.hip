@@ -1231,16 +1231,21 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     } else {
       wait_tiles_and_barrier<0>();  // every DMA has landed and no wave reads the ring any more: reuse it
     }
-    // arrival order: the look for the next tile goes out now and is used when this tile has been stored
+    // arrival order: the look for the next tile goes out while this tile is being stored and is used when it has been.
+    // Issued behind the epilogue's own loads (the scales), not in front of them: loads retire in order, so the wait
+    // for the scales would otherwise be a wait for the draw's round trip as well.
     int arr_flag = 0, arr_cnt = 0, arr_t = 0;
-    bool arr_drawn = false;
-    if (arrival && wave == 0) {
-      arr_look(arr_flag, arr_cnt);
-      // and the draw, unless a tile is in hand already or the own list is known to be empty
-      const int my_x = arr_nx_f() > 1 ? (int)blockIdx.x % arr_nx_f() : 0;
-      arr_drawn = arr_get(kArrHeld) == -1 && ((arr_get(kArrDead) >> my_x) & 1) == 0;
-      if (arr_drawn) arr_t = arr_draw(my_x);
-    }
+    bool arr_drawn = false, arr_issued = false;
+    auto arr_issue = [&]() {
+      if (arrival && wave == 0 && !arr_issued) {
+        arr_look(arr_flag, arr_cnt);
+        // and the draw, unless a tile is in hand already or the own list is known to be empty
+        const int my_x = arr_nx_f() > 1 ? (int)blockIdx.x % arr_nx_f() : 0;
+        arr_drawn = arr_get(kArrHeld) == -1 && ((arr_get(kArrDead) >> my_x) & 1) == 0;
+        if (arr_drawn) arr_t = arr_draw(my_x);
+      }
+      arr_issued = true;
+    };
     lds_u8 const epi = (kEarly && early) ? smem + C::kABytes + wave * (64 * C::kEpiPitch) : smem + wave * C::kEpiBytes;
     // The epilogue's lane-dependent addresses are the same for every tile; computed from these opaque copies they are
     // rebuilt per tile (a few dozen instructions) instead of being held in ~100 registers across the K loop.
@@ -1556,6 +1561,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         };
         static_for<kGroups>([&](auto g_c) { stage_fast(std::integral_constant<int, 0>{}, g_c); });
         __builtin_amdgcn_sched_barrier(0);
+        arr_issue();
+        __builtin_amdgcn_sched_barrier(0);
         int4v v[kPasses];
         auto read_piece = [&](int i, int u) {
           v[u] = *(const TDIST_AS3 int4v*)(rbase[u % kReadPhases] + (32 * (blocks_in_turn ? i % 2 : i) + u * kRowsPerPass) * C::kEpiPitch);
@@ -1641,8 +1648,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       store_rows(0, C::kWaveM);
     }
+    arr_issue();   // (the epilogue forms that did not issue the look themselves)
     if (arrival) {
-      // the next tile, by the look taken when the epilogue began (wave 0 is done reading its staging rows, which is
+      // the next tile, by the look taken while the epilogue ran (wave 0 is done reading its staging rows, which is
       // where the gate words lie)
       if (wave == 0) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
