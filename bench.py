@@ -30,11 +30,46 @@ PEAK = {"bf16": 2.5e15, "fp8": 5.0e15, "hbm": 8.0e12}  # MI355X published dense 
 # HBM-side bytes per launch, read off two rocprofv3 counter passes over this same script (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch, each scaled by what the counter reads for the 1 GiB copy kernel: x2.000 and
 # x1.000). Counters cannot be collected inside a timed run, so the figures are carried here as constants;
-# the summaries are kept under profiles/.
+# the summaries are kept under profiles/. Each figure names the kernel sources it was measured on, and
+# MEASURED_SOURCE_DIGEST holds those sources' digests at the time: a figure whose sources have changed since is
+# reported as null, not as a measurement (tests/test_bench_constants.py fails until it is measured again).
 MEASURED_TRAFFIC_BYTES = {
-    "c2_gemm": 839.2e6, "c2_reduce": 151.0e6, "c1_gemm": 130.3e6, "c3_gemm": 1646.6e6, "c4_dispatch": 265.8e6,
-    "c4_combine": 296.7e6, "c5_split_kv": 4316.1e6,
+    "c2_gemm": (840.0e6, ("gemm.hip", "common.h")), "c2_reduce": (151.0e6, ("reduce.hip", "common.h")),
+    "c1_gemm": (130.4e6, ("gemm.hip", "common.h")), "c3_gemm": (1648.2e6, ("gemm.hip", "common.h")),
+    "c4_dispatch": (265.8e6, ("moe.hip", "common.h")), "c4_dispatch_from_ids": (267.3e6, ("moe.hip", "common.h")),
+    "c4_combine": (296.7e6, ("moe.hip", "common.h")), "c5_split_kv": (4318.1e6, ("decode.hip", "common.h")),
 }
+MEASURED_SOURCE_DIGEST = {
+    "common.h": "29a71d5d51010d68",
+    "decode.hip": "5f8c13ce9a3fc0d7",
+    "gemm.hip": "3544be2cf1008870",
+    "moe.hip": "e5e7e316eca5a2e9",
+    "reduce.hip": "469689d34df1b205",
+}
+CSRC = os.path.join(ROOT, "triton-distributed_amd", "csrc")
+
+
+def source_digest(name):
+    """sha256 (first 16 hex digits) of a kernel source with comments and white space taken out, so that only a
+    change of code makes a measurement stale."""
+    import hashlib
+    import re
+    text = open(os.path.join(CSRC, name)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    return hashlib.sha256("".join(text.split()).encode()).hexdigest()[:16]
+
+
+def measured_traffic(key):
+    """The measured HBM-side bytes of one launch, or None when a source the figure was measured on has changed."""
+    value, sources = MEASURED_TRAFFIC_BYTES[key]
+    for name in sources:
+        if source_digest(name) != MEASURED_SOURCE_DIGEST.get(name):
+            log("traffic of %s: %s has changed since the counters were read; reporting null" % (key, name))
+            return None
+    return value
+
+
 LIVE_PRODUCER = True  # --no-live-producer clears it
 METRIC = "AG-GEMM/GEMM-RS TFLOPS (% MFMA peak); decode & A2A GB/s (% HBM peak)"
 
@@ -214,7 +249,7 @@ def bench_c2(dev, steps, warmup):
     else:
         cpu = {"value": round(flops / 8 / probe / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                "sample": "1/8 of the rows (1024 of 8192) of the fp32 up-cast golden GEMM, %.2f s" % probe}
-    gemm_roof = roof("mfma", flops, gemm_s, "bf16", MEASURED_TRAFFIC_BYTES["c2_gemm"])
+    gemm_roof = roof("mfma", flops, gemm_s, "bf16", measured_traffic("c2_gemm"))
     # The same launch on constant operands (all ones): the matrix cores then draw far less power and the clock stays
     # up, so this rate shows the schedule's cycles rather than the power limit that the seeded random operands run into.
     ones_a, ones_b = torch.ones_like(a_d), torch.ones_like(b_d)
@@ -226,7 +261,7 @@ def bench_c2(dev, steps, warmup):
                                       "hipblaslt_us_per_launch": round(lib_const_s * 1e6, 2),
                                       "hipblaslt_frac": round(flops / lib_const_s / PEAK["bf16"], 4)}
     del ones_a, ones_b, lib_out
-    return (step_s, gemm_roof, roof("hbm", red_bytes, red_s, "hbm", MEASURED_TRAFFIC_BYTES["c2_reduce"]), cpu, err)
+    return (step_s, gemm_roof, roof("hbm", red_bytes, red_s, "hbm", measured_traffic("c2_reduce")), cpu, err)
 
 
 def bench_c1(dev, steps, warmup):
@@ -253,7 +288,7 @@ def bench_c1(dev, steps, warmup):
     flags = torch.ones(world, dtype=torch.int32, device=dev)
     out = torch.empty((world * mpr, N), dtype=torch.bfloat16, device=dev)
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 1024, rank, world, sk_workspace=ctx.sk_workspace), steps, warmup)
-    r = roof("mfma", flops, pre_s, "bf16", MEASURED_TRAFFIC_BYTES["c1_gemm"])
+    r = roof("mfma", flops, pre_s, "bf16", measured_traffic("c1_gemm"))
     cs, cores = cpu_time(lambda: golden.torch_ag_gemm(shards, b))
     r["cpu_baseline"] = {"value": round(flops / cs / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                          "sample": "the whole config once (torch golden: cat + matmul), %.2f s" % cs}
@@ -297,7 +332,7 @@ def bench_c3(dev, steps, warmup):
     pre_s = time_launches(lambda: gated_gemm(full, None, 0, b_d, out, flags, 2048, rank, world, row_scale=sa, col_scale=sb,
                                              sk_workspace=ctx.sk_workspace),
                           steps, warmup)
-    r = roof("mfma", flops, pre_s, "fp8", MEASURED_TRAFFIC_BYTES["c3_gemm"])
+    r = roof("mfma", flops, pre_s, "fp8", measured_traffic("c3_gemm"))
     sa_c, sb_c = sa.cpu(), sb.cpu()
     cs, cores = cpu_time(lambda: golden.fp8_scaled_gemm_fp32(shards[0][:1024], sa_c[:1024], b, sb_c))
     r["cpu_baseline"] = {"value": round(flops / 16 / cs / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
@@ -338,7 +373,7 @@ def bench_c4(dev, steps, warmup):
     n = T * topk
     disp_bytes = T * H + n * H + T * 4 + n * 4 + n * 4          # unique row reads + row writes + scales + gather index
     comb_bytes = n * H + n * 4 + n * 4 + n * 4 + T * H * 2      # row reads + scales + weights + scatter index + bf16 out
-    d = roof("hbm", disp_bytes, disp_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_dispatch"])
+    d = roof("hbm", disp_bytes, disp_s, "hbm", measured_traffic("c4_dispatch"))
 
     def cpu_dispatch():
         _, c_cumsum, _, c_gather, _ = golden.moe_preprocess(ids, G)
@@ -352,6 +387,7 @@ def bench_c4(dev, steps, warmup):
     # tensors, no allocation), then the row movement; the ids' 131 KB are added to the bytes
     d["with_index_build"] = {"us": round(both_s * 1e6, 2), "achieved_GBps": round((disp_bytes + n * 4) / both_s / 1e9, 1),
                              "frac": round((disp_bytes + n * 4) / both_s / PEAK["hbm"], 4),
+                             "traffic": measured_traffic("c4_dispatch_from_ids"),
                              "as_two_launches_us": round(two_s * 1e6, 2)}
     # the step after the dispatch: align / sort of the same ids for the grouped GEMM (8 rank segments, block 128)
     from triton_dist.kernels.amd import sort_topk_ids_align_block_size
@@ -366,7 +402,7 @@ def bench_c4(dev, steps, warmup):
     qd_bytes = T * H * 2 + n * H + n * (H // 128) * 4 + n * 4
     d["online_quant_dispatch"] = {"us_per_launch": round(qd_s * 1e6, 2), "achieved_GBps": round(qd_bytes / qd_s / 1e9, 1),
                                   "frac": round(qd_bytes / qd_s / PEAK["hbm"], 4)}
-    c = roof("hbm", comb_bytes, comb_s, "hbm", MEASURED_TRAFFIC_BYTES["c4_combine"])
+    c = roof("hbm", comb_bytes, comb_s, "hbm", measured_traffic("c4_combine"))
     _, _, c_scatter, c_gather, _ = golden.moe_preprocess(ids, G)
     rows_f32 = q[c_gather.long()].float()
     cs, cores = cpu_time(lambda: golden.weighted_combine(rows_f32, s[c_gather.long()], c_scatter, w.cpu()))
@@ -421,7 +457,7 @@ def bench_c5(dev, steps, warmup):
     rank_s = time_launches(lambda: gqa_fwd_batch_decode_inter_rank_combine(all_out, all_lse, all_lens, final), steps, warmup)
     kv_bytes = 2 * B * L * Hkv * D * 2
     split_bytes = kv_bytes + q.numel() * 2 + table.numel() * 4 + out_split.numel() * 4 + lse_split.numel() * 4
-    r = roof("hbm", split_bytes, split_s, "hbm", MEASURED_TRAFFIC_BYTES["c5_split_kv"])
+    r = roof("hbm", split_bytes, split_s, "hbm", measured_traffic("c5_split_kv"))
     from oracle import golden
     pages1 = table[0].long()
     k1, v1, q1 = k[pages1].cpu(), v[pages1].cpu(), q[:1].cpu()
