@@ -108,6 +108,15 @@ int tdist_debug_get(int key);
  * rows touch (the reference's per-segment wait, kernels/nvidia/allgather_gemm.py:222-224), tiles are visited in row
  * order starting inside the own rank's rows, chunk_order must be NULL and the local shard must either start and end
  * on a multiple of 128 rows or be copied into A with its flags set (A_local = NULL).
+ * Tile order. Without a workspace, every workgroup walks a fixed list of tiles in the order above and waits at the
+ * flag of each. With sk_workspace, whole-tile chunks (m_per_chunk a multiple of the tile's rows, at most 64 chunks)
+ * and more tiles than workgroups, only a workgroup's first tile is fixed: after it, a workgroup draws its next tile
+ * from a list kept in the workspace header (one list per XCD, in the order above), puts a tile whose chunk has not
+ * arrived aside (at most two) and draws again, and comes back to a tile put aside as soon as its flag is up; only
+ * with nothing left to do does it wait, bounded by spin_limit as above. Rows that arrive late or out of order
+ * therefore delay only their own tiles. Every tile is computed whole by one workgroup, so C is bit for bit the same
+ * in either order and whatever the arrival order is. chunk_order, when given, is the order of the lists. The reference
+ * fixes the order by expected arrival instead (:193-206).
  * ------------------------------------------------------------------------------------------- */
 int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                 int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,
