@@ -299,11 +299,19 @@ def test_combine_reference_round_trip_bf16(cuda):
 @pytest.mark.parametrize("R,T,topk,E,BS,dtype", [(1, 4, 3, 4, 4, torch.int64), (8, 1024, 8, 256, 128, torch.int64),
                                                  (8, 512, 6, 64, 64, torch.int32), (3, 37, 4, 11, 8, torch.int64),
                                                  (2, 5, 2, 300, 1, torch.int32), (4, 1, 1, 1, 16, torch.int64),
-                                                 (16, 96, 8, 256, 128, torch.int64), (5, 300, 2, 7, 256, torch.int32)])
-def test_align_sort_bit_exact(cuda, R, T, topk, E, BS, dtype):
-    """sort_topk_ids_align_block_size against the oracle (the reference's align kernel restated)."""
+                                                 (16, 96, 8, 256, 128, torch.int64), (5, 300, 2, 7, 256, torch.int32),
+                                                 (8, 1024, 6, 64, 128, torch.int64), (3, 5461, 4, 32, 16, torch.int32),
+                                                 (2, 40000, 1, 8, 64, torch.int64)])
+@pytest.mark.parametrize("launches", ["one", "three"])
+def test_align_sort_bit_exact(cuda, switches, R, T, topk, E, BS, dtype, launches):
+    """sort_topk_ids_align_block_size against the oracle (the reference's align kernel restated): the one-launch form
+    that up to 65 536 entries take (blocks of 512 or of 1024 entries; 4096 groups do not fit it) and the three
+    launches behind it."""
+    from triton_dist import _lib
     from triton_dist.kernels.nvidia import sort_topk_ids_align_block_size
-    announce("moe align R=%d T=%d topk=%d E=%d BS=%d" % (R, T, topk, E, BS))
+    if launches == "three":
+        switches(_lib.TDIST_DEBUG_MOE_INDEX_FORM, 3)
+    announce("moe align R=%d T=%d topk=%d E=%d BS=%d (%s)" % (R, T, topk, E, BS, launches))
     g = torch.Generator().manual_seed(R * 1000 + T + E)
     if topk <= E:
         ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(R * T)])

@@ -294,14 +294,19 @@ __global__ __launch_bounds__(kThreads) void moe_index_fused_kernel(const int32_t
       }
     }
   };
+  // (no branch per id: one unsigned compare, and an id out of range counts into a word of its own lane behind the
+  // counters; with 64 ids per lane every instruction per id is a quarter of a microsecond per launch)
+  int32_t* const s_trash = s_mem + (kWaves + 3) * G + lane;
   auto count_others = [&](int64_t v0) {
 #pragma unroll
     for (int u = 0; u < kVecBatch; ++u) {
       const int64_t vi = v0 + (int64_t)u * kThreads;
       int32_t* const row = s_out + (vi * 4 < own_lo ? 0 : G);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (q[u][j] >= 0 && q[u][j] < G) atomicAdd(&row[q[u][j]], 1);
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t x = (uint32_t)q[u][j];
+        atomicAdd(x < (uint32_t)G ? row + x : s_trash, 1);
+      }
     }
   };
   if constexpr (kRecount) {
@@ -713,15 +718,28 @@ __global__ __launch_bounds__(kFdThreads) void moe_dispatch_fused_kernel(
       }
     }
   };
+  // (no branch per id: a vector that lies wholly in front of the workgroup's range or behind it, as all but one or
+  // two do, takes one unsigned compare per id, and what is not counted goes into a word of the lane's own)
+  int32_t* const s_trash = s_ids + ((own_n + 4 + 3) & ~3) + lane;
   auto count_others = [&](int64_t v0) {
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
       const int64_t vi = v0 + (int64_t)u * kFdThreads;
+      const int64_t i0 = vi * 4;
+      if (i0 + 3 < own_lo || i0 >= own_hi) {
+        int32_t* const row = i0 < own_lo ? s_before : s_behind;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int64_t i = vi * 4 + j;
-        const int x = q[u][j];
-        if (x >= 0 && x < G && (i < own_lo || i >= own_hi)) atomicAdd(i < own_lo ? &s_before[x] : &s_behind[x], 1);
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t x = (uint32_t)q[u][j];
+          atomicAdd(x < (uint32_t)G ? row + x : s_trash, 1);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int64_t i = i0 + j;
+          const int x = q[u][j];
+          if (x >= 0 && x < G && (i < own_lo || i >= own_hi)) atomicAdd(i < own_lo ? &s_before[x] : &s_behind[x], 1);
+        }
       }
     }
   };
@@ -1150,6 +1168,210 @@ __global__ __launch_bounds__(kPlaceThreads) void moe_align_place_kernel(
   if (k >= 0) sorted_ids[s_pad[k] + rank_in_group] = (int32_t)i;
 }
 
+// Align / sort in ONE launch for few entries (up to kRecountMaxBlocks blocks of 1024): the recounting index build above
+// with the composite keys formed on the way in and the groups' starts taken from the PADDED prefix, so that an entry's
+// rank is its place in the padded layout at once. Every block counts all entries (those in front of its range, its
+// own, those behind), works out the padded prefix over the G = R * E groups for itself and places its own entries;
+// the padding positions, the per-block expert / segment ids and the positions behind the padded total (up to fill_n)
+// are shared out among the blocks, groups in turn; block 0 writes the blocks per segment and the padded total.
+template <int kThreads, int kPerWave, bool kIds64>
+__global__ __launch_bounds__(kThreads) void moe_align_fused_kernel(
+    const void* __restrict__ ids_v, int64_t n, int per_iter, int E, int R, int nbits, int block_size,
+    int32_t* __restrict__ sorted_ids, int64_t fill_n, int32_t* __restrict__ expert_ids,
+    int32_t* __restrict__ block_barrier_ids, int32_t* __restrict__ rank_block_num, int32_t* __restrict__ total_post_pad,
+    uint32_t seg_magic) {
+  constexpr int kWaves = kThreads / 64, kItems = kWaves * kPerWave, kPasses = kPerWave / 64;
+  typedef __attribute__((__vector_size__(2 * sizeof(long long)))) long long long2v;
+  const int G = E * R;
+  extern __shared__ int32_t s_mem[];  // [kWaves][G] wave counters, [G] group sizes, [2][G] before / behind, then starts
+  int32_t* const s_cnt = s_mem;
+  int32_t* const s_col = s_mem + kWaves * G;
+  int32_t* const s_out = s_col + G;
+  int32_t* const s_start = s_out;     // [G + 1] padded exclusive prefix, once the two rows have been summed
+  __shared__ int32_t s_part[kWaves];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int B = gridDim.x, b = blockIdx.x;
+  const int32_t* const ids32 = (const int32_t*)ids_v;
+  const long long* const ids64 = (const long long*)ids_v;
+  const uint32_t per = (uint32_t)per_iter;
+  auto key_of = [&](uint32_t i, long long id) -> int {
+    return (id >= 0 && id < E) ? (int)__umulhi(i, seg_magic) * E + (int)id : -1;
+  };
+  // the wave's own entries first
+  const int64_t wbase = (int64_t)b * kItems + (int64_t)wave * kPerWave;
+  long long id_own[kPasses];
+#pragma unroll
+  for (int u = 0; u < kPasses; ++u) {
+    const int64_t i = wbase + u * 64 + lane;
+    id_own[u] = i < n ? (kIds64 ? ids64[i] : (long long)ids32[i]) : -1;
+  }
+  // everybody else's, four per lane and load, all of a batch in flight
+  constexpr int kVecBatch = 16;
+  const int64_t own_lo = (int64_t)b * kItems, own_hi = own_lo + kItems;
+  const int64_t n_vec = (n + 3) / 4;
+  int4v q32[kIds64 ? 1 : kVecBatch];
+  long2v q64[kIds64 ? 2 * kVecBatch : 1];
+  auto load_others = [&](int64_t v0) {
+#pragma unroll
+    for (int u = 0; u < kVecBatch; ++u) {
+      const int64_t vi = v0 + (int64_t)u * kThreads;
+      const bool take = vi < n_vec && !(vi * 4 >= own_lo && vi * 4 < own_hi);
+      const bool whole = vi * 4 + 3 < n;
+      if constexpr (kIds64) {
+        q64[2 * u] = long2v{-1, -1};
+        q64[2 * u + 1] = long2v{-1, -1};
+        if (take && whole) {
+          q64[2 * u] = ((const long2v*)ids64)[2 * vi];
+          q64[2 * u + 1] = ((const long2v*)ids64)[2 * vi + 1];
+        } else if (take) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (vi * 4 + j < n) q64[2 * u + j / 2][j % 2] = ids64[vi * 4 + j];
+        }
+      } else {
+        q32[u] = int4v{-1, -1, -1, -1};
+        if (take && whole) q32[u] = ((const int4v*)ids32)[vi];
+        else if (take) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (vi * 4 + j < n) q32[u][j] = ids32[vi * 4 + j];
+        }
+      }
+    }
+  };
+  // Counting is the kernel's longest phase (every lane counts n / kThreads entries), so an entry costs as few
+  // instructions as can be: the segment of a vector's first entry by a multiplication (seg_magic = ceil(2^32 / per),
+  // exact below 65536 entries), at most one segment boundary inside a vector (per >= 4), one unsigned compare for the
+  // id's range, and no branch: an id out of range counts into a word of its own lane behind the counters.
+  int32_t* const s_trash = s_mem + (kWaves + 3) * G + lane;
+  auto count_others = [&](int64_t v0) {
+#pragma unroll
+    for (int u = 0; u < kVecBatch; ++u) {
+      const int64_t vi = v0 + (int64_t)u * kThreads;
+      int32_t* const row = s_out + (vi * 4 < own_lo ? 0 : G);
+      const uint32_t i0 = (uint32_t)(vi * 4);
+      const uint32_t seg = __umulhi(i0, seg_magic);
+      const uint32_t to_next = (seg + 1) * per - i0;   // entries of this vector that are still in segment `seg`
+      int32_t* const row_seg = row + seg * (uint32_t)E;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t lo;
+        bool ok;
+        if constexpr (kIds64) {
+          const long long id = q64[2 * u + j / 2][j % 2];
+          lo = (uint32_t)id;
+          ok = (uint32_t)(id >> 32) == 0u && lo < (uint32_t)E;
+        } else {
+          lo = (uint32_t)q32[u][j];
+          ok = lo < (uint32_t)E;
+        }
+        int32_t* const at = row_seg + (j > 0 && (uint32_t)j >= to_next ? E : 0) + lo;
+        atomicAdd(ok ? at : s_trash, 1);
+      }
+    }
+  };
+  if (B > 1) load_others(threadIdx.x);
+  for (int g = threadIdx.x; g < (kWaves + 3) * G; g += kThreads) s_cnt[g] = 0;
+  __syncthreads();
+  int32_t* const my_cnt = s_cnt + wave * G;
+  int e_of[kPasses];
+#pragma unroll
+  for (int u = 0; u < kPasses; ++u) {
+    e_of[u] = key_of((uint32_t)(wbase + u * 64 + lane), id_own[u]);
+    if (e_of[u] >= 0) atomicAdd(&my_cnt[e_of[u]], 1);
+  }
+  if (B > 1) {
+    count_others(threadIdx.x);
+    for (int64_t v0 = threadIdx.x + (int64_t)kVecBatch * kThreads; v0 < n_vec; v0 += (int64_t)kVecBatch * kThreads) {
+      load_others(v0);
+      count_others(v0);
+    }
+  }
+  __syncthreads();
+  // group sizes; the waves' starts within their group (entries of the blocks in front, then of the earlier waves)
+  for (int g = threadIdx.x; g < G; g += kThreads) {
+    int32_t run = s_out[g], total = s_out[g] + s_out[G + g];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const int32_t c = s_cnt[w * G + g];
+      s_cnt[w * G + g] = run;
+      run += c;
+      total += c;
+    }
+    s_col[g] = total;
+  }
+  __syncthreads();
+  // exclusive scan of the PADDED group sizes: consecutive groups per thread, then across threads and waves
+  const int per_thread = (G + kThreads - 1) / kThreads;
+  const int g0 = threadIdx.x * per_thread;
+  auto padded = [&](int32_t c) { return (c + block_size - 1) / block_size * block_size; };
+  int32_t local_total = 0;
+  for (int j = 0; j < per_thread; ++j)
+    if (g0 + j < G) local_total += padded(s_col[g0 + j]);
+  int32_t incl = local_total;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int32_t t = __shfl_up(incl, off);
+    if (lane >= off) incl += t;
+  }
+  if (lane == 63) s_part[wave] = incl;
+  __syncthreads();
+  int32_t acc = incl - local_total;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) acc += w < wave ? s_part[w] : 0;
+  for (int j = 0; j < per_thread; ++j) {
+    const int g = g0 + j;
+    if (g < G) {
+      s_start[g] = acc;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) s_cnt[w * G + g] += acc;
+      acc += padded(s_col[g]);
+      if (g == G - 1) s_start[G] = acc;
+    }
+  }
+  __syncthreads();
+  const int32_t total = s_start[G];
+  if (b == 0) {
+    for (int r = threadIdx.x; r < R; r += kThreads) rank_block_num[r] = (s_start[(r + 1) * E] - s_start[r * E]) / block_size;
+    if (threadIdx.x == 0) *total_post_pad = total;
+  }
+  // the groups this block looks after (a wave each, in turn): their padding positions and their blocks' ids
+  for (int g = b + B * wave; g < G; g += B * kWaves) {
+    const int32_t st = s_start[g], c = s_col[g], pc = padded(c);
+    for (int32_t o = c + lane; o < pc; o += 64) sorted_ids[st + o] = (int32_t)n;
+    for (int32_t k = st / block_size + lane; k < (st + pc) / block_size; k += 64) {
+      expert_ids[k] = g % E;
+      block_barrier_ids[k] = g / E;
+    }
+  }
+  // and its share of the positions behind the padded total
+  if (fill_n > total) {
+    const int64_t share = (fill_n - total + B - 1) / B;
+    const int64_t lo = total + share * b, hi = lo + share < fill_n ? lo + share : fill_n;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) sorted_ids[i] = (int32_t)n;
+  }
+  // the wave's entries in flat order, 64 at a time (as in moe_rank_kernel)
+  volatile int32_t* pos = my_cnt;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+  for (int u = 0; u < kPasses; ++u) {
+    if (wbase + u * 64 >= n) break;
+    const int64_t i = wbase + u * 64 + lane;
+    const int e = e_of[u];
+    const bool valid = e >= 0;
+    uint64_t peers = __ballot(valid);
+    for (int bit = 0; bit < nbits; ++bit) {
+      const bool one = (e >> bit) & 1;
+      const uint64_t m = __ballot(valid && one);
+      peers &= one ? m : ~m;
+    }
+    if (valid) sorted_ids[pos[e] + __popcll(peers & lt_mask)] = (int32_t)i;
+    __builtin_amdgcn_wave_barrier();
+    if (valid && (peers & lt_mask) == 0) pos[e] = pos[e] + __popcll(peers);
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
 static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, int32_t* splits, int32_t* cumsum,
                             int32_t* scatter_idx, int32_t* gather_idx, int32_t* topk_idx, void* workspace,
                             int64_t workspace_bytes, hipStream_t stream, bool want_index, const char* who) {
@@ -1181,7 +1403,7 @@ static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, 
   constexpr int kRowsRecount = kRowsPlain + 2;         // and the ids before / behind the block
   constexpr int kSmall = kFusedThreads;                // ids per block of the recounting forms: 512, or 1024
   const int64_t n1 = n_ids > 0 ? n_ids : 1;
-  const bool can_recount = form_dbg != 2 && kRowsRecount * G * 4 <= kLdsLimit && aligned16(ids);
+  const bool can_recount = form_dbg != 2 && kRowsRecount * G * 4 + 256 <= kLdsLimit && aligned16(ids);
   // 0: blocks of 2048 ids that exchange their histograms; 1 / 2: blocks of 512 / 1024 ids that count everything
   const int form = !can_recount ? 0 : ceil_div(n1, kSmall) <= kRecountMaxBlocks ? 1 : ceil_div(n1, 2 * kSmall) <= kRecountMaxBlocks ? 2 : 0;
   if (di.ok == 1 && fused_blocks <= di.num_cus && form_dbg != 3 && (form != 0 || form_dbg == 2)) {
@@ -1197,7 +1419,7 @@ static int moe_index_common(const int32_t* ids, int64_t n_ids, int topk, int G, 
         return fail(TDIST_ERR_LAUNCH, "%s: cannot reserve LDS for the index kernel", who);
       attr_set[form] = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kFusedThreads), (size_t)rows * G * 4, stream,
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kFusedThreads), (size_t)rows * G * 4 + (form != 0 ? 256 : 0), stream,
                        ids, n_ids, want_index ? topk : 1, G, id_bits(G), hist, scan_counter, splits, cumsum,
                        want_index ? scatter_idx : nullptr, gather_idx, topk_idx);
     return launch_status(who);
@@ -1351,7 +1573,7 @@ int tdist_moe_dispatch_tokens_from_ids(const void* tokens, int64_t row_bytes, co
   if ((int64_t)world_size * max_m > 0x7fffffff) return fail(TDIST_ERR_UNSUPPORTED, "%s: world_size * max_m too large", who);
   const int G = (int)G64;
   const int windows = (int)ceil_div(row_bytes, 8192);
-  const int64_t lds = ((int64_t)3 * G + ((G + 1 + 3) & ~3) + kFdWaves * topk + 4) * 4;
+  const int64_t lds = ((int64_t)3 * G + ((G + 1 + 3) & ~3) + kFdWaves * topk + 8 + 64) * 4;   // (+ a word per lane for what is not counted)
   if (n_tokens * topk > kFusedDispatchMaxIds || windows > kFdWaves || kFdWaves % windows != 0 || lds > 160 * 1024 - 256)
     return fail(TDIST_ERR_UNSUPPORTED, "%s: more than %lld ids, rows above %d bytes (or no power-of-two number of 8 KB windows), or too "
                 "many experts for one workgroup's counters: use tdist_moe_scatter_index + tdist_moe_dispatch_tokens", who,
@@ -1498,6 +1720,35 @@ int tdist_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t n_to
   int32_t* splits = gather + n_total;
   int32_t* cumsum = splits + (G + 1);
   const int64_t blocks = ceil_div(n_total > 0 ? n_total : 1, 256);
+  // Few entries: one launch in which every block counts all of them (see moe_align_fused_kernel).
+  {
+    constexpr int kLdsLimit = 160 * 1024 - 256;
+    constexpr int kRows = kFusedThreads / 64 + 3;
+    const int64_t n1 = n_total > 0 ? n_total : 1;
+    const int form = ceil_div(n1, kFusedThreads) <= kRecountMaxBlocks ? 1 : ceil_div(n1, 2 * kFusedThreads) <= kRecountMaxBlocks ? 2 : 0;
+    const int64_t per_iter = n_per_iteration > 0 ? n_per_iteration : 1;
+    // (a vector of four entries may cross one segment boundary, not two; the segment of an entry by multiplication)
+    const uint32_t seg_magic = per_iter >= 65536 ? 0u : (uint32_t)(((1ull << 32) + per_iter - 1) / per_iter);
+    if (form != 0 && device_info().ok == 1 && kRows * G * 4 + 256 <= kLdsLimit && aligned16(topk_ids) &&
+        (per_iter >= 4 || num_iterations == 1) && debug_get(TDIST_DEBUG_MOE_INDEX_FORM) != 3) {
+      auto kern = form == 1 ? (ids_int64 ? moe_align_fused_kernel<kFusedThreads, kFusedThreads / 8, true>
+                                         : moe_align_fused_kernel<kFusedThreads, kFusedThreads / 8, false>)
+                            : (ids_int64 ? moe_align_fused_kernel<kFusedThreads, kFusedThreads / 4, true>
+                                         : moe_align_fused_kernel<kFusedThreads, kFusedThreads / 4, false>);
+      static bool attr_set[4] = {false, false, false, false};
+      const int which = (form - 1) * 2 + (ids_int64 ? 1 : 0);
+      if (!attr_set[which]) {
+        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit) != hipSuccess)
+          return fail(TDIST_ERR_LAUNCH, "%s: cannot reserve LDS for the align kernel", who);
+        attr_set[which] = true;
+      }
+      const int64_t nblk = ceil_div(n1, form == 1 ? kFusedThreads : 2 * kFusedThreads);
+      hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(kFusedThreads), (size_t)kRows * G * 4 + 256, st, topk_ids, n_total,
+                         (int)per_iter, num_experts, num_iterations, id_bits((int)G), block_size, sorted_token_ids, sorted_fill,
+                         expert_ids, block_barrier_ids, rank_block_num, total_tokens_post_pad, seg_magic);
+      return launch_status(who);
+    }
+  }
   // three launches: keys (and the pre-fill of the padding positions), the stable index on the keys, padding + placement
   const int64_t key_items = n_total > sorted_fill ? n_total : sorted_fill;
   if (key_items > 0)

@@ -17,6 +17,9 @@ from triton_dist import _lib
 from triton_dist.kernels.amd.common_ops import fill_flags
 
 
+_ALIGN_PLANS = {}   # (ids, experts, ranks, topk, block size) -> scratch bytes and the layout of the results
+
+
 def sort_topk_ids_align_block_size(
     topk_ids: torch.Tensor,
     num_experts: int,
@@ -43,28 +46,39 @@ def sort_topk_ids_align_block_size(
     topk_ids = topk_ids.contiguous()
     num_topk = topk_ids.shape[1]
     dev = topk_ids.device
-    n_per = num_tokens_per_rank * num_topk
     n_total = topk_ids.numel()
+    n_per = num_tokens_per_rank * num_topk
     assert n_total == n_per * num_ranks, "topk_ids must hold num_ranks * num_tokens_per_rank tokens"
-    # the five results are views of one allocation (sizes as in the reference, :100-121; every view 16-byte aligned)
-    n_sorted = (n_per + num_experts * (block_size - 1)) * num_ranks
-    n_blocks = (n_per + num_experts) * num_ranks
-    up4 = lambda n: (n + 3) // 4 * 4
-    flat = torch.empty(up4(n_sorted) + 2 * up4(n_blocks) + up4(num_ranks) + 4, dtype=torch.int32, device=dev)
+    # sizes and scratch bytes once per shape: the call itself costs less than working them out again
+    key = (n_total, num_experts, num_ranks, num_topk, block_size)
+    plan = _ALIGN_PLANS.get(key)
+    if plan is None:
+        ws_bytes = _lib.load().tdist_moe_align_workspace_bytes(n_total, num_experts, num_ranks)
+        if ws_bytes == 0:
+            raise _lib.TdistError(_lib.TDIST_ERR_UNSUPPORTED,
+                                  "num_experts * num_ranks = %d is above what the align kernel handles" % (num_experts * num_ranks))
+        # the five results are views of one allocation (sizes as in the reference, :100-121; every view 16-byte aligned)
+        n_sorted = (n_per + num_experts * (block_size - 1)) * num_ranks
+        n_blocks = (n_per + num_experts) * num_ranks
+        sizes = (n_sorted, n_blocks, n_blocks, num_ranks, 1)
+        starts, at = [], 0
+        for n in sizes:
+            starts.append(at)
+            at += (n + 3) // 4 * 4
+        plan = _ALIGN_PLANS[key] = (ws_bytes, at, tuple(starts), sizes)
+    ws_bytes, n_flat, starts, sizes = plan
+    flat = torch.empty(n_flat, dtype=torch.int32, device=dev)
     sorted_ids, expert_ids, block_barrier_ids, rank_block_num, num_tokens_post_pad = (
-        t[:n] for t, n in zip(flat.split([up4(n_sorted), up4(n_blocks), up4(n_blocks), up4(num_ranks), 4]),
-                              (n_sorted, n_blocks, n_blocks, num_ranks, 1)))
-    ws_bytes = _lib.load().tdist_moe_align_workspace_bytes(n_total, num_experts, num_ranks)
-    if ws_bytes == 0:
-        raise _lib.TdistError(_lib.TDIST_ERR_UNSUPPORTED,
-                              "num_experts * num_ranks = %d is above what the align kernel handles" % (num_experts * num_ranks))
+        flat[a:a + n] for a, n in zip(starts, sizes))
+    base = flat.data_ptr()
+    ids_ptr, ids_int64 = topk_ids.data_ptr(), 1 if topk_ids.dtype == torch.int64 else 0
+
     def launch(stream):
         workspace = _lib.zeroed_scratch(ws_bytes, dev)   # (cached per stream: current is `stream` here)
-        # (sorted_ids.fill_(numel) of the reference, :103, is done by the call's first kernel)
-        _lib.call("tdist_moe_align_block_size", topk_ids.data_ptr(), 1 if topk_ids.dtype == torch.int64 else 0, n_total,
-                  num_experts, num_ranks, n_per, block_size, sorted_ids.data_ptr(), n_sorted, expert_ids.data_ptr(),
-                  block_barrier_ids.data_ptr(), rank_block_num.data_ptr(), num_tokens_post_pad.data_ptr(),
-                  workspace.data_ptr(), ws_bytes, stream.cuda_stream)
+        # (sorted_ids.fill_(numel) of the reference, :103, is done inside the call)
+        _lib.call("tdist_moe_align_block_size", ids_ptr, ids_int64, n_total, num_experts, num_ranks, n_per, block_size,
+                  base + 4 * starts[0], sizes[0], base + 4 * starts[1], base + 4 * starts[2], base + 4 * starts[3],
+                  base + 4 * starts[4], workspace.data_ptr(), ws_bytes, stream.cuda_stream)
 
     if moe_stream is None:
         launch(torch.cuda.current_stream())      # no stream switch, event or allocator bookkeeping to pay for
