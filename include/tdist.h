@@ -66,8 +66,8 @@ typedef enum tdist_debug_key {
                                       call's row blocks and K admit it */
   TDIST_DEBUG_GEMM_SPLIT_K = 1,    /* 0: whole tiles only; 1: split a last round wherever the workspace allows */
   TDIST_DEBUG_GEMM_SK_COHERENT = 2,/* 1: the split-round exchange always through device-coherent stores */
-  TDIST_DEBUG_GEMM_SCHEDULE = 3,   /* 0: tiles in the static chunk-major order; 1: in arrival order (the default
-                                      for gated calls, see tdist_gemm_chunk_gated_bf16) */
+  TDIST_DEBUG_GEMM_SCHEDULE = 3,   /* 0: every workgroup takes its tiles in the static order; 1: in arrival
+                                      order (the default for gated calls, see tdist_gemm_chunk_gated_bf16) */
   TDIST_DEBUG_DECODE_WAVE_HEADS = 4,      /* 0: never the kv-head-per-wave form; 2: wherever the heads allow it, whatever
                                              the lengths; 4: likewise, its 4-wave workgroups only */
   TDIST_DEBUG_DECODE_SPLITS_PER_TEAM = 5, /* >= 1: splits one workgroup of that form streams through */
@@ -108,15 +108,16 @@ int tdist_debug_get(int key);
  * rows touch (the reference's per-segment wait, kernels/nvidia/allgather_gemm.py:222-224), tiles are visited in row
  * order starting inside the own rank's rows, chunk_order must be NULL and the local shard must either start and end
  * on a multiple of 128 rows or be copied into A with its flags set (A_local = NULL).
- * Tile order. Without a workspace, every workgroup walks a fixed list of tiles in the order above and waits at the
- * flag of each. With sk_workspace, whole-tile chunks (m_per_chunk a multiple of the tile's rows, at most 64 chunks)
- * and more tiles than workgroups, only a workgroup's first tile is fixed: after it, a workgroup draws its next tile
- * from a list kept in the workspace header (one list per XCD, in the order above), puts a tile whose chunk has not
- * arrived aside (at most two) and draws again, and comes back to a tile put aside as soon as its flag is up; only
- * with nothing left to do does it wait, bounded by spin_limit as above. Rows that arrive late or out of order
- * therefore delay only their own tiles. Every tile is computed whole by one workgroup, so C is bit for bit the same
- * in either order and whatever the arrival order is. chunk_order, when given, is the order of the lists. The reference
- * fixes the order by expected arrival instead (:193-206).
+ * Tile order. Every workgroup owns a fixed list of tiles, one per round of the grid, in the order above. With
+ * whole-tile chunks (m_per_chunk a multiple of the tile's rows, at most 64 chunks) and 2 to 64 rounds it takes them in
+ * the order in which their chunks arrive: when it has finished a tile it takes the earliest of its rounds whose
+ * chunk's flag is up, and only with none of them up does it wait, bounded by spin_limit as above; the look at the
+ * flags is taken while the tile before is being stored, so a call whose rows are all there pays nothing for it, and
+ * the rows of a chunk are acquired once per workgroup, not once per tile. Rows that arrive late or out of order
+ * therefore delay only their own tiles. Every tile is computed whole by the workgroup that owns it, so C is bit for
+ * bit the same whatever the arrival order is. Otherwise (a single round, ragged chunks, more chunks or rounds) a
+ * workgroup waits at the flag of each of its tiles in turn. chunk_order, when given, is the order of the rounds.
+ * The reference fixes the order by expected arrival instead (:193-206).
  * ------------------------------------------------------------------------------------------- */
 int tdist_gemm_chunk_gated_bf16(const void* A, int64_t lda, const void* A_local, int64_t lda_local,
                                 int local_row_begin, int local_rows, const void* B, int64_t ldb, void* C,

@@ -86,24 +86,25 @@ struct GemmParams {
   int sk_mode;
   int sk_l2_local;   // 1: workgroup i has been seen to run on XCD i mod num_xcds (tdist_init), so pieces that the
                      // schedule puts on one XCD may exchange through that XCD's L2 alone
-  // Tiles in arrival order (sched_ctrl != NULL; gated calls with whole-tile chunks, at most kSchedMaxChunks of them, and
-  // more than one round of tiles). The static schedule parks a workgroup on the flag of the chunk its position names,
-  // also while rows of other chunks have long arrived, and gives every workgroup a fixed list of tiles whatever
-  // happens (the reference orders its tiles by expected arrival for the same reason,
-  // kernels/amd/all_gather_gemm.py:193-206). Here only the first round is static (workgroup w owns the tile at
-  // position w of the static order). From the second round on, the tiles that the static schedule gives to the
-  // workgroups of one XCD form that XCD's LIST, in the static order, and a workgroup that needs work draws the list's
-  // next tile with one atomic add on the XCD's counter (a workgroup whose own list has run out draws from the other
-  // XCDs' lists), so the workgroups of an XCD still work on neighbouring tiles and share operand panels in that
-  // XCD's L2. A tile whose chunk has not arrived is put aside (two per workgroup at most) and the next one is drawn;
-  // tiles put aside come first again as soon as their flag is up. With nothing to do, the workgroup polls the flags
-  // of what it holds, bounded as the static order's flag wait is. The draw and the look at the flags (wave 0, one
-  // lane per chunk) are issued when the current tile's epilogue begins and used when it ends, so in a call whose rows
-  // are all there the schedule costs no waiting at all. Every tile is computed whole and by one workgroup, so the
-  // result does not depend on who computes it or when.
-  // The counters live in spare words of the workspace header: zero between launches (the last workgroup out clears
-  // them), so launches that share a workspace must be ordered, as for the split rounds.
-  int32_t* sched_ctrl;
+  // Tiles in arrival order (sched_rounds > 0; gated calls with whole-tile chunks, at most kSchedMaxChunks of them, and
+  // 2 .. 64 rounds of tiles). The static schedule parks a workgroup on the flag of the chunk its position names, also
+  // while rows of other chunks have long arrived (the reference orders its tiles by expected arrival for the same
+  // reason, kernels/amd/all_gather_gemm.py:193-206). Here a workgroup keeps the tiles the static schedule gives it
+  // (position w + r G of the static order in round r: the workgroups of an XCD still work on neighbouring tiles and
+  // share operand panels in that XCD's L2) but takes them in the order in which their chunks arrive: when it has
+  // finished a tile it takes the earliest round whose chunk has arrived; only with none of its tiles ready does it
+  // wait, polling the flags, bounded as the static order's flag wait is. The look at the flags (wave 0, one lane per
+  // chunk) is issued when the current tile's epilogue begins and used when it ends, so in a call whose rows are all
+  // there the schedule costs no waiting at all (the static order pays a trip to memory for the flag of every tile).
+  // Every tile is computed whole and by the workgroup the static schedule names, so neither the result nor the
+  // balance of the work depends on the arrival order; nothing is shared between workgroups and no workspace is used.
+  // (An earlier form let the workgroups of an XCD draw tiles from a common list with an atomic add per tile: with 32
+  // workgroups drawing at the same moment the draws queued up behind each other for 2-5 us per tile.)
+  int sched_rounds;
+  // (host-side constants of that schedule, so that the kernel divides by multiplying: ceil(2^32 / d) for d = tiles
+  // per chunk and d = world_size; the host takes the schedule only while positions x d stay below 2^31, where the
+  // product's high word is the quotient)
+  uint32_t sched_tpc_magic, sched_ws_magic;
 };
 
 // Workspace header, in int32 words
@@ -114,13 +115,8 @@ constexpr int kSkFlagsOff = 1024;        // [kSkMaxWorkgroups] tag of the partia
 constexpr int kSkAcksOff = 2048;         // [kSkMaxWorkgroups] readers that are done with the slot, ever
 constexpr int kSkHeaderWords = 3072;
 constexpr int64_t kSkHeaderBytes = (int64_t)kSkHeaderWords * 4;
-// words [kSchedOff, kSkFlagsOff) of the header: the arrival-order schedule's done counter and, a cache line apart,
-// one draw counter per XCD
-constexpr int kSchedOff = 16, kSchedDone = 0, kSchedCounters = 16, kSchedCounterStride = 16;
 constexpr int kSchedMaxChunks = 64;      // one lane of the deciding wave per chunk
-constexpr int kSchedMaxXcds = 8;
-constexpr int kSchedAside = 2;           // tiles a workgroup may put aside
-static_assert(kSchedOff + kSchedCounters + kSchedMaxXcds * kSchedCounterStride <= 1024, "draw counters within the header's spare words");
+constexpr int kSchedMaxRounds = 64;      // and per round of this workgroup's tiles
 constexpr int kSkTagStride = 16;         // tags per launch (rounds that may be split)
 // a flag word is the tag (low 27 bits) with the XCD the piece ran on above it
 constexpr int kSkTagBits = 27, kSkTagMask = (1 << kSkTagBits) - 1, kSkTagWrap = kSkTagMask - 0x10000;
@@ -442,152 +438,101 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   int sk_split = 1;
   if (p.sk_mode == 1 && sk_tail_tiles > 0) sk_split = sk_split_for(G, sk_tail_tiles, KT);
 
-  // ---- tiles in arrival order (see GemmParams::sched_ctrl); everything here is wave 0's, one lane per chunk ----------
-  const bool arrival = !kGrouped && !kPlain && p.sched_ctrl != nullptr;
-  // (small functions of the launch, recomputed where they are needed rather than held in scalar registers across the
-  // K loop, whose wave has no second wave to hide a reload behind)
-  auto arr_nx_f = [&]() { return (p.num_xcds > 1 && p.num_xcds <= kSchedMaxXcds && G % p.num_xcds == 0) ? p.num_xcds : 1; };
-  bool arr_first = true, arr_decided = false;
-  // The schedule's state lives in ONE vector register, a word per lane (wave 0's copy is the one that counts), and is
-  // read and written with v_readlane / v_writelane where a tile is chosen: positions in the static order of the tile
-  // drawn but not yet begun (kArrHeld; -1 = none, kArrNone once every list has run out) and of the tiles put aside
-  // (-1 = none), the XCDs whose lists this workgroup has found empty (a bit each), and the looks a wait may take (1
-  // once any wait of the launch has expired).
-  constexpr int kArrNone = -2;
-  enum { kArrHeld = 0, kArrAside0 = 1, kArrDead = 1 + kSchedAside, kArrLimit = 2 + kSchedAside };
-  int arr_v = -1;
+  // ---- tiles in arrival order (see GemmParams::sched_rounds); everything here is wave 0's ------------------------------
+  const bool arrival = !kGrouped && !kPlain && p.sched_rounds > 0;
+  bool arr_decided = false;
+  // The schedule's state lives in ONE vector register, a word per lane (wave 0's copy), read and written with
+  // v_readlane / v_writelane where a tile is chosen, so that nothing of it is held in scalar registers across the K
+  // loop: the rounds of this workgroup that are done with (taken or given up; 64 bits in two lanes), the looks a wait
+  // may take (1 once any wait of the launch has expired) and the chunks whose rows this workgroup has acquired.
+  enum { kArrDoneLo = 0, kArrDoneHi = 1, kArrLimit = 2, kArrSeenLo = 3, kArrSeenHi = 4 };
+  int arr_v = 0;
   asm volatile("" : "+v"(arr_v));
   auto arr_get = [&](int i) { return __builtin_amdgcn_readlane(arr_v, i); };
   // (the lane is an immediate: a second scalar operand would be one too many for the instruction)
 #define TDIST_ARR_SET(LANE, VAL) \
   asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(arr_v) : "s"(__builtin_amdgcn_readfirstlane(VAL)), "n"(LANE))
-  if (arrival) {
-    TDIST_ARR_SET(kArrDead, 0);
-    TDIST_ARR_SET(kArrLimit, p.spin_limit);
-  }
-  // draw t of XCD x's list → position in the static order (rounds from the second on), or -1 behind the list's end
-  auto arr_position = [&](int x, int t) {
-    const int gx = G / arr_nx_f();               // workgroups per XCD = tiles of a round in one XCD's list
-    const int sidx = (1 + t / gx) * G + x * gx + t % gx;
-    return t >= 0 && sidx < total_sched ? sidx : -1;
+  if (arrival) TDIST_ARR_SET(kArrLimit, p.spin_limit);
+  // chunk of the tile at position sidx of the static order (chunk_of with its divisions as multiplications)
+  auto arr_chunk_at = [&](int sidx) {
+    const int oc = (int)__umulhi((uint32_t)sidx, p.sched_tpc_magic);
+    if (p.order_mode == 1) {
+      const int sweep = (int)__umulhi((uint32_t)oc, p.sched_ws_magic);
+      int r = oc - sweep * p.world_size + p.rank;
+      r -= r >= p.world_size ? p.world_size : 0;
+      return r * p.chunks_per_rank + sweep;
+    }
+    return chunk_of(p, oc);
   };
-  auto arr_chunk_at = [&](int sidx) { return chunk_of(p, sidx / tiles_per_chunk); };
   auto arr_is_local = [&](int ch) {
     const int cm0 = ch * p.m_per_chunk;
     return p.A_local != nullptr && cm0 >= p.local_row_begin && cm0 < p.local_row_begin + p.local_rows;
   };
-  // One look: lane c loads chunk c's flag (system scope), lane x the draw counter of XCD x (device scope). Two
-  // independent loads with nothing branching around them: they go out at once and are waited for at their first use.
-  auto arr_look = [&](int& flag, int& cnt) {
+  // One look: lane c loads chunk c's flag (system scope); issued at once, waited for at its first use.
+  auto arr_look = [&]() {
     int l = lane;
     asm volatile("" : "+v"(l));   // (nothing of this is computed ahead and held across the K loop)
-    flag = __hip_atomic_load(p.flags + min(l, n_chunks - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    cnt = __hip_atomic_load(p.sched_ctrl + kSchedCounters + min(l, arr_nx_f() - 1) * kSchedCounterStride, __ATOMIC_RELAXED,
-                            __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(p.flags + min(l, n_chunks - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   };
-  // the draw: one lane's atomic add on XCD x's counter (the raw counter value, valid in every lane afterwards)
-  auto arr_draw = [&](int x) {
-    int t = 0;
-    if (lane == 0)
-      t = __hip_atomic_fetch_add(p.sched_ctrl + kSchedCounters + x * kSchedCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return t;
-  };
-  // The next tile of this workgroup, given a look (flag, cnt) and, if one was issued with it, a draw from the own
-  // XCD's list (drawn = true, t its raw result in lane 0). Returns the tile's position in the static order, or -1 when
-  // there is nothing left to do.
-  auto arr_next = [&](int flag, int cnt, bool drawn, int t_raw) -> int {
+  // The next tile of this workgroup given a look (lane c: chunk c's flag): its position in the static order with its
+  // chunk in the low six bits, or -1 when there is nothing left to do. Lane r stands for round r of this workgroup.
+  auto arr_next = [&](int flag) -> int {
     int l = lane;
     asm volatile("" : "+v"(l));
-    const int arr_nx = arr_nx_f(), arr_my_x = arr_nx > 1 ? (int)blockIdx.x % arr_nx : 0;
-    int arr_held = arr_get(kArrHeld), arr_dead = arr_get(kArrDead), arr_limit = arr_get(kArrLimit);
-    int arr_aside[kSchedAside];
-#pragma unroll
-    for (int i = 0; i < kSchedAside; ++i) arr_aside[i] = arr_get(kArrAside0 + i);
-    if (drawn) {
-      const int pos = arr_position(arr_my_x, __shfl(t_raw, 0));
-      arr_held = pos >= 0 ? pos : -1;
-      if (pos < 0) arr_dead |= 1 << arr_my_x;
-    }
+    uint64_t done = ((uint64_t)(uint32_t)arr_get(kArrDoneHi) << 32) | (uint32_t)arr_get(kArrDoneLo);
+    uint64_t seen = ((uint64_t)(uint32_t)arr_get(kArrSeenHi) << 32) | (uint32_t)arr_get(kArrSeenLo);
+    int arr_limit = arr_get(kArrLimit);
+    // this lane's round: its position, whether there is a tile there, its chunk
+    const int sidx = l * G + wg_pos;
+    const bool exists = l < p.sched_rounds && sidx < total_sched;
+    const int ch = exists ? arr_chunk_at(sidx) : 0;
+    const bool local = arr_is_local(ch);
     int looks = 0, next = -1;
     for (;;) {
-      // chunk c has arrived (lane c's verdict); the lists that are empty by their counters (counters only grow)
-      const uint64_t arrived = __ballot(l < n_chunks && (flag == p.wait_value || arr_is_local(l)));
-      arr_dead |= (int)__ballot(l < arr_nx && arr_position(l, cnt) < 0);
-      auto ready = [&](int sidx) { return ((arrived >> arr_chunk_at(sidx)) & 1) != 0; };
-      // 1. a tile put aside whose chunk has arrived, the oldest first
-      bool took = false;
-#pragma unroll
-      for (int i = 0; i < kSchedAside; ++i) {
-        if (!took && arr_aside[i] >= 0 && ready(arr_aside[i])) {
-          next = arr_aside[i];
-#pragma unroll
-          for (int j = i; j + 1 < kSchedAside; ++j) arr_aside[j] = arr_aside[j + 1];
-          arr_aside[kSchedAside - 1] = -1;
-          took = true;
+      const uint64_t open = __ballot(exists) & ~done;          // rounds still to be done
+      if (open == 0) break;                                      // nothing left (next = -1)
+      // the chunk of this lane's round has arrived (its flag is lane ch's)
+      const int flag_ch = __shfl(flag, ch);   // (by every lane: a lane that sits out answers nobody)
+      const bool arrived = local || flag_ch == p.wait_value;
+      const uint64_t ready = __ballot(exists && arrived) & open;
+      if (ready != 0) {
+        const int r = __builtin_amdgcn_readfirstlane(__builtin_ctzll(ready));   // the earliest round that can be done
+        done |= 1ull << r;
+        const int c_next = __builtin_amdgcn_readlane(ch, r);
+        next = ((r * G + wg_pos) << 6) | c_next;
+        // Acquire, once per chunk and workgroup at most: an invalidate drops every line the XCD's L2 holds for the
+        // other workgroups too, operand panels included, so it is issued only for a chunk whose rows this workgroup
+        // has not acquired yet, and it then covers every chunk whose flag this look has seen (with all rows there at
+        // the start: once per launch, where the static order invalidates once per tile). The wait behind it also
+        // waits for the last tile's stores, which is why it must be rare.
+        if (!__builtin_amdgcn_readlane((int)local, r) && ((seen >> c_next) & 1) == 0) {
+          seen |= __ballot(l < n_chunks && flag == p.wait_value);
+          asm volatile("buffer_inv sc0 sc1\n\ts_waitcnt vmcnt(0)" ::: "memory");
         }
+        break;
       }
-      if (took) break;
-      // 2. the tile in hand, or a new draw: the own list first, then the other XCDs' while any has tiles left
-      if (arr_held == -1) {
-        for (int dx = 0; dx < arr_nx && arr_held == -1; ++dx) {
-          const int x = (arr_my_x + dx) % arr_nx;
-          if ((arr_dead >> x) & 1) continue;
-          const int pos = arr_position(x, __shfl(arr_draw(x), 0));
-          if (pos >= 0) arr_held = pos;
-          else arr_dead |= 1 << x;
-        }
-        if (arr_held == -1) arr_held = kArrNone;
-      }
-      if (arr_held >= 0) {
-        if (ready(arr_held)) {
-          next = arr_held;
-          arr_held = -1;
-          break;
-        }
-        if (arr_aside[kSchedAside - 1] < 0) {   // room to put it aside: do, and draw again
-#pragma unroll
-          for (int i = 0; i < kSchedAside; ++i) {
-            if (arr_aside[i] < 0) {
-              arr_aside[i] = arr_held;
-              break;
-            }
-          }
-          arr_held = -1;
-          continue;
-        }
-      } else if (arr_aside[0] < 0) {
-        break;   // every list is empty and nothing is put aside: done (next = -1)
-      }
-      // 3. everything this workgroup holds waits for a flag: look again, as the static order's flag wait does (bounded;
-      // once any wait of the launch has expired, one look is all the others get)
+      // every tile left waits for a flag: look again, as the static order's flag wait does (bounded; once any wait of
+      // the launch has expired, one look is all the others get)
       if (looks == 0 && p.status != nullptr && __hip_atomic_load(p.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) arr_limit = 1;
       if (++looks >= arr_limit) {
-        // expired: the oldest tile is given up (skipped, as a tile whose flag wait expires is) and reported
-        const int lost = arr_aside[0] >= 0 ? arr_aside[0] : arr_held;
-        if (arr_aside[0] >= 0) {
-#pragma unroll
-          for (int j = 0; j + 1 < kSchedAside; ++j) arr_aside[j] = arr_aside[j + 1];
-          arr_aside[kSchedAside - 1] = -1;
-        } else {
-          arr_held = -1;
-        }
+        // expired: the earliest round is given up (skipped, as a tile whose flag wait expires is) and reported
+        const int r = __builtin_amdgcn_readfirstlane(__builtin_ctzll(open));
+        done |= 1ull << r;
         if (l == 0 && p.status != nullptr) {
-          if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = arr_chunk_at(lost);
+          if (atomicCAS(p.status, 0, TDIST_ERR_TIMEOUT) == 0) p.status[1] = __builtin_amdgcn_readlane(ch, r);
         }
         arr_limit = 1;
         looks = 0;
         continue;
       }
       __builtin_amdgcn_s_sleep(4);
-      arr_look(flag, cnt);
+      flag = arr_look();
     }
-    TDIST_ARR_SET(kArrHeld, arr_held);
-    TDIST_ARR_SET(kArrDead, arr_dead);
+    TDIST_ARR_SET(kArrDoneLo, (int)(uint32_t)done);
+    TDIST_ARR_SET(kArrDoneHi, (int)(uint32_t)(done >> 32));
     TDIST_ARR_SET(kArrLimit, arr_limit);
-    static_assert(kSchedAside == 2, "one write per tile put aside");
-    TDIST_ARR_SET(kArrAside0, arr_aside[0]);
-    TDIST_ARR_SET(kArrAside0 + 1, arr_aside[1]);
-    if (next >= 0 && !arr_is_local(arr_chunk_at(next))) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    TDIST_ARR_SET(kArrSeenLo, (int)(uint32_t)seen);
+    TDIST_ARR_SET(kArrSeenHi, (int)(uint32_t)(seen >> 32));
     return next;
   };
 
@@ -620,35 +565,18 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     if (arrival) {
       if (!arr_decided && wave == 0) {
         // not decided while the last tile was stored: the first tile, or a position that turned out to hold no tile
-        int next = -1;
-        bool quick = false;
-        if (arr_first && wg_pos < total_sched) {
-          // the first round is static: this workgroup's own tile, which nobody else can take
-          const int ch = arr_chunk_at(wg_pos);
-          if (arr_is_local(ch) || __hip_atomic_load(p.flags + ch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == p.wait_value) {
-            if (!arr_is_local(ch)) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-            next = wg_pos;
-            quick = true;
-          } else {
-            TDIST_ARR_SET(kArrHeld, wg_pos);
-          }
-        }
-        if (!quick) {
-          int flag, cnt;
-          arr_look(flag, cnt);
-          next = arr_next(flag, cnt, false, 0);
-        }
+        const int next = arr_next(arr_look());
         if (lane == 0) s_gate[0] = next;
       }
-      arr_first = false;
       arr_decided = false;
-      __syncthreads();
+      // (barriers that wait for LDS only: the last tile's stores stay in flight)
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       const int next = __builtin_amdgcn_readfirstlane(s_gate[0]);
-      __syncthreads();
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       if (next < 0) break;
-      oc = next / tiles_per_chunk;
-      within = next - oc * tiles_per_chunk;
-      arr_chunk = chunk_of(p, oc);
+      oc = (int)__umulhi((uint32_t)(next >> 6), p.sched_tpc_magic);
+      within = (next >> 6) - oc * tiles_per_chunk;
+      arr_chunk = next & 63;
     } else {
       int sidx;
       if (sbase >= total_sched) break;
@@ -1234,15 +1162,26 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // arrival order: the look for the next tile goes out while this tile is being stored and is used when it has been.
     // Issued behind the epilogue's own loads (the scales), not in front of them: loads retire in order, so the wait
     // for the scales would otherwise be a wait for the draw's round trip as well.
-    int arr_flag = 0, arr_cnt = 0, arr_t = 0;
-    bool arr_drawn = false, arr_issued = false;
-    auto arr_issue = [&]() {
+    int arr_flag = 0;
+    int arr_behind = 0;
+    bool arr_issued = false;
+    // stores_behind: the 16-byte stores this wave still issues behind the look (all of them, or none)
+    auto arr_issue = [&](int stores_behind) {
       if (arrival && wave == 0 && !arr_issued) {
-        arr_look(arr_flag, arr_cnt);
-        // and the draw, unless a tile is in hand already or the own list is known to be empty
-        const int my_x = arr_nx_f() > 1 ? (int)blockIdx.x % arr_nx_f() : 0;
-        arr_drawn = arr_get(kArrHeld) == -1 && ((arr_get(kArrDead) >> my_x) & 1) == 0;
-        if (arr_drawn) arr_t = arr_draw(my_x);
+        if constexpr (kFixedAcc) {
+          // The look lands in an accumulator register of the row block that has just been staged (a0: nothing uses
+          // it before the next tile clears it) and is fetched from there when the tile is chosen, behind a wait that
+          // leaves this wave's stores in flight. Left to the compiler, the wait for a load's result is a wait for
+          // everything the wave has issued, stores included: it does not count on loads and stores retiring in order
+          // through the one counter, as they do here.
+          int l = lane;
+          asm volatile("" : "+v"(l));
+          const uint32_t flag_off = (uint32_t)min(l, n_chunks - 1) * 4u;
+          asm volatile("global_load_dword a0, %0, %1 sc0 sc1" : : "v"(flag_off), "s"(p.flags) : "memory");
+          arr_behind = stores_behind;
+        } else {
+          arr_flag = arr_look();
+        }
       }
       arr_issued = true;
     };
@@ -1561,7 +1500,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         };
         static_for<kGroups>([&](auto g_c) { stage_fast(std::integral_constant<int, 0>{}, g_c); });
         __builtin_amdgcn_sched_barrier(0);
-        arr_issue();
+        arr_issue(kRowBlocks * kPasses);
         __builtin_amdgcn_sched_barrier(0);
         int4v v[kPasses];
         auto read_piece = [&](int i, int u) {
@@ -1648,13 +1587,22 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       store_rows(0, C::kWaveM);
     }
-    arr_issue();   // (the epilogue forms that did not issue the look themselves)
+    arr_issue(0);   // (the epilogue forms that did not issue the look themselves)
     if (arrival) {
       // the next tile, by the look taken while the epilogue ran (wave 0 is done reading its staging rows, which is
       // where the gate words lie)
       if (wave == 0) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const int next = arr_next(arr_flag, arr_cnt, arr_drawn, arr_t);
+        if constexpr (kFixedAcc) {
+          constexpr int kBehind = kRowBlocks * (32 / kRowsPerPass);   // the fast epilogue's stores per wave
+          static_assert(kBehind > 0 && kBehind < 60, "vmcnt is a 6-bit counter");
+          if (arr_behind != 0) {
+            asm volatile("s_waitcnt vmcnt(%1)\n\tv_accvgpr_read_b32 %0, a0" : "=v"(arr_flag) : "n"(kBehind) : "memory");
+          } else {
+            asm volatile("s_waitcnt vmcnt(0)\n\tv_accvgpr_read_b32 %0, a0" : "=v"(arr_flag) : : "memory");
+          }
+        }
+        const int next = arr_next(arr_flag);
         if (lane == 0) s_gate[0] = next;
       }
       arr_decided = true;
@@ -1662,15 +1610,6 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // the next tile's prologue overwrites the ring: every wave must be done reading its staging area
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if constexpr (kEarly) prefetched = early;
-  }
-  // ---- leave: the last workgroup out puts the ticket counters back to zero for the next launch ------------------
-  if (!kGrouped && p.sched_ctrl != nullptr && threadIdx.x == 0) {
-    int32_t* const done = p.sched_ctrl + kSchedDone;
-    if (__hip_atomic_fetch_add(done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == G - 1) {
-      for (int x = 0; x < kSchedMaxXcds; ++x)
-        __hip_atomic_store(p.sched_ctrl + kSchedCounters + x * kSchedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(done, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    }
   }
   // ---- the last workgroup out advances the workspace's tag base for the next launch --------------------------
   if (p.sk_mode != 0 && threadIdx.x == 0) {
@@ -1888,7 +1827,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   p.sk_partials = nullptr;
   p.sk_mode = 0;
   p.sk_l2_local = 0;
-  p.sched_ctrl = nullptr;
+  p.sched_rounds = 0; p.sched_tpc_magic = 0; p.sched_ws_magic = 0;
   p.k_tail_bytes = k_tail_bytes;
 
   if (c.scatter_bufs) {
@@ -1946,11 +1885,17 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   if (use_sk) {
     grid = cap_wgs;
     sk_attach(p, c.sk_workspace, 1);
-  } else if (c.flags && !c.scatter_bufs && !ragged && c.sk_workspace != nullptr && p.n_chunks <= kSchedMaxChunks &&
-             sched > grid && debug_get(TDIST_DEBUG_GEMM_SCHEDULE) != 0) {
-    // gated, whole-tile chunks, more than one round of tiles, a workspace for the ticket counters: tiles in arrival
-    // order (a single round is static either way: every workgroup owns its one tile)
-    p.sched_ctrl = (int32_t*)c.sk_workspace + kSchedOff;
+  } else if (c.flags && !c.scatter_bufs && !ragged && p.n_chunks <= kSchedMaxChunks && sched > grid &&
+             sched <= (int64_t)kSchedMaxRounds * grid && debug_get(TDIST_DEBUG_GEMM_SCHEDULE) != 0) {
+    // gated, whole-tile chunks, 2 .. 64 rounds of tiles: every workgroup takes its tiles in arrival order (a single
+    // round is static either way: every workgroup owns its one tile)
+    const int64_t tpc = (int64_t)(p.m_per_chunk / BM) * ceil_div(c.N, BN);
+    if (sched * tpc < 0x7fffffffll && sched < (1 << 25)) {
+      p.sched_rounds = (int)ceil_div(sched, grid);
+      p.sched_tpc_magic = (uint32_t)(((1ull << 32) + tpc - 1) / tpc);
+      const int64_t wsz = c.world_size > 0 ? c.world_size : 1;
+      p.sched_ws_magic = (uint32_t)(((1ull << 32) + wsz - 1) / wsz);   // (positions of chunks: at most 64)
+    }
   }
   const bool scales = elem == kElemFP8 && (c.row_scale || c.col_scale);
 
@@ -2103,7 +2048,7 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   p.sk_partials = nullptr;
   p.sk_mode = 0;
   p.sk_l2_local = 0;
-  p.sched_ctrl = nullptr;
+  p.sched_rounds = 0; p.sched_tpc_magic = 0; p.sched_ws_magic = 0;
   p.gate_rows = p.m_per_chunk;
   p.k_tail_bytes = 0;
 
