@@ -3,7 +3,7 @@ run. Every constant is tied to the kernel sources it was measured on: this test 
 changed (comments and white space aside) since the counters were last read, so that a stale figure cannot be
 reported as a measurement, and checks that every constant has a summary under profiles/ that holds it."""
 import glob
-import importlib.util
+import types
 import os
 import re
 
@@ -11,9 +11,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def load_bench():
-    spec = importlib.util.spec_from_file_location("bench_under_test", os.path.join(ROOT, "bench.py"))
-    mod = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(mod)
+    # (compiled from the source text: no bytecode cache between the file and the test)
+    path = os.path.join(ROOT, "bench.py")
+    mod = types.ModuleType("bench_under_test")
+    mod.__file__ = path
+    exec(compile(open(path).read(), path, "exec"), mod.__dict__)
     return mod
 
 
