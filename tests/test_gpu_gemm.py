@@ -304,6 +304,43 @@ def test_tiles_in_arrival_order(cuda, switches, schedule, dtype):
         assert torch.equal(out.cpu(), want)
 
 
+@pytest.mark.parametrize("max_workgroups,late", [(48, False), (48, True), (2, False), (2, True)])
+def test_arrival_order_on_a_capped_grid(cuda, max_workgroups, late):
+    """A grid held to a few workgroups: 96 tiles of 256 x 256 are 2 rounds on 48 workgroups (every workgroup takes its
+    tiles in arrival order) and 48 rounds on 2; held to one workgroup they are more rounds than the schedule keeps
+    track of, and the workgroup waits at each tile's flag in turn. With the flags up from the start and with all but
+    the own chunk released late and last chunk first, against the oracle bit for bit."""
+    from triton_dist import _lib
+    from triton_dist.kernels.amd import gated_gemm
+    from triton_dist.kernels.amd.common_ops import set_signal
+    announce("gemm arrival order with %d workgroups, late=%s" % (max_workgroups, late))
+    world, mpc, N, K, rank = 4, 512, 3072, 256, 1
+    M = world * mpc
+    g = torch.Generator().manual_seed(77)
+    a = torch.randint(-2, 3, (M, K), generator=g).float()
+    b = torch.randint(-2, 3, (N, K), generator=g).float()
+    want = golden.ag_gemm_fp32([a], b).to(torch.bfloat16)
+    a_d, b_d = a.to(torch.bfloat16).to(cuda), b.to(torch.bfloat16).to(cuda)
+    for cap in (max_workgroups, 1):
+        flags = torch.ones(world, dtype=torch.int32, device=cuda)
+        c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+        status = torch.zeros(2, dtype=torch.int32, device=cuda)
+        if late:
+            flags.zero_()
+            flags[rank] = 1
+            side = torch.cuda.Stream()
+            stamp = torch.zeros(1, dtype=torch.int64, device=cuda)
+            torch.cuda.synchronize()
+            _lib.call("tdist_producer_mark", stamp.data_ptr(), side.cuda_stream)
+            _lib.call("tdist_producer_wait_until", stamp.data_ptr(), 100000, side.cuda_stream)
+            for chunk in (3, 2, 0):
+                set_signal(flags.data_ptr() + 4 * chunk, 1, side)
+        gated_gemm(a_d, None, 0, b_d, c, flags, mpc, rank, world, status=status, max_workgroups=cap)
+        torch.cuda.synchronize()
+        assert status.tolist() == [0, 0], cap
+        assert torch.equal(c.cpu(), want), cap
+
+
 def test_gemm_rs_small_and_owner_mapping(cuda):
     from triton_dist.kernels.amd import create_gemm_rs_intra_node_context, gemm_rs_intra_node
     announce("gemm_rs small")
