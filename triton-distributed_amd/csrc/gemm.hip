@@ -105,6 +105,12 @@ struct GemmParams {
   // per chunk and d = world_size; the host takes the schedule only while positions x d stay below 2^31, where the
   // product's high word is the quotient)
   uint32_t sched_tpc_magic, sched_ws_magic;
+  // Chunks of few row tiles (1, 2 or 4) are scheduled group_s at a time (a power of two; 1: chunk by chunk): the
+  // positions of a group run down the rows of all its chunks before they move on to the next column of tiles, so that
+  // the block of tiles an XCD's workgroups work on is 8 rows x 4 columns (or 4 x 8) instead of 2 x 16 or 1 x 32, and
+  // fetches 12 operand panels instead of 18 or 33 (16384 x 7168 x 8192 e4m3 in chunks of 512 rows: 615 -> 597 us).
+  // Every tile is still gated by the flag of its own chunk. The sched_tpc_magic is then that of a group's tiles.
+  int group_s, group_rows_shift, cm_shift;
 };
 
 // Workspace header, in int32 words
@@ -454,8 +460,23 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
   asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(arr_v) : "s"(__builtin_amdgcn_readfirstlane(VAL)), "n"(LANE))
   if (arrival) TDIST_ARR_SET(kArrLimit, p.spin_limit);
   // chunk of the tile at position sidx of the static order (chunk_of with its divisions as multiplications)
+  // position sidx of the static order -> the chunk's place in the chunk order and the tile within the chunk (column *
+  // cm + row), with the divisions as multiplications and shifts (see GemmParams::group_s)
+  auto arr_locate = [&](int sidx, int& oc, int& within) {
+    const int og = (int)__umulhi((uint32_t)sidx, p.sched_tpc_magic);
+    const int win = sidx - og * (p.group_s * tiles_per_chunk);
+    if (p.group_s > 1) {
+      const int pn = win >> p.group_rows_shift, j = win & ((1 << p.group_rows_shift) - 1);
+      oc = og * p.group_s + (j >> p.cm_shift);
+      within = pn * cm + (j & (cm - 1));
+    } else {
+      oc = og;
+      within = win;
+    }
+  };
   auto arr_chunk_at = [&](int sidx) {
-    const int oc = (int)__umulhi((uint32_t)sidx, p.sched_tpc_magic);
+    int oc, within_unused;
+    arr_locate(sidx, oc, within_unused);
     if (p.order_mode == 1) {
       const int sweep = (int)__umulhi((uint32_t)oc, p.sched_ws_magic);
       int r = oc - sweep * p.world_size + p.rank;
@@ -574,8 +595,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
       const int next = __builtin_amdgcn_readfirstlane(s_gate[0]);
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       if (next < 0) break;
-      oc = (int)__umulhi((uint32_t)(next >> 6), p.sched_tpc_magic);
-      within = (next >> 6) - oc * tiles_per_chunk;
+      arr_locate(next >> 6, oc, within);
       arr_chunk = next & 63;
     } else {
       int sidx;
@@ -596,8 +616,16 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         sidx = round_base + wg_pos;
         if (sidx >= total_sched) continue;
       }
-      oc = sidx / tiles_per_chunk;
-      within = sidx - oc * tiles_per_chunk;
+      if (!kGrouped && p.group_s > 1) {
+        const int rows_g = p.group_s * cm, tpg = rows_g * num_pid_n;
+        const int og = sidx / tpg, win = sidx - og * tpg;
+        const int pn = win >> p.group_rows_shift, j = win & (rows_g - 1);
+        oc = og * p.group_s + (j >> p.cm_shift);
+        within = pn * cm + (j & (cm - 1));
+      } else {
+        oc = sidx / tiles_per_chunk;
+        within = sidx - oc * tiles_per_chunk;
+      }
     }
     const int KTp = kb - ka;
     const int chunk = kGrouped ? (oc + p.first_block) % n_chunks : arr_chunk >= 0 ? arr_chunk : chunk_of(p, oc);
@@ -1828,6 +1856,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   p.sk_mode = 0;
   p.sk_l2_local = 0;
   p.sched_rounds = 0; p.sched_tpc_magic = 0; p.sched_ws_magic = 0;
+  p.group_s = 1; p.group_rows_shift = 0; p.cm_shift = 0;
   p.k_tail_bytes = k_tail_bytes;
 
   if (c.scatter_bufs) {
@@ -1870,6 +1899,23 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
     } else {
       p.order_mode = 0;
     }
+    // chunks of 1, 2 or 4 row tiles: scheduled several at a time, so that an XCD's block of tiles is 8 (or 4) rows
+    // high (see GemmParams::group_s); the chunks of a group are neighbours in the expected order of arrival
+    const int cmh = c.m_per_chunk / BM;
+    if (cmh == 1 || cmh == 2 || cmh == 4) {
+      const int per_xcd = di.num_xcds > 0 && cap_wgs % di.num_xcds == 0 ? cap_wgs / di.num_xcds : cap_wgs;
+      const int tiles_n = (int)ceil_div(c.N, BN);
+      const bool fits8 = per_xcd % 8 == 0 && tiles_n % (per_xcd / 8) == 0;
+      const bool fits4 = per_xcd % 4 == 0 && tiles_n % (per_xcd / 4) == 0;
+      int gs = (fits8 || !fits4 ? 8 : 4) / cmh;
+      while (gs > 1 && (p.n_chunks % gs != 0 || (p.order_mode == 1 && c.world_size % gs != 0))) gs /= 2;
+      if (gs > 1) {
+        auto log2i = [](int v) { int n = 0; while ((1 << n) < v) ++n; return n; };
+        p.group_s = gs;
+        p.cm_shift = log2i(cmh);
+        p.group_rows_shift = log2i(gs * cmh);
+      }
+    }
   } else {
     // plain GEMM: schedule in groups of 4 row tiles
     // Row tiles per group: an XCD's workgroups (one in num_xcds of the grid) work on a block of `rows` x `cols` tiles
@@ -1908,7 +1954,7 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
              sched <= (int64_t)kSchedMaxRounds * grid && debug_get(TDIST_DEBUG_GEMM_SCHEDULE) != 0) {
     // gated, whole-tile chunks, 2 .. 64 rounds of tiles: every workgroup takes its tiles in arrival order (a single
     // round is static either way: every workgroup owns its one tile)
-    const int64_t tpc = (int64_t)(p.m_per_chunk / BM) * ceil_div(c.N, BN);
+    const int64_t tpc = (int64_t)p.group_s * (p.m_per_chunk / BM) * ceil_div(c.N, BN);   // tiles of a group of chunks
     if (sched * tpc < 0x7fffffffll && sched < (1 << 25)) {
       p.sched_rounds = (int)ceil_div(sched, grid);
       p.sched_tpc_magic = (uint32_t)(((1ull << 32) + tpc - 1) / tpc);
@@ -2068,6 +2114,7 @@ static int run_group_gemm(const GroupGemmCall& c, GemmElem elem) {
   p.sk_mode = 0;
   p.sk_l2_local = 0;
   p.sched_rounds = 0; p.sched_tpc_magic = 0; p.sched_ws_magic = 0;
+  p.group_s = 1; p.group_rows_shift = 0; p.cm_shift = 0;
   p.gate_rows = p.m_per_chunk;
   p.k_tail_bytes = 0;
 
