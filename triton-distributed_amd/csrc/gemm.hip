@@ -1189,7 +1189,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     }
     // arrival order: the look for the next tile goes out while this tile is being stored and is used when it has been.
     // Issued behind the epilogue's own loads (the scales), not in front of them: loads retire in order, so the wait
-    // for the scales would otherwise be a wait for the draw's round trip as well.
+    // for the scales would otherwise be a wait for the look's round trip as well.
     int arr_flag = 0;
     int arr_behind = 0;
     bool arr_issued = false;
@@ -1820,6 +1820,17 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
   }
   const int BM = kChoices[pick].bm;
   const int BN = kChoices[pick].bn;
+  // An XCD's workgroups (one in num_xcds of the grid) work on a block of rows x cols tiles at a time and fetch the
+  // operand rows of rows + cols panels for it: the bytes of such a block per tile, a little more where a side does not
+  // divide the tile count (the blocks then wrap around the matrix's edge and their panels are shared by fewer tiles);
+  // 0 if the XCD's workgroups do not make whole rows.
+  auto xcd_block_cost = [&](int rows) -> double {
+    const int per_xcd = di.num_xcds > 0 && cap_wgs % di.num_xcds == 0 ? cap_wgs / di.num_xcds : cap_wgs;
+    if (rows <= 0 || per_xcd % rows != 0) return 0;
+    const int cols = per_xcd / rows;
+    const int tiles_m = (int)ceil_div(c.M, BM), tiles_n = (int)ceil_div(c.N, BN);
+    return ((double)rows * BM + (double)cols * BN) * (1.0 + (tiles_n % cols != 0 ? 0.125 : 0.0) + (tiles_m % rows != 0 ? 0.125 : 0.0));
+  };
 
   GemmParams p;
   p.A = (const unsigned char*)c.A;
@@ -1903,12 +1914,16 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
     // high (see GemmParams::group_s); the chunks of a group are neighbours in the expected order of arrival
     const int cmh = c.m_per_chunk / BM;
     if (cmh == 1 || cmh == 2 || cmh == 4) {
-      const int per_xcd = di.num_xcds > 0 && cap_wgs % di.num_xcds == 0 ? cap_wgs / di.num_xcds : cap_wgs;
-      const int tiles_n = (int)ceil_div(c.N, BN);
-      const bool fits8 = per_xcd % 8 == 0 && tiles_n % (per_xcd / 8) == 0;
-      const bool fits4 = per_xcd % 4 == 0 && tiles_n % (per_xcd / 4) == 0;
-      int gs = (fits8 || !fits4 ? 8 : 4) / cmh;
-      while (gs > 1 && (p.n_chunks % gs != 0 || (p.order_mode == 1 && c.world_size % gs != 0))) gs /= 2;
+      int gs = 1;
+      double best = 0;
+      for (int cand = 1; cand * cmh <= 16; cand *= 2) {
+        if (p.n_chunks % cand != 0 || (cand > 1 && p.order_mode == 1 && c.world_size % cand != 0)) continue;
+        const double cost = xcd_block_cost(cand * cmh);
+        if (cost > 0 && (best == 0 || cost < best)) {
+          best = cost;
+          gs = cand;
+        }
+      }
       if (gs > 1) {
         auto log2i = [](int v) { int n = 0; while ((1 << n) < v) ++n; return n; };
         p.group_s = gs;
@@ -1917,21 +1932,14 @@ static int run_gemm(const GemmCall& c, GemmElem elem) {
       }
     }
   } else {
-    // plain GEMM: schedule in groups of 4 row tiles
-    // Row tiles per group: an XCD's workgroups (one in num_xcds of the grid) work on a block of `rows` x `cols` tiles
-    // at a time and fetch rows + cols operand panels for it, so the block should be near square, and its sides should
-    // divide the tile counts, or the blocks wrap around the matrix's edge and the panels are shared by fewer tiles
-    // (16384 x 7168 x 8192 e4m3, 28 column tiles, constant operands: 472 us in blocks of 4 x 8, 455 in blocks of 8 x 4).
+    // ungated GEMM: scheduled in groups of row tiles, of the size that gives an XCD's block of tiles its best shape
+    // (16384 x 7168 x 8192 e4m3, 28 column tiles, constant operands: 472 us in blocks of 4 x 8, 455 in blocks of 8 x 4)
     int rows_per_group = 4;
     {
-      const int per_xcd = di.num_xcds > 0 && cap_wgs % di.num_xcds == 0 ? cap_wgs / di.num_xcds : cap_wgs;
-      const int tiles_m = (int)ceil_div(c.M, BM), tiles_n = (int)ceil_div(c.N, BN);
-      int best = 1 << 30;
+      double best = 0;
       for (int rows : {4, 8, 2, 16}) {
-        if (per_xcd % rows != 0) continue;
-        const int cols = per_xcd / rows;
-        const int cost = rows + cols + (tiles_n % cols != 0 ? 4 : 0) + (tiles_m % rows != 0 ? 4 : 0);
-        if (cost < best) {
+        const double cost = xcd_block_cost(rows);
+        if (cost > 0 && (best == 0 || cost < best)) {
           best = cost;
           rows_per_group = rows;
         }
