@@ -42,7 +42,7 @@ MEASURED_TRAFFIC_BYTES = {
 MEASURED_SOURCE_DIGEST = {
     "common.h": "29a71d5d51010d68",
     "decode.hip": "5f8c13ce9a3fc0d7",
-    "gemm.hip": "67362246a78561b8",
+    "gemm.hip": "5b1de058c7b76344",
     "moe.hip": "3ab3dfd4ffc67cea",
     "reduce.hip": "469689d34df1b205",
 }

@@ -854,7 +854,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
     // accumulators: fixed registers a[0 .. kAccRegs) for the 16-row MFMA blocks, else the compiler's
     typename E::acc_t acc[kFixedAcc ? 1 : C::kTN][kFixedAcc ? 1 : C::kTM];
     if constexpr (kFixedAcc) {
-      acc_clear<kAccRegs>();
+      // (the split ring's K loops clear them behind the first loads' issue: 256 register writes that the loads' round
+      // trip hides there)
+      if constexpr (!(C::kSplit && E::kRows == 16)) acc_clear<kAccRegs>();
     } else {
 #pragma unroll
       for (int j = 0; j < C::kTN; ++j)
@@ -903,6 +905,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         // A(0), B(0) and B(1) went out before the last tile's epilogue; its stores are allowed to be still on their way
 #pragma unroll
         for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+        acc_clear<kAccRegs>();
         wait_tiles_and_barrier<kEarly ? C::kBInstr + kEpiStores + C::kAInstr : 0>();
       } else {
 #pragma unroll
@@ -913,6 +916,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
 #pragma unroll
         for (int q = 0; q < kProDma; ++q) issue_list(-1, q);
+        acc_clear<kAccRegs>();
         wait_tiles_and_barrier<C::kAInstr + kProDma>();
       }
 #pragma unroll
@@ -992,6 +996,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         // A(0), B(0) and B(1) went out before the last tile's epilogue; its stores are allowed to be still on their way
 #pragma unroll
         for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
+        acc_clear<kAccRegs>();
         wait_tiles_and_barrier<kEarly ? C::kBInstr + kEpiStores + C::kAInstr : 0>();
       } else {
 #pragma unroll
@@ -1002,6 +1007,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
         for (int t = 0; t < C::kAInstr; ++t) issue_a(1, t);
 #pragma unroll
         for (int q = 0; q < C::kDmaPerStep; ++q) issue_list(-1, q);
+        acc_clear<kAccRegs>();
         wait_tiles_and_barrier<C::kAInstr + C::kDmaPerStep>();
       }
       load_frags(0, 0, a_cur, b_cur);
@@ -1201,11 +1207,13 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(const GemmParams 
           // it before the next tile clears it) and is fetched from there when the tile is chosen, behind a wait that
           // leaves this wave's stores in flight. Left to the compiler, the wait for a load's result is a wait for
           // everything the wave has issued, stores included: it does not count on loads and stores retiring in order
-          // through the one counter, as they do here.
+          // through the one counter, as they do here. The register is first set to a value that is no chunk's
+          // go-ahead: should the wait ever let go with the load still out, the choice sees "not arrived" and polls.
           int l = lane;
           asm volatile("" : "+v"(l));
           const uint32_t flag_off = (uint32_t)min(l, n_chunks - 1) * 4u;
-          asm volatile("global_load_dword a0, %0, %1 sc0 sc1" : : "v"(flag_off), "s"(p.flags) : "memory");
+          const int not_yet = p.wait_value ^ 0x40000000;
+          asm volatile("v_accvgpr_write_b32 a0, %2\n\tglobal_load_dword a0, %0, %1 sc0 sc1" : : "v"(flag_off), "s"(p.flags), "v"(not_yet) : "memory");
           arr_behind = stores_behind;
         } else {
           arr_flag = arr_look();
