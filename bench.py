@@ -41,7 +41,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 MEASURED_SOURCE_DIGEST = {
     "common.h": "29a71d5d51010d68",
-    "decode.hip": "5f8c13ce9a3fc0d7",
+    "decode.hip": "5f65cc9c7465e64c",
     "gemm.hip": "5b1de058c7b76344",
     "moe.hip": "3ab3dfd4ffc67cea",
     "reduce.hip": "469689d34df1b205",

@@ -417,13 +417,13 @@ def test_head_dimensions_that_are_no_power_of_two(cuda, D, num_heads, kv_lens, S
 @pytest.mark.parametrize("kv_lens,S,block_size", [([1320, 18, 463], 4, 16), ([1, 54, 293, 70], 8, 1), ([777, 0, 5, 2047], 3, 16),
                                                   ([100, 31], 1, 16)])
 @pytest.mark.parametrize("dtype,soft_cap", [(torch.bfloat16, 0), (torch.float16, 30)])
-@pytest.mark.parametrize("splits_per_team", [1, 3])
+@pytest.mark.parametrize("splits_per_team", [1, 3, 4])
 def test_a_kv_head_per_wave(cuda, switches, D, num_heads, force, kv_lens, S, block_size, dtype, soft_cap, splits_per_team):
     """The form in which every wave of a workgroup takes a kv head of its own (chosen by itself only for grids that
     fill the chip; forced here on small cases): per-split partials and LSE against the oracle, the one-launch form bit
     for bit against split + combine with the counters back at zero, and both within the oracle's bar of the other
     form's results. A workgroup of this form streams through several consecutive splits of its sequence (as many as
-    fill the chip best; forced here too): splits_per_team = 3 leaves a last workgroup with fewer, and empty splits
+    fill the chip best; forced here too, 4 being the most any instance takes): splits_per_team = 3 leaves a last workgroup with fewer, and empty splits
     inside a workgroup's range."""
     from triton_dist.kernels.amd.flash_decode import _split_kv, decode_combine, decode_fused
     from triton_dist import _lib

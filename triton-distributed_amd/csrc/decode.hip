@@ -100,8 +100,9 @@ struct MmaF16 {
   }
 };
 
-// kWaveHeads: splits one workgroup may stream through (the results of all but the last wait in registers: D / 4 each)
-constexpr int decode_max_splits_per_team(int d) { return d <= 64 ? 4 : d <= 128 ? 3 : 2; }
+// kWaveHeads: splits one workgroup may stream through (the results of all but the last wait in registers: D / 4 each).
+// `heavy`: the instances that already fill their registers (soft cap, fused merge, padded rows).
+constexpr int decode_max_splits_per_team(int d, bool heavy) { return d <= 64 ? 4 : d <= 128 ? (heavy ? 3 : 4) : 2; }
 constexpr int kTableSlots = 8;  // ring of page-table rows per wave (>= 2P+2)
 
 // what the DMA lanes of a padded head dimension read for the dimensions that do not exist
@@ -510,7 +511,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeParams& prm) {
       }
     }
     // results of the splits before the team's last one, held until the stream ends
-    constexpr int kMaxHeld = decode_max_splits_per_team(D) - 1;
+    constexpr int kMaxHeld = decode_max_splits_per_team(D, kSoftCap || kFuse || kPadded) - 1;
     float4v held[kMaxHeld][D / 16];
     float held_lse[kMaxHeld];
 #pragma unroll
@@ -1007,7 +1008,7 @@ static int run_decode(const DecodeCall& c, bool fuse) {
     const int cus = device_info().num_cus > 0 ? device_info().num_cus : 256;
     int64_t best_cost = 0;
     int best_w = 1;
-    const int max_w = std::min(c.num_splits, decode_max_splits_per_team(dv));
+    const int max_w = std::min(c.num_splits, decode_max_splits_per_team(dv, c.soft_cap > 0.f || fuse || padded));
     for (int w = 1; w <= max_w; ++w) {
       const int64_t teams = heads_seqs * ((c.num_splits + w - 1) / w);
       const int64_t cost = ((teams + cus - 1) / cus) * w;
